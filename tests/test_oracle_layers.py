@@ -1,0 +1,325 @@
+"""Pins the CPU oracle (oracle/oracle.c) against independent statements of the same
+mathematics: brute-force loops, fp64 numpy/scipy/torch-CPU library routines and closed
+forms.  None of these reuse the oracle's own formulas."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+TOL = 2e-5
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def tf_geometry(n, k, s, padding):
+    """TensorFlow's documented rule, written independently of the reference's code path."""
+    if padding == "same":
+        out = -(-n // s)
+        total = max((out - 1) * s + k - n, 0)
+        return out, total // 2, total - total // 2
+    return (n - k) // s + 1 if n >= k else 0, 0, 0
+
+
+@pytest.mark.parametrize("padding", ["same", "valid"])
+def test_window_geometry_table(oracle, padding):
+    for n, k, s in itertools.product(range(1, 12), range(1, 6), range(1, 4)):
+        if padding == "valid" and n < k:
+            continue
+        g = oracle.window_geometry(n, n + 1, k, k, s, s, padding)
+        out, before, after = tf_geometry(n, k, s, padding)
+        assert (g["out_h"], g["pad_top"], g["pad_bottom"]) == (out, before, after), (n, k, s)
+        out, before, after = tf_geometry(n + 1, k, s, padding)
+        assert (g["out_w"], g["pad_left"], g["pad_right"]) == (out, before, after), (n, k, s)
+
+
+def test_window_geometry_causal(oracle):
+    g = oracle.window_geometry(7, 9, 3, 5, 1, 1, "causal")
+    assert (g["pad_top"], g["pad_bottom"], g["pad_left"], g["pad_right"]) == (2, 0, 4, 0)
+    assert (g["out_h"], g["out_w"]) == (7, 9)
+
+
+def torch_conv(x, w_oihw, b, strides, dilation, padding, groups=1):
+    import torch
+    import torch.nn.functional as F
+    h, w = x.shape[:2]
+    kh, kw = w_oihw.shape[2:]
+    ek = ((kh - 1) * dilation[0] + 1, (kw - 1) * dilation[1] + 1)
+    pads = []
+    for n, k, s in ((w, ek[1], strides[1]), (h, ek[0], strides[0])):
+        _, before, after = tf_geometry(n, k, s, padding)
+        pads += [before, after]
+    xt = torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None]
+    xt = F.pad(xt, pads)
+    y = F.conv2d(xt, torch.from_numpy(w_oihw.astype(np.float64)),
+                 None if b is None else torch.from_numpy(b.astype(np.float64)),
+                 stride=strides, dilation=dilation, groups=groups)
+    return y[0].permute(1, 2, 0).numpy()
+
+
+CONV_CASES = [
+    # h, w, cin, cout, kh, kw, strides, dilation, padding
+    (8, 9, 3, 5, 3, 3, (1, 1), (1, 1), "same"),
+    (8, 9, 3, 5, 3, 3, (1, 1), (1, 1), "valid"),
+    (11, 10, 4, 6, 3, 2, (2, 2), (1, 1), "same"),
+    (11, 10, 4, 6, 3, 2, (2, 3), (1, 1), "valid"),
+    (12, 12, 2, 3, 3, 3, (1, 1), (2, 2), "same"),
+    (12, 13, 2, 3, 2, 3, (1, 1), (2, 3), "valid"),
+    (9, 9, 8, 4, 1, 1, (1, 1), (1, 1), "valid"),
+    (9, 9, 8, 4, 1, 1, (2, 2), (1, 1), "same"),
+    (15, 15, 3, 8, 7, 7, (2, 2), (1, 1), "valid"),
+    (6, 7, 5, 7, 5, 5, (1, 1), (1, 1), "same"),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_vs_torch_fp64(oracle, case):
+    h, w, cin, cout, kh, kw, strides, dilation, padding = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = rng.standard_normal((h, w, cin)).astype(np.float32)
+    wj = rng.standard_normal((cout, kh, kw, cin)).astype(np.float32)  # converted-JSON order
+    b = rng.standard_normal(cout).astype(np.float32)
+    got = oracle.conv2d(x, oracle.conv2d_prepare(wj, cout, kh, kw, cin), b, cout, kh, kw, strides, dilation, padding)
+    want = torch_conv(x, wj.transpose(0, 3, 1, 2), b, strides, dilation, padding)
+    assert got.shape == want.shape
+    assert rel(got, want) < TOL
+
+
+def test_conv2d_brute_force(oracle):
+    rng = np.random.default_rng(3)
+    h, w, cin, cout, k = 5, 6, 2, 3, 3
+    x = rng.standard_normal((h, w, cin)).astype(np.float32)
+    wj = rng.standard_normal((cout, k, k, cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    got = oracle.conv2d(x, oracle.conv2d_prepare(wj, cout, k, k, cin), b, cout, k, k, (1, 1), (1, 1), "valid")
+    want = np.zeros((h - 2, w - 2, cout))
+    for y, xx, n, fy, fx, c in itertools.product(range(h - 2), range(w - 2), range(cout), range(k), range(k), range(cin)):
+        want[y, xx, n] += float(wj[n, fy, fx, c]) * float(x[y + fy, xx + fx, c])
+    want += b
+    assert rel(got, want) < TOL
+
+
+def test_conv2d_closed_forms(oracle):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((6, 7, 4)).astype(np.float32)
+    # 1x1 conv == matmul over channels
+    wj = rng.standard_normal((5, 1, 1, 4)).astype(np.float32)
+    got = oracle.conv2d(x, oracle.conv2d_prepare(wj, 5, 1, 1, 4), None, 5, 1, 1)
+    assert rel(got, x.astype(np.float64) @ wj.reshape(5, 4).T.astype(np.float64)) < TOL
+    # all-ones 3x3 kernel on one channel == box sum; same padding keeps size
+    x1 = x[:, :, :1]
+    got = oracle.conv2d(x1, np.ones(9, np.float32), None, 1, 3, 3, padding="same")
+    padded = np.pad(x1[:, :, 0].astype(np.float64), 1)
+    want = sum(padded[i:i + 6, j:j + 7] for i in range(3) for j in range(3))
+    assert rel(got[:, :, 0], want) < TOL
+    # delta kernel at (0, 2) == shift (cross-correlation, no flip)
+    delta = np.zeros((1, 3, 3, 1), np.float32)
+    delta[0, 0, 2, 0] = 1
+    got = oracle.conv2d(x1, oracle.conv2d_prepare(delta, 1, 3, 3, 1), None, 1, 3, 3, padding="valid")
+    assert np.array_equal(got[:, :, 0], x1[0:4, 2:7, 0])
+
+
+@pytest.mark.parametrize("case", [
+    (9, 8, 6, 3, 3, (1, 1), (1, 1), "same"), (9, 8, 6, 3, 3, (2, 2), (1, 1), "same"),
+    (10, 11, 5, 3, 3, (2, 2), (1, 1), "valid"), (12, 12, 4, 3, 3, (1, 1), (2, 2), "same"),
+    (7, 7, 3, 5, 2, (1, 2), (1, 1), "valid")])
+def test_depthwise_vs_torch_fp64(oracle, case):
+    h, w, c, kh, kw, strides, dilation, padding = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = rng.standard_normal((h, w, c)).astype(np.float32)
+    wj = rng.standard_normal((c, kh, kw)).astype(np.float32)
+    b = rng.standard_normal(c).astype(np.float32)
+    got = oracle.depthwise_conv2d(x, wj, b, kh, kw, strides, dilation, padding)
+    want = torch_conv(x, wj[:, None], b, strides, dilation, padding, groups=c)
+    assert got.shape == want.shape
+    assert rel(got, want) < TOL
+
+
+def test_dense_any_rank(oracle):
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((7, 4)).astype(np.float32)
+    b = rng.standard_normal(4).astype(np.float32)
+    for shape in [(7,), (3, 7), (2, 3, 7), (2, 2, 3, 7)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        got = oracle.dense(x, w.reshape(-1), b, 4)
+        assert got.shape == shape[:-1] + (4,)
+        assert rel(got, x.astype(np.float64) @ w.astype(np.float64) + b) < TOL
+
+
+def test_softmax_vs_scipy(oracle):
+    from scipy.special import softmax
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((5, 3, 17)) * 8).astype(np.float32)
+    assert rel(oracle.softmax(x), softmax(x.astype(np.float64), axis=-1)) < TOL
+    big = np.array([[1000.0, -1000.0, 999.0]], np.float32)
+    got = oracle.softmax(big)
+    assert np.isfinite(got).all() and abs(got.sum() - 1) < 1e-6
+
+
+@pytest.mark.parametrize("affine", [True, False])
+def test_layernorm_vs_torch(oracle, affine):
+    import torch
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal((6, 33)) * 3 + 1).astype(np.float32)
+    g = rng.standard_normal(33).astype(np.float32) if affine else None
+    b = rng.standard_normal(33).astype(np.float32) if affine else None
+    want = torch.nn.functional.layer_norm(
+        torch.from_numpy(x.astype(np.float64)), (33,),
+        None if g is None else torch.from_numpy(g.astype(np.float64)),
+        None if b is None else torch.from_numpy(b.astype(np.float64)), eps=1e-3).numpy()
+    assert rel(oracle.layernorm(x, g, b, 1e-3), want) < TOL
+    # two trailing axes normalised together == layer norm of the flattened rows
+    x3 = x.reshape(2, 3, 33)
+    got = oracle.layernorm(x3, None, None, 1e-3, n_axes=2)
+    flat = x3.reshape(2, 99).astype(np.float64)
+    want = (flat - flat.mean(1, keepdims=True)) / np.sqrt(flat.var(1, keepdims=True) + 1e-3)
+    assert rel(got.reshape(2, 99), want) < TOL
+
+
+def test_batchnorm_formula(oracle):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    mean, beta = rng.standard_normal(6).astype(np.float32), rng.standard_normal(6).astype(np.float32)
+    var, gamma = (0.5 + rng.random(6)).astype(np.float32), (0.5 + rng.random(6)).astype(np.float32)
+    want = (x.astype(np.float64) - mean) / np.sqrt(var.astype(np.float64) + 1e-3) * gamma + beta
+    assert rel(oracle.batchnorm(x, mean, var, gamma, beta, 1e-3), want) < TOL
+    want = (x.astype(np.float64) - mean) / np.sqrt(var.astype(np.float64) + 1e-3)
+    assert rel(oracle.batchnorm(x, mean, var, None, None, 1e-3), want) < TOL
+
+
+def test_relu_family_and_gelu(oracle):
+    from scipy.special import erf
+    x = np.linspace(-8, 8, 161).astype(np.float32)
+    assert np.array_equal(oracle.relu(x), np.maximum(x, 0))
+    assert np.array_equal(oracle.relu(x, 6.0, 0.0, 0.0), np.clip(x, 0, 6))
+    got = oracle.relu(x, 4.0, 0.1, 1.0)  # x>=4 -> 4; 1<=x<4 -> x; else 0.1*(x-1)
+    want = np.where(x >= 4, 4, np.where(x >= 1, x, np.float32(0.1) * (x - 1)))
+    assert rel(got, want) < 1e-7
+    xd = x.astype(np.float64)
+    assert rel(oracle.gelu(x), 0.5 * xd * (1 + erf(xd / math.sqrt(2)))) < TOL
+
+
+@pytest.mark.parametrize("case", [(8, 8, 2, 2, "valid"), (9, 7, 3, 2, "same"), (9, 7, 3, 2, "valid"),
+                                  (5, 5, 2, 1, "same"), (7, 10, 3, 3, "same")])
+@pytest.mark.parametrize("mode", ["max", "avg"])
+def test_pool2d_vs_torch(oracle, case, mode):
+    import torch
+    import torch.nn.functional as F
+    h, w, k, s, padding = case
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((h, w, 3)).astype(np.float32)
+    got = oracle.pool2d(x, (k, k), (s, s), padding, mode)
+    _, pt, pb = tf_geometry(h, k, s, padding)
+    _, pl, pr = tf_geometry(w, k, s, padding)
+    xt = torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None]
+    if mode == "max":
+        want = F.max_pool2d(F.pad(xt, (pl, pr, pt, pb), value=-1e30), k, s)
+    else:  # padded taps are excluded from the divisor
+        ones = F.pad(torch.ones_like(xt), (pl, pr, pt, pb))
+        want = F.avg_pool2d(F.pad(xt, (pl, pr, pt, pb)), k, s) / F.avg_pool2d(ones, k, s)
+    want = want[0].permute(1, 2, 0).numpy()
+    assert got.shape == want.shape
+    assert rel(got, want) < TOL
+
+
+def test_global_pool_add_embedding_argmax(oracle):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    assert rel(oracle.global_pool(x, "avg"), x.astype(np.float64).mean((0, 1))) < TOL
+    assert np.array_equal(oracle.global_pool(x, "max"), x.max((0, 1)))
+    assert oracle.global_pool(x, "avg", keepdims=True).shape == (1, 1, 6)
+    y = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    assert np.array_equal(oracle.add(x, y), x + y)
+    assert np.array_equal(oracle.add(x, y[:1, :, :]), x + y[:1])
+    table = rng.standard_normal((11, 3)).astype(np.float32)
+    ids = np.array([0, 10, 3.7, 3], np.float32)  # floats are truncated
+    assert np.array_equal(oracle.embedding(ids, table.reshape(-1), 11, 3), table[[0, 10, 3, 3]])
+    with pytest.raises(RuntimeError):
+        oracle.embedding(np.array([11], np.float32), table.reshape(-1), 11, 3)
+    assert oracle.argmax(np.array([1, 5, 5, 2], np.float32)) == 1  # first maximum wins
+    assert oracle.argmax(np.array([-3, -1, -1], np.float32)) == 1
+
+
+def numpy_mha(q, v, k, heads, dk, dv, w, use_bias):
+    q, v, k = (a.astype(np.float64) for a in (q, v, k))
+    if use_bias:
+        qw, qb, kw, kb, vw, vb, ow, ob = [a.astype(np.float64) for a in w]
+    else:
+        qw, kw, vw, ow = [a.astype(np.float64) for a in w]
+        qb = kb = vb = ob = 0.0
+    d = q.shape[1]
+    Q = np.einsum("td,dhk->htk", q, qw.reshape(d, heads, dk)) + (np.reshape(qb, (heads, 1, dk)) if use_bias else 0)
+    K = np.einsum("sd,dhk->hsk", k, kw.reshape(d, heads, dk)) + (np.reshape(kb, (heads, 1, dk)) if use_bias else 0)
+    V = np.einsum("sd,dhk->hsk", v, vw.reshape(d, heads, dv)) + (np.reshape(vb, (heads, 1, dv)) if use_bias else 0)
+    S = np.einsum("htk,hsk->hts", Q, K) / math.sqrt(dk)
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    O = np.einsum("hts,hsk->thk", P, V).reshape(q.shape[0], heads * dv)
+    return O @ ow.reshape(heads * dv, -1) + ob
+
+
+@pytest.mark.parametrize("heads,dk,dv,use_bias,sep_key", [(1, 4, 4, True, False), (3, 4, 5, True, True),
+                                                          (2, 8, 8, False, False), (2, 3, 6, True, False)])
+def test_mha_vs_numpy(oracle, heads, dk, dv, use_bias, sep_key):
+    rng = np.random.default_rng(11)
+    t, s, d = 5, 7, 6
+    q = rng.standard_normal((t, d)).astype(np.float32)
+    v = rng.standard_normal((s, d)).astype(np.float32)
+    k = rng.standard_normal((s, d)).astype(np.float32) if sep_key else None
+    shapes = []
+    for dim in (dk, dk, dv):
+        shapes.append((d, heads, dim))
+        if use_bias:
+            shapes.append((heads, dim))
+    shapes.append((heads, dv, d))
+    if use_bias:
+        shapes.append((d,))
+    w = [rng.standard_normal(sh).astype(np.float32).reshape(-1) * 0.5 for sh in shapes]
+    got = oracle.mha(q, v, k, heads, dk, dv, w, use_bias)
+    want = numpy_mha(q, v, v if k is None else k, heads, dk, dv, w, use_bias)
+    assert rel(got, want) < TOL
+    # permuting key/value rows together leaves the output unchanged (no positional term, no mask)
+    perm = rng.permutation(s)
+    got2 = oracle.mha(q, v[perm], None if k is None else k[perm], heads, dk, dv, w, use_bias)
+    assert rel(got2, got) < TOL
+
+
+def test_mha_torch_sdpa_crosscheck(oracle):
+    import torch
+    rng = np.random.default_rng(12)
+    t, d = 6, 8
+    x = rng.standard_normal((t, d)).astype(np.float32)
+    eye = np.eye(d, dtype=np.float32)
+    # one head, identity projections: plain softmax(x x^T / sqrt(d)) x
+    got = oracle.mha(x, x, None, 1, d, d, [eye.reshape(-1)] * 4, False)
+    xt = torch.from_numpy(x.astype(np.float64))[None]
+    want = torch.nn.functional.scaled_dot_product_attention(xt, xt, xt)[0].numpy()
+    assert rel(got, want) < TOL
+
+
+@pytest.mark.parametrize("eq,xs,ks,bias_axes", [
+    ("abc,cd->abd", (3, 4), (4, 5), "d"), ("abc,cde->abde", (3, 4), (4, 2, 5), "de"),
+    ("abc,cde->abde", (3, 4), (4, 2, 5), "ed"), ("abcd,cde->abe", (3, 4, 2), (4, 2, 5), "e"),
+    ("abc,cd->abd", (3, 4), (4, 5), None)])
+def test_einsum_dense_vs_numpy(oracle, eq, xs, ks, bias_axes):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal(xs).astype(np.float32)
+    k = rng.standard_normal(ks).astype(np.float32)
+    lhs, rest = eq.split(",")
+    rk, rhs = rest.split("->")
+    sizes = dict(zip(lhs, (1,) + xs))
+    sizes.update(zip(rk, ks))
+    bias = None
+    want = np.einsum(eq, x[None].astype(np.float64), k.astype(np.float64))
+    if bias_axes:
+        # the stored bias follows the order of the output subscripts, whatever order bias_axes spells
+        bchars = [c for c in rhs if c in bias_axes]
+        bias = rng.standard_normal([sizes[c] for c in bchars]).astype(np.float32)
+        want = want + np.einsum("".join(bchars) + "->" + "".join(c if c in bchars else "" for c in rhs),
+                                bias.astype(np.float64)).reshape([sizes[c] if c in bchars else 1 for c in rhs])
+    got = oracle.einsum_dense(x, eq, k, list(ks), bias, bias_axes)
+    assert got.shape == want.shape[1:]
+    assert rel(got, want[0]) < TOL
