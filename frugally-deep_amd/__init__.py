@@ -1,1 +1,285 @@
-"""placeholder, replaced below"""
+"""ctypes binding of libfdx.so, the C ABI declared in include/fdx.h.
+
+The forward path runs only on the GPU through the HIP library; there is no CPU
+fallback.  Importing this module without a built libfdx.so raises ImportError with the
+build command (``python -c "import __graft_entry__ as g; g.build()"`` or
+``make -C frugally-deep_amd/csrc``).
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfdx.so")
+
+c_float_p = ctypes.POINTER(ctypes.c_float)
+c_void_pp = ctypes.POINTER(ctypes.c_void_p)
+
+ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+FLT_MAX = float(np.finfo(np.float32).max)
+PAD = {"valid": 0, "same": 1, "causal": 2}
+
+
+class Act(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int), ("max_value", ctypes.c_float), ("negative_slope", ctypes.c_float),
+                ("threshold", ctypes.c_float)]
+
+
+class GemmBatch(ctypes.Structure):
+    _fields_ = [("batch", ctypes.c_int), ("inner", ctypes.c_int)] + [
+        (n, ctypes.c_int64) for n in ("a_outer", "a_inner", "b_outer", "b_inner", "c_outer", "c_inner")]
+
+
+class FdxError(RuntimeError):
+    pass
+
+
+def build_library():
+    import subprocess
+    subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "-j8"])
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("libfdx.so is not built (run `make -C %s`); the fdx forward path has no fallback"
+                          % os.path.join(_HERE, "csrc"))
+    return ctypes.CDLL(LIB_PATH)
+
+
+lib = _load()
+lib.fdx_last_error.restype = ctypes.c_char_p
+lib.fdx_mha_scratch_bytes.restype = ctypes.c_size_t
+
+
+def check(status):
+    if status != 0:
+        raise FdxError(lib.fdx_last_error().decode("utf-8", "replace"))
+
+
+def relu_act(max_value=None, negative_slope=0.0, threshold=0.0):
+    return Act(ACT_RELU, FLT_MAX if max_value is None else max_value, negative_slope, threshold)
+
+
+def gelu_act():
+    return Act(ACT_GELU, FLT_MAX, 0.0, 0.0)
+
+
+def _act_ref(act):
+    return None if act is None else ctypes.byref(act)
+
+
+class DevBuf:
+    """Device buffer owned by the library's allocator; holds fp32 (or raw bytes)."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        p = ctypes.c_void_p()
+        check(lib.fdx_dev_alloc(ctypes.c_size_t(max(self.nbytes, 4)), ctypes.byref(p)))
+        self.ptr = p
+
+    @classmethod
+    def from_host(cls, arr, dtype=np.float32):
+        arr = np.ascontiguousarray(arr, dtype=dtype)
+        buf = cls(arr.nbytes)
+        if arr.nbytes:
+            check(lib.fdx_h2d(buf.ptr, arr.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(arr.nbytes)))
+        return buf
+
+    def to_host(self, shape, dtype=np.float32):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes, (out.nbytes, self.nbytes)
+        check(lib.fdx_d2h(out.ctypes.data_as(ctypes.c_void_p), self.ptr, ctypes.c_size_t(out.nbytes)))
+        return out
+
+    def free(self):
+        if self.ptr:
+            check(lib.fdx_dev_free(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _dp(buf):
+    return None if buf is None else ctypes.cast(buf.ptr, c_float_p)
+
+
+def sync():
+    check(lib.fdx_sync())
+
+
+def window_geometry(in_h, in_w, k_h, k_w, s_h, s_w, padding):
+    g = (ctypes.c_int * 6)()
+    check(lib.fdx_window_geometry(in_h, in_w, k_h, k_w, s_h, s_w, PAD[padding], g))
+    return dict(pad_top=g[0], pad_bottom=g[1], pad_left=g[2], pad_right=g[3], out_h=g[4], out_w=g[5])
+
+
+# ------------------------------------------------------------------ host-array conveniences
+# Each takes numpy arrays, stages them in HBM, launches the kernel through the C ABI and returns numpy.
+
+def conv2d(x, w, bias, strides=(1, 1), dilation=(1, 1), padding="valid", residual=None, act=None, extra_pad=None):
+    """x [n,h,w,cin]; w in converted-JSON order [cout,kh,kw,cin]."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, wd, cin = x.shape
+    cout, kh, kw, _ = w.shape
+    g = window_geometry(h, wd, (kh - 1) * dilation[0] + 1, (kw - 1) * dilation[1] + 1, strides[0], strides[1], padding)
+    dx, dw = DevBuf.from_host(x), DevBuf.from_host(w)
+    db = None if bias is None else DevBuf.from_host(bias)
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * cout)
+    check(lib.fdx_conv2d_nhwc_f32(_dp(dx), n, h, wd, cin, _dp(dw), _dp(db), cout, kh, kw, strides[0], strides[1],
+                                  dilation[0], dilation[1], g["pad_top"], g["pad_left"], g["out_h"], g["out_w"],
+                                  _dp(dr), _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], cout))
+
+
+def dwconv2d(x, w_chw, bias, strides=(1, 1), dilation=(1, 1), padding="valid", act=None):
+    """x [n,h,w,c]; w in converted-JSON order [c,kh,kw] (re-laid to [kh,kw,c] here, as the loader does)."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, wd, c = x.shape
+    _, kh, kw = w_chw.shape
+    g = window_geometry(h, wd, (kh - 1) * dilation[0] + 1, (kw - 1) * dilation[1] + 1, strides[0], strides[1], padding)
+    dx, dw = DevBuf.from_host(x), DevBuf.from_host(np.transpose(w_chw, (1, 2, 0)))
+    db = None if bias is None else DevBuf.from_host(bias)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * c)
+    check(lib.fdx_dwconv2d_nhwc_f32(_dp(dx), n, h, wd, c, _dp(dw), _dp(db), kh, kw, strides[0], strides[1],
+                                    dilation[0], dilation[1], g["pad_top"], g["pad_left"], g["out_h"], g["out_w"],
+                                    _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], c))
+
+
+def gemm(a, b_nk, bias=None, alpha=1.0, bias_per_row=False, residual=None, act=None):
+    a, b_nk = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b_nk, np.float32)
+    m, k = a.shape
+    n = b_nk.shape[0]
+    da, dbm = DevBuf.from_host(a), DevBuf.from_host(b_nk)
+    dbias = None if bias is None else DevBuf.from_host(bias)
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * m * n)
+    check(lib.fdx_gemm_bias_act_f32(_dp(da), ctypes.c_int64(k), _dp(dbm), ctypes.c_int64(k), m, n, k,
+                                    ctypes.c_float(alpha), _dp(dbias), int(bias_per_row), _dp(dr), _act_ref(act),
+                                    _dp(out), ctypes.c_int64(n), None))
+    return out.to_host((m, n))
+
+
+def pool2d(x, pool, strides, padding, mode, zero_frame=(0, 0, 0, 0)):
+    """zero_frame = (top, left, bottom, right) of an explicit ZeroPadding2D folded into the pool."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    zt, zl, zb, zr = zero_frame
+    g = window_geometry(h + zt + zb, w + zl + zr, pool[0], pool[1], strides[0], strides[1], padding)
+    dx = DevBuf.from_host(x)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * c)
+    check(lib.fdx_pool2d_nhwc_f32(_dp(dx), n, h, w, c, pool[0], pool[1], strides[0], strides[1],
+                                  g["pad_top"] + zt, g["pad_left"] + zl, zt, zl, zb, zr, g["out_h"], g["out_w"],
+                                  0 if mode == "max" else 1, _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], c))
+
+
+def global_pool(x, mode):
+    x = np.ascontiguousarray(x, np.float32)
+    n, c = x.shape[0], x.shape[-1]
+    pos = x.size // (n * c)
+    dx, out = DevBuf.from_host(x), DevBuf(4 * n * c)
+    check(lib.fdx_global_pool_f32(_dp(dx), n, pos, c, 0 if mode == "max" else 1, _dp(out)))
+    return out.to_host((n, c))
+
+
+def add(a, b, act=None):
+    a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+    da, db, out = DevBuf.from_host(a), DevBuf.from_host(b), DevBuf(a.nbytes)
+    check(lib.fdx_eltwise_add_f32(_dp(da), _dp(db), ctypes.c_size_t(a.size), ctypes.c_size_t(b.size), _act_ref(act),
+                                  _dp(out)))
+    return out.to_host(a.shape)
+
+
+def activation(x, act):
+    x = np.ascontiguousarray(x, np.float32)
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    check(lib.fdx_activation_f32(_dp(dx), ctypes.c_size_t(x.size), _act_ref(act), _dp(out)))
+    return out.to_host(x.shape)
+
+
+def channel_affine(x, scale, shift, act=None):
+    x = np.ascontiguousarray(x, np.float32)
+    c = x.shape[-1]
+    dx, ds, dh, out = DevBuf.from_host(x), DevBuf.from_host(scale), DevBuf.from_host(shift), DevBuf(x.nbytes)
+    check(lib.fdx_channel_affine_f32(_dp(dx), ctypes.c_size_t(x.size // c), c, _dp(ds), _dp(dh), _act_ref(act),
+                                     _dp(out)))
+    return out.to_host(x.shape)
+
+
+def zero_pad2d(x, pt, pb, pl, pr):
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    dx, out = DevBuf.from_host(x), DevBuf(4 * n * (h + pt + pb) * (w + pl + pr) * c)
+    check(lib.fdx_zero_pad2d_nhwc_f32(_dp(dx), n, h, w, c, pt, pb, pl, pr, _dp(out)))
+    return out.to_host((n, h + pt + pb, w + pl + pr, c))
+
+
+def layernorm(x, gamma, beta, eps):
+    x = np.ascontiguousarray(x, np.float32)
+    d = x.shape[-1]
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    dg = None if gamma is None else DevBuf.from_host(gamma)
+    db = None if beta is None else DevBuf.from_host(beta)
+    check(lib.fdx_layernorm_f32(_dp(dx), ctypes.c_int64(x.size // d), d, _dp(dg), _dp(db), ctypes.c_float(eps),
+                                _dp(out)))
+    return out.to_host(x.shape)
+
+
+def softmax(x, causal_period=0, causal_offset=0):
+    x = np.ascontiguousarray(x, np.float32)
+    d = x.shape[-1]
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    check(lib.fdx_softmax_f32(_dp(dx), ctypes.c_int64(x.size // d), d, causal_period, causal_offset, _dp(out)))
+    return out.to_host(x.shape)
+
+
+def embedding(ids, table):
+    ids = np.ascontiguousarray(ids, np.float32).reshape(-1)
+    table = np.ascontiguousarray(table, np.float32)
+    di, dt, out = DevBuf.from_host(ids), DevBuf.from_host(table), DevBuf(4 * ids.size * table.shape[1])
+    flag = DevBuf.from_host(np.zeros(1, np.int32), np.int32)
+    check(lib.fdx_embedding_f32(_dp(di), ctypes.c_int64(ids.size), _dp(dt), table.shape[0], table.shape[1], _dp(out),
+                                ctypes.cast(flag.ptr, ctypes.POINTER(ctypes.c_int))))
+    if flag.to_host((1,), np.int32)[0]:
+        raise FdxError("vocabulary item indices must all be strictly less than the value of input_dim")
+    return out.to_host((ids.size, table.shape[1]))
+
+
+def argmax(x):
+    x = np.ascontiguousarray(x, np.float32)
+    d = x.shape[-1]
+    rows = x.size // d
+    dx, oi, ov = DevBuf.from_host(x), DevBuf(4 * rows), DevBuf(4 * rows)
+    check(lib.fdx_argmax_f32(_dp(dx), ctypes.c_int64(rows), d, ctypes.cast(oi.ptr, ctypes.POINTER(ctypes.c_int32)),
+                             _dp(ov)))
+    return oi.to_host((rows,), np.int32), ov.to_host((rows,))
+
+
+def mha_prefill(q, k, v, heads, dk, dv, causal=False):
+    """q [b,t,heads*dk], k [b,s,heads*dk], v [b,s,heads*dv] (already projected)."""
+    q, k, v = (np.ascontiguousarray(a, np.float32) for a in (q, k, v))
+    b, t, _ = q.shape
+    s = k.shape[1]
+    dq, dk_, dv_ = DevBuf.from_host(q), DevBuf.from_host(k), DevBuf.from_host(v)
+    scratch = DevBuf(lib.fdx_mha_scratch_bytes(b, heads, t, s, dv))
+    out = DevBuf(4 * b * t * heads * dv)
+    check(lib.fdx_mha_prefill_f32(_dp(dq), _dp(dk_), _dp(dv_), b, t, s, heads, dk, dv, int(causal), _dp(out),
+                                  scratch.ptr))
+    return out.to_host((b, t, heads * dv))
+
+
+def mha_decode(q, k_cache, v_cache, heads, dk, dv, length):
+    """q [b,heads*dk]; caches [b,max_len,heads*dk|dv]."""
+    q, k_cache, v_cache = (np.ascontiguousarray(a, np.float32) for a in (q, k_cache, v_cache))
+    b, max_len = k_cache.shape[0], k_cache.shape[1]
+    dq, dkc, dvc = DevBuf.from_host(q), DevBuf.from_host(k_cache), DevBuf.from_host(v_cache)
+    out = DevBuf(4 * b * heads * dv)
+    check(lib.fdx_mha_decode_f32(_dp(dq), _dp(dkc), _dp(dvc), b, heads, dk, dv, length, max_len, _dp(out)))
+    return out.to_host((b, heads * dv))

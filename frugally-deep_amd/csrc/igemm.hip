@@ -1,0 +1,400 @@
+// Implicit-GEMM Conv2D and row-major GEMM on fp32 MFMA (v_mfma_f32_32x32x2_f32), gfx950.
+//
+// One kernel template serves both: the A operand is either a row-major matrix or the
+// virtual im2col matrix of an NHWC activation tensor (never materialised: padding is a
+// load predicate, the K axis walks (filter row, filter column, input channel) which is a
+// contiguous channel run in memory and also the storage order of the converted-JSON
+// filters, so weights need no re-layout).  B is always [N][K] with K contiguous.
+//
+// Tiling: a workgroup of WAVES_M x WAVES_N wave64s owns a BM x BN output tile and walks K
+// in slabs of 16.  Global loads are 16-byte per lane into registers, written to LDS rows
+// padded to 20 floats (conflict-free 128-bit fragment reads), double-buffered so one
+// barrier per slab suffices.  Each lane feeds four consecutive k values from one 128-bit
+// LDS read into four MFMAs (the k order inside a slab is permuted identically for A and
+// B, which a sum does not notice).  Epilogue: alpha, bias (per column or per row),
+// residual add, activation, fused on the accumulators before the only store.
+#include "common.hpp"
+
+namespace fdx {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmParams {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;
+    const float* residual;
+    int M, N, K;
+    int64_t lda, ldb, ldc;
+    float alpha;
+    int bias_per_row;
+    Act act;
+    int inner;
+    int64_t a_outer, a_inner, b_outer, b_inner, c_outer, c_inner;
+    // convolution view of A
+    int H, W, Cin, kh, kw, sy, sx, dy, dx, pad_top, pad_left, OH, OW;
+};
+
+enum { A_ROWS_VEC = 0, A_CONV_VEC = 1, A_CONV_SCALAR = 2, A_ROWS_SCALAR = 3 };
+
+constexpr int BK = 16;
+constexpr int LDS_STRIDE = BK + 4;
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int A_MODE, int B_VEC>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParams p)
+{
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_LOADS = (BM * 4 + NT - 1) / NT, B_LOADS = (BN * 4 + NT - 1) / NT;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
+    static_assert(NT % 4 == 0, "loader mapping assumes the k quarter is fixed per thread");
+
+    __shared__ __attribute__((aligned(16))) float As[2][BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN * LDS_STRIDE];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
+    // tiles so that tiles sharing an A row block also share that XCD's L2.
+    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+    const int total = tiles_m * tiles_n;
+    int id = blockIdx.x;
+    {
+        const int xcd = id & 7, local = id >> 3, per = total >> 3, rem = total & 7;
+        id = xcd * per + (xcd < rem ? xcd : rem) + local;
+    }
+    const int m0 = (id / tiles_n) * BM, n0 = (id % tiles_n) * BN;
+
+    const int z = blockIdx.z;
+    const float* __restrict__ A = p.A + (z / p.inner) * p.a_outer + (z % p.inner) * p.a_inner;
+    const float* __restrict__ B = p.B + (z / p.inner) * p.b_outer + (z % p.inner) * p.b_inner;
+    const int64_t c_off = (z / p.inner) * p.c_outer + (z % p.inner) * p.c_inner;
+    float* __restrict__ C = p.C + c_off;
+    const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
+
+    const int kq = t & 3; // which 4-float quarter of the 16-wide slab this thread loads
+
+    // ---- per-thread A row state (fixed for the whole K loop)
+    bool a_ok[A_LOADS];
+    const float* a_ptr[A_LOADS];
+    int a_iy0[A_LOADS], a_ix0[A_LOADS];
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int idx = t + i * NT;
+        const int m = m0 + (idx >> 2);
+        a_ok[i] = (idx < BM * 4) && (m < p.M);
+        a_ptr[i] = A;
+        a_iy0[i] = a_ix0[i] = 0;
+        if (a_ok[i]) {
+            if (A_MODE == A_ROWS_VEC || A_MODE == A_ROWS_SCALAR) {
+                a_ptr[i] = A + (int64_t)m * p.lda;
+            } else {
+                const int img = m / (p.OH * p.OW), rem = m - img * (p.OH * p.OW);
+                const int oy = rem / p.OW, ox = rem - oy * p.OW;
+                a_ptr[i] = A + (int64_t)img * p.H * p.W * p.Cin;
+                a_iy0[i] = oy * p.sy - p.pad_top;
+                a_ix0[i] = ox * p.sx - p.pad_left;
+            }
+        }
+    }
+    // conv k-state of this thread's quarter: input channel, filter column, filter row
+    int kc = 0, kfx = 0, kfy = 0;
+    if (A_MODE == A_CONV_VEC) {
+        const int kk = kq * 4, tap = kk / p.Cin;
+        kc = kk - tap * p.Cin;
+        kfy = tap / p.kw;
+        kfx = tap - kfy * p.kw;
+    }
+    bool b_ok[B_LOADS];
+    const float* b_ptr[B_LOADS];
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int idx = t + i * NT;
+        const int n = n0 + (idx >> 2);
+        b_ok[i] = (idx < BN * 4) && (n < p.N);
+        b_ptr[i] = b_ok[i] ? B + (int64_t)n * p.ldb : B;
+    }
+
+    f32x4 ra[A_LOADS], rb[B_LOADS];
+
+    auto load_tiles = [&](int kt) {
+        const int k = kt * BK + kq * 4;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            f32x4 v = { 0.f, 0.f, 0.f, 0.f };
+            if (A_MODE == A_ROWS_VEC) {
+                if (a_ok[i] && k < p.K)
+                    v = *reinterpret_cast<const f32x4*>(a_ptr[i] + k);
+            } else if (A_MODE == A_ROWS_SCALAR) {
+                if (a_ok[i]) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (k + j < p.K)
+                            v[j] = a_ptr[i][k + j];
+                }
+            } else if (A_MODE == A_CONV_VEC) {
+                const int iy = a_iy0[i] + kfy * p.dy, ix = a_ix0[i] + kfx * p.dx;
+                if (a_ok[i] && kfy < p.kh && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W)
+                    v = *reinterpret_cast<const f32x4*>(a_ptr[i] + ((int64_t)(iy * p.W + ix) * p.Cin + kc));
+            } else {
+                if (a_ok[i]) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int kk = k + j;
+                        if (kk < p.K) {
+                            const int tap = kk / p.Cin, c = kk - tap * p.Cin;
+                            const int fy = tap / p.kw, fx = tap - fy * p.kw;
+                            const int iy = a_iy0[i] + fy * p.dy, ix = a_ix0[i] + fx * p.dx;
+                            if (iy >= 0 && iy < p.H && ix >= 0 && ix < p.W)
+                                v[j] = a_ptr[i][(int64_t)(iy * p.W + ix) * p.Cin + c];
+                        }
+                    }
+                }
+            }
+            ra[i] = v;
+        }
+        if (A_MODE == A_CONV_VEC) { // advance the quarter's (fy, fx, c) by one slab
+            kc += BK;
+            while (kc >= p.Cin) {
+                kc -= p.Cin;
+                if (++kfx == p.kw) {
+                    kfx = 0;
+                    ++kfy;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            f32x4 v = { 0.f, 0.f, 0.f, 0.f };
+            if (B_VEC) {
+                if (b_ok[i] && k < p.K)
+                    v = *reinterpret_cast<const f32x4*>(b_ptr[i] + k);
+            } else if (b_ok[i]) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (k + j < p.K)
+                        v[j] = b_ptr[i][k + j];
+            }
+            rb[i] = v;
+        }
+    };
+    auto store_tiles = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int idx = t + i * NT;
+            if (idx < BM * 4)
+                *reinterpret_cast<f32x4*>(&As[buf][(idx >> 2) * LDS_STRIDE + kq * 4]) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const int idx = t + i * NT;
+            if (idx < BN * 4)
+                *reinterpret_cast<f32x4*>(&Bs[buf][(idx >> 2) * LDS_STRIDE + kq * 4]) = rb[i];
+        }
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                acc[i][j][e] = 0.f;
+
+    const int KT = (p.K + BK - 1) / BK;
+    const int fr = lane & 31, fh = lane >> 5;
+
+    load_tiles(0);
+    store_tiles(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < KT)
+            load_tiles(kt + 1);
+#pragma unroll
+        for (int k8 = 0; k8 < BK / 8; ++k8) {
+            f32x4 af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const f32x4*>(
+                    &As[buf][(wm * WTM + i * 32 + fr) * LDS_STRIDE + k8 * 8 + fh * 4]);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                bf[j] = *reinterpret_cast<const f32x4*>(
+                    &Bs[buf][(wn * WTN + j * 32 + fr) * LDS_STRIDE + k8 * 8 + fh * 4]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < KT)
+            store_tiles(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue.  32x32 accumulator layout: element e of lane l is
+    // row 8*(e/4) + 4*(l/32) + e%4, column l%32.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * WTN + j * 32 + fr;
+        if (n >= p.N)
+            continue;
+        const float bcol = (p.bias && !p.bias_per_row) ? p.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (e >> 2) + 4 * fh + (e & 3);
+                if (m < p.M) {
+                    float v = acc[i][j][e] * p.alpha + bcol;
+                    if (p.bias && p.bias_per_row)
+                        v += p.bias[m];
+                    const int64_t off = (int64_t)m * p.ldc + n;
+                    if (R)
+                        v += R[off];
+                    C[off] = apply_act(v, p.act);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ dispatch
+
+static int g_forced_tile = -1; // tests force a tile configuration through fdx_debug_force_tile
+
+template <int BM, int BN, int WM, int WN>
+static void launch_cfg(const GemmParams& p, int a_mode, int b_vec, int batch, hipStream_t s)
+{
+    const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    dim3 grid(tiles, 1, batch), block(64 * WM * WN);
+#define FDX_IGEMM_CASE(AM, BV)                                                              \
+    if (a_mode == AM && b_vec == BV) {                                                      \
+        hipLaunchKernelGGL((igemm_kernel<BM, BN, WM, WN, AM, BV>), grid, block, 0, s, p);   \
+        return;                                                                             \
+    }
+    FDX_IGEMM_CASE(A_ROWS_VEC, 1)
+    FDX_IGEMM_CASE(A_ROWS_VEC, 0)
+    FDX_IGEMM_CASE(A_CONV_VEC, 1)
+    FDX_IGEMM_CASE(A_CONV_VEC, 0)
+    FDX_IGEMM_CASE(A_CONV_SCALAR, 1)
+    FDX_IGEMM_CASE(A_CONV_SCALAR, 0)
+    FDX_IGEMM_CASE(A_ROWS_SCALAR, 1)
+    FDX_IGEMM_CASE(A_ROWS_SCALAR, 0)
+#undef FDX_IGEMM_CASE
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* family)
+{
+    int a_mode;
+    if (conv)
+        a_mode = (p.Cin % 4 == 0 && aligned16(p.A)) ? A_CONV_VEC : A_CONV_SCALAR;
+    else
+        a_mode = (p.K % 4 == 0 && p.lda % 4 == 0 && aligned16(p.A) && p.a_outer % 4 == 0 && p.a_inner % 4 == 0)
+            ? A_ROWS_VEC
+            : A_ROWS_SCALAR;
+    const int b_vec = (p.K % 4 == 0 && p.ldb % 4 == 0 && aligned16(p.B) && p.b_outer % 4 == 0 && p.b_inner % 4 == 0) ? 1 : 0;
+
+    // Tile choice: the largest tile that still yields at least ~2 waves of workgroups over
+    // the 256 CUs; narrow N picks the 32-wide tile.
+    int cfg;
+    auto blocks = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
+    if (p.N <= 32)
+        cfg = 2;
+    else if (p.N <= 64)
+        cfg = blocks(128, 64) >= 512 ? 1 : 3;
+    else if (blocks(128, 128) >= 512)
+        cfg = 0;
+    else if (blocks(128, 64) >= 512)
+        cfg = 1;
+    else
+        cfg = 3;
+    if (g_forced_tile >= 0)
+        cfg = g_forced_tile;
+
+    hipStream_t s = stream();
+    profile_begin();
+    switch (cfg) {
+    case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
+    case 1: launch_cfg<128, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+    case 2: launch_cfg<128, 32, 4, 1>(p, a_mode, b_vec, batch, s); break;
+    default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+    }
+    const double flops = 2.0 * p.M * (double)p.N * p.K * batch;
+    profile_end(family, flops, 0.0);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+} // namespace fdx
+
+using namespace fdx;
+
+extern "C" fdx_status fdx_debug_force_tile(int cfg)
+{
+    fdx::g_forced_tile = cfg;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_conv2d_nhwc_f32(const float* in, int n, int h, int w, int cin,
+    const float* weights, const float* bias, int cout, int kh, int kw,
+    int sy, int sx, int dy, int dx, int pad_top, int pad_left, int out_h, int out_w,
+    const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(in && weights && out, "conv2d: null pointer");
+    FDX_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0 && kh > 0 && kw > 0, "conv2d: bad shape");
+    FDX_REQUIRE(sy > 0 && sx > 0 && dy > 0 && dx > 0 && out_h > 0 && out_w > 0, "conv2d: bad stride/dilation/output");
+    FDX_REQUIRE(pad_top >= 0 && pad_left >= 0, "conv2d: negative padding");
+    // the last tap of the last output must not start beyond what padding can explain
+    FDX_REQUIRE((int64_t)n * out_h * out_w < (1LL << 31) && (int64_t)kh * kw * cin < (1LL << 31)
+            && (int64_t)h * w * cin < (1LL << 31),
+        "conv2d: dimension overflow");
+    GemmParams p {};
+    p.A = in; p.B = weights; p.C = out; p.bias = bias; p.residual = residual;
+    p.M = n * out_h * out_w; p.N = cout; p.K = kh * kw * cin;
+    p.lda = 0; p.ldb = p.K; p.ldc = cout;
+    p.alpha = 1.f; p.bias_per_row = 0; p.act = make_act(act);
+    p.inner = 1;
+    p.H = h; p.W = w; p.Cin = cin; p.kh = kh; p.kw = kw; p.sy = sy; p.sx = sx; p.dy = dy; p.dx = dx;
+    p.pad_top = pad_top; p.pad_left = pad_left; p.OH = out_h; p.OW = out_w;
+    const bool pointwise = kh == 1 && kw == 1 && sy == 1 && sx == 1 && pad_top == 0 && pad_left == 0
+        && out_h == h && out_w == w;
+    if (pointwise) { // a 1x1 stride-1 convolution is the plain GEMM [n*h*w][cin] x [cout][cin]^T
+        p.lda = cin;
+        return run_igemm(p, false, 1, "conv1x1_gemm_f32");
+    }
+    return run_igemm(p, true, 1, "conv_igemm_f32");
+}
+
+extern "C" fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const float* b_nk, int64_t ldb,
+    int m, int n, int k, float alpha, const float* bias, int bias_per_row,
+    const float* residual, const fdx_act* act, float* c, int64_t ldc, const fdx_gemm_batch* batch)
+{
+    FDX_REQUIRE(a && b_nk && c, "gemm: null pointer");
+    FDX_REQUIRE(m > 0 && n > 0 && k > 0 && lda >= k && ldb >= k && ldc >= n, "gemm: bad shape m=%d n=%d k=%d", m, n, k);
+    GemmParams p {};
+    p.A = a; p.B = b_nk; p.C = c; p.bias = bias; p.residual = residual;
+    p.M = m; p.N = n; p.K = k; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.alpha = alpha; p.bias_per_row = bias_per_row; p.act = make_act(act);
+    p.inner = 1;
+    int nb = 1;
+    if (batch) {
+        FDX_REQUIRE(batch->batch > 0 && batch->inner > 0 && batch->batch <= 65535, "gemm: bad batch");
+        nb = batch->batch;
+        p.inner = batch->inner;
+        p.a_outer = batch->a_outer; p.a_inner = batch->a_inner;
+        p.b_outer = batch->b_outer; p.b_inner = batch->b_inner;
+        p.c_outer = batch->c_outer; p.c_inner = batch->c_inner;
+    }
+    return run_igemm(p, false, nb, "gemm_f32");
+}

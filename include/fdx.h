@@ -1,0 +1,225 @@
+/*
+ * fdx -- C ABI of the MI355X (gfx950) forward path for frugally-deep models.
+ *
+ * Everything behind fdeep::load_model / model::predict / predict_multi runs through
+ * these entry points: the C++ facade in include/fdeep/fdeep.hpp, the ctypes
+ * binding and the tests call nothing else.  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every function returns fdx_status, 0 = ok; fdx_last_error() gives the text
+ *     (thread-local), which the C++ facade rethrows as std::runtime_error the way
+ *     include/fdeep/common.hpp:42-57 raises.
+ *   - tensors are fp32, channels-last, batch outermost: [n][h][w][c] / [n][rows][depth].
+ *   - "dev" pointers are device memory of the current GPU; the per-kernel launchers
+ *     take device pointers only and enqueue on the library stream (fdx_sync waits).
+ */
+#ifndef FDX_H
+#define FDX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int fdx_status;
+enum { FDX_OK = 0, FDX_ERR_INVALID = 1, FDX_ERR_HIP = 2, FDX_ERR_FORMAT = 3, FDX_ERR_UNSUPPORTED = 4 };
+
+/* activation fused into a producer's epilogue or applied stand-alone */
+enum { FDX_ACT_NONE = 0, FDX_ACT_RELU = 1, FDX_ACT_GELU = 2 };
+typedef struct fdx_act {
+    int kind;             /* FDX_ACT_*                                              */
+    float max_value;      /* relu family: x >= max -> max            (relu_layer.hpp:40-46) */
+    float negative_slope; /*              x < threshold -> slope * (x - threshold)  */
+    float threshold;
+} fdx_act;
+
+const char* fdx_last_error(void);
+fdx_status fdx_init(int device);
+
+/* ---- device memory plumbing for callers that do not link HIP themselves ---- */
+fdx_status fdx_dev_alloc(size_t bytes, void** out);
+fdx_status fdx_dev_free(void* p);
+fdx_status fdx_h2d(void* dst_dev, const void* src_host, size_t bytes);
+fdx_status fdx_d2h(void* dst_host, const void* src_dev, size_t bytes);
+fdx_status fdx_sync(void);
+/* HIP-event stopwatch on the library stream: start, run work, stop returns milliseconds */
+fdx_status fdx_timer_start(void);
+fdx_status fdx_timer_stop(float* ms);
+/* name and average duration (ms) of the dominant kernel family since the last reset,
+ * measured with HIP events around every launch while profiling is enabled */
+fdx_status fdx_profile_enable(int on);
+fdx_status fdx_profile_reset(void);
+fdx_status fdx_profile_get(int index, char* name, size_t name_len, uint64_t* launches, double* total_ms,
+    double* flops, double* bytes);
+
+/*
+ * Conv2D, cross-correlation, implicit GEMM on fp32 MFMA:
+ *   out[n][oy][ox][co] = act(bias[co] + sum_{fy,fx,ci} w[co][fy][fx][ci] * in[n][oy*sy+fy*dy-pad_top][ox*sx+fx*dx-pad_left][ci]
+ *                            (+ residual[n][oy][ox][co]))
+ * replaces convolve / convolve_accumulative (include/fdeep/convolution.hpp:398-429, 224-305).
+ * Weights in the converted-JSON order [cout][kh][kw][cin] (keras_export/convert_model.py:197-200).
+ * Out-of-range taps read zero, which is pad_tensor's zero fill (include/fdeep/tensor.hpp:490-517);
+ * pad_top/pad_left and out_h/out_w come from fdx_window_geometry.
+ * bias and residual may be NULL.
+ */
+fdx_status fdx_conv2d_nhwc_f32(const float* in, int n, int h, int w, int cin,
+    const float* weights, const float* bias, int cout, int kh, int kw,
+    int sy, int sx, int dy, int dx, int pad_top, int pad_left, int out_h, int out_w,
+    const float* residual, const fdx_act* act, float* out);
+
+/*
+ * DepthwiseConv2D (depth multiplier 1); replaces depthwise_convolve
+ * (include/fdeep/depthwise_convolution.hpp:21-99).  weights_hwc is [kh][kw][c]
+ * (the converted-JSON slice_weights [c][kh][kw] transposed once at load).
+ */
+fdx_status fdx_dwconv2d_nhwc_f32(const float* in, int n, int h, int w, int c,
+    const float* weights_hwc, const float* bias, int kh, int kw,
+    int sy, int sx, int dy, int dx, int pad_top, int pad_left, int out_h, int out_w,
+    const fdx_act* act, float* out);
+
+/*
+ * Row-major GEMM with fused epilogue, fp32 MFMA:
+ *   c[m][n] = act(alpha * sum_k a[m][k] * b_nk[n][k] + bias + residual[m][n])
+ * replaces dense_layer::apply_impl (include/fdeep/layers/dense_layer.hpp:76-86; weights arrive
+ * [in][out] and are transposed once at load to [out][in]) and dot_product_tensors
+ * (include/fdeep/tensor.hpp:814-884).  bias_per_row selects bias[m] instead of bias[n].
+ * batch > 1 runs `batch` independent problems; problem i uses
+ *   a + (i / inner) * a_outer + (i % inner) * a_inner   (same for b, c); residual follows c.
+ */
+typedef struct fdx_gemm_batch {
+    int batch, inner;
+    int64_t a_outer, a_inner, b_outer, b_inner, c_outer, c_inner;
+} fdx_gemm_batch;
+fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const float* b_nk, int64_t ldb,
+    int m, int n, int k, float alpha, const float* bias, int bias_per_row,
+    const float* residual, const fdx_act* act, float* c, int64_t ldc, const fdx_gemm_batch* batch);
+
+/* [rows][cols] -> [cols][rows] (load-time weight re-layout) */
+fdx_status fdx_transpose_f32(const float* in, int rows, int cols, float* out);
+
+/*
+ * Max / average pooling with TF padding; mode 0 = max, 1 = average.  Window taps outside
+ * [0,h)x[0,w) are ignored by max and excluded from the average's divisor
+ * (include/fdeep/layers/max_pooling_3d_layer.hpp:17-38, average_pooling_3d_layer.hpp:17-42).
+ * zero_top/left/bottom/right describe an explicit ZeroPadding2D folded into this call: taps in
+ * that frame (still outside the stored tensor) contribute the value 0 and count as real elements.
+ */
+fdx_status fdx_pool2d_nhwc_f32(const float* in, int n, int h, int w, int c, int ph, int pw, int sy, int sx,
+    int pad_top, int pad_left, int zero_top, int zero_left, int zero_bottom, int zero_right,
+    int out_h, int out_w, int mode, float* out);
+
+/* global max (mode 0) / average (mode 1) over all positions of each sample:
+ * include/fdeep/layers/global_average_pooling_3d_layer.hpp:25-41 */
+fdx_status fdx_global_pool_f32(const float* in, int n, int positions, int c, int mode, float* out);
+
+/* out = act(a + b), b broadcast if b_count < count (b_count divides count; trailing dims match):
+ * add_layer / sum_tensors, include/fdeep/tensor.hpp:642-680 */
+fdx_status fdx_eltwise_add_f32(const float* a, const float* b, size_t count, size_t b_count,
+    const fdx_act* act, float* out);
+/* out = act(x) ; relu family and erf-GELU (include/fdeep/layers/relu_layer.hpp:32-48,
+ * include/fdeep/recurrent_ops.hpp:73-76) */
+fdx_status fdx_activation_f32(const float* x, size_t count, const fdx_act* act, float* out);
+/* out = act(x * scale[c] + shift[c]) along the last axis: a BatchNormalization that could not be
+ * folded into its producer (include/fdeep/tensor.hpp:773-793) */
+fdx_status fdx_channel_affine_f32(const float* x, size_t positions, int c, const float* scale,
+    const float* shift, const fdx_act* act, float* out);
+/* explicit zero padding, zero_padding_3d_layer / pad_tensor (include/fdeep/tensor.hpp:490-517) */
+fdx_status fdx_zero_pad2d_nhwc_f32(const float* in, int n, int h, int w, int c, int pt, int pb, int pl, int pr,
+    float* out);
+
+/* LayerNormalization over the last `depth` elements of each row
+ * (include/fdeep/layers/layer_normalization_layer.hpp:37-63, tensor.hpp:758-793); gamma/beta may be NULL */
+fdx_status fdx_layernorm_f32(const float* x, int64_t rows, int depth, const float* gamma, const float* beta,
+    float eps, float* out);
+/* softmax over the last axis in the reference's exp(x - m - log(sum)) form (tensor.hpp:1165-1192);
+ * causal_period > 0 masks row r to its first (r % causal_period) + 1 + causal_offset entries
+ * (the prefix identity of causal self-attention; no counterpart in the reference, which has no mask) */
+fdx_status fdx_softmax_f32(const float* x, int64_t rows, int depth, int causal_period, int causal_offset,
+    float* out);
+/* rows of `table` selected by float ids truncated to size_t (include/fdeep/layers/embedding_layer.hpp:38-58).
+ * error_flag_dev (may be NULL) is set to 1 on the device if an id is out of range. */
+fdx_status fdx_embedding_f32(const float* ids, int64_t count, const float* table, int input_dim, int output_dim,
+    float* out, int* error_flag_dev);
+/* first maximum of each row (tensor_max_pos, include/fdeep/tensor.hpp:281-302) */
+fdx_status fdx_argmax_f32(const float* x, int64_t rows, int depth, int32_t* out_idx, float* out_val);
+
+/*
+ * MultiHeadAttention core for already projected q/k/v (prefill shape):
+ *   out[b][t][h][:] = softmax_s(scale * q[b][t][h] . k[b][s][h]) * v[b][s][h]
+ * q [b][t][heads*dk], k [b][s][heads*dk], v [b][s][heads*dv], out [b][t][heads*dv]
+ * (apply_head, include/fdeep/layers/multi_head_attention_layer.hpp:74-95).  causal != 0 lets query t
+ * see keys 0..t+(s-t_len) only.  scratch_dev must hold fdx_mha_scratch_bytes().
+ */
+size_t fdx_mha_scratch_bytes(int batch, int heads, int t, int s, int dv);
+fdx_status fdx_mha_prefill_f32(const float* q, const float* k, const float* v, int batch, int t, int s,
+    int heads, int dk, int dv, int causal, float* out, void* scratch_dev);
+/*
+ * Decode step: one query row per sequence against a key/value cache.
+ * q [b][heads*dk]; k_cache [b][max_len][heads*dk], v_cache [b][max_len][heads*dv] (token-major, so the
+ * projection GEMM of a new token writes its row in place); len = keys visible (incl. the newest).
+ */
+fdx_status fdx_mha_decode_f32(const float* q, const float* k_cache, const float* v_cache, int batch, int heads,
+    int dk, int dv, int len, int max_len, float* out);
+
+/* TF window geometry shared by conv and pooling (include/fdeep/convolution.hpp:320-396):
+ * padding 0 valid, 1 same, 2 causal; geom = pad_top, pad_bottom, pad_left, pad_right, out_h, out_w */
+fdx_status fdx_window_geometry(int in_h, int in_w, int k_h, int k_w, int s_h, int s_w, int padding, int* geom);
+
+/* ---------------------------------------------------------------- whole models */
+typedef struct fdx_model fdx_model;
+typedef struct fdx_session fdx_session;
+
+/*
+ * Parses a converted-JSON model (the output format of keras_export/convert_model.py:971-1001),
+ * uploads the weights once (they stay resident in HBM) and builds the launch plan.
+ * Replaces read_model (include/fdeep/model.hpp:198-281).  verify != 0 replays the file's embedded
+ * test cases with absolute tolerance verify_epsilon (model.hpp:254-267, import_model.hpp:1990-2021).
+ */
+fdx_status fdx_model_create(const char* json, size_t len, int verify, float verify_epsilon, fdx_model** out);
+fdx_status fdx_model_destroy(fdx_model* m);
+fdx_status fdx_model_name(const fdx_model* m, const char** name, const char** hash);
+/* number of inputs/outputs and their shapes: rank and dims (-1 = variable), model.hpp:66-96 */
+fdx_status fdx_model_io_count(const fdx_model* m, int* n_inputs, int* n_outputs);
+fdx_status fdx_model_io_shape(const fdx_model* m, int is_output, int index, int* rank, int64_t* dims5);
+/*
+ * predict / predict_multi (include/fdeep/model.hpp:23-42,132-151): `batch` independent samples in one
+ * launch sequence.  in[i] points at batch * volume(in_dims[i]) floats (sample-major); in_dims holds
+ * 5 right-aligned dims per input and in_ranks its rank (the reference rejects a rank mismatch,
+ * tensor_shape.hpp:246-250).  Outputs: out[i] receives batch * volume floats; out_dims/out_ranks are
+ * written per output.  Host-pointer and device-pointer variants.
+ */
+fdx_status fdx_model_predict(fdx_model* m, int batch, const float* const* in, const int64_t* in_dims,
+    const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks);
+fdx_status fdx_model_predict_dev(fdx_model* m, int batch, const float* const* in_dev, const int64_t* in_dims,
+    const int* in_ranks, float* const* out_dev, int64_t* out_dims, int* out_ranks);
+/* output shapes for given input shapes without running anything */
+fdx_status fdx_model_infer_shapes(fdx_model* m, const int64_t* in_dims, const int* in_ranks, int64_t* out_dims,
+    int* out_ranks);
+/* 2 * multiply-accumulates of the Conv2D/Dense/attention contractions of the last planned batch */
+fdx_status fdx_model_last_flops(const fdx_model* m, double* flops);
+
+/*
+ * Autoregressive session over a decoder model with inputs (ids, positions) and one logits output:
+ * causal self-attention with projected keys/values cached in HBM.  The reference has neither a mask
+ * nor a cache (layers/multi_head_attention_layer.hpp:74-95); position t of a session equals the
+ * reference's MultiHeadAttention(query = x[t:t+1], value = x[0:t+1]) (same file, :98-103).
+ * prefill consumes `t` ids per sequence ([batch][t], float), decode_step one id per sequence.
+ * logits_dev (may be NULL) receives [batch][vocab] of the last position; next_ids_dev (may be NULL)
+ * the greedy argmax as floats (first maximum wins, tensor.hpp:281-302).
+ */
+fdx_status fdx_session_create(fdx_model* m, int batch, int max_len, fdx_session** out);
+fdx_status fdx_session_destroy(fdx_session* s);
+fdx_status fdx_session_reset(fdx_session* s);
+fdx_status fdx_session_prefill(fdx_session* s, const float* ids_dev, int t, float* logits_dev, float* next_ids_dev);
+fdx_status fdx_session_decode_step(fdx_session* s, const float* ids_dev, float* logits_dev, float* next_ids_dev);
+/* runs `steps` greedy decode steps feeding each step's argmax back in; tokens_dev gets [steps][batch] floats */
+fdx_status fdx_session_decode_greedy(fdx_session* s, const float* first_ids_dev, int steps, float* tokens_dev,
+    float* last_logits_dev);
+fdx_status fdx_session_length(const fdx_session* s, int* len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -499,7 +499,9 @@ int fdo_mha(const float* query, int t, const float* value, const float* key, int
         free(q); free(k); free(v); free(sc); free(merged); free(wh);
         return -2;
     }
-    const float scale = (float)(1.0 / sqrt((double)dk));
+    /* 1 / std::sqrt(size_t) is a double; the float score is multiplied in double and
+     * narrowed on store (multi_head_attention_layer.hpp:92-93) */
+    const double scale = 1.0 / sqrt((double)dk);
     for (int h = 0; h < heads; ++h) {
         /* per-head weight slice along H: W[:, h, :] */
         for (int i = 0; i < d; ++i)
@@ -516,7 +518,7 @@ int fdo_mha(const float* query, int t, const float* value, const float* key, int
                 float acc = 0.0f;
                 for (int z = 0; z < dk; ++z)
                     acc += q[(size_t)i * dk + z] * k[(size_t)j * dk + z];
-                sc[(size_t)i * s + j] = acc * scale;
+                sc[(size_t)i * s + j] = (float)((double)acc * scale);
             }
         fdo_softmax(sc, t, s, sc);
         for (int i = 0; i < t; ++i) {

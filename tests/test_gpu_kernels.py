@@ -1,0 +1,284 @@
+"""Parity of every HIP kernel launcher of the C ABI against the CPU oracle on the same seeded
+inputs.  Tolerance (floating point, summation order differs): per output tensor
+max|gpu - ref| / max|ref| <= 1e-4; integer results (argmax) are exact."""
+import zlib
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def rng_for(*key):
+    return np.random.default_rng(zlib.crc32(repr(key).encode()))
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+CONV_CASES = [
+    # n, h, w, cin, cout, kh, kw, strides, dilation, padding
+    (2, 8, 9, 3, 5, 3, 3, (1, 1), (1, 1), "same"),       # scalar gather path (cin % 4 != 0)
+    (2, 32, 32, 3, 16, 3, 3, (1, 1), (1, 1), "same"),    # small-CNN first layer
+    (3, 15, 15, 16, 32, 3, 3, (1, 1), (1, 1), "valid"),  # small-CNN second layer
+    (1, 30, 30, 3, 64, 7, 7, (2, 2), (1, 1), "valid"),   # ResNet stem shape, K = 147
+    (2, 14, 14, 64, 64, 3, 3, (1, 1), (1, 1), "same"),   # bottleneck 3x3
+    (2, 14, 14, 64, 256, 1, 1, (1, 1), (1, 1), "valid"),  # pointwise -> plain GEMM path
+    (2, 14, 14, 256, 128, 1, 1, (2, 2), (1, 1), "valid"),  # strided pointwise
+    (1, 11, 10, 4, 6, 3, 2, (2, 3), (1, 1), "same"),     # cin = 4 < slab, ragged everything
+    (1, 12, 13, 8, 12, 2, 3, (1, 1), (2, 3), "same"),    # dilation
+    (1, 9, 9, 20, 40, 5, 5, (1, 1), (1, 1), "same"),     # cin not a multiple of the 16-wide slab
+    (4, 7, 7, 512, 160, 1, 1, (1, 1), (1, 1), "valid"),  # M = 196, N not a tile multiple
+    (1, 5, 5, 8, 8, 3, 3, (1, 1), (1, 1), "causal"),
+]
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_vs_oracle(fdx, oracle, case, tile):
+    n, h, w, cin, cout, kh, kw, strides, dilation, padding = case
+    say("conv2d", case, "tile", tile)
+    r = rng_for("conv", case)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, kh, kw, cin)) / np.sqrt(kh * kw * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, kh, kw, cin)
+    want = np.stack([oracle.conv2d(x[i], wo, b, cout, kh, kw, strides, dilation, padding) for i in range(n)])
+    fdx.lib.fdx_debug_force_tile(tile)
+    try:
+        got = fdx.conv2d(x, wj, b, strides, dilation, padding)
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(got, want) <= TOL
+
+
+def test_conv2d_epilogue_residual_relu(fdx, oracle):
+    say("conv2d epilogue")
+    r = rng_for("conv-epi")
+    n, h, w, cin, cout = 2, 10, 10, 32, 48
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, 3, 3, cin)) / np.sqrt(9 * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    res = r.standard_normal((n, h, w, cout)).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, 3, 3, cin)
+    conv = np.stack([oracle.conv2d(x[i], wo, b, cout, 3, 3, (1, 1), (1, 1), "same") for i in range(n)])
+    for act, f in [(fdx.relu_act(), lambda v: oracle.relu(v)), (fdx.relu_act(6.0), lambda v: oracle.relu(v, 6.0, 0.0, 0.0)),
+                   (fdx.relu_act(4.0, 0.1, 1.0), lambda v: oracle.relu(v, 4.0, 0.1, 1.0)), (fdx.gelu_act(), oracle.gelu),
+                   (None, lambda v: v)]:
+        got = fdx.conv2d(x, wj, b, padding="same", residual=res, act=act)
+        assert rel(got, f(oracle.add(res, conv))) <= TOL
+    got = fdx.conv2d(x, wj, None, padding="same")
+    want = np.stack([oracle.conv2d(x[i], wo, None, cout, 3, 3, (1, 1), (1, 1), "same") for i in range(n)])
+    assert rel(got, want) <= TOL
+
+
+GEMM_CASES = [(1, 10, 32), (16, 768, 768), (37, 50, 29), (256, 2048, 512), (130, 1000, 2048), (5, 3, 7), (64, 64, 16),
+              (300, 96, 100)]
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("m,n,k", GEMM_CASES)
+def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
+    say("gemm", m, n, k, "tile", tile)
+    r = rng_for("gemm", m, n, k)
+    a = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)  # Dense layout [in][out]
+    b = r.standard_normal(n).astype(np.float32)
+    want = oracle.dense(a, w.reshape(-1), b, n)
+    fdx.lib.fdx_debug_force_tile(tile)
+    try:
+        got = fdx.gemm(a, w.T, b)
+        got_gelu = fdx.gemm(a, w.T, b, act=fdx.gelu_act())
+        got_row = fdx.gemm(w.T, a, b, bias_per_row=True, alpha=0.5)  # swapped operands: (a w)^T
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(got, want) <= TOL
+    assert rel(got_gelu, oracle.gelu(want)) <= TOL
+    want_row = 0.5 * (a.astype(np.float64) @ w.astype(np.float64)).T + b[:, None]
+    assert rel(got_row, want_row) <= TOL
+
+
+@pytest.mark.parametrize("case", [
+    (2, 9, 8, 8, 3, 3, (1, 1), (1, 1), "same"), (2, 9, 8, 6, 3, 3, (2, 2), (1, 1), "same"),
+    (1, 10, 11, 5, 3, 3, (2, 2), (1, 1), "valid"), (2, 12, 12, 4, 3, 3, (1, 1), (2, 2), "same"),
+    (3, 28, 28, 96, 3, 3, (2, 2), (1, 1), "valid"), (2, 14, 14, 144, 3, 3, (1, 1), (1, 1), "same")])
+def test_dwconv_vs_oracle(fdx, oracle, case):
+    n, h, w, c, kh, kw, strides, dilation, padding = case
+    say("dwconv", case)
+    r = rng_for("dw", case)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    wj = r.standard_normal((c, kh, kw)).astype(np.float32)
+    b = r.standard_normal(c).astype(np.float32)
+    want = np.stack([oracle.depthwise_conv2d(x[i], wj, b, kh, kw, strides, dilation, padding) for i in range(n)])
+    assert rel(fdx.dwconv2d(x, wj, b, strides, dilation, padding), want) <= TOL
+    got6 = fdx.dwconv2d(x, wj, None, strides, dilation, padding, act=fdx.relu_act(6.0))
+    want6 = np.stack([oracle.relu(oracle.depthwise_conv2d(x[i], wj, None, kh, kw, strides, dilation, padding), 6.0, 0.0, 0.0)
+                      for i in range(n)])
+    assert rel(got6, want6) <= TOL
+
+
+@pytest.mark.parametrize("case", [(2, 8, 8, 5, 2, 2, "valid"), (2, 9, 7, 4, 3, 2, "same"), (1, 9, 7, 3, 3, 2, "valid"),
+                                  (2, 5, 5, 64, 2, 1, "same"), (1, 7, 10, 6, 3, 3, "same")])
+@pytest.mark.parametrize("mode", ["max", "avg"])
+def test_pool_vs_oracle(fdx, oracle, case, mode):
+    n, h, w, c, k, s, padding = case
+    say("pool", case, mode)
+    x = rng_for("pool", case).standard_normal((n, h, w, c)).astype(np.float32)
+    want = np.stack([oracle.pool2d(x[i], (k, k), (s, s), padding, mode) for i in range(n)])
+    got = fdx.pool2d(x, (k, k), (s, s), padding, mode)
+    assert rel(got, want) <= 1e-6
+
+
+def test_pool_with_folded_zero_padding(fdx, oracle):
+    say("pool folded zero pad")
+    x = rng_for("poolz").standard_normal((2, 10, 10, 8)).astype(np.float32) - 2.0  # mostly negative: zeros must win
+    for mode in ("max", "avg"):
+        for padding in ("valid", "same"):
+            padded = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0)))
+            want = np.stack([oracle.pool2d(padded[i], (3, 3), (2, 2), padding, mode) for i in range(2)])
+            got = fdx.pool2d(x, (3, 3), (2, 2), padding, mode, zero_frame=(1, 1, 1, 1))
+            assert rel(got, want) <= 1e-6
+
+
+def test_global_pool_add_act_affine_pad(fdx, oracle):
+    say("glue kernels")
+    r = rng_for("glue")
+    x = r.standard_normal((3, 7, 7, 100)).astype(np.float32)
+    for mode in ("avg", "max"):
+        want = np.stack([oracle.global_pool(x[i], mode) for i in range(3)])
+        assert rel(fdx.global_pool(x, mode), want) <= 1e-6
+    y = r.standard_normal(x.shape).astype(np.float32)
+    assert np.array_equal(fdx.add(x, y), x + y)
+    assert np.array_equal(fdx.add(x, y, fdx.relu_act()), np.maximum(x + y, 0))
+    assert np.array_equal(fdx.add(x, y[0]), x + y[0])  # broadcast over the batch
+    odd = r.standard_normal(1001).astype(np.float32)
+    assert np.array_equal(fdx.add(odd, odd), odd + odd)
+    assert rel(fdx.activation(x, fdx.gelu_act()), oracle.gelu(x)) <= 1e-6
+    assert np.array_equal(fdx.activation(x, fdx.relu_act(6.0)), oracle.relu(x, 6.0, 0.0, 0.0))
+    assert rel(fdx.activation(x, fdx.relu_act(4.0, 0.1, 1.0)), oracle.relu(x, 4.0, 0.1, 1.0)) <= 1e-6
+    mean, beta = r.standard_normal(100).astype(np.float32), r.standard_normal(100).astype(np.float32)
+    var, gamma = (0.5 + r.random(100)).astype(np.float32), (0.5 + r.random(100)).astype(np.float32)
+    inv = (gamma / np.sqrt(var + np.float32(1e-3))).astype(np.float32)
+    got = fdx.channel_affine(x, inv, (beta - mean * inv).astype(np.float32))
+    assert rel(got, oracle.batchnorm(x, mean, var, gamma, beta, 1e-3)) <= 1e-5
+    got = fdx.zero_pad2d(x, 1, 2, 3, 0)
+    assert np.array_equal(got, np.pad(x, ((0, 0), (1, 2), (3, 0), (0, 0))))
+
+
+@pytest.mark.parametrize("rows,depth", [(5, 33), (256, 512), (16, 768), (7, 1000), (3, 4097)])
+def test_layernorm_vs_oracle(fdx, oracle, rows, depth):
+    say("layernorm", rows, depth)
+    r = rng_for("ln", rows, depth)
+    x = (r.standard_normal((rows, depth)) * 3 + 1).astype(np.float32)
+    g, b = r.standard_normal(depth).astype(np.float32), r.standard_normal(depth).astype(np.float32)
+    assert rel(fdx.layernorm(x, g, b, 1e-3), oracle.layernorm(x, g, b, 1e-3)) <= TOL
+    assert rel(fdx.layernorm(x, None, None, 1e-5), oracle.layernorm(x, None, None, 1e-5)) <= TOL
+
+
+@pytest.mark.parametrize("rows,depth", [(4, 10), (64, 256), (5, 1000), (3, 50257), (9, 1)])
+def test_softmax_vs_oracle(fdx, oracle, rows, depth):
+    say("softmax", rows, depth)
+    x = (rng_for("sm", rows, depth).standard_normal((rows, depth)) * 6).astype(np.float32)
+    assert rel(fdx.softmax(x), oracle.softmax(x)) <= TOL
+    big = x * 100  # saturating inputs keep finite outputs that sum to one
+    got = fdx.softmax(big)
+    assert np.isfinite(got).all() and np.abs(got.sum(-1) - 1).max() < 1e-4
+
+
+def test_softmax_causal_prefix(fdx, oracle):
+    say("softmax causal")
+    t, s = 5, 8
+    x = rng_for("smc").standard_normal((3 * t, s)).astype(np.float32)
+    got = fdx.softmax(x, causal_period=t, causal_offset=s - t)
+    for row in range(3 * t):
+        vis = row % t + 1 + (s - t)
+        assert rel(got[row, :vis], oracle.softmax(x[row, :vis])) <= TOL
+        assert (got[row, vis:] == 0).all()
+
+
+def test_embedding_and_argmax(fdx, oracle):
+    say("embedding argmax")
+    r = rng_for("emb")
+    table = r.standard_normal((50, 24)).astype(np.float32)
+    ids = np.array([0, 49, 3.7, 3, 17], np.float32)
+    assert np.array_equal(fdx.embedding(ids, table), oracle.embedding(ids, table.reshape(-1), 50, 24))
+    with pytest.raises(fdx.FdxError):
+        fdx.embedding(np.array([50], np.float32), table)
+    x = r.standard_normal((6, 50257)).astype(np.float32)
+    x[0, 100] = x[0, 40000] = 50.0  # tie: the first maximum wins
+    x[1, :] = -1.0
+    idx, val = fdx.argmax(x)
+    want = [oracle.argmax(x[i]) for i in range(6)]
+    assert idx.tolist() == want and idx[0] == 100 and idx[1] == 0
+    assert np.array_equal(val, x[np.arange(6), idx])
+
+
+def numpy_attention(q, k, v, heads, dk, dv, causal):
+    b, t, _ = q.shape
+    s = k.shape[1]
+    out = np.zeros((b, t, heads * dv))
+    for bi in range(b):
+        for h in range(heads):
+            Q, K, V = q[bi, :, h * dk:(h + 1) * dk], k[bi, :, h * dk:(h + 1) * dk], v[bi, :, h * dv:(h + 1) * dv]
+            S = Q.astype(np.float64) @ K.astype(np.float64).T / np.sqrt(dk)
+            if causal:
+                S = np.where(np.arange(s)[None, :] <= np.arange(t)[:, None] + (s - t), S, -np.inf)
+            P = np.exp(S - S.max(-1, keepdims=True))
+            P /= P.sum(-1, keepdims=True)
+            out[bi, :, h * dv:(h + 1) * dv] = P @ V
+    return out
+
+
+@pytest.mark.parametrize("b,t,s,heads,dk,dv,causal", [(2, 5, 7, 3, 4, 5, False), (2, 16, 16, 2, 64, 64, True),
+                                                      (1, 33, 33, 4, 16, 16, True), (2, 64, 64, 8, 64, 64, False),
+                                                      (1, 3, 9, 2, 8, 8, True)])
+def test_mha_prefill(fdx, oracle, b, t, s, heads, dk, dv, causal):
+    say("mha prefill", b, t, s, heads, dk, dv, causal)
+    r = rng_for("mha", b, t, s, heads, dk, dv, causal)
+    q = r.standard_normal((b, t, heads * dk)).astype(np.float32)
+    k = r.standard_normal((b, s, heads * dk)).astype(np.float32)
+    v = r.standard_normal((b, s, heads * dv)).astype(np.float32)
+    got = fdx.mha_prefill(q, k, v, heads, dk, dv, causal)
+    assert rel(got, numpy_attention(q, k, v, heads, dk, dv, causal)) <= TOL
+    if not causal:  # the oracle's MultiHeadAttention with identity projections is this core
+        eye_k = np.zeros((heads * dk, heads, dk), np.float32)
+        eye_v = np.zeros((heads * dv, heads, dv), np.float32)
+        for h in range(heads):
+            eye_k[h * dk:(h + 1) * dk, h] = np.eye(dk)
+            eye_v[h * dv:(h + 1) * dv, h] = np.eye(dv)
+        if dk == dv:
+            w = [eye_k.reshape(-1), eye_k.reshape(-1), eye_v.reshape(-1), np.eye(heads * dv, dtype=np.float32).reshape(-1)]
+            want = oracle.mha(q[0], v[0], k[0], heads, dk, dv, w, False)
+            assert rel(got[0], want) <= TOL
+
+
+@pytest.mark.parametrize("b,heads,dk,dv,length,max_len", [(2, 3, 8, 8, 5, 9), (16, 12, 64, 64, 129, 256),
+                                                          (3, 2, 64, 32, 256, 256), (1, 1, 6, 10, 1, 4)])
+def test_mha_decode(fdx, b, heads, dk, dv, length, max_len):
+    say("mha decode", b, heads, dk, dv, length, max_len)
+    r = rng_for("dec", b, heads, dk, dv, length)
+    q = r.standard_normal((b, heads * dk)).astype(np.float32)
+    kc = r.standard_normal((b, max_len, heads * dk)).astype(np.float32)
+    vc = r.standard_normal((b, max_len, heads * dv)).astype(np.float32)
+    got = fdx.mha_decode(q, kc, vc, heads, dk, dv, length)
+    want = numpy_attention(q[:, None], kc[:, :length], vc[:, :length], heads, dk, dv, False)[:, 0]
+    assert rel(got, want) <= TOL
+
+
+def test_launcher_argument_errors(fdx):
+    say("argument errors")
+    a = fdx.DevBuf(64)
+    with pytest.raises(fdx.FdxError):
+        fdx.check(fdx.lib.fdx_gemm_bias_act_f32(None, 4, None, 4, 1, 1, 4, fdx.ctypes.c_float(1), None, 0, None, None, None, 1, None))
+    with pytest.raises(fdx.FdxError):
+        fdx.check(fdx.lib.fdx_pool2d_nhwc_f32(fdx._dp(a), 1, 2, 2, 1, 2, 2, 1, 1, 0, 0, 0, 0, 0, 0, 1, 1, 7, fdx._dp(a)))
+    with pytest.raises(fdx.FdxError):
+        fdx.window_geometry(0, 4, 3, 3, 1, 1, "same")
