@@ -283,3 +283,86 @@ def mha_decode(q, k_cache, v_cache, heads, dk, dv, length):
     out = DevBuf(4 * b * heads * dv)
     check(lib.fdx_mha_decode_f32(_dp(dq), _dp(dkc), _dp(dvc), b, heads, dk, dv, length, max_len, _dp(out)))
     return out.to_host((b, heads * dv))
+
+
+# ------------------------------------------------------------------ whole models
+
+class Model:
+    """A converted-JSON model resident on the GPU (fdx_model_*).  `source` is the file's bytes or a path."""
+
+    def __init__(self, source, verify=True, verify_epsilon=1e-4):
+        if isinstance(source, str):
+            if not os.path.exists(source):
+                raise FdxError("Can not open " + source)
+            with open(source, "rb") as f:
+                source = f.read()
+        self._h = ctypes.c_void_p()
+        check(lib.fdx_model_create(source, ctypes.c_size_t(len(source)), int(verify), ctypes.c_float(verify_epsilon),
+                                   ctypes.byref(self._h)))
+        ni, no = ctypes.c_int(), ctypes.c_int()
+        check(lib.fdx_model_io_count(self._h, ctypes.byref(ni), ctypes.byref(no)))
+        self.n_inputs, self.n_outputs = ni.value, no.value
+        self.input_shapes = [self._io_shape(0, i) for i in range(self.n_inputs)]
+        self.output_shapes = [self._io_shape(1, i) for i in range(self.n_outputs)]
+        name, hsh = ctypes.c_char_p(), ctypes.c_char_p()
+        check(lib.fdx_model_name(self._h, ctypes.byref(name), ctypes.byref(hsh)))
+        self.name, self.hash = name.value.decode(), hsh.value.decode()
+
+    def _io_shape(self, is_output, index):
+        rank, dims = ctypes.c_int(), (ctypes.c_int64 * 5)()
+        check(lib.fdx_model_io_shape(self._h, is_output, index, ctypes.byref(rank), dims))
+        return tuple(None if d < 0 else int(d) for d in list(dims)[5 - rank.value:])
+
+    def _dims(self, shapes):
+        dims = (ctypes.c_int64 * (5 * len(shapes)))(*([1] * (5 * len(shapes))))
+        ranks = (ctypes.c_int * len(shapes))()
+        for i, s in enumerate(shapes):
+            ranks[i] = len(s)
+            for k, d in enumerate(s):
+                dims[i * 5 + 5 - len(s) + k] = d
+        return dims, ranks
+
+    def infer_shapes(self, sample_shapes):
+        dims, ranks = self._dims(sample_shapes)
+        od, orank = (ctypes.c_int64 * (5 * self.n_outputs))(), (ctypes.c_int * self.n_outputs)()
+        check(lib.fdx_model_infer_shapes(self._h, dims, ranks, od, orank))
+        return [tuple(int(d) for d in od[i * 5 + 5 - orank[i]:i * 5 + 5]) for i in range(self.n_outputs)]
+
+    def predict(self, inputs):
+        """inputs: one array per model input, shaped [batch, *sample_shape]; returns arrays [batch, *out_shape].
+        All samples go through one batched launch sequence (predict_multi semantics)."""
+        inputs = [np.ascontiguousarray(x, np.float32) for x in inputs]
+        if len(inputs) != self.n_inputs:
+            raise FdxError("Invalid inputs shape.\nThe model takes %d inputs" % self.n_inputs)
+        batch = inputs[0].shape[0]
+        sample_shapes = [x.shape[1:] for x in inputs]
+        dims, ranks = self._dims(sample_shapes)
+        out_shapes = self.infer_shapes(sample_shapes)
+        outs = [np.empty((batch,) + s, np.float32) for s in out_shapes]
+        ip = (c_float_p * self.n_inputs)(*[x.ctypes.data_as(c_float_p) for x in inputs])
+        op = (c_float_p * self.n_outputs)(*[o.ctypes.data_as(c_float_p) for o in outs])
+        check(lib.fdx_model_predict(self._h, batch, ip, dims, ranks, op, None, None))
+        return outs
+
+    def predict_dev(self, batch, in_bufs, sample_shapes, out_bufs):
+        """Device-resident variant: in_bufs / out_bufs are DevBuf objects; asynchronous (call sync())."""
+        dims, ranks = self._dims(sample_shapes)
+        ip = (c_float_p * self.n_inputs)(*[_dp(b) for b in in_bufs])
+        op = (c_float_p * self.n_outputs)(*[_dp(b) for b in out_bufs])
+        check(lib.fdx_model_predict_dev(self._h, batch, ip, dims, ranks, op, None, None))
+
+    def last_flops(self):
+        f = ctypes.c_double()
+        check(lib.fdx_model_last_flops(self._h, ctypes.byref(f)))
+        return f.value
+
+    def close(self):
+        if self._h:
+            check(lib.fdx_model_destroy(self._h))
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

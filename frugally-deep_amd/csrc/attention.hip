@@ -11,7 +11,7 @@
 #include "common.hpp"
 
 namespace fdx {
-fdx_status transpose_launch(const float* in, int batch, int rows, int cols, float* out);
+fdx_status transpose_launch(const float* in, int batch, int rows, int cols, int64_t ld_in, int64_t in_batch, float* out);
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -103,8 +103,12 @@ extern "C" size_t fdx_mha_scratch_bytes(int batch, int heads, int t, int s, int 
     return sizeof(float) * ((size_t)batch * heads * t * s + (size_t)batch * heads * dv * s) + 256;
 }
 
-extern "C" fdx_status fdx_mha_prefill_f32(const float* q, const float* k, const float* v, int batch, int t, int s,
-    int heads, int dk, int dv, int causal, float* out, void* scratch_dev)
+namespace fdx {
+// q/k/v/out rows may be strided (ld*) and sequences apart by *_batch elements, so the key/value
+// operands can live in a token-major cache and q/k/v can be column blocks of one fused projection.
+fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, const float* k, int64_t ldk, int64_t k_batch,
+    const float* v, int64_t ldv, int64_t v_batch, int batch, int t, int s, int heads, int dk, int dv, int causal,
+    float* out, int64_t ldo, int64_t o_batch, void* scratch_dev)
 {
     FDX_REQUIRE(q && k && v && out && scratch_dev, "mha_prefill: null pointer");
     FDX_REQUIRE(batch > 0 && t > 0 && s > 0 && heads > 0 && dk > 0 && dv > 0, "mha_prefill: bad shape");
@@ -112,28 +116,37 @@ extern "C" fdx_status fdx_mha_prefill_f32(const float* q, const float* k, const 
     FDX_REQUIRE((int64_t)batch * heads <= 65535, "mha_prefill: batch * heads too large");
     float* scores = static_cast<float*>(scratch_dev);
     float* vt = scores + (((size_t)batch * heads * t * s + 3) & ~(size_t)3);
-    const int64_t qk_row = (int64_t)heads * dk, v_row = (int64_t)heads * dv;
+    const int64_t v_row = (int64_t)heads * dv;
     // 1 / sqrt(key_dim) applied to the scores after the product (multi_head_attention_layer.hpp:91-93)
     const float scale = (float)(1.0 / std::sqrt((double)dk));
     fdx_gemm_batch bt {};
     bt.batch = batch * heads;
     bt.inner = heads;
-    bt.a_outer = (int64_t)t * qk_row; bt.a_inner = dk;
-    bt.b_outer = (int64_t)s * qk_row; bt.b_inner = dk;
+    bt.a_outer = q_batch; bt.a_inner = dk;
+    bt.b_outer = k_batch; bt.b_inner = dk;
     bt.c_outer = (int64_t)heads * t * s; bt.c_inner = (int64_t)t * s;
-    fdx_status st = fdx_gemm_bias_act_f32(q, qk_row, k, qk_row, t, s, dk, scale, nullptr, 0, nullptr, nullptr, scores, s, &bt);
+    fdx_status st = fdx_gemm_bias_act_f32(q, ldq, k, ldk, t, s, dk, scale, nullptr, 0, nullptr, nullptr, scores, s, &bt);
     if (st != FDX_OK)
         return st;
     st = fdx_softmax_f32(scores, (int64_t)batch * heads * t, s, causal ? t : 0, causal ? s - t : 0, scores);
     if (st != FDX_OK)
         return st;
-    st = transpose_launch(v, batch, s, (int)v_row, vt); // [b][s][H*dv] -> [b][H*dv][s]
+    st = transpose_launch(v, batch, s, (int)v_row, ldv, v_batch, vt); // [b][s][H*dv] -> [b][H*dv][s]
     if (st != FDX_OK)
         return st;
     bt.a_outer = (int64_t)heads * t * s; bt.a_inner = (int64_t)t * s;
     bt.b_outer = v_row * s; bt.b_inner = (int64_t)dv * s;
-    bt.c_outer = (int64_t)t * v_row; bt.c_inner = dv;
-    return fdx_gemm_bias_act_f32(scores, s, vt, s, t, dv, s, 1.0f, nullptr, 0, nullptr, nullptr, out, v_row, &bt);
+    bt.c_outer = o_batch; bt.c_inner = dv;
+    return fdx_gemm_bias_act_f32(scores, s, vt, s, t, dv, s, 1.0f, nullptr, 0, nullptr, nullptr, out, ldo, &bt);
+}
+}
+
+extern "C" fdx_status fdx_mha_prefill_f32(const float* q, const float* k, const float* v, int batch, int t, int s,
+    int heads, int dk, int dv, int causal, float* out, void* scratch_dev)
+{
+    const int64_t qk = (int64_t)heads * dk, vr = (int64_t)heads * dv;
+    return fdx::mha_prefill_strided(q, qk, t * qk, k, qk, s * qk, v, vr, s * vr, batch, t, s, heads, dk, dv, causal, out, vr,
+        t * vr, scratch_dev);
 }
 
 extern "C" fdx_status fdx_mha_decode_f32(const float* q, const float* k_cache, const float* v_cache, int batch, int heads,

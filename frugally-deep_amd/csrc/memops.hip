@@ -230,20 +230,32 @@ __global__ void zero_pad_kernel(const float* __restrict__ in, float* __restrict_
     }
 }
 
-__global__ void transpose_kernel(const float* __restrict__ in, float* __restrict__ out, int rows, int cols)
+// in: rows x cols with row stride ld_in; out: cols x rows packed.  blockIdx.z walks independent matrices.
+__global__ void transpose_kernel(const float* __restrict__ in, float* __restrict__ out, int rows, int cols,
+    int64_t ld_in, int64_t in_batch, int64_t out_batch)
 {
     __shared__ float tile[32][33];
-    in += (int64_t)blockIdx.z * rows * cols; // blockIdx.z: independent matrices stored back to back
-    out += (int64_t)blockIdx.z * rows * cols;
+    in += (int64_t)blockIdx.z * in_batch;
+    out += (int64_t)blockIdx.z * out_batch;
     const int bx = blockIdx.x * 32, by = blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 256 threads: 8 rows per pass
     for (int r = ty; r < 32; r += 8)
         if (by + r < rows && bx + tx < cols)
-            tile[r][tx] = in[(int64_t)(by + r) * cols + bx + tx];
+            tile[r][tx] = in[(int64_t)(by + r) * ld_in + bx + tx];
     __syncthreads();
     for (int r = ty; r < 32; r += 8)
         if (bx + r < cols && by + tx < rows)
             out[(int64_t)(bx + r) * rows + by + tx] = tile[tx][r];
+}
+
+// out[r][:] = in[offset + r * row_stride + :]  (last position of every sequence, for instance)
+__global__ void gather_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int depth, int64_t row_stride,
+    int64_t offset)
+{
+    const float* src = in + offset + (int64_t)blockIdx.x * row_stride;
+    float* dst = out + (int64_t)blockIdx.x * depth;
+    for (int z = threadIdx.x; z < depth; z += blockDim.x)
+        dst[z] = src[z];
 }
 
 // ------------------------------------------------------------------ LayerNorm
@@ -539,11 +551,19 @@ extern "C" fdx_status fdx_zero_pad2d_nhwc_f32(const float* in, int n, int h, int
 }
 
 namespace fdx {
-fdx_status transpose_launch(const float* in, int batch, int rows, int cols, float* out)
+fdx_status transpose_launch(const float* in, int batch, int rows, int cols, int64_t ld_in, int64_t in_batch, float* out)
 {
-    FDX_REQUIRE(in && out && rows > 0 && cols > 0 && batch > 0 && batch <= 65535, "transpose: bad arguments");
+    FDX_REQUIRE(in && out && rows > 0 && cols > 0 && batch > 0 && batch <= 65535 && ld_in >= cols, "transpose: bad arguments");
     hipLaunchKernelGGL(transpose_kernel, dim3((cols + 31) / 32, (rows + 31) / 32, batch), dim3(256), 0, stream(), in, out,
-        rows, cols);
+        rows, cols, ld_in, in_batch, (int64_t)rows * cols);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+fdx_status gather_rows_launch(const float* in, int64_t rows, int depth, int64_t row_stride, int64_t offset, float* out)
+{
+    FDX_REQUIRE(in && out && rows > 0 && depth > 0, "gather_rows: bad arguments");
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)rows), dim3(256), 0, stream(), in, out, depth, row_stride, offset);
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }
@@ -551,7 +571,7 @@ fdx_status transpose_launch(const float* in, int batch, int rows, int cols, floa
 
 extern "C" fdx_status fdx_transpose_f32(const float* in, int rows, int cols, float* out)
 {
-    return fdx::transpose_launch(in, 1, rows, cols, out);
+    return fdx::transpose_launch(in, 1, rows, cols, cols, 0, out);
 }
 
 extern "C" fdx_status fdx_layernorm_f32(const float* x, int64_t rows, int depth, const float* gamma, const float* beta,

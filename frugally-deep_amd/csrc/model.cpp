@@ -1,0 +1,1409 @@
+// Loader, load-time fusion, launch planner and executor behind fdx_model_*.
+//
+// Reads the converted-JSON format that frugally-deep's read_model consumes
+// (include/fdeep/model.hpp:198-281, include/fdeep/import_model.hpp), turns the layer graph
+// into a flat op list, fuses what the GPU can do in one pass (BatchNormalization into the
+// preceding convolution's weights, ReLU/GELU and residual Add into GEMM epilogues,
+// ZeroPadding2D into the consumer's padding predicate), uploads the weights once, and runs
+// `batch` independent samples per launch with the batch as the outermost axis.
+#include "model.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <set>
+
+#include "json.hpp"
+
+using namespace fdx;
+using json::Value;
+
+namespace fdx {
+
+Plan::~Plan()
+{
+    for (auto& b : blocks)
+        if (b.p)
+            (void)hipFree(b.p);
+}
+
+float* plan_alloc(Plan& p, size_t bytes, int* block_index)
+{
+    bytes = (bytes + 255) & ~(size_t)255;
+    int best = -1;
+    for (size_t i = 0; i < p.blocks.size(); ++i)
+        if (!p.blocks[i].busy && p.blocks[i].bytes >= bytes && (best < 0 || p.blocks[i].bytes < p.blocks[best].bytes))
+            best = (int)i;
+    if (best < 0) {
+        Block b;
+        if (hipMalloc(&b.p, bytes) != hipSuccess)
+            return nullptr;
+        b.bytes = bytes;
+        p.blocks.push_back(b);
+        best = (int)p.blocks.size() - 1;
+    }
+    p.blocks[best].busy = true;
+    *block_index = best;
+    return static_cast<float*>(p.blocks[best].p);
+}
+
+namespace {
+
+    struct FormatError : std::runtime_error {
+        using std::runtime_error::runtime_error;
+    };
+    struct Unsupported : std::runtime_error {
+        using std::runtime_error::runtime_error;
+    };
+
+    // include/fdeep/import_model.hpp:274-297
+    std::vector<float> decode_floats(const Value& v)
+    {
+        if (!(v.is_array() || v.is_string()))
+            throw FormatError("invalid float array format");
+        std::vector<float> out;
+        if (v.is_array() && v.size() > 0 && v.arr[0].is_number()) {
+            out.reserve(v.size());
+            for (const auto& e : v.arr)
+                out.push_back((float)e.number());
+            return out;
+        }
+        std::vector<uint8_t> bytes;
+        auto feed = [&](const Value& s) {
+            if (!s.is_string() || !base64_decode_append(s.s, s.slen, bytes))
+                throw FormatError("invalid base64 float data");
+        };
+        if (v.is_string())
+            feed(v);
+        else {
+            size_t chars = 0;
+            for (const auto& e : v.arr)
+                chars += e.is_string() ? e.slen : 0;
+            bytes.reserve(chars / 4 * 3 + 8);
+            for (const auto& e : v.arr)
+                feed(e);
+        }
+        if (bytes.size() % 4 != 0)
+            throw FormatError("invalid float vector data");
+        out.resize(bytes.size() / 4);
+        std::memcpy(out.data(), bytes.data(), bytes.size());
+        return out;
+    }
+
+    struct Conn {
+        std::string layer;
+        int node, tensor;
+    };
+
+    // import_model.hpp:323-372
+    Conn conn_from_triple(const Value& v)
+    {
+        if (!v.is_array() || v.size() < 3)
+            throw FormatError("invalid format for inbound node");
+        return { v.at((size_t)0).str(), (int)v.at(1).integer(), (int)v.at(2).integer() };
+    }
+    std::vector<Conn> model_connections(const Value& v)
+    {
+        if (!v.is_array())
+            throw FormatError("input_layers/output_layers must be an array");
+        std::vector<Conn> r;
+        if (v.size() > 0 && !v.arr[0].is_array()) {
+            r.push_back(conn_from_triple(v));
+            return r;
+        }
+        for (const auto& e : v.arr)
+            r.push_back(conn_from_triple(e));
+        return r;
+    }
+    Conn conn_from_arg(const Value& a)
+    {
+        const Value* cfg = a.is_object() ? a.find("config") : nullptr;
+        const Value* kh = cfg ? cfg->find("keras_history") : nullptr;
+        if (!kh)
+            throw FormatError("No keras_history on node connection. Constant-value tensors are not supported.");
+        return conn_from_triple(*kh);
+    }
+    std::vector<std::vector<Conn>> inbound_nodes(const Value& layer)
+    {
+        std::vector<std::vector<Conn>> nodes;
+        const Value* in = layer.find("inbound_nodes");
+        if (!in || !in->is_array())
+            throw FormatError("no inbound nodes");
+        for (const auto& n : in->arr) {
+            const Value& args = n.at("args");
+            if (!args.is_array())
+                throw FormatError("node args need to be an array");
+            std::vector<Conn> c;
+            if (args.size() > 0 && args.arr[0].is_array()) {
+                if (args.size() != 1)
+                    throw FormatError("invalid args format");
+                for (const auto& a : args.arr[0].arr)
+                    c.push_back(conn_from_arg(a));
+            } else {
+                for (const auto& a : args.arr)
+                    c.push_back(conn_from_arg(a));
+            }
+            nodes.push_back(std::move(c));
+        }
+        return nodes;
+    }
+
+    int padding_from(const std::string& s)
+    {
+        if (s == "valid") return 0;
+        if (s == "same") return 1;
+        if (s == "causal") return 2;
+        throw FormatError("no padding");
+    }
+    void pair_from(const Value& v, int& a, int& b)
+    {
+        if (v.is_array() && v.size() == 2) {
+            a = (int)v.at((size_t)0).integer();
+            b = (int)v.at(1).integer();
+        } else if (v.is_array() && v.size() == 1) { // 1-D layers: width only
+            a = 1;
+            b = (int)v.at((size_t)0).integer();
+        } else {
+            a = b = (int)v.integer();
+        }
+    }
+
+    // Layer class names that are the identity at inference (import_model.hpp:1796-1838)
+    const std::set<std::string> kIdentity = { "Identity", "Dropout", "Masking", "ActivityRegularization", "AlphaDropout",
+        "FixedDropout", "SpatialDropout1D", "SpatialDropout2D", "SpatialDropout3D", "GaussianDropout", "GaussianNoise",
+        "RandomBrightness", "RandomContrast", "RandomCrop", "RandomFlip", "RandomHeight", "RandomRotation",
+        "RandomTranslation", "RandomWidth", "RandomZoom" };
+
+    // Sets an activation by name; returns false for "softmax" (caller schedules the softmax kernel).
+    // import_model.hpp:1649-1700; relu parameters only when max_value is present and non-null (:1289-1302).
+    enum class ActParse { Epilogue, Softmax, Linear };
+    ActParse parse_activation(const std::string& type, const Value* cfg, Act& act)
+    {
+        if (type == "linear")
+            return ActParse::Linear;
+        if (type == "softmax")
+            return ActParse::Softmax;
+        if (type == "relu") {
+            act = { FDX_ACT_RELU, 3.402823466e+38f, 0.f, 0.f };
+            const Value* mv = cfg ? cfg->find("max_value") : nullptr;
+            if (mv && !mv->is_null()) {
+                act.max_value = (float)mv->number();
+                act.negative_slope = (float)cfg->at("negative_slope").number();
+                act.threshold = (float)cfg->at("threshold").number();
+            }
+            return ActParse::Epilogue;
+        }
+        if (type == "relu6") {
+            act = { FDX_ACT_RELU, 6.f, 0.f, 0.f };
+            return ActParse::Epilogue;
+        }
+        if (type == "gelu") {
+            const Value* ap = cfg ? cfg->find("approximate") : nullptr;
+            if (ap && !ap->is_null() && ap->boolean())
+                throw FormatError("Gelu with approximate = True is not supported.");
+            act = { FDX_ACT_GELU, 3.402823466e+38f, 0.f, 0.f };
+            return ActParse::Epilogue;
+        }
+        throw Unsupported("unknown activation type: " + type);
+    }
+
+    struct Builder {
+        fdx_model& m;
+        const Value& params;
+        std::map<std::string, const Value*> layers;
+        std::map<std::pair<std::string, int>, int> memo;
+        std::map<std::string, int> input_ops;
+
+        const Value& param(const std::string& layer, const char* key)
+        {
+            const Value* l = params.find(layer.c_str());
+            if (!l)
+                throw FormatError("missing trainable_params for layer " + layer);
+            return l->at(key);
+        }
+
+        int add_op(Op&& op)
+        {
+            m.ops.push_back(std::move(op));
+            return (int)m.ops.size() - 1;
+        }
+
+        // applies config["activation"] after the op (import_model.hpp:1953-1962)
+        int with_fused_activation(int idx, const Value& cfg)
+        {
+            const Value* a = cfg.find("activation");
+            if (!a)
+                return idx;
+            if (!a->is_string())
+                throw FormatError("Layer activation must be a string.");
+            Act act = m.ops[idx].act;
+            switch (parse_activation(a->str(), nullptr, act)) {
+            case ActParse::Linear: return idx;
+            case ActParse::Softmax: m.ops[idx].softmax = true; return idx;
+            case ActParse::Epilogue: m.ops[idx].act = act; return idx;
+            }
+            return idx;
+        }
+
+        int build(const Conn& c)
+        {
+            auto key = std::make_pair(c.layer, c.node);
+            auto it = memo.find(key);
+            if (it != memo.end())
+                return it->second;
+            auto lit = layers.find(c.layer);
+            if (lit == layers.end())
+                throw FormatError("dangling connection to layer " + c.layer);
+            const Value& L = *lit->second;
+            const std::string cls = L.at("class_name").str();
+            const Value& cfg = L.at("config");
+            if (cls == "InputLayer") {
+                auto io = input_ops.find(c.layer);
+                if (io == input_ops.end())
+                    throw FormatError("input layer " + c.layer + " is not listed in input_layers");
+                return memo[key] = io->second;
+            }
+            if (c.tensor != 0)
+                throw Unsupported("layers with several output tensors are not supported: " + c.layer);
+            auto nodes = inbound_nodes(L);
+            if (c.node < 0 || c.node >= (int)nodes.size())
+                throw FormatError("invalid node index for layer " + c.layer);
+            std::vector<int> ins;
+            for (const auto& ic : nodes[c.node])
+                ins.push_back(build(ic));
+            if (ins.empty())
+                throw FormatError("layer without inputs: " + c.layer);
+
+            Op op;
+            op.name = c.layer;
+            op.cls = cls;
+            op.in = ins;
+            int result;
+            if (kIdentity.count(cls)) {
+                op.kind = OpKind::View;
+                result = add_op(std::move(op));
+            } else if (cls == "Conv2D" || cls == "Conv1D") {
+                op.kind = OpKind::Conv2D;
+                op.padding = padding_from(cfg.at("padding").str());
+                pair_from(cfg.at("strides"), op.sy, op.sx);
+                pair_from(cfg.at("dilation_rate"), op.dy, op.dx);
+                pair_from(cfg.at("kernel_size"), op.kh, op.kw);
+                op.cout = (int)cfg.at("filters").integer();
+                op.hw.resize(2);
+                op.hw[0] = decode_floats(param(c.layer, "weights"));
+                if (cfg.at("use_bias").boolean())
+                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                else
+                    op.hw[1].assign(op.cout, 0.f);
+                if ((int)op.hw[1].size() != op.cout)
+                    throw FormatError("size of bias does not match");
+                if (op.hw[0].size() % ((size_t)op.kh * op.kw * op.cout) != 0)
+                    throw FormatError("invalid number of weights");
+                op.n_in = (int)(op.hw[0].size() / ((size_t)op.kh * op.kw * op.cout));
+                result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (cls == "DepthwiseConv2D" || cls == "DepthwiseConv1D") {
+                op.kind = OpKind::DWConv2D;
+                op.padding = padding_from(cfg.at("padding").str());
+                pair_from(cfg.at("strides"), op.sy, op.sx);
+                pair_from(cfg.at("dilation_rate"), op.dy, op.dx);
+                pair_from(cfg.at("kernel_size"), op.kh, op.kw);
+                std::vector<float> sw = decode_floats(param(c.layer, "slice_weights"));
+                if (sw.size() % ((size_t)op.kh * op.kw) != 0)
+                    throw FormatError("invalid number of weights");
+                const int ch = (int)(sw.size() / ((size_t)op.kh * op.kw));
+                op.cout = op.n_in = ch;
+                op.hw.resize(2);
+                op.hw[0].resize(sw.size()); // [c][kh][kw] -> [kh][kw][c]
+                for (int z = 0; z < ch; ++z)
+                    for (int t = 0; t < op.kh * op.kw; ++t)
+                        op.hw[0][(size_t)t * ch + z] = sw[(size_t)z * op.kh * op.kw + t];
+                if (cfg.at("use_bias").boolean())
+                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                else
+                    op.hw[1].assign(ch, 0.f);
+                if ((int)op.hw[1].size() != ch)
+                    throw FormatError("size of bias does not match");
+                result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (cls == "Dense") {
+                op.kind = OpKind::Dense;
+                op.units = (int)cfg.at("units").integer();
+                std::vector<float> w = decode_floats(param(c.layer, "weights"));
+                op.hw.resize(2);
+                if (cfg.at("use_bias").boolean())
+                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                else
+                    op.hw[1].assign(op.units, 0.f);
+                if ((int)op.hw[1].size() != op.units || op.units == 0 || w.size() % (size_t)op.units != 0)
+                    throw FormatError("size of bias does not match");
+                op.n_in = (int)(w.size() / (size_t)op.units);
+                op.hw[0].resize(w.size()); // [in][out] -> [out][in]
+                for (int i = 0; i < op.n_in; ++i)
+                    for (int o = 0; o < op.units; ++o)
+                        op.hw[0][(size_t)o * op.n_in + i] = w[(size_t)i * op.units + o];
+                result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (cls == "BatchNormalization") {
+                op.kind = OpKind::Affine;
+                std::vector<float> mean = decode_floats(param(c.layer, "moving_mean"));
+                std::vector<float> var = decode_floats(param(c.layer, "moving_variance"));
+                std::vector<float> gamma, beta;
+                if (cfg.at("scale").boolean())
+                    gamma = decode_floats(param(c.layer, "gamma"));
+                if (cfg.at("center").boolean())
+                    beta = decode_floats(param(c.layer, "beta"));
+                const Value& ax = cfg.at("axis");
+                if (ax.is_array() && ax.size() != 1)
+                    throw FormatError("invalid axis configuration");
+                op.ln_axes = (int)(ax.is_array() ? ax.at((size_t)0).integer() : ax.integer()); // checked at plan time
+                const float eps = (float)cfg.at("epsilon").number();
+                if (var.size() != mean.size() || (!gamma.empty() && gamma.size() != mean.size())
+                    || (!beta.empty() && beta.size() != mean.size()))
+                    throw FormatError("invalid sizes");
+                // tensor.hpp:773-793: inv = gamma / sqrt(var + eps); y = x * inv + (beta - mean * inv)
+                op.hw.resize(2);
+                op.hw[0].resize(mean.size());
+                op.hw[1].resize(mean.size());
+                for (size_t i = 0; i < mean.size(); ++i) {
+                    const float inv = (1.0f / std::sqrt(var[i] + eps)) * (gamma.empty() ? 1.f : gamma[i]);
+                    op.hw[0][i] = inv;
+                    op.hw[1][i] = (beta.empty() ? 0.f : beta[i]) - mean[i] * inv;
+                }
+                op.cout = (int)mean.size();
+                result = add_op(std::move(op));
+            } else if (cls == "LayerNormalization") {
+                op.kind = OpKind::LayerNorm;
+                op.hw.resize(2);
+                if (cfg.at("scale").boolean())
+                    op.hw[0] = decode_floats(param(c.layer, "gamma"));
+                if (cfg.at("center").boolean())
+                    op.hw[1] = decode_floats(param(c.layer, "beta"));
+                op.eps = (float)cfg.at("epsilon").number();
+                const Value& ax = cfg.at("axis");
+                op.target_shape.clear();
+                if (ax.is_array())
+                    for (const auto& a : ax.arr)
+                        op.target_shape.push_back(a.integer());
+                else
+                    op.target_shape.push_back(ax.integer());
+                result = add_op(std::move(op));
+            } else if (cls == "ReLU") {
+                op.kind = OpKind::Act;
+                parse_activation("relu", &cfg, op.act);
+                result = add_op(std::move(op));
+            } else if (cls == "Activation") {
+                const std::string type = cfg.at("activation").str();
+                switch (parse_activation(type, &cfg, op.act)) {
+                case ActParse::Linear: op.kind = OpKind::View; break;
+                case ActParse::Softmax: op.kind = OpKind::Softmax; break;
+                case ActParse::Epilogue: op.kind = OpKind::Act; break;
+                }
+                result = add_op(std::move(op));
+            } else if (cls == "Softmax") {
+                op.kind = OpKind::Softmax;
+                result = add_op(std::move(op));
+            } else if (cls == "ZeroPadding2D") {
+                op.kind = OpKind::ZeroPad;
+                const Value& p = cfg.at("padding");
+                if (!p.is_array() || p.size() != 2 || !p.arr[0].is_array() || p.arr[0].size() != 2 || p.arr[1].size() != 2)
+                    throw FormatError("invalid padding format");
+                op.zp[0] = (int)p.arr[0].at((size_t)0).integer();
+                op.zp[1] = (int)p.arr[0].at(1).integer();
+                op.zp[2] = (int)p.arr[1].at((size_t)0).integer();
+                op.zp[3] = (int)p.arr[1].at(1).integer();
+                result = add_op(std::move(op));
+            } else if (cls == "MaxPooling2D" || cls == "AveragePooling2D") {
+                op.kind = OpKind::Pool;
+                op.pool_mode = cls[0] == 'M' ? 0 : 1;
+                pair_from(cfg.at("pool_size"), op.kh, op.kw);
+                const Value& st = cfg.at("strides");
+                if (st.is_null()) {
+                    op.sy = op.kh;
+                    op.sx = op.kw;
+                } else
+                    pair_from(st, op.sy, op.sx);
+                op.padding = padding_from(cfg.at("padding").str());
+                result = add_op(std::move(op));
+            } else if (cls == "GlobalAveragePooling2D" || cls == "GlobalMaxPooling2D" || cls == "GlobalAveragePooling1D"
+                || cls == "GlobalMaxPooling1D") {
+                op.kind = OpKind::GlobalPool;
+                op.pool_mode = cls.find("Max") != std::string::npos ? 0 : 1;
+                const Value* kd = cfg.find("keepdims");
+                op.keepdims = kd && kd->is_bool() && kd->boolean();
+                result = add_op(std::move(op));
+            } else if (cls == "Add") {
+                op.kind = OpKind::Add;
+                result = add_op(std::move(op));
+            } else if (cls == "Embedding") {
+                op.kind = OpKind::Embedding;
+                op.input_dim = (int)cfg.at("input_dim").integer();
+                op.output_dim = (int)cfg.at("output_dim").integer();
+                op.hw.resize(1);
+                op.hw[0] = decode_floats(param(c.layer, "weights"));
+                if (op.hw[0].size() != (size_t)op.input_dim * op.output_dim)
+                    throw FormatError("embedding weight size does not match input_dim * output_dim");
+                m.has_embedding = true;
+                result = add_op(std::move(op));
+            } else if (cls == "MultiHeadAttention") {
+                op.kind = OpKind::MHA;
+                op.heads = (int)cfg.at("num_heads").integer();
+                op.dk = (int)cfg.at("key_dim").integer();
+                op.dv = (int)cfg.at("value_dim").integer();
+                op.use_bias = cfg.at("use_bias").boolean();
+                if (ins.size() != 2 && ins.size() != 3)
+                    throw FormatError("Invalid number of inputs for MultiHeadAttention layer.");
+                const Value& shapes = param(c.layer, "weight_shapes");
+                const Value& vals = param(c.layer, "weights");
+                const size_t expect = op.use_bias ? 8 : 4;
+                if (!shapes.is_array() || !vals.is_array() || shapes.size() != expect || vals.size() != expect)
+                    throw FormatError("MultiHeadAttention expects q/k/v/output kernels (and biases)");
+                std::vector<std::vector<float>> w;
+                for (const auto& v : vals.arr)
+                    w.push_back(decode_floats(v));
+                const int step = op.use_bias ? 2 : 1;
+                const int H = op.heads;
+                // kernels arrive (D, H, dim): transpose to [H*dim][D], the B operand of the projection GEMM
+                auto kernel_t = [&](const std::vector<float>& k, int dim, int& d_in) {
+                    if (k.size() % ((size_t)H * dim) != 0)
+                        throw FormatError("Invalid weights shape for attention head dimension.");
+                    d_in = (int)(k.size() / ((size_t)H * dim));
+                    std::vector<float> t(k.size());
+                    const int n = H * dim;
+                    for (int i = 0; i < d_in; ++i)
+                        for (int o = 0; o < n; ++o)
+                            t[(size_t)o * d_in + i] = k[(size_t)i * n + o];
+                    return t;
+                };
+                auto bias_of = [&](int idx, int n) {
+                    std::vector<float> b = op.use_bias ? w[(size_t)idx * step + 1] : std::vector<float>((size_t)n, 0.f);
+                    if ((int)b.size() != n)
+                        throw FormatError("Invalid biases shape for attention head dimension.");
+                    return b;
+                };
+                op.hw.resize(8);
+                int dq = 0, dkk = 0, dvv = 0;
+                op.hw[0] = kernel_t(w[0], op.dk, dq);
+                op.hw[1] = bias_of(0, H * op.dk);
+                op.hw[2] = kernel_t(w[(size_t)step], op.dk, dkk);
+                op.hw[3] = bias_of(1, H * op.dk);
+                op.hw[4] = kernel_t(w[(size_t)2 * step], op.dv, dvv);
+                op.hw[5] = bias_of(2, H * op.dv);
+                if (dq != dkk || dq != dvv)
+                    throw FormatError("MultiHeadAttention kernels disagree on the input depth");
+                op.d_in = dq;
+                const std::vector<float>& ow = w[(size_t)3 * step]; // (H, dv, Dout) = [H*dv][Dout] -> [Dout][H*dv]
+                const int kin = H * op.dv;
+                if (ow.size() % (size_t)kin != 0)
+                    throw FormatError("Invalid output kernel shape for MultiHeadAttention");
+                op.dout = (int)(ow.size() / (size_t)kin);
+                op.hw[6].resize(ow.size());
+                for (int i = 0; i < kin; ++i)
+                    for (int o = 0; o < op.dout; ++o)
+                        op.hw[6][(size_t)o * kin + i] = ow[(size_t)i * op.dout + o];
+                op.hw[7] = bias_of(3, op.dout);
+                result = add_op(std::move(op));
+            } else if (cls == "Flatten") {
+                op.kind = OpKind::View;
+                op.flatten = true;
+                result = add_op(std::move(op));
+            } else if (cls == "Reshape") {
+                op.kind = OpKind::View;
+                for (const auto& d : cfg.at("target_shape").arr)
+                    op.target_shape.push_back(d.integer());
+                result = add_op(std::move(op));
+            } else {
+                throw Unsupported("unknown layer type: " + cls);
+            }
+            return memo[key] = result;
+        }
+    };
+
+    void replace_uses(fdx_model& m, int from, int to)
+    {
+        for (auto& o : m.ops) {
+            for (auto& i : o.in)
+                if (i == from)
+                    i = to;
+            if (o.residual == from)
+                o.residual = to;
+        }
+        for (auto& o : m.outputs)
+            if (o == from)
+                o = to;
+    }
+
+    void count_consumers(fdx_model& m)
+    {
+        for (auto& o : m.ops)
+            o.consumers = 0;
+        for (auto& o : m.ops) {
+            if (o.dead)
+                continue;
+            for (int i : o.in)
+                m.ops[i].consumers++;
+            if (o.residual >= 0)
+                m.ops[o.residual].consumers++;
+        }
+        for (int o : m.outputs)
+            m.ops[o].consumers++;
+    }
+
+    bool is_gemm_like(const Op& o) { return o.kind == OpKind::Conv2D || o.kind == OpKind::Dense; }
+
+    fdx_status infer_shapes(const fdx_model& m, const std::vector<Shape>& in_shapes, std::vector<Shape>& shapes,
+        const std::vector<int>& order);
+
+    std::vector<int> topo_order(const fdx_model& m)
+    {
+        std::vector<int> order;
+        std::vector<char> seen(m.ops.size(), 0);
+        std::function<void(int)> visit = [&](int i) {
+            if (seen[i])
+                return;
+            seen[i] = 1;
+            for (int p : m.ops[i].in)
+                visit(p);
+            if (m.ops[i].residual >= 0)
+                visit(m.ops[i].residual);
+            order.push_back(i);
+        };
+        for (int i : m.inputs)
+            visit(i);
+        for (int o : m.outputs)
+            visit(o);
+        return order;
+    }
+
+    void fuse(fdx_model& m)
+    {
+        // shapes with every variable dimension set to a dummy extent decide which Adds are plain
+        // (equal-shape) sums
+        std::vector<Shape> dummy;
+        for (const auto& s : m.in_decl) {
+            Shape d = s;
+            for (auto& v : d)
+                if (v < 0)
+                    v = 6;
+            dummy.push_back(d);
+        }
+        std::vector<Shape> shapes;
+        const bool have_shapes = infer_shapes(m, dummy, shapes, topo_order(m)) == FDX_OK;
+
+        count_consumers(m);
+        // 1. BatchNormalization on the channel axis into the producing convolution / dense weights
+        for (size_t i = 0; i < m.ops.size(); ++i) {
+            Op& bn = m.ops[i];
+            if (bn.dead || bn.kind != OpKind::Affine)
+                continue;
+            Op& p = m.ops[bn.in[0]];
+            const bool producer_ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D) && p.act.kind == FDX_ACT_NONE
+                && !p.softmax && p.consumers == 1 && p.residual < 0;
+            if (!producer_ok || !have_shapes)
+                continue;
+            const int rank = (int)shapes[i].size();
+            const int axis = bn.ln_axes < 0 ? bn.ln_axes + rank + 1 : bn.ln_axes;
+            const int ch = p.kind == OpKind::Dense ? p.units : p.cout;
+            if (axis != rank || bn.cout != ch)
+                continue;
+            const size_t per = p.hw[0].size() / (size_t)ch;
+            if (p.kind == OpKind::DWConv2D) { // filter is [kh][kw][c]
+                for (size_t t = 0; t < per; ++t)
+                    for (int c = 0; c < ch; ++c)
+                        p.hw[0][t * ch + c] *= bn.hw[0][c];
+            } else { // [cout][k]
+                for (int c = 0; c < ch; ++c)
+                    for (size_t t = 0; t < per; ++t)
+                        p.hw[0][(size_t)c * per + t] *= bn.hw[0][c];
+            }
+            for (int c = 0; c < ch; ++c)
+                p.hw[1][c] = p.hw[1][c] * bn.hw[0][c] + bn.hw[1][c];
+            bn.dead = true;
+            replace_uses(m, (int)i, bn.in[0]);
+            count_consumers(m);
+        }
+        // 2. stand-alone ReLU / GELU into the producer's epilogue
+        for (size_t i = 0; i < m.ops.size(); ++i) {
+            Op& a = m.ops[i];
+            if (a.dead || a.kind != OpKind::Act)
+                continue;
+            Op& p = m.ops[a.in[0]];
+            const bool ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D || p.kind == OpKind::Add || p.kind == OpKind::Affine)
+                && p.act.kind == FDX_ACT_NONE && !p.softmax && p.consumers == 1;
+            if (!ok)
+                continue;
+            p.act = a.act;
+            a.dead = true;
+            replace_uses(m, (int)i, a.in[0]);
+            count_consumers(m);
+        }
+        // 3. ZeroPadding2D into the consumer's load predicate
+        for (size_t i = 0; i < m.ops.size(); ++i) {
+            Op& c = m.ops[i];
+            if (c.dead || !(c.kind == OpKind::Conv2D || c.kind == OpKind::DWConv2D || c.kind == OpKind::Pool))
+                continue;
+            Op& z = m.ops[c.in[0]];
+            if (z.dead || z.kind != OpKind::ZeroPad || z.consumers != 1)
+                continue;
+            for (int k = 0; k < 4; ++k)
+                c.zp[k] = z.zp[k];
+            c.in[0] = z.in[0];
+            z.dead = true;
+            count_consumers(m);
+        }
+        // 4. two-input equal-shape Add into the epilogue of the convolution / dense that feeds it
+        for (size_t i = 0; i < m.ops.size() && have_shapes; ++i) {
+            Op& add = m.ops[i];
+            if (add.dead || add.kind != OpKind::Add || add.in.size() != 2 || add.in[0] == add.in[1])
+                continue;
+            if (shapes[add.in[0]] != shapes[add.in[1]])
+                continue;
+            for (int side = 1; side >= 0; --side) {
+                Op& p = m.ops[add.in[side]];
+                if (is_gemm_like(p) && p.consumers == 1 && p.residual < 0 && !p.softmax && p.act.kind == FDX_ACT_NONE
+                    && !p.dead) {
+                    p.residual = add.in[1 - side];
+                    p.act = add.act;
+                    add.dead = true;
+                    replace_uses(m, (int)i, add.in[side]);
+                    count_consumers(m);
+                    break;
+                }
+            }
+        }
+    }
+
+    fdx_status upload(fdx_model& m)
+    {
+        for (auto& o : m.ops) {
+            if (o.dead) {
+                o.hw.clear();
+                continue;
+            }
+            o.dw.assign(o.hw.size(), nullptr);
+            for (size_t i = 0; i < o.hw.size(); ++i) {
+                if (o.hw[i].empty())
+                    continue;
+                float* d = nullptr;
+                FDX_HIP(hipMalloc(&d, o.hw[i].size() * sizeof(float)));
+                m.device_allocs.push_back(d);
+                FDX_HIP(hipMemcpy(d, o.hw[i].data(), o.hw[i].size() * sizeof(float), hipMemcpyHostToDevice));
+                o.dw[i] = d;
+            }
+            o.hw.clear();
+            o.hw.shrink_to_fit();
+        }
+        FDX_HIP(hipMalloc(&m.err_flag, sizeof(int)));
+        FDX_HIP(hipMemset(m.err_flag, 0, sizeof(int)));
+        return FDX_OK;
+    }
+
+    fdx_status window(int h, int w, const Op& o, bool dilated, int* g)
+    {
+        const int ekh = dilated ? (o.kh - 1) * o.dy + 1 : o.kh, ekw = dilated ? (o.kw - 1) * o.dx + 1 : o.kw;
+        return fdx_window_geometry(h + o.zp[0] + o.zp[1], w + o.zp[2] + o.zp[3], ekh, ekw, o.sy, o.sx, o.padding, g);
+    }
+
+    fdx_status infer_shapes(const fdx_model& m, const std::vector<Shape>& in_shapes, std::vector<Shape>& shapes,
+        const std::vector<int>& order)
+    {
+        shapes.assign(m.ops.size(), Shape());
+        for (int idx : order) {
+            const Op& o = m.ops[idx];
+            if (o.dead)
+                continue;
+            Shape& out = shapes[idx];
+            const Shape* in0 = o.in.empty() ? nullptr : &shapes[o.in[0]];
+            int g[6];
+            switch (o.kind) {
+            case OpKind::Input:
+                out = in_shapes[o.input_index];
+                break;
+            case OpKind::Conv2D:
+            case OpKind::DWConv2D: {
+                Shape s = *in0;
+                if (s.size() == 2)
+                    s.insert(s.begin(), 1); // 1-D convolution: height 1
+                FDX_REQUIRE(s.size() == 3, "%s: convolution needs a (height, width, depth) input", o.name.c_str());
+                FDX_REQUIRE(s[2] == o.n_in, "invalid filter depth");
+                if (window((int)s[0], (int)s[1], o, true, g) != FDX_OK)
+                    return FDX_ERR_INVALID;
+                FDX_REQUIRE(g[4] > 0 && g[5] > 0, "%s: empty convolution output", o.name.c_str());
+                out = { g[4], g[5], o.cout };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
+                break;
+            }
+            case OpKind::Dense:
+                FDX_REQUIRE(!in0->empty() && in0->back() == o.n_in, "%s: Dense input depth %lld does not match weights (%d)",
+                    o.name.c_str(), in0->empty() ? 0LL : (long long)in0->back(), o.n_in);
+                out = *in0;
+                out.back() = o.units;
+                break;
+            case OpKind::Affine:
+            case OpKind::Act:
+            case OpKind::Softmax:
+            case OpKind::LayerNorm:
+                out = *in0;
+                break;
+            case OpKind::ZeroPad:
+                FDX_REQUIRE(in0->size() == 3, "%s: ZeroPadding2D needs a rank-3 input", o.name.c_str());
+                out = { (*in0)[0] + o.zp[0] + o.zp[1], (*in0)[1] + o.zp[2] + o.zp[3], (*in0)[2] };
+                break;
+            case OpKind::Pool:
+                FDX_REQUIRE(in0->size() == 3, "%s: pooling needs a rank-3 input", o.name.c_str());
+                if (window((int)(*in0)[0], (int)(*in0)[1], o, false, g) != FDX_OK)
+                    return FDX_ERR_INVALID;
+                FDX_REQUIRE(g[4] > 0 && g[5] > 0, "%s: empty pooling output", o.name.c_str());
+                out = { g[4], g[5], (*in0)[2] };
+                break;
+            case OpKind::GlobalPool:
+                FDX_REQUIRE(in0->size() >= 2, "%s: global pooling needs rank >= 2", o.name.c_str());
+                if (o.keepdims) {
+                    out.assign(in0->size(), 1);
+                    out.back() = in0->back();
+                } else
+                    out = { in0->back() };
+                break;
+            case OpKind::Add: {
+                out = *in0;
+                for (size_t k = 1; k < o.in.size(); ++k) {
+                    const Shape& b = shapes[o.in[k]];
+                    if (b == out)
+                        continue;
+                    // size-1 broadcasting is supported when the smaller operand, leading ones dropped, equals
+                    // the trailing dimensions of the larger one (it then repeats as a contiguous block)
+                    const Shape& big = volume(b) > volume(out) ? b : out;
+                    Shape small = volume(b) > volume(out) ? out : b;
+                    while (!small.empty() && small.front() == 1)
+                        small.erase(small.begin());
+                    bool ok = small.size() <= big.size() && std::equal(small.begin(), small.end(), big.end() - (long)small.size());
+                    FDX_REQUIRE(ok, "%s: unsupported broadcast in Add", o.name.c_str());
+                    out = Shape(big);
+                }
+                break;
+            }
+            case OpKind::Embedding:
+                FDX_REQUIRE(in0->size() == 1, "size_dim_5, size_dim_4, height and width dimension must be 1");
+                out = { (*in0)[0], o.output_dim };
+                break;
+            case OpKind::MHA: {
+                const Shape& q = shapes[o.in[0]];
+                const Shape& v = shapes[o.in[1]];
+                const Shape& k = shapes[o.in.size() > 2 ? o.in[2] : o.in[1]];
+                FDX_REQUIRE(q.size() == 2 && v.size() == 2 && k.size() == 2 && q[1] == v[1] && q[1] == k[1] && v[0] == k[0],
+                    "Invalid shapes; need a query tensor of shape (B, T, dim) and a value/key tensor of shape (B, S, dim).");
+                FDX_REQUIRE(q[1] == o.d_in, "%s: attention input depth does not match the kernels", o.name.c_str());
+                out = { q[0], o.dout };
+                break;
+            }
+            case OpKind::View:
+                if (o.flatten)
+                    out = { volume(*in0) };
+                else if (!o.target_shape.empty()) {
+                    out = o.target_shape;
+                    int64_t known = 1, unknown = -1;
+                    for (size_t d = 0; d < out.size(); ++d)
+                        if (out[d] < 0)
+                            unknown = (int64_t)d;
+                        else
+                            known *= out[d];
+                    if (unknown >= 0)
+                        out[(size_t)unknown] = volume(*in0) / std::max<int64_t>(known, 1);
+                    FDX_REQUIRE(volume(out) == volume(*in0), "Invalid target shape");
+                } else
+                    out = *in0;
+                break;
+            }
+        }
+        return FDX_OK;
+    }
+
+    double op_flops(const Op& o, const Shape& out, const std::vector<Shape>& shapes, int batch)
+    {
+        switch (o.kind) {
+        case OpKind::Conv2D: return 2.0 * batch * volume(out) * o.kh * o.kw * o.n_in;
+        case OpKind::Dense: return 2.0 * batch * volume(out) * o.n_in;
+        case OpKind::MHA: {
+            const double t = (double)shapes[o.in[0]][0], s = (double)shapes[o.in[1]][0];
+            return 2.0 * batch * (t * o.d_in * o.heads * o.dk + s * o.d_in * o.heads * (o.dk + o.dv)
+                       + (double)o.heads * t * s * (o.dk + o.dv) + t * o.heads * o.dv * o.dout);
+        }
+        default: return 0.0;
+        }
+    }
+
+} // namespace
+
+fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out)
+{
+    if (m->plan && m->plan->batch == batch && m->plan->in_shapes == in_shapes) {
+        *out = m->plan.get();
+        return FDX_OK;
+    }
+    FDX_HIP(hipStreamSynchronize(stream()));
+    m->plan.reset();
+    std::unique_ptr<Plan> p(new Plan);
+    p->batch = batch;
+    p->in_shapes = in_shapes;
+    p->order = topo_order(*m);
+    fdx_status st = infer_shapes(*m, in_shapes, p->shapes, p->order);
+    if (st != FDX_OK)
+        return st;
+    const size_t n = m->ops.size();
+    p->out.assign(n, nullptr);
+    p->block_of.assign(n, -1);
+    p->last_use.assign(n, -1);
+    p->temps.assign(n, {});
+    // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
+    std::vector<int> root(n);
+    for (int idx : p->order) {
+        const Op& o = m->ops[idx];
+        root[idx] = (o.kind == OpKind::View) ? root[o.in[0]] : idx;
+    }
+    for (size_t pos = 0; pos < p->order.size(); ++pos) {
+        const Op& o = m->ops[p->order[pos]];
+        for (int i : o.in)
+            p->last_use[root[i]] = (int)pos;
+        if (o.residual >= 0)
+            p->last_use[root[o.residual]] = (int)pos;
+    }
+    for (int o : m->outputs)
+        p->last_use[root[o]] = 1 << 30;
+    for (int i : m->inputs)
+        p->last_use[root[i]] = 1 << 30; // input staging buffers persist across calls
+    for (size_t pos = 0; pos < p->order.size(); ++pos) {
+        const int idx = p->order[pos];
+        const Op& o = m->ops[idx];
+        if (o.kind == OpKind::View) {
+            p->out[idx] = p->out[o.in[0]];
+        } else {
+            const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(p->shapes[idx]);
+            p->out[idx] = plan_alloc(*p, bytes, &p->block_of[idx]);
+            if (!p->out[idx]) {
+                set_error("out of device memory while planning %s", o.name.c_str());
+                return FDX_ERR_HIP;
+            }
+        }
+        if (o.kind == OpKind::MHA) { // per-op scratch: placed while inputs and output are live, free again afterwards
+            const int64_t T = p->shapes[o.in[0]][0], S = p->shapes[o.in[1]][0];
+            const size_t nk = (size_t)o.heads * o.dk, nv = (size_t)o.heads * o.dv, fb = sizeof(float) * (size_t)batch;
+            const size_t sizes[5] = { fb * T * nk, fb * S * nk, fb * S * nv, fb * T * nv,
+                fdx_mha_scratch_bytes(batch, o.heads, (int)T, (int)S, o.dv) };
+            std::vector<int> held;
+            for (size_t sz : sizes) {
+                int b = -1;
+                float* t = plan_alloc(*p, sz, &b);
+                if (!t) {
+                    set_error("out of device memory while planning %s", o.name.c_str());
+                    return FDX_ERR_HIP;
+                }
+                p->temps[idx].push_back(t);
+                held.push_back(b);
+            }
+            for (int b : held)
+                p->blocks[b].busy = false;
+        }
+        p->flops += op_flops(o, p->shapes[idx], p->shapes, batch);
+        // release buffers whose last consumer is this op (the op's own output is already placed, so a
+        // producer never writes over one of its live inputs)
+        for (size_t q = 0; q < n; ++q)
+            if (p->block_of[q] >= 0 && p->last_use[q] == (int)pos && p->blocks[p->block_of[q]].busy)
+                p->blocks[p->block_of[q]].busy = false;
+        if (p->last_use[idx] < 0 && p->block_of[idx] >= 0) // produced but never read
+            p->blocks[p->block_of[idx]].busy = false;
+    }
+    m->plan = std::move(p);
+    *out = m->plan.get();
+    return FDX_OK;
+}
+
+namespace {
+
+    fdx_act to_c(const Act& a) { return { a.kind, a.max_value, a.negative_slope, a.threshold }; }
+
+    fdx_status run_op(fdx_model& m, Plan& p, int idx)
+    {
+        const Op& o = m.ops[idx];
+        const int B = p.batch;
+        const Shape& os = p.shapes[idx];
+        float* out = p.out[idx];
+        const float* in0 = o.in.empty() ? nullptr : p.out[o.in[0]];
+        const Shape* is = o.in.empty() ? nullptr : &p.shapes[o.in[0]];
+        const fdx_act act = to_c(o.act);
+        const fdx_act* actp = o.act.kind == FDX_ACT_NONE ? nullptr : &act;
+        const float* res = o.residual >= 0 ? p.out[o.residual] : nullptr;
+        int g[6];
+        fdx_status st = FDX_OK;
+        switch (o.kind) {
+        case OpKind::Input:
+        case OpKind::View:
+            return FDX_OK;
+        case OpKind::Conv2D:
+        case OpKind::DWConv2D: {
+            const bool one_d = is->size() == 2;
+            const int h = one_d ? 1 : (int)(*is)[0], w = (int)(*is)[one_d ? 0 : 1], c = (int)is->back();
+            if ((st = window(h, w, o, true, g)) != FDX_OK)
+                return st;
+            if (o.kind == OpKind::Conv2D)
+                st = fdx_conv2d_nhwc_f32(in0, B, h, w, c, o.dw[0], o.dw[1], o.cout, o.kh, o.kw, o.sy, o.sx, o.dy, o.dx,
+                    g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5], res, actp, out);
+            else
+                st = fdx_dwconv2d_nhwc_f32(in0, B, h, w, c, o.dw[0], o.dw[1], o.kh, o.kw, o.sy, o.sx, o.dy, o.dx,
+                    g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5], actp, out);
+            break;
+        }
+        case OpKind::Dense: {
+            const int64_t rows = (int64_t)B * volume(*is) / o.n_in;
+            FDX_REQUIRE(rows < (1LL << 31), "%s: too many rows", o.name.c_str());
+            st = fdx_gemm_bias_act_f32(in0, o.n_in, o.dw[0], o.n_in, (int)rows, o.units, o.n_in, 1.0f, o.dw[1], 0, res, actp,
+                out, o.units, nullptr);
+            break;
+        }
+        case OpKind::Affine: {
+            const int rank = (int)is->size();
+            const int axis = o.ln_axes < 0 ? o.ln_axes + rank + 1 : o.ln_axes;
+            if (axis != rank || is->back() != o.cout) {
+                set_error("%s: BatchNormalization is supported on the last axis only", o.name.c_str());
+                return FDX_ERR_UNSUPPORTED;
+            }
+            st = fdx_channel_affine_f32(in0, (size_t)B * (size_t)volume(*is) / (size_t)o.cout, o.cout, o.dw[0], o.dw[1], actp, out);
+            break;
+        }
+        case OpKind::LayerNorm: {
+            const int rank = (int)is->size();
+            std::vector<int64_t> axes = o.target_shape;
+            for (auto& a : axes)
+                a = a < 0 ? a + rank + 1 : a;
+            std::sort(axes.begin(), axes.end());
+            int64_t depth = 1;
+            for (size_t k = 0; k < axes.size(); ++k) {
+                if (axes[k] != rank - (int64_t)axes.size() + 1 + (int64_t)k) {
+                    set_error("%s: LayerNormalization is supported over trailing axes only", o.name.c_str());
+                    return FDX_ERR_UNSUPPORTED;
+                }
+                depth *= (*is)[(size_t)axes[k] - 1];
+            }
+            st = fdx_layernorm_f32(in0, (int64_t)B * volume(*is) / depth, (int)depth, o.dw[0], o.dw[1], o.eps, out);
+            break;
+        }
+        case OpKind::Act:
+            st = fdx_activation_f32(in0, (size_t)B * (size_t)volume(*is), actp, out);
+            break;
+        case OpKind::Softmax:
+            st = fdx_softmax_f32(in0, (int64_t)B * volume(*is) / is->back(), (int)is->back(), 0, 0, out);
+            break;
+        case OpKind::ZeroPad:
+            st = fdx_zero_pad2d_nhwc_f32(in0, B, (int)(*is)[0], (int)(*is)[1], (int)(*is)[2], o.zp[0], o.zp[1], o.zp[2], o.zp[3], out);
+            break;
+        case OpKind::Pool:
+            if ((st = window((int)(*is)[0], (int)(*is)[1], o, false, g)) != FDX_OK)
+                return st;
+            st = fdx_pool2d_nhwc_f32(in0, B, (int)(*is)[0], (int)(*is)[1], (int)(*is)[2], o.kh, o.kw, o.sy, o.sx, g[0] + o.zp[0],
+                g[2] + o.zp[2], o.zp[0], o.zp[2], o.zp[1], o.zp[3], g[4], g[5], o.pool_mode, out);
+            break;
+        case OpKind::GlobalPool:
+            st = fdx_global_pool_f32(in0, B, (int)(volume(*is) / is->back()), (int)is->back(), o.pool_mode, out);
+            break;
+        case OpKind::Add: {
+            // left fold (tensor.hpp:677-680); the last step carries the fused activation
+            const float* acc = in0;
+            int64_t acc_vol = volume(*is);
+            for (size_t k = 1; k < o.in.size() && st == FDX_OK; ++k) {
+                const float* b = p.out[o.in[k]];
+                const int64_t bv = volume(p.shapes[o.in[k]]);
+                const fdx_act* a = k + 1 == o.in.size() ? actp : nullptr;
+                if (bv == acc_vol || B == 1) {
+                    const size_t big = (size_t)B * (size_t)std::max(acc_vol, bv), small = (size_t)B * (size_t)std::min(acc_vol, bv);
+                    st = fdx_eltwise_add_f32(acc_vol >= bv ? acc : b, acc_vol >= bv ? b : acc, big, small, a, out);
+                } else {
+                    // broadcast inside each sample: run sample by sample so the smaller operand repeats per sample
+                    const int64_t big = std::max(acc_vol, bv), small = std::min(acc_vol, bv);
+                    for (int s = 0; s < B && st == FDX_OK; ++s) {
+                        const float* pa = acc + (size_t)s * (size_t)acc_vol;
+                        const float* pb = b + (size_t)s * (size_t)bv;
+                        st = fdx_eltwise_add_f32(acc_vol >= bv ? pa : pb, acc_vol >= bv ? pb : pa, (size_t)big, (size_t)small, a,
+                            out + (size_t)s * (size_t)big);
+                    }
+                }
+                acc = out;
+                acc_vol = std::max(acc_vol, bv);
+            }
+            if (o.in.size() == 1)
+                st = fdx_activation_f32(in0, (size_t)B * (size_t)acc_vol, actp, out);
+            break;
+        }
+        case OpKind::Embedding:
+            st = fdx_embedding_f32(in0, (int64_t)B * (*is)[0], o.dw[0], o.input_dim, o.output_dim, out, m.err_flag);
+            break;
+        case OpKind::MHA: {
+            const Shape& qs = p.shapes[o.in[0]];
+            const Shape& vs = p.shapes[o.in[1]];
+            const int T = (int)qs[0], S = (int)vs[0], D = o.d_in, H = o.heads;
+            const float* xq = p.out[o.in[0]];
+            const float* xv = p.out[o.in[1]];
+            const float* xk = p.out[o.in.size() > 2 ? o.in[2] : o.in[1]];
+            const int64_t nk = (int64_t)H * o.dk, nv = (int64_t)H * o.dv;
+            const std::vector<float*>& tmp = p.temps[idx];
+            float *q = tmp[0], *k = tmp[1], *v = tmp[2], *merged = tmp[3], *scratch = tmp[4];
+            if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[0], D, B * T, (int)nk, D, 1.f, o.dw[1], 0, nullptr, nullptr, q, nk, nullptr)) != FDX_OK)
+                return st;
+            if ((st = fdx_gemm_bias_act_f32(xk, D, o.dw[2], D, B * S, (int)nk, D, 1.f, o.dw[3], 0, nullptr, nullptr, k, nk, nullptr)) != FDX_OK)
+                return st;
+            if ((st = fdx_gemm_bias_act_f32(xv, D, o.dw[4], D, B * S, (int)nv, D, 1.f, o.dw[5], 0, nullptr, nullptr, v, nv, nullptr)) != FDX_OK)
+                return st;
+            if ((st = fdx_mha_prefill_f32(q, k, v, B, T, S, H, o.dk, o.dv, 0, merged, scratch)) != FDX_OK)
+                return st;
+            st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, B * T, o.dout, (int)nv, 1.f, o.dw[7], 0, nullptr, nullptr, out,
+                o.dout, nullptr);
+            break;
+        }
+        }
+        if (st != FDX_OK)
+            return st;
+        if (o.softmax) // fused "softmax" activation of a conv / dense layer, in place
+            st = fdx_softmax_f32(out, (int64_t)B * volume(os) / os.back(), (int)os.back(), 0, 0, out);
+        return st;
+    }
+
+    std::string shape_str(const Shape& s)
+    {
+        std::string r = "(";
+        for (size_t i = 0; i < s.size(); ++i)
+            r += (i ? ", " : "") + (s[i] < 0 ? std::string("None") : std::to_string(s[i]));
+        return r + ")";
+    }
+
+    fdx_status shapes_from_args(const fdx_model& m, const int64_t* in_dims, const int* in_ranks, std::vector<Shape>& shapes)
+    {
+        shapes.clear();
+        for (size_t i = 0; i < m.inputs.size(); ++i) {
+            const int rank = in_ranks[i];
+            FDX_REQUIRE(rank >= 1 && rank <= 5, "input %zu: rank must be 1..5", i);
+            Shape s(in_dims + i * 5 + (5 - rank), in_dims + i * 5 + 5);
+            // rank and every fixed dimension must match (model.hpp:134-139, tensor_shape.hpp:246-250)
+            const Shape& d = m.in_decl[i];
+            bool ok = d.size() == s.size();
+            for (size_t k = 0; ok && k < s.size(); ++k)
+                ok = s[k] > 0 && (d[k] < 0 || d[k] == s[k]);
+            if (!ok) {
+                std::string want, got;
+                for (const auto& ds : m.in_decl)
+                    want += shape_str(ds);
+                set_error("Invalid inputs shape.\nThe model takes %s but input %zu has shape %s", want.c_str(), i,
+                    shape_str(s).c_str());
+                return FDX_ERR_INVALID;
+            }
+            shapes.push_back(std::move(s));
+        }
+        return FDX_OK;
+    }
+
+    void write_out_shapes(const fdx_model& m, const Plan& p, int64_t* out_dims, int* out_ranks)
+    {
+        for (size_t i = 0; i < m.outputs.size(); ++i) {
+            const Shape& s = p.shapes[m.outputs[i]];
+            if (out_ranks)
+                out_ranks[i] = (int)s.size();
+            if (out_dims) {
+                for (int k = 0; k < 5; ++k)
+                    out_dims[i * 5 + k] = 1;
+                for (size_t k = 0; k < s.size(); ++k)
+                    out_dims[i * 5 + 5 - s.size() + k] = s[k];
+            }
+        }
+    }
+
+    fdx_status execute(fdx_model& m, Plan& p)
+    {
+        for (int idx : p.order) {
+            if (m.ops[idx].dead)
+                continue;
+            fdx_status st = run_op(m, p, idx);
+            if (st != FDX_OK)
+                return st;
+        }
+        m.last_flops = p.flops;
+        return FDX_OK;
+    }
+
+    fdx_status check_embedding_flag(fdx_model& m)
+    {
+        if (!m.has_embedding)
+            return FDX_OK;
+        int flag = 0;
+        FDX_HIP(hipMemcpyAsync(&flag, m.err_flag, sizeof(int), hipMemcpyDeviceToHost, stream()));
+        FDX_HIP(hipStreamSynchronize(stream()));
+        if (flag) {
+            FDX_HIP(hipMemsetAsync(m.err_flag, 0, sizeof(int), stream()));
+            set_error("vocabulary item indices must all be strictly less than the value of input_dim");
+            return FDX_ERR_INVALID;
+        }
+        return FDX_OK;
+    }
+
+    fdx_status predict_impl(fdx_model* m, int batch, const float* const* in, bool in_on_device, const int64_t* in_dims,
+        const int* in_ranks, float* const* out, bool out_on_device, int64_t* out_dims, int* out_ranks)
+    {
+        FDX_REQUIRE(m && in && in_dims && in_ranks && out, "predict: null argument");
+        FDX_REQUIRE(batch > 0, "predict: batch must be positive");
+        std::lock_guard<std::mutex> lock(m->mu);
+        std::vector<Shape> shapes;
+        fdx_status st = shapes_from_args(*m, in_dims, in_ranks, shapes);
+        if (st != FDX_OK)
+            return st;
+        Plan* p = nullptr;
+        if ((st = get_plan(m, batch, shapes, &p)) != FDX_OK)
+            return st;
+        for (size_t i = 0; i < m->inputs.size(); ++i) {
+            FDX_REQUIRE(in[i], "predict: null input %zu", i);
+            const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(shapes[i]);
+            FDX_HIP(hipMemcpyAsync(p->out[m->inputs[i]], in[i], bytes, in_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                stream()));
+        }
+        if ((st = execute(*m, *p)) != FDX_OK)
+            return st;
+        for (size_t i = 0; i < m->outputs.size(); ++i) {
+            FDX_REQUIRE(out[i], "predict: null output %zu", i);
+            const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(p->shapes[m->outputs[i]]);
+            FDX_HIP(hipMemcpyAsync(out[i], p->out[m->outputs[i]], bytes, out_on_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost,
+                stream()));
+        }
+        write_out_shapes(*m, *p, out_dims, out_ranks);
+        if (!out_on_device || m->has_embedding) {
+            FDX_HIP(hipStreamSynchronize(stream()));
+            if ((st = check_embedding_flag(*m)) != FDX_OK)
+                return st;
+        }
+        return FDX_OK;
+    }
+
+    Shape decl_shape(const Value& v)
+    {
+        Shape s;
+        if (!v.is_array())
+            throw FormatError("shape must be an array");
+        for (const auto& d : v.arr)
+            s.push_back(d.is_null() ? -1 : d.integer());
+        return s;
+    }
+
+    fdx_status run_embedded_tests(fdx_model* m, const Value& tests, float eps)
+    {
+        for (const auto& t : tests.arr) {
+            const Value& ins = t.at("inputs");
+            const Value& outs = t.at("outputs");
+            FDX_REQUIRE(ins.is_array() && outs.is_array(), "test needs inputs and outputs");
+            FDX_REQUIRE(ins.size() == m->inputs.size() && outs.size() == m->outputs.size(), "test case arity does not match the model");
+            std::vector<std::vector<float>> iv, ov;
+            std::vector<const float*> ip;
+            std::vector<int64_t> dims(5 * ins.size(), 1);
+            std::vector<int> ranks(ins.size());
+            for (size_t i = 0; i < ins.size(); ++i) {
+                Shape s = decl_shape(ins.arr[i].at("shape"));
+                iv.push_back(decode_floats(ins.arr[i].at("values")));
+                FDX_REQUIRE((int64_t)iv.back().size() == volume(s), "test input %zu: values do not fill the shape", i);
+                ranks[i] = (int)s.size();
+                for (size_t k = 0; k < s.size(); ++k)
+                    dims[i * 5 + 5 - s.size() + k] = s[k];
+            }
+            for (auto& v : iv)
+                ip.push_back(v.data());
+            std::vector<Shape> shapes;
+            fdx_status st = shapes_from_args(*m, dims.data(), ranks.data(), shapes);
+            if (st != FDX_OK)
+                return st;
+            Plan* p = nullptr;
+            {
+                std::lock_guard<std::mutex> lock(m->mu);
+                if ((st = get_plan(m, 1, shapes, &p)) != FDX_OK)
+                    return st;
+                ov.resize(outs.size());
+                for (size_t i = 0; i < outs.size(); ++i)
+                    ov[i].resize((size_t)volume(p->shapes[m->outputs[i]]));
+            }
+            std::vector<float*> op;
+            for (auto& v : ov)
+                op.push_back(v.data());
+            if ((st = predict_impl(m, 1, ip.data(), false, dims.data(), ranks.data(), op.data(), false, nullptr, nullptr)) != FDX_OK)
+                return st;
+            // import_model.hpp:1990-2021: absolute tolerance, NaN == NaN passes
+            for (size_t i = 0; i < outs.size(); ++i) {
+                std::vector<float> want = decode_floats(outs.arr[i].at("values"));
+                FDX_REQUIRE(want.size() == ov[i].size(), "test failed: output %zu has %zu values, the file holds %zu", i, ov[i].size(),
+                    want.size());
+                for (size_t k = 0; k < want.size(); ++k) {
+                    const float a = ov[i][k], b = want[k];
+                    if (!(std::fabs(a - b) <= eps || (std::isnan(a) && std::isnan(b)))) {
+                        set_error("test failed: output=%zu pos=%zu value=%.9g target=%.9g", i, k, a, b);
+                        return FDX_ERR_INVALID;
+                    }
+                }
+            }
+        }
+        return FDX_OK;
+    }
+
+} // namespace
+} // namespace fdx
+
+fdx_model::~fdx_model()
+{
+    (void)hipStreamSynchronize(fdx::stream());
+    plan.reset();
+    for (float* p : device_allocs)
+        (void)hipFree(p);
+    if (err_flag)
+        (void)hipFree(err_flag);
+}
+
+extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int verify, float verify_epsilon, fdx_model** out)
+{
+    FDX_REQUIRE(json_text && out, "model_create: null argument");
+    *out = nullptr;
+    if (fdx_sync() != FDX_OK)
+        return FDX_ERR_HIP;
+    std::unique_ptr<fdx_model> m(new fdx_model);
+    try {
+        json::Parser parser(json_text, len);
+        const Value root = parser.parse();
+        const Value* fmt = root.find("image_data_format");
+        if (!fmt || !fmt->is_string() || fmt->str() != "channels_last")
+            throw FormatError("only channels_last data format supported");
+        const Value& arch = root.at("architecture");
+        const Value& cfg = arch.at("config");
+        m->name = cfg.at("name").str();
+        if (const Value* h = root.find("hash"))
+            if (h->is_string())
+                m->hash = h->str();
+        const Value& layers = cfg.at("layers");
+        if (!layers.is_array())
+            throw FormatError("missing layers array");
+        static const Value empty_params = [] { Value v; v.type = Value::Object; return v; }();
+        const Value* tp = root.find("trainable_params");
+        Builder b { *m, tp ? *tp : empty_params, {}, {}, {} };
+        for (const auto& l : layers.arr) {
+            const std::string name = l.at("name").str();
+            if (b.layers.count(name))
+                throw FormatError("layer names must be unique: " + name);
+            const std::string cls = l.at("class_name").str();
+            if (cls == "Functional" || cls == "Model" || cls == "Sequential")
+                throw Unsupported("nested models are not supported yet: " + name);
+            b.layers[name] = &l;
+        }
+        for (const auto& s : root.at("input_shapes").arr)
+            m->in_decl.push_back(decl_shape(s));
+        for (const auto& s : root.at("output_shapes").arr)
+            m->out_decl.push_back(decl_shape(s));
+        const auto ins = model_connections(cfg.at("input_layers"));
+        const auto outs = model_connections(cfg.at("output_layers"));
+        if (ins.size() != m->in_decl.size())
+            throw FormatError("input_shapes does not match input_layers");
+        for (size_t i = 0; i < ins.size(); ++i) {
+            auto lit = b.layers.find(ins[i].layer);
+            if (lit == b.layers.end() || lit->second->at("class_name").str() != "InputLayer")
+                throw FormatError("input_layers must name InputLayer layers");
+            const Value* nodes = lit->second->find("inbound_nodes");
+            if (nodes && nodes->size() != 0)
+                throw FormatError("input layer is not allowed to have inbound nodes");
+            Op op;
+            op.kind = OpKind::Input;
+            op.name = ins[i].layer;
+            op.cls = "InputLayer";
+            op.input_index = (int)i;
+            m->ops.push_back(std::move(op));
+            m->inputs.push_back((int)m->ops.size() - 1);
+            b.input_ops[ins[i].layer] = m->inputs.back();
+        }
+        for (const auto& o : outs)
+            m->outputs.push_back(b.build(o));
+        fuse(*m);
+        fdx_status st = upload(*m);
+        if (st != FDX_OK)
+            return st;
+        const Value* tests = root.find("tests");
+        if (verify && tests && tests->is_array()) {
+            st = run_embedded_tests(m.get(), *tests, verify_epsilon);
+            if (st != FDX_OK)
+                return st;
+        }
+    } catch (const Unsupported& e) {
+        set_error("%s", e.what());
+        return FDX_ERR_UNSUPPORTED;
+    } catch (const std::exception& e) {
+        set_error("%s", e.what());
+        return FDX_ERR_FORMAT;
+    }
+    *out = m.release();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_destroy(fdx_model* m)
+{
+    delete m;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_name(const fdx_model* m, const char** name, const char** hash)
+{
+    FDX_REQUIRE(m, "model_name: null model");
+    if (name) *name = m->name.c_str();
+    if (hash) *hash = m->hash.c_str();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_io_count(const fdx_model* m, int* n_inputs, int* n_outputs)
+{
+    FDX_REQUIRE(m, "model_io_count: null model");
+    if (n_inputs) *n_inputs = (int)m->inputs.size();
+    if (n_outputs) *n_outputs = (int)m->outputs.size();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_io_shape(const fdx_model* m, int is_output, int index, int* rank, int64_t* dims5)
+{
+    FDX_REQUIRE(m && rank && dims5, "model_io_shape: null argument");
+    const auto& decl = is_output ? m->out_decl : m->in_decl;
+    FDX_REQUIRE(index >= 0 && index < (int)decl.size(), "model_io_shape: index out of range");
+    const Shape& s = decl[index];
+    *rank = (int)s.size();
+    for (int k = 0; k < 5; ++k)
+        dims5[k] = 1;
+    for (size_t k = 0; k < s.size(); ++k)
+        dims5[5 - s.size() + k] = s[k];
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_predict(fdx_model* m, int batch, const float* const* in, const int64_t* in_dims,
+    const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks)
+{
+    return predict_impl(m, batch, in, false, in_dims, in_ranks, out, false, out_dims, out_ranks);
+}
+
+extern "C" fdx_status fdx_model_predict_dev(fdx_model* m, int batch, const float* const* in_dev, const int64_t* in_dims,
+    const int* in_ranks, float* const* out_dev, int64_t* out_dims, int* out_ranks)
+{
+    return predict_impl(m, batch, in_dev, true, in_dims, in_ranks, out_dev, true, out_dims, out_ranks);
+}
+
+extern "C" fdx_status fdx_model_infer_shapes(fdx_model* m, const int64_t* in_dims, const int* in_ranks, int64_t* out_dims,
+    int* out_ranks)
+{
+    FDX_REQUIRE(m && in_dims && in_ranks, "infer_shapes: null argument");
+    std::lock_guard<std::mutex> lock(m->mu);
+    std::vector<Shape> shapes;
+    fdx_status st = shapes_from_args(*m, in_dims, in_ranks, shapes);
+    if (st != FDX_OK)
+        return st;
+    Plan tmp;
+    tmp.order = topo_order(*m);
+    if ((st = infer_shapes(*m, shapes, tmp.shapes, tmp.order)) != FDX_OK)
+        return st;
+    write_out_shapes(*m, tmp, out_dims, out_ranks);
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_model_last_flops(const fdx_model* m, double* flops)
+{
+    FDX_REQUIRE(m && flops, "last_flops: null argument");
+    *flops = m->last_flops;
+    return FDX_OK;
+}

@@ -1,0 +1,103 @@
+// In-memory form of a loaded model: a flat list of device ops (after load-time fusion),
+// resident weights, and per-input-shape launch plans.
+#pragma once
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace fdx {
+
+enum class OpKind {
+    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View
+};
+
+using Shape = std::vector<int64_t>; // dims of one sample, no batch axis
+
+inline int64_t volume(const Shape& s)
+{
+    int64_t v = 1;
+    for (auto d : s)
+        v *= d;
+    return v;
+}
+
+struct Op {
+    OpKind kind = OpKind::View;
+    std::string name, cls;
+    std::vector<int> in; // producer op indices
+    int residual = -1;   // op whose output is added in the producer's epilogue
+    bool dead = false;
+    int consumers = 0;
+
+    // attributes
+    int cout = 0, kh = 1, kw = 1, sy = 1, sx = 1, dy = 1, dx = 1, padding = 0;
+    int zp[4] = { 0, 0, 0, 0 }; // folded explicit zero padding: top, bottom, left, right
+    Act act { FDX_ACT_NONE, 3.402823466e+38f, 0.f, 0.f };
+    bool softmax = false; // fused "softmax" activation runs as a second kernel
+    int pool_mode = 0;
+    bool keepdims = false;
+    float eps = 0.f;
+    int ln_axes = 1;
+    int heads = 0, dk = 0, dv = 0, dout = 0, d_in = 0;
+    bool use_bias = true;
+    int input_dim = 0, output_dim = 0, units = 0, n_in = 0;
+    Shape target_shape;
+    bool flatten = false;
+    int input_index = -1;
+
+    // host weights (released after upload)
+    std::vector<std::vector<float>> hw;
+    // device weights, indexed like hw
+    std::vector<float*> dw;
+};
+
+struct Block {
+    void* p = nullptr;
+    size_t bytes = 0;
+    bool busy = false;
+};
+
+struct Plan {
+    int batch = 0;
+    std::vector<Shape> in_shapes;
+    std::vector<Shape> shapes;   // per op
+    std::vector<float*> out;     // per op output buffer (device)
+    std::vector<int> order;      // execution order (live ops)
+    std::vector<int> block_of;   // per op: index into blocks, -1 = alias / external
+    std::vector<int> last_use;   // position in order of the last consumer
+    std::vector<Block> blocks;
+    std::vector<std::vector<float*>> temps; // per op: scratch placed at plan time
+    double flops = 0;
+    ~Plan();
+};
+
+} // namespace fdx
+
+struct fdx_model {
+    std::string name, hash;
+    std::vector<fdx::Op> ops;
+    std::vector<int> inputs, outputs;   // op indices
+    std::vector<fdx::Shape> in_decl, out_decl; // declared shapes, -1 = variable
+    std::vector<float*> device_allocs;
+    int* err_flag = nullptr;
+    bool has_embedding = false;
+    std::unique_ptr<fdx::Plan> plan;
+    std::mutex mu;
+    double last_flops = 0;
+    ~fdx_model();
+};
+
+namespace fdx {
+// builds (or reuses) the plan for this batch and these per-sample input shapes
+fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out);
+float* plan_alloc(Plan& p, size_t bytes, int* block_index);
+fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, const float* k, int64_t ldk, int64_t k_batch,
+    const float* v, int64_t ldv, int64_t v_batch, int batch, int t, int s, int heads, int dk, int dv, int causal,
+    float* out, int64_t ldo, int64_t o_batch, void* scratch_dev);
+fdx_status argmax_launch(const float* x, int64_t rows, int depth, int32_t* out_idx, float* out_val, float* out_idx_f);
+fdx_status gather_rows_launch(const float* in, int64_t rows, int depth, int64_t row_stride, int64_t offset, float* out);
+}

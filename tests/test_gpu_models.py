@@ -1,0 +1,136 @@
+"""Whole-model parity: converted-JSON files written by the package's model writers, loaded through
+fdx_model_create and run batched on the GPU, against the CPU oracle walking the same file sample by sample.
+Tolerance: per output tensor max|gpu - ref| / max|ref| <= 1e-4 (fp32, summation order differs)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def with_taps(spec, names):
+    """Adds intermediate layers as extra model outputs so that parity is checked before a saturating softmax."""
+    cfg = spec["architecture"]["config"]
+    cfg["output_layers"] = cfg["output_layers"] + [[n, 0, 0] for n in names]
+    spec["output_shapes"] = spec["output_shapes"] + [None] * len(names)  # placeholders, fixed below
+    return spec
+
+
+def run_both(fdx, oracle, modelgen, spec, inputs, tol=TOL):
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    n = inputs[0].shape[0]
+    want = [ref.predict([x[i] for x in inputs]) for i in range(n)]
+    want = [np.stack([w[k] for w in want]) for k in range(len(want[0]))]
+    model = fdx.Model(js)
+    got = model.predict(inputs)
+    errs = [rel(g, w) for g, w in zip(got, want)]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= tol
+    return got, want, model
+
+
+def fix_tap_shapes(spec, oracle, modelgen, sample_inputs):
+    tmp = dict(spec)
+    tmp["output_shapes"] = [[1]] * len(spec["output_shapes"])
+    ref = oracle.OracleModel(modelgen.dumps(tmp))
+    outs = ref.predict(sample_inputs)
+    spec["output_shapes"] = [list(o.shape) for o in outs]
+    return spec
+
+
+def test_small_cnn_256_samples(fdx, oracle, modelgen):
+    say("small_cnn")
+    spec = modelgen.small_cnn()
+    x = np.random.default_rng(11).uniform(-1, 1, (256, 32, 32, 3)).astype(np.float32)
+    got, want, model = run_both(fdx, oracle, modelgen, spec, [x])
+    assert np.abs(got[0].sum(-1) - 1).max() < 1e-5
+    # predict_class semantics: argmax with first-max-wins equals the oracle's
+    assert [int(np.argmax(g)) for g in got[0]] == [oracle.argmax(w) for w in want[0]]
+    # batch 1 equals row 0 of the batched run (samples are independent)
+    one = model.predict([x[:1]])
+    assert rel(one[0], got[0][:1]) <= 1e-6
+
+
+def test_embedded_self_test_and_failure(fdx, oracle, modelgen):
+    say("embedded tests")
+    spec = modelgen.small_cnn()
+    x = np.random.default_rng(12).uniform(-1, 1, (32, 32, 3)).astype(np.float32)
+    ref = oracle.OracleModel(modelgen.dumps(spec))
+    y = ref.predict([x])[0]
+    spec["tests"] = [{"inputs": [x], "outputs": [y]}]
+    fdx.Model(modelgen.dumps(spec), verify=True, verify_epsilon=1e-5)  # passes
+    spec["tests"] = [{"inputs": [x], "outputs": [y + 0.01]}]
+    with pytest.raises(fdx.FdxError, match="test failed"):
+        fdx.Model(modelgen.dumps(spec), verify=True)
+    fdx.Model(modelgen.dumps(spec), verify=False)  # verification is optional
+
+
+def test_resnet_scaled_down(fdx, oracle, modelgen):
+    say("resnet scaled")
+    spec = modelgen.resnet50(seed=21, input_size=64, width=16, blocks=(2, 2, 2, 2), classes=20, random_bn=True)
+    spec = with_taps(spec, ["avg_pool", "conv2_block1_out", "pool1_pool"])
+    x = np.random.default_rng(13).uniform(0, 1, (3, 64, 64, 3)).astype(np.float32)
+    spec = fix_tap_shapes(spec, oracle, modelgen, [x[0]])
+    run_both(fdx, oracle, modelgen, spec, [x])
+
+
+def test_resnet50_full_width_two_images(fdx, oracle, modelgen):
+    say("resnet50 full")
+    spec = modelgen.resnet50()
+    spec = with_taps(spec, ["avg_pool"])
+    x = np.random.default_rng(14).uniform(0, 1, (2, 224, 224, 3)).astype(np.float32)
+    spec = fix_tap_shapes(spec, oracle, modelgen, [x[0]])
+    got, want, model = run_both(fdx, oracle, modelgen, spec, [x])
+    assert abs(model.last_flops() - 2 * modelgen.model_flops(spec)) / (2 * modelgen.model_flops(spec)) < 1e-9
+
+
+def test_mobilenet_v2_truncated(fdx, oracle, modelgen):
+    say("mobilenet")
+    spec = modelgen.mobilenet_v2(seed=22, input_size=96, classes=30, random_bn=True, truncate=8)
+    spec = with_taps(spec, ["global_average_pooling2d", "block_3_depthwise_relu"])
+    x = np.random.default_rng(15).uniform(0, 1, (3, 96, 96, 3)).astype(np.float32)
+    spec = fix_tap_shapes(spec, oracle, modelgen, [x[0]])
+    run_both(fdx, oracle, modelgen, spec, [x])
+
+
+def test_encoder_small(fdx, oracle, modelgen):
+    say("encoder")
+    spec = modelgen.encoder(seed=23, layers=2, seq=24, d_model=64, heads=4, ffn=128, bias_std=0.1, random_affine=True)
+    x = np.random.default_rng(16).standard_normal((3, 24, 64)).astype(np.float32)
+    run_both(fdx, oracle, modelgen, spec, [x])
+
+
+def test_gpt2_tiny_predict_is_unmasked(fdx, oracle, modelgen):
+    say("gpt2 tiny predict")
+    spec = modelgen.gpt2(seed=24, layers=2, d_model=32, heads=4, vocab=97, max_pos=32, bias_std=0.1, random_affine=True,
+                         std=0.2)
+    r = np.random.default_rng(17)
+    ids = r.integers(0, 97, (2, 9)).astype(np.float32)
+    pos = np.tile(np.arange(9, dtype=np.float32), (2, 1))
+    run_both(fdx, oracle, modelgen, spec, [ids, pos])
+
+
+def test_input_shape_errors(fdx, modelgen):
+    say("shape errors")
+    model = fdx.Model(modelgen.dumps(modelgen.small_cnn()))
+    with pytest.raises(fdx.FdxError, match="Invalid inputs shape"):
+        model.predict([np.zeros((1, 32, 32, 4), np.float32)])
+    with pytest.raises(fdx.FdxError, match="Invalid inputs shape"):
+        model.predict([np.zeros((1, 32 * 32 * 3), np.float32)])  # same volume, wrong rank
+    with pytest.raises(fdx.FdxError):
+        fdx.Model(b'{"image_data_format": "channels_first"}')
+    bad = modelgen.small_cnn()
+    bad["architecture"]["config"]["layers"][1]["class_name"] = "Conv9D"
+    with pytest.raises(fdx.FdxError, match="unknown layer type: Conv9D"):
+        fdx.Model(modelgen.dumps(bad))
