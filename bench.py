@@ -1,11 +1,16 @@
-"""Benchmark of the forward hot path on one MI355X.
+"""Benchmark of the forward hot path on one MI355X.  Prints ONE JSON line.
 
-Primary line (BASELINE.json metric, configs[1]): ResNet50-architecture CNN, fp32, batch 64, 224x224x3,
-random-init He-normal weights, synthetic uniform[0,1] inputs already resident in HBM.  One step = one
-batched predict (fdx_model_predict_dev) of 64 images.  Prints ONE JSON line.
+Primary figure (BASELINE.json metric, configs[1]): ResNet50-architecture CNN, fp32, batch 64, 224x224x3,
+random-init He-normal weights, synthetic uniform[0,1] inputs already resident in HBM.  One step = one batched
+predict (fdx_model_predict_dev) of 64 images; `value` = images / second.
+
+Second half of the metric, reported under "gpt2_decode": GPT-2-small-shaped decoder (12 layers, d 768, 12 heads,
+vocab 50257, untied head), batch 16, prompt 128 random ids, then 128 greedy tokens with the key/value cache;
+tokens / second over the decode loop and the fraction of the HBM roofline for the bytes a step must stream.
 """
 import argparse
 import concurrent.futures
+import ctypes
 import importlib
 import json
 import os
@@ -30,7 +35,6 @@ def load_package():
 
 
 def profile_families(fdx):
-    import ctypes
     fams = {}
     i = 0
     while True:
@@ -58,19 +62,7 @@ def cpu_baseline_resnet(js, x, cores, passes=2):
     return cores * passes / dt
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (samples are independent; more GPUs would each take a "
-                 "slice of the batch with their own copy of the weights) -- use --gpus 1")
-
-    fdx, modelgen = load_package()
+def bench_resnet(fdx, modelgen, args):
     batch = args.batch
     spec = modelgen.resnet50()
     flops_per_image = modelgen.model_flops(spec)
@@ -87,7 +79,6 @@ def main():
     for _ in range(args.warmup):
         model.predict_dev(batch, [d_in], shapes, [d_out])
     fdx.sync()
-    import ctypes
     ms = ctypes.c_float()
     t0 = time.perf_counter()
     fdx.check(fdx.lib.fdx_timer_start())
@@ -102,9 +93,10 @@ def main():
     assert np.isfinite(probs).all() and np.abs(probs.sum(-1) - 1).max() < 1e-3
 
     # per-kernel pass: HIP events around every launch on the library stream (same work, outside the timed region)
+    prof_steps = max(2, args.steps // 4)
     fdx.check(fdx.lib.fdx_profile_enable(1))
     fdx.check(fdx.lib.fdx_profile_reset())
-    for _ in range(max(2, args.steps // 4)):
+    for _ in range(prof_steps):
         model.predict_dev(batch, [d_in], shapes, [d_out])
     fdx.sync()
     fams = profile_families(fdx)
@@ -144,7 +136,7 @@ def main():
             "share_of_step_time": round(mf_ms / total_ms, 4) if total_ms else None,
             "traffic": None,
         },
-        "kernel_ms_per_step": {k: round(v["ms"] / max(2, args.steps // 4), 4) for k, v in sorted(fams.items())},
+        "kernel_ms_per_step": {k: round(v["ms"] / prof_steps, 4) for k, v in sorted(fams.items())},
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
         "load_seconds": round(load_s, 2),
     }
@@ -154,6 +146,89 @@ def main():
         result["cpu_baseline"] = {"value": round(cpu, 3), "unit": "img/s", "cores": cores, "kind": "port",
                                   "sample": "%d ResNet50 predictions per pass (one per core, in parallel threads), "
                                             "1 warm-up + 2 timed passes of the CPU oracle" % cores}
+    model.close()
+    return result
+
+
+def gpt2_step_bytes(L, batch=16, layers=12, d=768, ffn=3072, vocab=50257):
+    """Bytes one decode step must stream at context length L (keys visible incl. the new token)."""
+    w_layers = layers * (4 * d * d + 4 * d + 2 * d * ffn + ffn + d + 4 * d) * 4
+    w_head = (d * vocab + vocab) * 4
+    kv = layers * 2 * L * d * 4 * batch
+    logits = batch * vocab * 4
+    return w_layers + w_head + kv + logits
+
+
+def bench_gpt2(fdx, modelgen, args):
+    batch, prompt, new = 16, 128, 128
+    spec = modelgen.gpt2()
+    js = modelgen.dumps(spec)
+    del spec
+    t0 = time.perf_counter()
+    model = fdx.Model(js, verify=False)
+    load_s = time.perf_counter() - t0
+    del js
+    ids = np.random.default_rng(99).integers(0, 50257, (batch, prompt)).astype(np.float32)
+    sess = fdx.Session(model, batch, prompt + new)
+    d_ids = fdx.DevBuf.from_host(ids)
+    d_first, d_tok, d_log = fdx.DevBuf(4 * batch), fdx.DevBuf(4 * new * batch), fdx.DevBuf(4 * batch * 50257)
+    ms = ctypes.c_float()
+    best = None
+    for rep in range(1 + max(1, args.decode_reps)):  # first repetition is the warm-up
+        sess.reset()
+        fdx.check(fdx.lib.fdx_timer_start())
+        fdx.check(fdx.lib.fdx_session_prefill(sess._h, fdx._dp(d_ids), prompt, None, fdx._dp(d_first)))
+        fdx.check(fdx.lib.fdx_timer_stop(ctypes.byref(ms)))
+        prefill_ms = ms.value
+        fdx.check(fdx.lib.fdx_timer_start())
+        fdx.check(fdx.lib.fdx_session_decode_greedy(sess._h, fdx._dp(d_first), new, fdx._dp(d_tok), fdx._dp(d_log)))
+        fdx.check(fdx.lib.fdx_timer_stop(ctypes.byref(ms)))
+        if rep > 0 and (best is None or ms.value < best[0]):
+            best = (ms.value, prefill_ms)
+    decode_ms, prefill_ms = best
+    tokens = d_tok.to_host((new, batch))
+    assert np.isfinite(tokens).all() and tokens.min() >= 0 and tokens.max() < 50257
+    total_bytes = sum(gpt2_step_bytes(prompt + 1 + i) for i in range(new))
+    achieved = total_bytes / (decode_ms / 1e3) / 1e9
+    out = {
+        "metric": "GPT-2-small-shape KV-cache greedy decode tok/s (fp32, batch 16, prompt 128 + 128 new)",
+        "value": round(batch * new / (decode_ms / 1e3), 1),
+        "unit": "tok/s",
+        "ms_per_step": round(decode_ms / new, 4),
+        "prefill_ms": round(prefill_ms, 3),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "bytes_per_step_mean": round(total_bytes / new),
+                     "traffic": None},
+        "load_seconds": round(load_s, 2),
+    }
+    sess.close()
+    model.close()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--decode-reps", type=int, default=2)
+    ap.add_argument("--workload", choices=["all", "resnet50", "gpt2"], default="all")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (samples are independent; more GPUs would each take a "
+                 "slice of the batch with their own copy of the weights) -- use --gpus 1")
+    fdx, modelgen = load_package()
+    result = {}
+    if args.workload in ("all", "resnet50"):
+        result = bench_resnet(fdx, modelgen, args)
+    if args.workload in ("all", "gpt2"):
+        g = bench_gpt2(fdx, modelgen, args)
+        if result:
+            result["gpt2_decode"] = g
+        else:
+            result = g
     print(json.dumps(result), flush=True)
 
 

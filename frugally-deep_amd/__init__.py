@@ -366,3 +366,54 @@ class Model:
             self.close()
         except Exception:
             pass
+
+
+class Session:
+    """Autoregressive decoding with a key/value cache over a decoder Model (fdx_session_*)."""
+
+    def __init__(self, model, batch, max_len):
+        self.model, self.batch, self.max_len = model, batch, max_len
+        self.vocab = model.output_shapes[0][-1]
+        self._h = ctypes.c_void_p()
+        check(lib.fdx_session_create(model._h, batch, max_len, ctypes.byref(self._h)))
+
+    def length(self):
+        n = ctypes.c_int()
+        check(lib.fdx_session_length(self._h, ctypes.byref(n)))
+        return n.value
+
+    def reset(self):
+        check(lib.fdx_session_reset(self._h))
+
+    def prefill(self, ids):
+        """ids [batch, t]; returns (logits [batch, vocab] of the last position, greedy next ids [batch])."""
+        ids = np.ascontiguousarray(ids, np.float32)
+        assert ids.shape[0] == self.batch
+        d_ids, d_log, d_next = DevBuf.from_host(ids), DevBuf(4 * self.batch * self.vocab), DevBuf(4 * self.batch)
+        check(lib.fdx_session_prefill(self._h, _dp(d_ids), ids.shape[1], _dp(d_log), _dp(d_next)))
+        return d_log.to_host((self.batch, self.vocab)), d_next.to_host((self.batch,)).astype(np.int64)
+
+    def decode_step(self, ids):
+        ids = np.ascontiguousarray(ids, np.float32).reshape(self.batch)
+        d_ids, d_log, d_next = DevBuf.from_host(ids), DevBuf(4 * self.batch * self.vocab), DevBuf(4 * self.batch)
+        check(lib.fdx_session_decode_step(self._h, _dp(d_ids), _dp(d_log), _dp(d_next)))
+        return d_log.to_host((self.batch, self.vocab)), d_next.to_host((self.batch,)).astype(np.int64)
+
+    def decode_greedy(self, first_ids, steps):
+        """Feeds each step's argmax back in; returns (tokens [steps, batch], logits of the last step)."""
+        first = np.ascontiguousarray(first_ids, np.float32).reshape(self.batch)
+        d_first, d_tok = DevBuf.from_host(first), DevBuf(4 * steps * self.batch)
+        d_log = DevBuf(4 * self.batch * self.vocab)
+        check(lib.fdx_session_decode_greedy(self._h, _dp(d_first), steps, _dp(d_tok), _dp(d_log)))
+        return d_tok.to_host((steps, self.batch)).astype(np.int64), d_log.to_host((self.batch, self.vocab))
+
+    def close(self):
+        if self._h:
+            check(lib.fdx_session_destroy(self._h))
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

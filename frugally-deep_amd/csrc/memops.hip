@@ -560,6 +560,22 @@ fdx_status transpose_launch(const float* in, int batch, int rows, int cols, int6
     return FDX_OK;
 }
 
+__global__ void positions_kernel(float* __restrict__ out, int batch, int t, int start)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < batch * t)
+        out[i] = (float)(start + i % t);
+}
+
+// out[b][j] = start + j : the position ids of `t` new tokens of every sequence
+fdx_status positions_launch(float* out, int batch, int t, int start)
+{
+    FDX_REQUIRE(out && batch > 0 && t > 0 && start >= 0, "positions: bad arguments");
+    hipLaunchKernelGGL(positions_kernel, dim3((batch * t + 255) / 256), dim3(256), 0, stream(), out, batch, t, start);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
 fdx_status gather_rows_launch(const float* in, int64_t rows, int depth, int64_t row_stride, int64_t offset, float* out)
 {
     FDX_REQUIRE(in && out && rows > 0 && depth > 0, "gather_rows: bad arguments");

@@ -552,7 +552,10 @@ namespace {
     fdx_status infer_shapes(const fdx_model& m, const std::vector<Shape>& in_shapes, std::vector<Shape>& shapes,
         const std::vector<int>& order);
 
-    std::vector<int> topo_order(const fdx_model& m)
+} // namespace
+
+std::vector<int> topo_order(const fdx_model& m)
+{
     {
         std::vector<int> order;
         std::vector<char> seen(m.ops.size(), 0);
@@ -572,6 +575,9 @@ namespace {
             visit(o);
         return order;
     }
+}
+
+namespace {
 
     void fuse(fdx_model& m)
     {

@@ -95,6 +95,8 @@ namespace fdx {
 // builds (or reuses) the plan for this batch and these per-sample input shapes
 fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out);
 float* plan_alloc(Plan& p, size_t bytes, int* block_index);
+std::vector<int> topo_order(const fdx_model& m); // producers before consumers, dead ops skipped by callers
+fdx_status positions_launch(float* out, int batch, int t, int start);
 fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, const float* k, int64_t ldk, int64_t k_batch,
     const float* v, int64_t ldv, int64_t v_batch, int batch, int t, int s, int heads, int dk, int dv, int causal,
     float* out, int64_t ldo, int64_t o_batch, void* scratch_dev);
