@@ -13,29 +13,14 @@
 // LDS read into four MFMAs (the k order inside a slab is permuted identically for A and
 // B, which a sum does not notice).  Epilogue: alpha, bias (per column or per row),
 // residual add, activation, fused on the accumulators before the only store.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+
 #include "common.hpp"
+#include "igemm_params.hpp"
 
 namespace fdx {
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-struct GemmParams {
-    const float* A;
-    const float* B;
-    float* C;
-    const float* bias;
-    const float* residual;
-    int M, N, K;
-    int64_t lda, ldb, ldc;
-    float alpha;
-    int bias_per_row;
-    Act act;
-    int inner;
-    int64_t a_outer, a_inner, b_outer, b_inner, c_outer, c_inner;
-    // convolution view of A
-    int H, W, Cin, kh, kw, sy, sx, dy, dx, pad_top, pad_left, OH, OW;
-};
 
 enum { A_ROWS_VEC = 0, A_CONV_VEC = 1, A_CONV_SCALAR = 2, A_ROWS_SCALAR = 3 };
 
@@ -267,6 +252,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParam
     }
 }
 
+
+#include "igemm_fast.hpp"
+
 // ------------------------------------------------------------------ dispatch
 
 static int g_forced_tile = -1; // tests force a tile configuration through fdx_debug_force_tile
@@ -292,7 +280,101 @@ static void launch_cfg(const GemmParams& p, int a_mode, int b_vec, int batch, hi
 #undef FDX_IGEMM_CASE
 }
 
+// Persistent launch: as many workgroups as fit on the chip at once (occupancy x CUs, cached per
+// kernel), or one per tile when there are fewer tiles than that.
+static int g_persist_scale = 0; // 0 = resident workgroups; tests and tuning may override the grid cap
+template <typename K>
+static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStream_t s)
+{
+    static int resident = 0; // one instance per kernel instantiation
+    if (resident == 0) {
+        int per_cu = 1, dev = 0;
+        hipDeviceProp_t prop;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1)
+            per_cu = 1;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+            prop.multiProcessorCount = 256;
+        resident = per_cu * prop.multiProcessorCount;
+    }
+    const int cap = g_persist_scale > 0 ? g_persist_scale : resident;
+    const int grid = tiles < cap ? tiles : cap;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, q);
+}
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static void launch_fast(int cfg, const GemmParams& q, bool conv, int batch, hipStream_t s)
+{
+#define FDX_FAST(BM_, BN_, BK_)                                                                                  \
+    {                                                                                                            \
+        const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
+        if (conv)                                                                                                \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s);                        \
+        else                                                                                                     \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s);                       \
+    }
+        switch (cfg) {
+        case 10: FDX_FAST(128, 128, 16) break;
+        case 11: FDX_FAST(128, 64, 16) break;
+        case 12: FDX_FAST(64, 64, 16) break;
+        case 13: FDX_FAST(128, 128, 32) break;
+        case 14: FDX_FAST(128, 64, 32) break;
+        default: FDX_FAST(64, 64, 32) break;
+        }
+#undef FDX_FAST
+}
+
+// First sight of a problem shape on the fast path: time every tile configuration once on the
+// real operands (the launches are idempotent) and remember the winner.  Tile count versus
+// resident workgroups, K depth and output width interact too irregularly for a closed rule.
+struct TuneKey {
+    int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
+    bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }
+};
+static std::map<TuneKey, int> g_tuned;
+static int g_autotune = -1;
+
+static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s)
+{
+    if (g_autotune < 0) {
+        const char* e = std::getenv("FDX_AUTOTUNE");
+        g_autotune = (e && e[0] == '0') ? 0 : 1;
+    }
+    if (!g_autotune)
+        return -1;
+    TuneKey key;
+    std::memset(&key, 0, sizeof key);
+    key.conv = conv; key.M = q.M; key.N = q.N; key.K = q.K; key.Cin = conv ? q.Cin : 0; key.kh = conv ? q.kh : 0;
+    key.kw = conv ? q.kw : 0; key.sy = conv ? q.sy : 0; key.sx = conv ? q.sx : 0; key.batch = batch; key.res = q.residual != nullptr;
+    auto it = g_tuned.find(key);
+    if (it != g_tuned.end())
+        return it->second;
+    hipEvent_t a, b;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess)
+        return -1;
+    int best = -1;
+    float best_ms = 1e30f;
+    for (int cfg = 10; cfg <= 15; ++cfg) {
+        if (cfg >= 13 && unit % 32 != 0)
+            continue;
+        launch_fast(cfg, q, conv, batch, s); // warm-up
+        (void)hipEventRecord(a, s);
+        for (int r = 0; r < 3; ++r)
+            launch_fast(cfg, q, conv, batch, s);
+        (void)hipEventRecord(b, s);
+        float ms = 1e30f;
+        if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
+            continue;
+        if (ms < best_ms) {
+            best_ms = ms;
+            best = cfg;
+        }
+    }
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    g_tuned[key] = best;
+    return best;
+}
 
 static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* family)
 {
@@ -305,30 +387,74 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             : A_ROWS_SCALAR;
     const int b_vec = (p.K % 4 == 0 && p.ldb % 4 == 0 && aligned16(p.B) && p.b_outer % 4 == 0 && p.b_inner % 4 == 0) ? 1 : 0;
 
-    // Tile choice: the largest tile that still yields at least ~2 waves of workgroups over
-    // the 256 CUs; narrow N picks the 32-wide tile.
-    int cfg;
     auto blocks = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * batch; };
-    if (p.N <= 32)
-        cfg = 2;
-    else if (p.N <= 64)
-        cfg = blocks(128, 64) >= 512 ? 1 : 3;
-    else if (blocks(128, 128) >= 512)
-        cfg = 0;
-    else if (blocks(128, 64) >= 512)
-        cfg = 1;
-    else
-        cfg = 3;
-    if (g_forced_tile >= 0)
-        cfg = g_forced_tile;
-
     hipStream_t s = stream();
+
+    // ---- fast path eligibility (see igemm_fast_kernel)
+    const bool out_ok = p.N % 4 == 0 && p.ldc % 4 == 0 && aligned16(p.C) && p.c_outer % 4 == 0 && p.c_inner % 4 == 0
+        && (!p.residual || aligned16(p.residual)) && (!p.bias || aligned16(p.bias)) && !p.bias_per_row;
+    const int64_t b_bytes = ((int64_t)(p.N - 1) * p.ldb + p.K) * 4;
+    int64_t a_bytes, a_shift = 0;
+    bool a_ok;
+    if (conv) {
+        a_shift = ((int64_t)p.pad_top * p.W + p.pad_left) * p.Cin;
+        a_bytes = ((int64_t)(p.M / (p.OH * p.OW)) * p.H * p.W * p.Cin + a_shift) * 4 + 64;
+        a_ok = a_mode == A_CONV_VEC && p.Cin % 16 == 0 && p.kh * p.kw <= 64;
+    } else {
+        a_bytes = ((int64_t)(p.M - 1) * p.lda + p.K) * 4;
+        a_ok = a_mode == A_ROWS_VEC && p.K % 16 == 0;
+    }
+    const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31);
+    const int unit = conv ? p.Cin : p.K;
+
+    int cfg = g_forced_tile;
+    if (cfg >= 10 && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
+        cfg = -1;
+    if (cfg < 0) {
+        if (fast_ok && p.N >= 64 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
+            GemmParams q = p;
+            q.A = p.A - a_shift;
+            q.a_records = (uint32_t)a_bytes;
+            q.b_records = (uint32_t)b_bytes;
+            q.batch = batch;
+            cfg = autotune(q, conv, batch, unit, s);
+        }
+        if (cfg >= 10) {
+        } else if (fast_ok && p.N >= 64) {
+            // the largest tile that still gives every CU a few workgroups
+            if (blocks(128, 128) >= 1024 && p.N % 128 == 0)
+                cfg = 10;
+            else if (blocks(128, 64) >= 1024)
+                cfg = 11;
+            else
+                cfg = unit % 32 == 0 ? 15 : 12;
+        } else if (p.N <= 32)
+            cfg = 2;
+        else if (p.N <= 64)
+            cfg = blocks(128, 64) >= 512 ? 1 : 3;
+        else if (blocks(128, 128) >= 512)
+            cfg = 0;
+        else if (blocks(128, 64) >= 512)
+            cfg = 1;
+        else
+            cfg = 3;
+    }
+
     profile_begin();
-    switch (cfg) {
-    case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
-    case 1: launch_cfg<128, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
-    case 2: launch_cfg<128, 32, 4, 1>(p, a_mode, b_vec, batch, s); break;
-    default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+    if (cfg >= 10) {
+        GemmParams q = p;
+        q.A = p.A - a_shift;
+        q.a_records = (uint32_t)a_bytes;
+        q.b_records = (uint32_t)b_bytes;
+        q.batch = batch;
+        launch_fast(cfg, q, conv, batch, s);
+    } else {
+        switch (cfg) {
+        case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        case 1: launch_cfg<128, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        case 2: launch_cfg<128, 32, 4, 1>(p, a_mode, b_vec, batch, s); break;
+        default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        }
     }
     const double flops = 2.0 * p.M * (double)p.N * p.K * batch;
     profile_end(family, flops, 0.0);

@@ -1,0 +1,242 @@
+// Fast path of the implicit-GEMM Conv2D / GEMM (included inside namespace fdx by igemm.hip).
+//
+// Same tiling and MFMA schedule as igemm_kernel, with the per-slab overhead stripped for the
+// shapes that dominate real networks (Cin, or K for a plain GEMM, a multiple of the slab; N a
+// multiple of 4), and the workgroups made persistent:
+//
+//  * Operands are fetched with raw buffer loads: each lane keeps ONE 32-bit byte offset per
+//    tile row for the whole K loop, the walk along K is a scalar offset shared by the
+//    workgroup (filter tap and channel are uniform within a slab), and a padded or
+//    out-of-range tap is an offset beyond the buffer's extent, which the hardware answers
+//    with zeros -- no branches, no per-slab address arithmetic.  A's base is shifted down by
+//    the top-left padding so offsets stay non-negative.
+//  * A workgroup walks a strided list of output tiles.  Before it writes a finished tile it
+//    already has the first slab of its next tile in flight, and the tile's stores drain while
+//    the next tile computes: output traffic and first-load latency overlap with MFMA work
+//    instead of adding to it (with one tile per workgroup all workgroups of a round reach
+//    their epilogue together and the matrix cores idle while HBM drains).
+//  * The epilogue goes through LDS so that bias, residual and output move as 16-byte
+//    accesses along the channel axis.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV>
+__global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
+{
+    constexpr int NT = 256;
+    static_assert(WAVES_M * WAVES_N == 4, "256 threads");
+    constexpr int STRIDE = BKT + 4;
+    constexpr int CPR = BKT / 4;  // 16-byte chunks per tile row
+    constexpr int RPP = NT / CPR; // tile rows filled per loader pass
+    constexpr int A_LOADS = BM / RPP, B_LOADS = BN / RPP;
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must be a multiple of the loader pass");
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int OSTRIDE = WTN + 4; // epilogue scratch row
+    static_assert(2 * (BM + BN) * STRIDE >= 4 * 32 * OSTRIDE, "epilogue scratch must fit in the operand buffers");
+    constexpr uint32_t OOB = 0x80000000u; // beyond any extent this path accepts: the load returns zeros
+
+    __shared__ __attribute__((aligned(16))) float smem[2 * (BM + BN) * STRIDE];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int kq = t % CPR, r0 = t / CPR;
+    const int fr = lane & 31, fh = lane >> 5;
+
+    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+    const int per_problem = tiles_m * tiles_n;
+    const int total = per_problem * p.batch;
+    // XCD x (workgroups with blockIdx % 8 == x) owns the contiguous tile range [lo, hi) so tiles
+    // that share an A row block also share that XCD's L2; its workgroups stride through it.
+    const int xcd = blockIdx.x & 7, wg_in_xcd = blockIdx.x >> 3;
+    const int wgs_in_xcd = ((int)gridDim.x - xcd + 7) >> 3;
+    const int per = total >> 3, rem = total & 7;
+    const int lo = xcd * per + (xcd < rem ? xcd : rem), hi = lo + per + (xcd < rem ? 1 : 0);
+
+    // ---- per-tile loader state
+    uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+    uint64_t a_mask[A_LOADS];
+    __amdgpu_buffer_rsrc_t srd_a, srd_b;
+    int tap, fx, fy, c0, soff_a, soff_b;
+    f32x4 ra[A_LOADS], rb[B_LOADS];
+
+    auto setup = [&](int tile, int& m0, int& n0, int64_t& c_off) {
+        const int z = tile / per_problem, id = tile - z * per_problem;
+        m0 = (id / tiles_n) * BM;
+        n0 = (id % tiles_n) * BN;
+        const float* A = p.A + (z / p.inner) * p.a_outer + (z % p.inner) * p.a_inner;
+        const float* B = p.B + (z / p.inner) * p.b_outer + (z % p.inner) * p.b_inner;
+        c_off = (z / p.inner) * p.c_outer + (z % p.inner) * p.c_inner;
+        srd_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, (int)p.a_records, 0x00020000);
+        srd_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, (int)p.b_records, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const int m = m0 + r0 + i * RPP;
+            a_voff[i] = OOB;
+            a_mask[i] = 0;
+            if (m < p.M) {
+                if (CONV) {
+                    const int img = m / (p.OH * p.OW), rm = m - img * (p.OH * p.OW);
+                    const int oy = rm / p.OW, ox = rm - oy * p.OW;
+                    const int iy0 = oy * p.sy - p.pad_top, ix0 = ox * p.sx - p.pad_left;
+                    // byte offset from the shifted base (shift = (pad_top*W + pad_left)*Cin elements)
+                    a_voff[i] = (uint32_t)(((img * p.H + oy * p.sy) * p.W + ox * p.sx) * p.Cin) * 4u + kq * 16;
+                    uint64_t mk = 0;
+                    for (int y = 0; y < p.kh; ++y) {
+                        const int iy = iy0 + y * p.dy;
+                        for (int x = 0; x < p.kw; ++x) {
+                            const int ix = ix0 + x * p.dx;
+                            if (iy >= 0 && iy < p.H && ix >= 0 && ix < p.W)
+                                mk |= 1ull << (y * p.kw + x);
+                        }
+                    }
+                    a_mask[i] = mk;
+                } else {
+                    a_voff[i] = (uint32_t)((int64_t)m * p.lda) * 4u + kq * 16;
+                    a_mask[i] = ~0ull;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const int n = n0 + r0 + i * RPP;
+            b_voff[i] = n < p.N ? (uint32_t)((int64_t)n * p.ldb) * 4u + kq * 16 : OOB;
+        }
+        tap = fx = fy = c0 = 0;
+        soff_a = soff_b = 0;
+    };
+    auto load_tiles = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const uint32_t vo = CONV ? (((a_mask[i] >> tap) & 1) ? a_voff[i] : OOB) : a_voff[i];
+            ra[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_a, (int)vo, soff_a, 0));
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i)
+            rb[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, (int)b_voff[i], soff_b, 0));
+        soff_b += BKT * 4;
+        if (CONV) {
+            c0 += BKT;
+            if (c0 == p.Cin) {
+                c0 = 0;
+                ++tap;
+                if (++fx == p.kw) {
+                    fx = 0;
+                    ++fy;
+                }
+            }
+            soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.Cin + c0) * 4;
+        } else {
+            soff_a += BKT * 4;
+        }
+    };
+    auto store_tiles = [&](int buf) {
+        float* as = smem + buf * (BM + BN) * STRIDE;
+        float* bs = as + BM * STRIDE;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+            *reinterpret_cast<f32x4*>(&as[(r0 + i * RPP) * STRIDE + kq * 4]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i)
+            *reinterpret_cast<f32x4*>(&bs[(r0 + i * RPP) * STRIDE + kq * 4]) = rb[i];
+    };
+
+    const int KT = p.K / BKT;
+    int tile = lo + wg_in_xcd;
+    if (tile >= hi)
+        return; // uniform per workgroup
+    int m0, n0;
+    int64_t c_off;
+    setup(tile, m0, n0, c_off);
+    load_tiles();
+
+    for (;;) {
+        f32x16 acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0.f;
+
+        store_tiles(0);
+        __syncthreads();
+        for (int kt = 0; kt < KT; ++kt) {
+            const int buf = kt & 1;
+            if (kt + 1 < KT)
+                load_tiles();
+            const float* as = smem + buf * (BM + BN) * STRIDE;
+            const float* bs = as + BM * STRIDE;
+#pragma unroll
+            for (int k8 = 0; k8 < BKT / 8; ++k8) {
+                f32x4 af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    af[i] = *reinterpret_cast<const f32x4*>(&as[(wm * WTM + i * 32 + fr) * STRIDE + k8 * 8 + fh * 4]);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    bf[j] = *reinterpret_cast<const f32x4*>(&bs[(wn * WTN + j * 32 + fr) * STRIDE + k8 * 8 + fh * 4]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+            }
+            if (kt + 1 < KT)
+                store_tiles(buf ^ 1);
+            __syncthreads();
+        }
+
+        // this tile's coordinates for the epilogue; the loader state moves on to the next tile
+        const int em0 = m0, en0 = n0;
+        float* __restrict__ C = p.C + c_off;
+        const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
+        tile += wgs_in_xcd;
+        const bool more = tile < hi;
+        if (more) {
+            setup(tile, m0, n0, c_off);
+            load_tiles(); // in flight while this tile is written out
+        }
+
+        // ---- epilogue: accumulators -> per-wave LDS scratch [32][WTN] -> 16-byte row accesses
+        float* scratch = smem + wave * 32 * OSTRIDE;
+        constexpr int LPR = WTN / 4;  // lanes per scratch row
+        constexpr int RPS = 64 / LPR; // rows per store pass
+        const int srow = lane / LPR, scol = (lane % LPR) * 4;
+        const int n = en0 + wn * WTN + scol;
+        const bool n_ok = n < p.N; // N is a multiple of 4 on this path
+        f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
+        if (p.bias && n_ok)
+            bias4 = *reinterpret_cast<const f32x4*>(p.bias + n);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    scratch[(8 * (e >> 2) + 4 * fh + (e & 3)) * OSTRIDE + j * 32 + fr] = acc[i][j][e];
+            __syncthreads();
+#pragma unroll
+            for (int ps = 0; ps < 32 / RPS; ++ps) {
+                const int row = ps * RPS + srow;
+                const int m = em0 + wm * WTM + i * 32 + row;
+                if (m < p.M && n_ok) {
+                    f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
+                    const int64_t off = (int64_t)m * p.ldc + n;
+                    f32x4 r = { 0.f, 0.f, 0.f, 0.f };
+                    if (R)
+                        r = *reinterpret_cast<const f32x4*>(R + off);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = apply_act(v[e] * p.alpha + bias4[e] + r[e], p.act);
+                    *reinterpret_cast<f32x4*>(C + off) = v;
+                }
+            }
+            __syncthreads();
+        }
+        if (!more)
+            break;
+    }
+}

@@ -1,0 +1,31 @@
+// Launch parameters shared by the implicit-GEMM kernels.
+#pragma once
+#include "common.hpp"
+
+namespace fdx {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmParams {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;
+    const float* residual;
+    int M, N, K;
+    int64_t lda, ldb, ldc;
+    float alpha;
+    int bias_per_row;
+    Act act;
+    int inner;
+    int64_t a_outer, a_inner, b_outer, b_inner, c_outer, c_inner;
+    // convolution view of A
+    int H, W, Cin, kh, kw, sy, sx, dy, dx, pad_top, pad_left, OH, OW;
+    // fast path only: byte extents of one problem's A (counted from the shifted base) and B operands
+    uint32_t a_records, b_records;
+    int batch; // number of independent problems folded into the persistent tile walk
+};
+
+
+} // namespace fdx

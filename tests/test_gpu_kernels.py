@@ -41,7 +41,7 @@ CONV_CASES = [
 ]
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("case", CONV_CASES)
 def test_conv2d_vs_oracle(fdx, oracle, case, tile):
     n, h, w, cin, cout, kh, kw, strides, dilation, padding = case
@@ -84,7 +84,7 @@ GEMM_CASES = [(1, 10, 32), (16, 768, 768), (37, 50, 29), (256, 2048, 512), (130,
               (300, 96, 100)]
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("m,n,k", GEMM_CASES)
 def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
     say("gemm", m, n, k, "tile", tile)
