@@ -1,0 +1,656 @@
+// Decode-shape kernels (gfx950): a handful of activation rows against a whole weight matrix.
+//
+// With at most 16 rows the GEMMs of a decode step are pure weight streaming: every byte of W
+// is used once, so the kernel is HBM-bound and latency-bound, and the job is to put every
+// load in flight at once and add nothing to the launch.  One workgroup of 8 wave64s owns 16
+// output columns; the waves split K; each lane issues ALL its 16-byte weight and activation
+// loads for a chunk of slabs before the first use, and v_mfma_f32_16x16x4_f32 does the 16x16
+// products (it also performs the reduction along K that a VALU formulation would need
+// cross-lane shuffles for).  The eight partial 16x16 tiles meet in LDS; bias, activation and
+// residual are applied before the only store.
+//
+// A LayerNormalization in front of the GEMM costs no pass over the rows: with gamma folded
+// into the weights (W' = W * gamma along k), their row sums s[n] and b' = b + W beta
+// precomputed once, LN(x) W^T + b = rstd * (x W'^T - mean * s) + b', so the kernel multiplies
+// the raw rows and only needs each row's mean and 1/sqrt(var + eps); both come from the
+// activation registers the lanes already hold (two-pass variance, as the reference computes
+// it) while the weight loads are still in flight.
+//
+// Up to three output segments let one launch write q and the new key / value cache rows.
+#include <cfloat>
+#include <cmath>
+#include <cstring>
+
+#include "common.hpp"
+#include "skinny.hpp"
+
+namespace fdx {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int SK_WAVES = 8;
+constexpr int SK_CHUNK = 8;       // slabs of 16 k-values whose loads are issued together (8 waves x 8 x 16 = 1024 k)
+constexpr int SK_CHUNK_LONG = 24; // long-K launches (up to 3072) still issue everything at once, one workgroup per CU
+
+// SINGLE: the workgroup's K range fits one chunk per wave (only one register set is live, which
+// triples the number of resident workgroups).  gridDim.y > 1 splits K across workgroups: partial
+// tiles go to a workspace and the last workgroup to arrive at a column group (atomic ticket) adds
+// them in split order -- deterministic, no spinning -- and runs the epilogue.
+template <int CHUNK, bool SINGLE>
+__global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
+{
+    __shared__ float red[SK_WAVES * 256];
+    __shared__ int is_last;
+    __shared__ float stat[SK_WAVES * 16];
+    __shared__ float row_mean[16], row_rstd[16];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int i = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int K = p.K;
+
+    // K range of this workgroup (split index blockIdx.y) and of this wave, multiples of 16
+    const int ksplit = gridDim.y;
+    const int per_wg = ((K + ksplit * 16 - 1) / (ksplit * 16)) * 16;
+    const int wg_begin = blockIdx.y * per_wg;
+    const int wg_end = wg_begin + per_wg < K ? wg_begin + per_wg : K;
+    const int per_wave = ((per_wg + SK_WAVES * 16 - 1) / (SK_WAVES * 16)) * 16;
+    const int k_begin = wg_begin + wave * per_wave;
+    const int k_end = k_begin + per_wave < wg_end ? k_begin + per_wave : wg_end;
+    const int slabs = k_end > k_begin ? (k_end - k_begin + 15) / 16 : 0;
+
+    const int n = n0 + i;
+    const bool n_ok = n < p.N, m_ok = i < p.M;
+    const float* wrow = p.W + (int64_t)(n_ok ? n : 0) * p.ldw;
+    const int spw = per_wave / 16; // slabs per wave in the packed layout
+    const float* xrow = p.X + (int64_t)(m_ok ? i : 0) * p.ldx;
+    // two named register sets (indexing one array with a run-time buffer number would push it to scratch)
+    f32x4 w0[CHUNK], a0[CHUNK];
+    auto load_chunk = [&](f32x4 (&wreg)[CHUNK], f32x4 (&areg)[CHUNK], int s0) {
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s) {
+            const int k = k_begin + (s0 + s) * 16 + kq * 4;
+            const bool k_ok = s0 + s < slabs && k < k_end;
+            f32x4 wv = { 0.f, 0.f, 0.f, 0.f }, av = { 0.f, 0.f, 0.f, 0.f };
+            if (p.packed) {
+                // pre-packed operand: this wave's slab is one contiguous 1 KB run, zeros baked in
+                if (s0 + s < spw)
+                    wv = reinterpret_cast<const f32x4*>(p.W)[(((int64_t)blockIdx.x * SK_WAVES + wave) * spw + (s0 + s)) * 64 + lane];
+            } else if (n_ok && k_ok)
+                wv = *reinterpret_cast<const f32x4*>(wrow + k);
+            if (m_ok && k_ok)
+                av = *reinterpret_cast<const f32x4*>(xrow + k);
+            wreg[s] = wv;
+            areg[s] = av;
+        }
+    };
+    load_chunk(w0, a0, 0);
+
+    // epilogue operands of this thread's output element travel with the weights instead of costing a
+    // second dependent round trip after the reduction
+    const int em = t >> 4, ecol = n0 + (t & 15);
+    const bool e_ok = t < 256 && em < p.M && ecol < p.N;
+    float e_bias = 0.f, e_res = 0.f, e_wsum = 0.f;
+    int64_t e_shift = 0;
+    int e_seg = 0;
+    if (e_ok) {
+        if (p.bias)
+            e_bias = p.bias[ecol];
+        if (p.residual)
+            e_res = p.residual[(int64_t)em * p.ldr + ecol];
+        if (p.ln)
+            e_wsum = p.w_rowsum[ecol];
+        if (p.n_seg > 1 && ecol >= p.seg[1].col_begin)
+            e_seg = 1;
+        if (p.n_seg > 2 && ecol >= p.seg[2].col_begin)
+            e_seg = 2;
+        if (p.seg[e_seg].len_stride)
+            e_shift = (int64_t)(*p.len_dev) * p.seg[e_seg].len_stride;
+    }
+
+    // 16x16x4 MFMA: A operand lane (m = i, k slot = kq), B operand lane (n = i, k slot = kq);
+    // lane l ends up with D[4*(l/16) + e][l%16], e = 0..3.
+    f32x4 acc = { 0.f, 0.f, 0.f, 0.f };
+    auto compute_chunk = [&](const f32x4 (&wreg)[CHUNK], const f32x4 (&areg)[CHUNK]) {
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[s][e], wreg[s][e], acc, 0, 0, 0);
+    };
+
+    if (p.ln) {
+        // rows fit one chunk (host guarantees K <= 8 * CHUNK * 16): statistics from the registers
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < CHUNK; ++c)
+            s += (a0[c][0] + a0[c][1]) + (a0[c][2] + a0[c][3]);
+        s += __shfl_xor(s, 16, 64);
+        s += __shfl_xor(s, 32, 64);
+        if (kq == 0)
+            stat[wave * 16 + i] = s;
+        __syncthreads();
+        if (t < 16) {
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+                tot += stat[w * 16 + t];
+            row_mean[t] = tot / (float)K;
+        }
+        __syncthreads();
+        const float mean = row_mean[i];
+        float q = 0.f;
+#pragma unroll
+        for (int c = 0; c < CHUNK; ++c) {
+            const int k = k_begin + c * 16 + kq * 4;
+            if (c < slabs && k < k_end) { // padding lanes hold zeros, not row values
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float d = a0[c][e] - mean;
+                    q += d * d;
+                }
+            }
+        }
+        q += __shfl_xor(q, 16, 64);
+        q += __shfl_xor(q, 32, 64);
+        __syncthreads();
+        if (kq == 0)
+            stat[wave * 16 + i] = q;
+        __syncthreads();
+        if (t < 16) {
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+                tot += stat[w * 16 + t];
+            row_rstd[t] = 1.0f / sqrtf(tot / (float)K + p.ln_eps);
+        }
+        compute_chunk(w0, a0);
+    } else if (SINGLE) {
+        compute_chunk(w0, a0);
+    } else {
+        f32x4 w1[CHUNK], a1[CHUNK];
+        for (int s0 = 0; s0 < slabs; s0 += 2 * CHUNK) {
+            if (s0 + CHUNK < slabs)
+                load_chunk(w1, a1, s0 + CHUNK);
+            compute_chunk(w0, a0);
+            if (s0 + 2 * CHUNK < slabs)
+                load_chunk(w0, a0, s0 + 2 * CHUNK);
+            if (s0 + CHUNK < slabs)
+                compute_chunk(w1, a1);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        red[wave * 256 + (4 * kq + e) * 16 + i] = acc[e];
+    __syncthreads();
+    float v = 0.f;
+    if (t < 256) {
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w)
+            v += red[w * 256 + t];
+    }
+    if (ksplit > 1) {
+        // Publish this split's partial tile with device-scope stores (they go past the XCD's L2), wait for
+        // them, then take a ticket; only the last arrival continues and adds the partials in split order,
+        // which makes the sum independent of arrival order.  No fence that writes back the whole L2.
+        float* part = p.workspace + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256;
+        if (t < 256)
+            __hip_atomic_store(part + t, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (t == 0) {
+            const int ticket = __hip_atomic_fetch_add(p.tickets + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = ticket == ksplit - 1;
+            if (is_last)
+                __hip_atomic_store(p.tickets + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // next launch
+        }
+        __syncthreads();
+        if (!is_last)
+            return;
+        if (t < 256) {
+            v = 0.f;
+            for (int ks = 0; ks < ksplit; ++ks)
+                v += __hip_atomic_load(p.workspace + ((int64_t)ks * gridDim.x + blockIdx.x) * 256 + t, __ATOMIC_RELAXED,
+                    __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (e_ok) {
+        if (p.ln)
+            v = row_rstd[em] * (v - row_mean[em] * e_wsum);
+        v = apply_act(v + e_bias + e_res, p.act);
+        const SkinnySegment& sg = p.seg[e_seg];
+        sg.ptr[e_shift + (int64_t)em * sg.ld + (ecol - sg.col_begin)] = v;
+    }
+}
+
+// [N][K] -> [column tile][wave][slab][lane] 16-byte pieces in exactly the order the GEMM's lanes consume
+// them (lane l of wave w, slab s holds W[tile*16 + l%16][w*per_wave + s*16 + (l/16)*4 ..+3], zero beyond N or K),
+// so every wave-wide load is one contiguous kilobyte
+__global__ __launch_bounds__(64) void pack_weights_kernel(const float* __restrict__ w, int N, int K, int64_t ldw, int per_wave,
+    float* __restrict__ out)
+{
+    const int spw = per_wave / 16;
+    const int64_t blk = blockIdx.x; // ((tile * 8 + wave) * spw + slab)
+    const int slab = (int)(blk % spw), wave = (int)((blk / spw) % SK_WAVES), tile = (int)(blk / ((int64_t)spw * SK_WAVES));
+    const int lane = threadIdx.x;
+    const int n = tile * 16 + (lane & 15), k = wave * per_wave + slab * 16 + (lane >> 4) * 4;
+    f32x4 v = { 0.f, 0.f, 0.f, 0.f };
+    if (n < N) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (k + e < K && k + e < (wave + 1) * per_wave)
+                v[e] = w[(int64_t)n * ldw + k + e];
+    }
+    reinterpret_cast<f32x4*>(out)[blk * 64 + lane] = v;
+}
+
+// W'[n][k] = W[n][k] * gamma[k];  s[n] = sum_k W'[n][k];  b'[n] = b[n] + sum_k W[n][k] * beta[k]
+__global__ __launch_bounds__(256) void fold_layernorm_kernel(const float* __restrict__ gamma, const float* __restrict__ beta,
+    const float* __restrict__ w, const float* __restrict__ bias, int k, float* __restrict__ w_out, float* __restrict__ wsum,
+    float* __restrict__ bias_out)
+{
+    __shared__ float sa[4], sb[4];
+    const int n = blockIdx.x;
+    const float* wr = w + (int64_t)n * k;
+    float* wo = w_out + (int64_t)n * k;
+    float s = 0.f, bsum = 0.f;
+    for (int z = threadIdx.x; z < k; z += 256) {
+        const float wv = wr[z];
+        const float folded = wv * (gamma ? gamma[z] : 1.f);
+        wo[z] = folded;
+        s += folded;
+        bsum += wv * (beta ? beta[z] : 0.f);
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o, 64);
+        bsum += __shfl_xor(bsum, o, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        sa[threadIdx.x >> 6] = s;
+        sb[threadIdx.x >> 6] = bsum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        wsum[n] = (sa[0] + sa[1]) + (sa[2] + sa[3]);
+        bias_out[n] = (bias ? bias[n] : 0.f) + ((sb[0] + sb[1]) + (sb[2] + sb[3]));
+    }
+}
+
+// out[b][:] = table_a[ids[b]][:] + table_b[*len_dev][:]  (token + position embedding of one new token);
+// also clears this sequence's packed arg-max cell for the step's last kernel
+__global__ void embed_add_kernel(const float* __restrict__ ids, const float* __restrict__ ta, int dim_a,
+    const float* __restrict__ tb, int dim_b, const int* __restrict__ len_dev, int depth, float* __restrict__ out,
+    int* __restrict__ err, unsigned long long* __restrict__ amax)
+{
+    const int b = blockIdx.x;
+    const float f = ids[b];
+    int64_t id = (f >= 0.f && f < 9.0e18f) ? (int64_t)f : -1;
+    const int64_t pos = *len_dev;
+    const bool ok = id >= 0 && id < dim_a && pos < dim_b;
+    if (!ok && err && threadIdx.x == 0)
+        atomicExch(err, 1);
+    if (amax && threadIdx.x == 0)
+        amax[b] = 0ull;
+    for (int z = threadIdx.x; z < depth; z += blockDim.x)
+        out[(int64_t)b * depth + z] = ok ? ta[id * depth + z] + tb[pos * depth + z] : 0.f;
+}
+
+// One workgroup per (sequence, head); the number of visible keys is *len_dev + 1 (the new token's
+// key / value row was written by the projection kernel just before).
+__global__ __launch_bounds__(256) void mha_decode_dyn_kernel(const float* __restrict__ q, int64_t ldq,
+    const float* __restrict__ kc, const float* __restrict__ vc, float* __restrict__ out, int heads, int dk, int dv,
+    const int* __restrict__ len_dev, int max_len, float scale)
+{
+    extern __shared__ float smem[]; // [dk] query, [max_len] scores, [256] reduction scratch
+    const int len = *len_dev + 1;
+    float* sq = smem;
+    float* sp = smem + dk;
+    float* red = sp + max_len;
+    const int b = blockIdx.x / heads, h = blockIdx.x % heads, tid = threadIdx.x;
+    const int64_t krow = (int64_t)heads * dk, vrow = (int64_t)heads * dv;
+    for (int d = tid; d < dk; d += 256)
+        sq[d] = q[(int64_t)b * ldq + h * dk + d];
+    __syncthreads();
+    // scores: 16 lanes share one key row (each lane 16 contiguous bytes per pass), so a wave reads four
+    // whole rows per load; four passes are issued together to keep more rows in flight
+    float m = -FLT_MAX;
+    const int part = tid & 15, slot = tid >> 4;
+    const float* kbase = kc + (int64_t)b * max_len * krow + h * dk;
+    if (dk == 64) {
+        const f32x4 qv = *reinterpret_cast<const f32x4*>(sq + part * 4);
+        for (int j0 = 0; j0 < len; j0 += 64) {
+            f32x4 kv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + u * 16 + slot;
+                kv[u] = f32x4 { 0.f, 0.f, 0.f, 0.f };
+                if (j < len)
+                    kv[u] = *reinterpret_cast<const f32x4*>(kbase + (int64_t)j * krow + part * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + u * 16 + slot;
+                float s = qv[0] * kv[u][0] + qv[1] * kv[u][1] + qv[2] * kv[u][2] + qv[3] * kv[u][3];
+                for (int o = 8; o > 0; o >>= 1)
+                    s += __shfl_xor(s, o, 64);
+                if (j < len) {
+                    s *= scale;
+                    if (part == 0)
+                        sp[j] = s;
+                    m = fmaxf(m, s);
+                }
+            }
+        }
+    } else {
+        for (int j0 = 0; j0 < len; j0 += 16) {
+            const int j = j0 + slot;
+            float s = 0.f;
+            if (j < len)
+                for (int d = part; d < dk; d += 16)
+                    s += sq[d] * kbase[(int64_t)j * krow + d];
+            for (int o = 8; o > 0; o >>= 1)
+                s += __shfl_xor(s, o, 64);
+            if (j < len) {
+                s *= scale;
+                if (part == 0)
+                    sp[j] = s;
+                m = fmaxf(m, s);
+            }
+        }
+    }
+    __syncthreads();
+    for (int o = 32; o > 0; o >>= 1)
+        m = fmaxf(m, __shfl_xor(m, o, 64));
+    if ((tid & 63) == 0)
+        red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float sum = 0.f;
+    for (int j = tid; j < len; j += 256)
+        sum += expf(sp[j] - m);
+    for (int o = 32; o > 0; o >>= 1)
+        sum += __shfl_xor(sum, o, 64);
+    __syncthreads();
+    if ((tid & 63) == 0)
+        red[tid >> 6] = sum;
+    __syncthreads();
+    const float ls = logf(red[0] + red[1] + red[2] + red[3]);
+    for (int j = tid; j < len; j += 256) {
+        const float pr = expf(sp[j] - m - ls);
+        sp[j] = isinf(pr) ? 0.f : pr;
+    }
+    __syncthreads();
+    // P V: lanes along the value depth, 256/dv key partitions; eight rows in flight per thread
+    const int parts = dv <= 256 ? 256 / dv : 1;
+    const float* vbase = vc + (int64_t)b * max_len * vrow + h * dv;
+    for (int d0 = 0; d0 < dv; d0 += 256) {
+        const int d = d0 + (parts > 1 ? tid % dv : tid), prt = parts > 1 ? tid / dv : 0;
+        float acc = 0.f;
+        if (d < dv && prt < parts) {
+            for (int j0 = prt; j0 < len; j0 += 8 * parts) {
+                float vv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int j = j0 + u * parts;
+                    vv[u] = j < len ? vbase[(int64_t)j * vrow + d] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int j = j0 + u * parts;
+                    if (j < len)
+                        acc += sp[j] * vv[u];
+                }
+            }
+        }
+        if (parts > 1) {
+            __syncthreads();
+            red[tid] = acc;
+            __syncthreads();
+            if (tid < dv) {
+                float r = red[tid];
+                for (int pidx = 1; pidx < parts; ++pidx)
+                    r += red[pidx * dv + tid];
+                out[(int64_t)b * vrow + h * dv + tid] = r;
+            }
+        } else if (d < dv) {
+            out[(int64_t)b * vrow + h * dv + d] = acc;
+        }
+    }
+}
+
+// Packs (value, column) so that an unsigned 64-bit max picks the largest value and, among equal values,
+// the smallest column: the first maximum wins, as in the reference's tensor_max_pos.
+__device__ __forceinline__ unsigned long long pack_max(float v, int col)
+{
+    unsigned int u = __float_as_uint(v);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u); // order-preserving map of floats to unsigned
+    return ((unsigned long long)u << 32) | (unsigned long long)(0xFFFFFFFFu - (unsigned int)col);
+}
+
+// per-row partial arg-max over a slice of columns, merged with a 64-bit atomic max
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ x, int depth, int cols_per_block,
+    unsigned long long* __restrict__ amax)
+{
+    __shared__ unsigned long long sm[4];
+    const int row = blockIdx.y, c0 = blockIdx.x * cols_per_block;
+    const int c1 = c0 + cols_per_block < depth ? c0 + cols_per_block : depth;
+    const float* xr = x + (int64_t)row * depth;
+    unsigned long long best = 0ull;
+    for (int z = c0 + threadIdx.x; z < c1; z += 256) {
+        const unsigned long long pk = pack_max(xr[z], z);
+        best = pk > best ? pk : best;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(best, o, 64);
+        best = other > best ? other : best;
+    }
+    if ((threadIdx.x & 63) == 0)
+        sm[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            best = sm[w] > best ? sm[w] : best;
+        atomicMax(&amax[row], best);
+    }
+}
+
+// packed winners -> float ids; optionally advances the session length (every other kernel of the step
+// has finished by stream order)
+__global__ void argmax_finish_kernel(const unsigned long long* __restrict__ amax, int rows, float* __restrict__ out_idx_f,
+    int* __restrict__ len_dev, float* __restrict__ history)
+{
+    const int r = threadIdx.x;
+    if (r < rows) {
+        const unsigned long long pk = amax[r];
+        const float id = pk == 0ull ? 0.f : (float)(0xFFFFFFFFu - (unsigned int)(pk & 0xFFFFFFFFull));
+        out_idx_f[r] = id;
+        if (history && len_dev)
+            history[(int64_t)(*len_dev) * rows + r] = id; // row = position of the token that produced these logits
+    }
+    __syncthreads();
+    if (len_dev && r == 0)
+        *len_dev += 1;
+}
+
+__global__ void set_int_kernel(int* p, int v) { *p = v; }
+
+// library-owned scratch of the split-K path: partial tiles and one ticket per column tile (zero between launches)
+constexpr int64_t kSplitWsFloats = 1 << 20;
+constexpr int kSplitTickets = 4096;
+static float* g_splitk_ws = nullptr;
+static int* g_splitk_tickets = nullptr;
+static bool ensure_splitk_workspace()
+{
+    if (g_splitk_ws && g_splitk_tickets)
+        return true;
+    if (hipMalloc(&g_splitk_ws, sizeof(float) * kSplitWsFloats) != hipSuccess)
+        return false;
+    if (hipMalloc(&g_splitk_tickets, sizeof(int) * kSplitTickets) != hipSuccess
+        || hipMemset(g_splitk_tickets, 0, sizeof(int) * kSplitTickets) != hipSuccess)
+        return false;
+    return true;
+}
+
+// allocates the split-K scratch ahead of time (it must not happen inside a stream capture)
+fdx_status skinny_prepare()
+{
+    if (!ensure_splitk_workspace()) {
+        set_error("dense_rows: out of device memory for the split-K workspace");
+        return FDX_ERR_HIP;
+    }
+    return FDX_OK;
+}
+
+fdx_status skinny_gemm_launch(const SkinnyParams& p)
+{
+    FDX_REQUIRE(p.X && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0, "dense_rows: bad arguments");
+    FDX_REQUIRE(p.K % 4 == 0 && p.ldx % 4 == 0 && p.ldw % 4 == 0, "dense_rows: K and row strides must be multiples of 4");
+    FDX_REQUIRE(p.n_seg >= 1 && p.n_seg <= 3, "dense_rows: 1 to 3 output segments");
+    FDX_REQUIRE(!p.ln || (p.K <= SK_WAVES * SK_CHUNK * 16 && p.w_rowsum), "dense_rows: the LayerNorm prologue needs K <= %d",
+        SK_WAVES * SK_CHUNK * 16);
+    FDX_REQUIRE(!p.residual || p.residual != p.seg[0].ptr, "dense_rows: the residual is read before the output is written; they must not alias");
+    const int tiles = (p.N + 15) / 16;
+    // split K across workgroups when a launch would otherwise leave most CUs idle or a wave would need
+    // more than one chunk; LayerNorm launches keep whole rows in one workgroup
+    int ksplit = 1;
+    SkinnyParams q = p;
+    if (!p.ln && !p.packed && ensure_splitk_workspace()) {
+        // spread a narrow projection over the chip: a CU pulls only a few tens of GB/s on its own
+        // long K only: below that the ticket exchange costs more than the idle CUs
+        while (ksplit < 8 && p.K / ksplit > SK_WAVES * SK_CHUNK * 16 && p.K / (ksplit * 2) >= 128)
+            ksplit *= 2;
+        if (ksplit > 1)
+            while (ksplit < 8 && tiles * ksplit < 192 && p.K / (ksplit * 2) >= 256)
+                ksplit *= 2;
+        if ((int64_t)tiles * ksplit * 256 > kSplitWsFloats || tiles > kSplitTickets)
+            ksplit = 1;
+        q.workspace = g_splitk_ws;
+        q.tickets = g_splitk_tickets;
+    }
+    const int per_wg = ((p.K + ksplit * 16 - 1) / (ksplit * 16)) * 16; // as the kernel derives it
+    const dim3 grid((unsigned)tiles, (unsigned)ksplit);
+    profile_begin();
+    // every load of a workgroup in flight at once when its K range fits 8 (or 24) slabs per wave
+    if (per_wg <= SK_WAVES * SK_CHUNK * 16)
+        hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK, true>), grid, dim3(512), 0, stream(), q);
+    else if (per_wg <= SK_WAVES * SK_CHUNK_LONG * 16)
+        hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK_LONG, true>), grid, dim3(512), 0, stream(), q);
+    else
+        hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK, false>), grid, dim3(512), 0, stream(), q);
+    profile_end("dense_rows_f32", 2.0 * p.M * (double)p.N * p.K, 4.0 * ((double)p.N * p.K + (double)p.M * (p.K + p.N)));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+// number of floats pack_weights_launch writes for an [n][k] operand
+int64_t packed_weight_floats(int n, int k)
+{
+    const int per_wave = ((k + SK_WAVES * 16 - 1) / (SK_WAVES * 16)) * 16;
+    return (int64_t)((n + 15) / 16) * SK_WAVES * (per_wave / 16) * 64 * 4;
+}
+
+fdx_status pack_weights_launch(const float* w, int n, int k, int64_t ldw, float* out)
+{
+    FDX_REQUIRE(w && out && n > 0 && k > 0, "pack_weights: bad arguments");
+    const int per_wave = ((k + SK_WAVES * 16 - 1) / (SK_WAVES * 16)) * 16;
+    const int64_t blocks = (int64_t)((n + 15) / 16) * SK_WAVES * (per_wave / 16);
+    hipLaunchKernelGGL(pack_weights_kernel, dim3((unsigned)blocks), dim3(64), 0, stream(), w, n, k, ldw, per_wave, out);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+fdx_status fold_layernorm_launch(const float* gamma, const float* beta, const float* w, const float* bias, int n, int k,
+    float* w_out, float* wsum, float* bias_out)
+{
+    FDX_REQUIRE(w && w_out && wsum && bias_out && n > 0 && k > 0, "fold_layernorm: bad arguments");
+    hipLaunchKernelGGL(fold_layernorm_kernel, dim3((unsigned)n), dim3(256), 0, stream(), gamma, beta, w, bias, k, w_out, wsum, bias_out);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+fdx_status embed_add_launch(const float* ids, int batch, const float* ta, int dim_a, const float* tb, int dim_b,
+    const int* len_dev, int depth, float* out, int* err, unsigned long long* amax)
+{
+    FDX_REQUIRE(ids && ta && tb && len_dev && out && batch > 0 && depth > 0, "embed_add: bad arguments");
+    profile_begin();
+    hipLaunchKernelGGL(embed_add_kernel, dim3(batch), dim3(256), 0, stream(), ids, ta, dim_a, tb, dim_b, len_dev, depth, out, err, amax);
+    profile_end("embed_add_f32", 0.0, 12.0 * batch * depth);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+bool mha_decode_fast_launch(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch, int heads,
+    int dk, int dv, const int* len_dev, int max_len, hipStream_t s);
+
+fdx_status mha_decode_dyn_launch(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch,
+    int heads, int dk, int dv, const int* len_dev, int max_len, int len_hint)
+{
+    FDX_REQUIRE(q && kc && vc && out && len_dev && batch > 0 && heads > 0 && dk > 0 && dv > 0 && max_len > 0, "mha_decode: bad arguments");
+    const size_t smem = sizeof(float) * ((size_t)dk + max_len + 256);
+    FDX_REQUIRE(smem <= 64 * 1024, "mha_decode: max_len %d exceeds the single-pass kernel's LDS budget", max_len);
+    const float scale = (float)(1.0 / std::sqrt((double)dk));
+    profile_begin();
+    if (!mha_decode_fast_launch(q, ldq, kc, vc, out, batch, heads, dk, dv, len_dev, max_len, stream()))
+        hipLaunchKernelGGL(mha_decode_dyn_kernel, dim3(batch * heads), dim3(256), smem, stream(), q, ldq, kc, vc, out, heads, dk, dv,
+            len_dev, max_len, scale);
+    profile_end("mha_decode_f32", 4.0 * batch * heads * (double)len_hint * dk, 4.0 * (double)batch * len_hint * heads * (dk + dv));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+// amax must hold zeros on entry (embed_add_kernel clears it at the start of every step)
+fdx_status argmax_bump_launch(const float* x, int rows, int depth, float* out_idx_f, int* len_dev, unsigned long long* amax,
+    float* history)
+{
+    FDX_REQUIRE(x && out_idx_f && amax && rows > 0 && rows <= 1024 && depth > 0, "argmax: bad arguments");
+    const int cols_per_block = 2048;
+    profile_begin();
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3((unsigned)((depth + cols_per_block - 1) / cols_per_block), (unsigned)rows), dim3(256), 0,
+        stream(), x, depth, cols_per_block, amax);
+    hipLaunchKernelGGL(argmax_finish_kernel, dim3(1), dim3(1024), 0, stream(), amax, rows, out_idx_f, len_dev, history);
+    profile_end("argmax_f32", 0.0, 4.0 * rows * depth);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+fdx_status set_int_launch(int* p, int v)
+{
+    hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, stream(), p, v);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+} // namespace fdx
+
+// ---- C ABI (include/fdx.h documents the semantics)
+extern "C" fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
+    const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(x && w_nk && out, "dense_rows: null pointer");
+    fdx::SkinnyParams p;
+    std::memset(&p, 0, sizeof p);
+    p.X = x; p.ldx = k; p.W = w_nk; p.ldw = k; p.M = m; p.N = n; p.K = k; p.bias = bias; p.residual = residual; p.ldr = n;
+    p.act = fdx::make_act(act);
+    p.n_seg = 1;
+    p.seg[0] = { out, n, 0, 0 };
+    return fdx::skinny_gemm_launch(p);
+}
+
+extern "C" fdx_status fdx_fold_layernorm_f32(const float* gamma, const float* beta, const float* w_nk, const float* bias, int n,
+    int k, float* w_folded, float* w_rowsum, float* bias_folded)
+{
+    return fdx::fold_layernorm_launch(gamma, beta, w_nk, bias, n, k, w_folded, w_rowsum, bias_folded);
+}
+
+extern "C" fdx_status fdx_layernorm_dense_rows_f32(const float* x, int m, int k, float ln_eps, const float* w_folded,
+    const float* w_rowsum, const float* bias_folded, int n, const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(x && w_folded && w_rowsum && out, "layernorm_dense_rows: null pointer");
+    fdx::SkinnyParams p;
+    std::memset(&p, 0, sizeof p);
+    p.X = x; p.ldx = k; p.W = w_folded; p.ldw = k; p.M = m; p.N = n; p.K = k; p.bias = bias_folded; p.residual = residual; p.ldr = n;
+    p.act = fdx::make_act(act);
+    p.ln = 1; p.ln_eps = ln_eps; p.w_rowsum = w_rowsum;
+    p.n_seg = 1;
+    p.seg[0] = { out, n, 0, 0 };
+    return fdx::skinny_gemm_launch(p);
+}

@@ -8,9 +8,12 @@
 // other than attention works on rows independently, so caching K/V of earlier rows and attending the
 // new rows to the visible prefix computes exactly that.
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <map>
 
 #include "model.hpp"
+#include "skinny.hpp"
 
 using namespace fdx;
 
@@ -27,6 +30,30 @@ struct fdx_session {
         size_t bytes, used;
     };
     std::vector<Chunk> chunks;
+
+    // ---- decode fast path (one new token per sequence, batch <= 16): a fixed list of fused launches
+    // over buffers allocated once; built at creation when the graph has the expected decoder structure
+    struct Step {
+        enum Kind { EmbedAdd, Gemm, Attn, LayerNorm, Add, Act, Softmax } kind;
+        SkinnyParams g;                 // Gemm
+        const float *a = nullptr, *b = nullptr; // operands of the other kinds
+        float* out = nullptr;
+        int op = -1;                    // model op this step realises
+        int depth = 0;
+    };
+    bool fast = false;
+    std::vector<Step> steps;
+    std::vector<void*> owned;           // device buffers of the fast path
+    int* len_dev = nullptr;             // tokens already cached, read by the fast-path kernels
+    float* ids_buf = nullptr;           // ids consumed by the next step (argmax writes them)
+    const float* logits_buf = nullptr;
+    unsigned long long* amax = nullptr; // per sequence: packed running arg-max of the step's logits
+    float* history = nullptr;           // [max_len][batch] greedy ids by the position that produced them
+    hipGraphExec_t step_graph = nullptr; // one decode step (ids_buf -> ids_buf) captured for replay
+    float* splitk_ws = nullptr;         // partial tiles of split-K decode GEMMs
+    int* splitk_tickets = nullptr;
+    static constexpr int64_t kWsFloats = 1 << 20;
+    static constexpr int kTickets = 4096;
     float* positions = nullptr;
     ~fdx_session()
     {
@@ -37,6 +64,10 @@ struct fdx_session {
             (void)hipFree(kv.second);
         for (auto& kv : vc)
             (void)hipFree(kv.second);
+        for (void* p : owned)
+            (void)hipFree(p);
+        if (step_graph)
+            (void)hipGraphExecDestroy(step_graph);
     }
     void arena_reset()
     {
@@ -258,6 +289,392 @@ fdx_status run(fdx_session* s, const float* ids_dev, int T, float* logits_dev, f
     return FDX_OK;
 }
 
+// ---------------------------------------------------------------- decode fast path
+// Turns the op list into fused decode launches: token+position embedding in one kernel; a
+// LayerNorm that only feeds Dense / attention layers becomes the prologue of their weight-
+// streaming GEMM; q, k and v come from one GEMM that writes the new cache rows in place; the
+// residual Add after attention rides in the output projection's epilogue.  Returns false (and
+// leaves the generic path in charge) when the graph does not have that structure.
+bool build_fast_plan(fdx_session* s)
+{
+    fdx_model& m = *s->m;
+    const int B = s->batch;
+    if (B > 16)
+        return false;
+    std::vector<int> dmemo(m.ops.size(), -1);
+    std::vector<float*> buf(m.ops.size(), nullptr);
+    std::vector<int> lazy_ln(m.ops.size(), -1); // LayerNorm op applied inside its consumers' GEMMs
+    std::vector<int> consumers(m.ops.size(), 0);
+    std::vector<std::vector<int>> users(m.ops.size());
+    for (int idx : s->order) {
+        const Op& o = m.ops[idx];
+        if (o.dead)
+            continue;
+        for (int i : o.in)
+            users[i].push_back(idx);
+        if (o.residual >= 0)
+            users[o.residual].push_back(idx);
+    }
+    auto alloc = [&](size_t floats) -> float* {
+        void* p = nullptr;
+        if (hipMalloc(&p, floats * sizeof(float)) != hipSuccess)
+            return nullptr;
+        s->owned.push_back(p);
+        return static_cast<float*>(p);
+    };
+    {
+        void* p = nullptr;
+        if (hipMalloc(&p, sizeof(int)) != hipSuccess)
+            return false;
+        s->owned.push_back(p);
+        s->len_dev = static_cast<int*>(p);
+    }
+    s->ids_buf = alloc((size_t)B);
+    s->amax = reinterpret_cast<unsigned long long*>(alloc((size_t)2 * B + 4));
+    if (!s->ids_buf || !s->amax)
+        return false;
+    if (hipMemset(s->amax, 0, sizeof(unsigned long long) * B) != hipSuccess)
+        return false;
+    s->history = alloc((size_t)s->max_len * B);
+    if (!s->history || skinny_prepare() != FDX_OK)
+        return false;
+    s->splitk_ws = alloc((size_t)fdx_session::kWsFloats);
+    s->splitk_tickets = reinterpret_cast<int*>(alloc((size_t)fdx_session::kTickets));
+    if (!s->splitk_ws || !s->splitk_tickets || hipMemset(s->splitk_tickets, 0, sizeof(int) * fdx_session::kTickets) != hipSuccess)
+        return false;
+    std::vector<char> skip(m.ops.size(), 0);
+    const int ids_op = m.inputs[0], pos_op = m.inputs[1];
+
+    for (int idx : s->order) {
+        const Op& o = m.ops[idx];
+        if (o.dead || skip[idx] || o.kind == OpKind::Input)
+            continue;
+        const int depth = depth_of(m, idx, dmemo);
+        fdx_session::Step st;
+        st.op = idx;
+        st.depth = depth;
+        // operand of a weight-streaming GEMM; a pending LayerNorm is folded into copies of the weights
+        // (W * gamma, row sums, bias + W beta) so the launch works on the raw rows
+        auto gemm_input = [&](int src, SkinnyParams& g, const float* w, const float* bias, int n, int k) -> bool {
+            g.W = w;
+            g.bias = bias;
+            if (lazy_ln[src] < 0) {
+                g.X = buf[src];
+                g.ln = 0;
+                return g.X != nullptr;
+            }
+            const Op& ln = m.ops[src];
+            float* wf = alloc((size_t)n * k);
+            float* ws = alloc((size_t)n);
+            float* bf = alloc((size_t)n);
+            if (!wf || !ws || !bf || fold_layernorm_launch(ln.dw[0], ln.dw[1], w, bias, n, k, wf, ws, bf) != FDX_OK)
+                return false;
+            g.X = buf[ln.in[0]];
+            g.ln = 1;
+            g.ln_eps = ln.eps;
+            g.W = wf;
+            g.w_rowsum = ws;
+            g.bias = bf;
+            return g.X != nullptr;
+        };
+        switch (o.kind) {
+        case OpKind::View:
+            buf[idx] = buf[o.in[0]];
+            continue;
+        case OpKind::Embedding: {
+            // only as one half of Add(Embedding(ids), Embedding(positions))
+            if (users[idx].size() != 1)
+                return false;
+            const Op& add = m.ops[users[idx][0]];
+            if (add.kind != OpKind::Add || add.in.size() != 2 || add.act.kind != FDX_ACT_NONE)
+                return false;
+            const Op& ea = m.ops[add.in[0]];
+            const Op& eb = m.ops[add.in[1]];
+            if (ea.kind != OpKind::Embedding || eb.kind != OpKind::Embedding || users[add.in[0]].size() != 1
+                || users[add.in[1]].size() != 1 || ea.output_dim != eb.output_dim)
+                return false;
+            const bool a_is_ids = ea.in[0] == ids_op && eb.in[0] == pos_op;
+            const bool b_is_ids = eb.in[0] == ids_op && ea.in[0] == pos_op;
+            if (!a_is_ids && !b_is_ids)
+                return false;
+            if (idx != add.in[0])
+                continue; // emitted when the first operand is visited
+            const Op& tok = a_is_ids ? ea : eb;
+            const Op& pos = a_is_ids ? eb : ea;
+            st.kind = fdx_session::Step::EmbedAdd;
+            st.a = tok.dw[0];
+            st.b = pos.dw[0];
+            st.g.M = tok.input_dim;
+            st.g.N = pos.input_dim;
+            st.depth = tok.output_dim;
+            st.out = alloc((size_t)B * tok.output_dim);
+            if (!st.out)
+                return false;
+            st.op = users[idx][0];
+            buf[st.op] = st.out;
+            skip[st.op] = 1;
+            s->steps.push_back(st);
+            continue;
+        }
+        case OpKind::LayerNorm: {
+            bool all_gemm = !users[idx].empty() && o.target_shape.size() == 1 && depth <= 1024 && depth % 4 == 0;
+            for (int u : users[idx]) {
+                const Op& c = m.ops[u];
+                const bool feeds_gemm = (c.kind == OpKind::Dense && c.in[0] == idx && c.residual != idx)
+                    || (c.kind == OpKind::MHA);
+                all_gemm = all_gemm && feeds_gemm;
+            }
+            for (int out : m.outputs)
+                all_gemm = all_gemm && out != idx;
+            if (all_gemm) {
+                lazy_ln[idx] = o.in[0];
+                continue;
+            }
+            st.kind = fdx_session::Step::LayerNorm;
+            st.a = buf[o.in[0]];
+            break;
+        }
+        case OpKind::Dense: {
+            st.kind = fdx_session::Step::Gemm;
+            SkinnyParams& g = st.g;
+            std::memset(&g, 0, sizeof g);
+            if (!gemm_input(o.in[0], g, o.dw[0], o.dw[1], o.units, o.n_in))
+                return false;
+            g.ldx = o.n_in;
+            g.ldw = o.n_in;
+            g.M = B;
+            g.N = o.units;
+            g.K = o.n_in;
+            g.act = o.act;
+            if (o.residual >= 0) {
+                if (lazy_ln[o.residual] >= 0)
+                    return false;
+                g.residual = buf[o.residual];
+                g.ldr = o.units;
+            }
+            if (o.softmax)
+                return false;
+            break;
+        }
+        case OpKind::MHA: {
+            const int H = o.heads, D = o.d_in;
+            const int nk = H * o.dk, nv = H * o.dv, nqkv = 2 * nk + nv;
+            // fused projection weights [q | k | v][D] and bias
+            float* wqkv = alloc((size_t)nqkv * D);
+            float* bqkv = alloc((size_t)nqkv);
+            float* q = alloc((size_t)B * nk);
+            float* merged = alloc((size_t)B * nv);
+            if (!wqkv || !bqkv || !q || !merged)
+                return false;
+            const size_t f = sizeof(float);
+            if (hipMemcpy(wqkv, o.dw[0], f * nk * D, hipMemcpyDeviceToDevice) != hipSuccess
+                || hipMemcpy(wqkv + (size_t)nk * D, o.dw[2], f * nk * D, hipMemcpyDeviceToDevice) != hipSuccess
+                || hipMemcpy(wqkv + (size_t)2 * nk * D, o.dw[4], f * nv * D, hipMemcpyDeviceToDevice) != hipSuccess
+                || hipMemcpy(bqkv, o.dw[1], f * nk, hipMemcpyDeviceToDevice) != hipSuccess
+                || hipMemcpy(bqkv + nk, o.dw[3], f * nk, hipMemcpyDeviceToDevice) != hipSuccess
+                || hipMemcpy(bqkv + 2 * nk, o.dw[5], f * nv, hipMemcpyDeviceToDevice) != hipSuccess)
+                return false;
+            fdx_session::Step pr;
+            pr.kind = fdx_session::Step::Gemm;
+            pr.op = idx;
+            SkinnyParams& g = pr.g;
+            std::memset(&g, 0, sizeof g);
+            if (!gemm_input(o.in[0], g, wqkv, bqkv, nqkv, D))
+                return false;
+            g.ldx = D; g.ldw = D; g.M = B; g.N = nqkv; g.K = D;
+            g.act = Act { FDX_ACT_NONE, 3.402823466e+38f, 0.f, 0.f };
+            g.n_seg = 3;
+            g.seg[0] = { q, nk, 0, 0 };
+            g.seg[1] = { s->kc[idx], (int64_t)s->max_len * nk, nk, nk };
+            g.seg[2] = { s->vc[idx], (int64_t)s->max_len * nv, 2 * nk, nv };
+            g.len_dev = s->len_dev;
+            s->steps.push_back(pr);
+            fdx_session::Step at;
+            at.kind = fdx_session::Step::Attn;
+            at.op = idx;
+            at.a = q;
+            at.out = merged;
+            s->steps.push_back(at);
+            // output projection; a following two-input Add becomes its residual operand
+            st.kind = fdx_session::Step::Gemm;
+            SkinnyParams& og = st.g;
+            std::memset(&og, 0, sizeof og);
+            og.X = merged; og.ldx = nv; og.W = o.dw[6]; og.ldw = nv; og.M = B; og.N = o.dout; og.K = nv; og.bias = o.dw[7];
+            og.act = Act { FDX_ACT_NONE, 3.402823466e+38f, 0.f, 0.f };
+            bool is_output = false;
+            for (int out : m.outputs)
+                is_output = is_output || out == idx;
+            if (!is_output && users[idx].size() == 1) {
+                const int ai = users[idx][0];
+                const Op& add = m.ops[ai];
+                if (add.kind == OpKind::Add && add.in.size() == 2 && add.in[0] != add.in[1]) {
+                    const int other = add.in[0] == idx ? add.in[1] : add.in[0];
+                    if (buf[other] && lazy_ln[other] < 0) {
+                        og.residual = buf[other];
+                        og.ldr = o.dout;
+                        og.act = add.act;
+                        st.op = ai;
+                        skip[ai] = 1;
+                    }
+                }
+            }
+            break;
+        }
+        case OpKind::Add:
+            if (o.in.size() != 2 || lazy_ln[o.in[0]] >= 0 || lazy_ln[o.in[1]] >= 0)
+                return false;
+            st.kind = fdx_session::Step::Add;
+            st.a = buf[o.in[0]];
+            st.b = buf[o.in[1]];
+            break;
+        case OpKind::Act:
+            st.kind = fdx_session::Step::Act;
+            st.a = buf[o.in[0]];
+            break;
+        case OpKind::Softmax:
+            st.kind = fdx_session::Step::Softmax;
+            st.a = buf[o.in[0]];
+            break;
+        default:
+            return false;
+        }
+        if (st.kind != fdx_session::Step::Gemm && !st.a)
+            return false;
+        if (st.kind == fdx_session::Step::Gemm && !st.g.X)
+            return false;
+        st.out = alloc((size_t)B * st.depth);
+        if (!st.out)
+            return false;
+        if (st.kind == fdx_session::Step::Gemm) {
+            st.g.n_seg = 1;
+            st.g.seg[0] = { st.out, st.g.N, 0, 0 };
+            st.g.len_dev = s->len_dev;
+        }
+        buf[st.op] = st.out;
+        if (st.op != idx)
+            buf[idx] = st.out;
+        s->steps.push_back(st);
+    }
+    for (auto& stp : s->steps)
+        if (stp.kind == fdx_session::Step::Gemm) {
+            // decode-time copy of the operand in the order the kernel's lanes read it; narrow or long-K
+            // projections without LayerNorm stay row-major because they run split along K instead
+            const bool split_candidate = !stp.g.ln && stp.g.K > 1024;
+            if (!split_candidate) {
+                float* packed = alloc((size_t)packed_weight_floats(stp.g.N, stp.g.K));
+                if (!packed || pack_weights_launch(stp.g.W, stp.g.N, stp.g.K, stp.g.ldw, packed) != FDX_OK)
+                    return false;
+                stp.g.W = packed;
+                stp.g.packed = 1;
+            }
+            stp.g.workspace = nullptr; // split-K stays off: its device-scope fences cost more than the idle CUs
+            stp.g.workspace_floats = fdx_session::kWsFloats;
+            stp.g.tickets = s->splitk_tickets;
+            stp.g.ticket_count = fdx_session::kTickets;
+        }
+    s->logits_buf = buf[m.outputs[0]];
+    if (!s->logits_buf || lazy_ln[m.outputs[0]] >= 0)
+        return false;
+    // the embedding launch opens every step and clears the packed arg-max cells the last launch fills
+    if (s->steps.empty() || s->steps.front().kind != fdx_session::Step::EmbedAdd)
+        return false;
+    return set_int_launch(s->len_dev, 0) == FDX_OK;
+}
+
+// enqueues the fused launches of one decode step; ids_dev [batch] floats, greedy ids go to next_dev
+fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
+{
+    fdx_model& m = *s->m;
+    const int B = s->batch;
+    fdx_status st = FDX_OK;
+    for (const auto& step : s->steps) {
+        const Op& o = m.ops[step.op];
+        const fdx_act act = to_c(o.act);
+        const fdx_act* actp = o.act.kind == FDX_ACT_NONE ? nullptr : &act;
+        switch (step.kind) {
+        case fdx_session::Step::EmbedAdd:
+            st = embed_add_launch(ids_dev, B, step.a, step.g.M, step.b, step.g.N, s->len_dev, step.depth, step.out, m.err_flag, s->amax);
+            break;
+        case fdx_session::Step::Gemm:
+            st = skinny_gemm_launch(step.g);
+            break;
+        case fdx_session::Step::Attn:
+            st = mha_decode_dyn_launch(step.a, (int64_t)o.heads * o.dk, s->kc[step.op], s->vc[step.op], step.out, B, o.heads, o.dk, o.dv,
+                s->len_dev, s->max_len, s->len + 1);
+            break;
+        case fdx_session::Step::LayerNorm:
+            st = fdx_layernorm_f32(step.a, B, step.depth, o.dw[0], o.dw[1], o.eps, step.out);
+            break;
+        case fdx_session::Step::Add:
+            st = fdx_eltwise_add_f32(step.a, step.b, (size_t)B * step.depth, (size_t)B * step.depth, actp, step.out);
+            break;
+        case fdx_session::Step::Act:
+            st = fdx_activation_f32(step.a, (size_t)B * step.depth, actp, step.out);
+            break;
+        case fdx_session::Step::Softmax:
+            st = fdx_softmax_f32(step.a, B, step.depth, 0, 0, step.out);
+            break;
+        }
+        if (st != FDX_OK)
+            return st;
+    }
+    // greedy ids (first maximum wins); the same launch records them by position and advances the cached
+    // length on the device
+    return argmax_bump_launch(s->logits_buf, B, s->vocab, next_dev, s->len_dev, s->amax, s->history);
+}
+
+// one decode step, eager launches
+fdx_status run_fast(fdx_session* s, const float* ids_dev, float* logits_dev, float* next_ids_dev)
+{
+    fdx_model& m = *s->m;
+    FDX_REQUIRE(ids_dev, "session: null ids");
+    FDX_REQUIRE(s->len + 1 <= s->max_len, "session: sequence length %d exceeds max_len %d", s->len + 1, s->max_len);
+    std::lock_guard<std::mutex> lock(m.mu);
+    fdx_status st = launch_steps(s, ids_dev, next_ids_dev ? next_ids_dev : s->ids_buf);
+    if (st != FDX_OK)
+        return st;
+    if (logits_dev)
+        FDX_HIP(hipMemcpyAsync(logits_dev, s->logits_buf, sizeof(float) * (size_t)s->batch * s->vocab, hipMemcpyDeviceToDevice, stream()));
+    s->len += 1;
+    return FDX_OK;
+}
+
+// `steps` greedy steps as replays of one captured step graph: the step reads its ids from ids_buf and
+// writes the next ids back there, the visible length lives in device memory, so every replay launches
+// the identical kernel sequence.  Ids are collected from the per-position history afterwards.
+fdx_status run_fast_greedy(fdx_session* s, const float* first_ids_dev, int steps, float* tokens_dev, float* last_logits_dev)
+{
+    fdx_model& m = *s->m;
+    FDX_REQUIRE(s->len + steps <= s->max_len, "session: sequence length %d exceeds max_len %d", s->len + steps, s->max_len);
+    std::lock_guard<std::mutex> lock(m.mu);
+    const int B = s->batch;
+    hipStream_t st = stream();
+    FDX_HIP(hipMemcpyAsync(s->ids_buf, first_ids_dev, sizeof(float) * B, hipMemcpyDeviceToDevice, st));
+    if (!s->step_graph) {
+        hipGraph_t graph = nullptr;
+        FDX_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        const fdx_status ls = launch_steps(s, s->ids_buf, s->ids_buf);
+        const hipError_t ce = hipStreamEndCapture(st, &graph);
+        if (ls != FDX_OK) {
+            if (graph)
+                (void)hipGraphDestroy(graph);
+            return ls;
+        }
+        FDX_HIP(ce);
+        const hipError_t ie = hipGraphInstantiate(&s->step_graph, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        FDX_HIP(ie);
+    }
+    const int start = s->len;
+    for (int i = 0; i < steps; ++i)
+        FDX_HIP(hipGraphLaunch(s->step_graph, st));
+    s->len += steps;
+    FDX_HIP(hipMemcpyAsync(tokens_dev, s->history + (size_t)start * B, sizeof(float) * (size_t)steps * B, hipMemcpyDeviceToDevice, st));
+    if (last_logits_dev)
+        FDX_HIP(hipMemcpyAsync(last_logits_dev, s->logits_buf, sizeof(float) * (size_t)B * s->vocab, hipMemcpyDeviceToDevice, st));
+    return FDX_OK;
+}
+
 } // namespace
 
 extern "C" fdx_status fdx_session_create(fdx_model* m, int batch, int max_len, fdx_session** out)
@@ -302,6 +719,9 @@ extern "C" fdx_status fdx_session_create(fdx_model* m, int batch, int max_len, f
     }
     std::vector<int> memo(m->ops.size(), -1);
     s->vocab = depth_of(*m, m->outputs[0], memo);
+    s->fast = build_fast_plan(s.get());
+    if (!s->fast)
+        s->steps.clear();
     *out = s.release();
     return FDX_OK;
 }
@@ -316,6 +736,8 @@ extern "C" fdx_status fdx_session_reset(fdx_session* s)
 {
     FDX_REQUIRE(s, "session_reset: null session");
     s->len = 0;
+    if (s->len_dev)
+        return set_int_launch(s->len_dev, 0);
     return FDX_OK;
 }
 
@@ -329,12 +751,17 @@ extern "C" fdx_status fdx_session_length(const fdx_session* s, int* len)
 extern "C" fdx_status fdx_session_prefill(fdx_session* s, const float* ids_dev, int t, float* logits_dev, float* next_ids_dev)
 {
     FDX_REQUIRE(s, "session_prefill: null session");
-    return run(s, ids_dev, t, logits_dev, next_ids_dev);
+    fdx_status st = run(s, ids_dev, t, logits_dev, next_ids_dev);
+    if (st == FDX_OK && s->len_dev)
+        st = set_int_launch(s->len_dev, s->len);
+    return st;
 }
 
 extern "C" fdx_status fdx_session_decode_step(fdx_session* s, const float* ids_dev, float* logits_dev, float* next_ids_dev)
 {
     FDX_REQUIRE(s, "session_decode_step: null session");
+    if (s->fast)
+        return run_fast(s, ids_dev, logits_dev, next_ids_dev);
     return run(s, ids_dev, 1, logits_dev, next_ids_dev);
 }
 
@@ -342,9 +769,18 @@ extern "C" fdx_status fdx_session_decode_greedy(fdx_session* s, const float* fir
     float* last_logits_dev)
 {
     FDX_REQUIRE(s && first_ids_dev && tokens_dev && steps > 0, "session_decode_greedy: bad arguments");
+    // FDX_DECODE_GRAPH=0 keeps the eager launches (tools that intercept HIP calls may not cope with graphs)
+    static const bool use_graph = [] {
+        const char* e = std::getenv("FDX_DECODE_GRAPH");
+        return !(e && e[0] == '0');
+    }();
+    if (s->fast && use_graph && !profiling())
+        return run_fast_greedy(s, first_ids_dev, steps, tokens_dev, last_logits_dev);
     for (int i = 0; i < steps; ++i) {
         const float* ids = i == 0 ? first_ids_dev : tokens_dev + (size_t)(i - 1) * s->batch;
-        fdx_status st = run(s, ids, 1, i + 1 == steps ? last_logits_dev : nullptr, tokens_dev + (size_t)i * s->batch);
+        float* logits = i + 1 == steps ? last_logits_dev : nullptr;
+        float* next = tokens_dev + (size_t)i * s->batch;
+        fdx_status st = s->fast ? run_fast(s, ids, logits, next) : run(s, ids, 1, logits, next);
         if (st != FDX_OK)
             return st;
     }

@@ -1,0 +1,52 @@
+// Launch parameters of the decode-shape kernels (decode_kernels.hip).
+#pragma once
+#include "common.hpp"
+
+namespace fdx {
+
+struct SkinnySegment {
+    float* ptr;         // output base of this column range
+    int64_t ld;         // row stride in floats
+    int col_begin;      // first output column stored here
+    int64_t len_stride; // if non-zero the base is advanced by *len_dev * len_stride floats (cache rows)
+};
+
+struct SkinnyParams {
+    const float* X;     // [M][K] activation rows, M <= 16
+    int64_t ldx;
+    const float* W;     // [N][K], K contiguous (LayerNorm gamma already folded in when ln != 0)
+    int64_t ldw;
+    int packed;         // W is in the pre-packed tile/wave/slab/lane order written by pack_weights_launch
+    int M, N, K;
+    const float* bias;  // [N] or null (LayerNorm beta already folded in when ln != 0)
+    const float* residual; // [M][N] (row stride ldr) or null
+    int64_t ldr;
+    Act act;
+    int ln;             // rows of X are layer-normalised over K before the product
+    float ln_eps;
+    const float* w_rowsum; // [N] row sums of the folded W, needed when ln != 0
+    int n_seg;
+    SkinnySegment seg[3];
+    const int* len_dev; // device int read by segments with len_stride != 0
+    // optional split-K support: partial tiles [split][tile][256] and one zero-initialised ticket per tile
+    float* workspace;
+    int64_t workspace_floats;
+    int* tickets;
+    int ticket_count;
+};
+
+fdx_status skinny_gemm_launch(const SkinnyParams& p);
+fdx_status skinny_prepare();
+int64_t packed_weight_floats(int n, int k);
+fdx_status pack_weights_launch(const float* w, int n, int k, int64_t ldw, float* out);
+fdx_status fold_layernorm_launch(const float* gamma, const float* beta, const float* w, const float* bias, int n, int k,
+    float* w_out, float* wsum, float* bias_out);
+fdx_status embed_add_launch(const float* ids, int batch, const float* ta, int dim_a, const float* tb, int dim_b,
+    const int* len_dev, int depth, float* out, int* err, unsigned long long* amax);
+fdx_status mha_decode_dyn_launch(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch,
+    int heads, int dk, int dv, const int* len_dev, int max_len, int len_hint);
+fdx_status argmax_bump_launch(const float* x, int rows, int depth, float* out_idx_f, int* len_dev, unsigned long long* amax,
+    float* history);
+fdx_status set_int_launch(int* p, int v);
+
+} // namespace fdx

@@ -96,6 +96,24 @@ fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const float* b_nk,
     int m, int n, int k, float alpha, const float* bias, int bias_per_row,
     const float* residual, const fdx_act* act, float* c, int64_t ldc, const fdx_gemm_batch* batch);
 
+/*
+ * Dense on at most 16 rows (the decode shape): out[m][:] = act(x[m][:] * w_nk^T + bias + residual[m][:]),
+ * an HBM-bound weight-streaming kernel (layers/dense_layer.hpp:76-86 at batch <= 16).
+ */
+fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
+    const float* residual, const fdx_act* act, float* out);
+/*
+ * LayerNormalization followed by Dense in one launch (layers/layer_normalization_layer.hpp:37-63 then
+ * layers/dense_layer.hpp:76-86).  fdx_fold_layernorm_f32 prepares, once per layer pair,
+ *   w_folded[n][k] = w[n][k] * gamma[k],  w_rowsum[n] = sum_k w_folded[n][k],  bias_folded[n] = bias[n] + sum_k w[n][k] * beta[k]
+ * (gamma / beta / bias may be NULL); the launch then computes rstd[m] * (x w_folded^T - mean[m] * w_rowsum) + bias_folded
+ * with each row's mean and biased two-pass variance taken from x itself.  k <= 1024.
+ */
+fdx_status fdx_fold_layernorm_f32(const float* gamma, const float* beta, const float* w_nk, const float* bias, int n,
+    int k, float* w_folded, float* w_rowsum, float* bias_folded);
+fdx_status fdx_layernorm_dense_rows_f32(const float* x, int m, int k, float ln_eps, const float* w_folded,
+    const float* w_rowsum, const float* bias_folded, int n, const float* residual, const fdx_act* act, float* out);
+
 /* [rows][cols] -> [cols][rows] (load-time weight re-layout) */
 fdx_status fdx_transpose_f32(const float* in, int rows, int cols, float* out);
 

@@ -282,3 +282,52 @@ def test_launcher_argument_errors(fdx):
         fdx.check(fdx.lib.fdx_pool2d_nhwc_f32(fdx._dp(a), 1, 2, 2, 1, 2, 2, 1, 1, 0, 0, 0, 0, 0, 0, 1, 1, 7, fdx._dp(a)))
     with pytest.raises(fdx.FdxError):
         fdx.window_geometry(0, 4, 3, 3, 1, 1, "same")
+
+
+DENSE_ROWS = [(16, 768, 2304), (16, 768, 768), (16, 3072, 768), (3, 64, 100), (16, 768, 50257), (5, 20, 33), (7, 1024, 40),
+              (16, 100, 64), (1, 2048, 48)]
+
+
+@pytest.mark.parametrize("m,k,n", DENSE_ROWS)
+def test_dense_rows_decode_shape(fdx, oracle, m, k, n):
+    """The weight-streaming Dense for <= 16 rows (split along K for long K) against the oracle's Dense."""
+    say("dense_rows", m, k, n)
+    r = rng_for("dense_rows", m, k, n)
+    x = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    b = r.standard_normal(n).astype(np.float32)
+    res = r.standard_normal((m, n)).astype(np.float32)
+    want = oracle.gelu(oracle.dense(x, np.ascontiguousarray(w.T).reshape(-1), b, n) + res)
+    dx, dw, db, dr = (fdx.DevBuf.from_host(a) for a in (x, w, b, res))
+    out = fdx.DevBuf(4 * m * n)
+    act = fdx.gelu_act()
+    for _ in range(2):  # twice: the split-K tickets must be back at zero after a launch
+        fdx.check(fdx.lib.fdx_dense_rows_f32(fdx._dp(dx), m, k, fdx._dp(dw), fdx._dp(db), n, fdx._dp(dr), fdx.ctypes.byref(act),
+                                             fdx._dp(out)))
+        assert rel(out.to_host((m, n)), want) <= TOL
+
+
+@pytest.mark.parametrize("m,k,n", [(16, 768, 2304), (3, 64, 100), (16, 768, 50257), (7, 1024, 40), (16, 100, 64)])
+def test_layernorm_dense_rows_folded(fdx, oracle, m, k, n):
+    """LayerNormalization + Dense in one launch through folded weights against oracle LN followed by oracle Dense,
+    on rows with a mean far from zero (the folded form subtracts mean * rowsum after the product)."""
+    say("layernorm_dense_rows", m, k, n)
+    r = rng_for("ln_dense_rows", m, k, n)
+    x = (r.standard_normal((m, k)) * 2 + 3.0).astype(np.float32)
+    w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    b = r.standard_normal(n).astype(np.float32)
+    g, be = r.standard_normal(k).astype(np.float32), r.standard_normal(k).astype(np.float32)
+    want = oracle.dense(oracle.layernorm(x, g, be, 1e-5), np.ascontiguousarray(w.T).reshape(-1), b, n)
+    dx, dw, db, dg, dbe = (fdx.DevBuf.from_host(a) for a in (x, w, b, g, be))
+    wf, ws, bf, out = fdx.DevBuf(4 * n * k), fdx.DevBuf(4 * n), fdx.DevBuf(4 * n), fdx.DevBuf(4 * m * n)
+    fdx.check(fdx.lib.fdx_fold_layernorm_f32(fdx._dp(dg), fdx._dp(dbe), fdx._dp(dw), fdx._dp(db), n, k, fdx._dp(wf), fdx._dp(ws),
+                                             fdx._dp(bf)))
+    fdx.check(fdx.lib.fdx_layernorm_dense_rows_f32(fdx._dp(dx), m, k, fdx.ctypes.c_float(1e-5), fdx._dp(wf), fdx._dp(ws),
+                                                   fdx._dp(bf), n, None, None, fdx._dp(out)))
+    assert rel(out.to_host((m, n)), want) <= TOL
+    # no gamma / beta / bias
+    fdx.check(fdx.lib.fdx_fold_layernorm_f32(None, None, fdx._dp(dw), None, n, k, fdx._dp(wf), fdx._dp(ws), fdx._dp(bf)))
+    fdx.check(fdx.lib.fdx_layernorm_dense_rows_f32(fdx._dp(dx), m, k, fdx.ctypes.c_float(1e-3), fdx._dp(wf), fdx._dp(ws),
+                                                   fdx._dp(bf), n, None, None, fdx._dp(out)))
+    want = oracle.dense(oracle.layernorm(x, None, None, 1e-3), np.ascontiguousarray(w.T).reshape(-1), None, n)
+    assert rel(out.to_host((m, n)), want) <= TOL
