@@ -232,6 +232,80 @@ def layernorm(x, gamma, beta, eps):
     return out.to_host(x.shape)
 
 
+def _dims5(shape):
+    shape = tuple(int(v) for v in shape)
+    return (ctypes.c_int64 * 5)(*((1,) * (5 - len(shape)) + shape))
+
+
+def layernorm_axes(x, axes, gamma, beta, eps):
+    """x: (batch, ...sample dims); axes: 1-based positions in the sample's rank, negative from the end."""
+    x = np.ascontiguousarray(x, np.float32)
+    rank = x.ndim - 1
+    mask = 0
+    for a in axes:
+        a = a + rank + 1 if a < 0 else a
+        mask |= 1 << (5 - rank + a - 1)
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    dg = None if gamma is None else DevBuf.from_host(gamma)
+    db = None if beta is None else DevBuf.from_host(beta)
+    check(lib.fdx_layernorm_axes_f32(_dp(dx), x.shape[0], _dims5(x.shape[1:]), ctypes.c_uint(mask), _dp(dg), _dp(db),
+                                     ctypes.c_float(eps), _dp(out)))
+    return out.to_host(x.shape)
+
+
+def broadcast_add(a, b, act=None):
+    """a, b: (batch, ...sample dims) with right-aligned size-1 broadcasting between the samples."""
+    a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+    batch = a.shape[0]
+    od = (ctypes.c_int64 * 5)()
+    rank = max(a.ndim, b.ndim) - 1
+    pa, pb = (1,) * (rank - a.ndim + 1) + a.shape[1:], (1,) * (rank - b.ndim + 1) + b.shape[1:]
+    out = DevBuf(4 * batch * int(np.prod([max(x, y) for x, y in zip(pa, pb)])))
+    da, db = DevBuf.from_host(a), DevBuf.from_host(b)
+    check(lib.fdx_broadcast_add_f32(_dp(da), _dims5(a.shape[1:]), _dp(db), _dims5(b.shape[1:]), batch, _act_ref(act),
+                                    _dp(out), od))
+    got = tuple(od)[5 - rank:]
+    return out.to_host((batch,) + got)
+
+
+def concat(xs, axis):
+    """xs: arrays of shape (batch, ...); axis: 1-based in the sample's rank (batch = 0), negative from the end."""
+    xs = [np.ascontiguousarray(x, np.float32) for x in xs]
+    rank = xs[0].ndim - 1
+    a = axis + rank + 1 if axis < 0 else axis
+    outer = int(np.prod(xs[0].shape[:a]))
+    inner = (ctypes.c_int64 * len(xs))(*[int(np.prod(x.shape[a:])) for x in xs])
+    bufs = [DevBuf.from_host(x) for x in xs]
+    ptrs = (ctypes.c_void_p * len(xs))(*[b.ptr.value for b in bufs])
+    shape = list(xs[0].shape)
+    shape[a] = sum(x.shape[a] for x in xs)
+    out = DevBuf(4 * int(np.prod(shape)))
+    check(lib.fdx_concat_f32(ptrs, len(xs), inner, ctypes.c_int64(outer), _dp(out)))
+    return out.to_host(tuple(shape))
+
+
+def einsum_dense(x, equation, kernel, bias=None, bias_axes=None, full_output_shape=None, act=None):
+    """x carries every lhs character it has (a leading batch is just the first one); returns the full rhs array."""
+    x, kernel = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(kernel, np.float32)
+    rhs = equation.split("->")[1]
+    dx, dk = DevBuf.from_host(x), DevBuf.from_host(kernel)
+    db = None if bias is None else DevBuf.from_host(np.ascontiguousarray(bias, np.float32))
+    lhs, ker = equation.split("->")[0].split(",")
+    size = dict(zip(ker[len(ker) - kernel.ndim:], kernel.shape))
+    size.update(zip(lhs[len(lhs) - x.ndim:], x.shape))
+    for i, c in enumerate(rhs):
+        if c not in size:
+            size[c] = 1 if c in lhs else int(full_output_shape[i])
+    out = DevBuf(4 * int(np.prod([size[c] for c in rhs])))
+    in_dims = (ctypes.c_int64 * x.ndim)(*x.shape)
+    k_dims = (ctypes.c_int64 * kernel.ndim)(*kernel.shape)
+    full = None if full_output_shape is None else (ctypes.c_int64 * len(rhs))(*[int(v) for v in full_output_shape])
+    orank, odims = ctypes.c_int(0), (ctypes.c_int64 * 6)()
+    check(lib.fdx_einsum_dense_f32(equation.encode(), (bias_axes or "").encode(), _dp(dx), x.ndim, in_dims, _dp(dk),
+                                   kernel.ndim, k_dims, _dp(db), full, _act_ref(act), _dp(out), ctypes.byref(orank), odims))
+    return out.to_host(tuple(odims)[:orank.value])
+
+
 def softmax(x, causal_period=0, causal_offset=0):
     x = np.ascontiguousarray(x, np.float32)
     d = x.shape[-1]

@@ -13,7 +13,9 @@
 #include <cstring>
 #include <functional>
 #include <set>
+#include <tuple>
 
+#include "einsum.hpp"
 #include "json.hpp"
 
 using namespace fdx;
@@ -208,19 +210,40 @@ namespace {
         throw Unsupported("unknown activation type: " + type);
     }
 
+    // One level of the layer graph: the top-level model or one application of a nested
+    // Functional model (create_model_layer, import_model.hpp:397-424).  A nested level reads its
+    // parameters under "<outer names>_<layer>" and its InputLayers are bound to the outer operands.
+    struct Scope {
+        std::map<std::string, const Value*> layers;
+        std::string prefix;
+        std::map<std::string, int> input_ops;
+        std::map<std::tuple<std::string, int, int>, int> memo;
+    };
+
     struct Builder {
         fdx_model& m;
         const Value& params;
-        std::map<std::string, const Value*> layers;
-        std::map<std::pair<std::string, int>, int> memo;
-        std::map<std::string, int> input_ops;
+        std::vector<std::unique_ptr<Scope>> scopes;
 
-        const Value& param(const std::string& layer, const char* key)
+        const Value& param(const Scope& sc, const std::string& layer, const char* key)
         {
-            const Value* l = params.find(layer.c_str());
+            const std::string full = sc.prefix + layer;
+            const Value* l = params.find(full.c_str());
             if (!l)
-                throw FormatError("missing trainable_params for layer " + layer);
+                throw FormatError("missing trainable_params for layer " + full);
             return l->at(key);
+        }
+
+        static void index_layers(Scope& sc, const Value& layers)
+        {
+            if (!layers.is_array())
+                throw FormatError("missing layers array");
+            for (const auto& l : layers.arr) {
+                const std::string name = l.at("name").str();
+                if (sc.layers.count(name))
+                    throw FormatError("layer names must be unique");
+                sc.layers[name] = &l;
+            }
         }
 
         int add_op(Op&& op)
@@ -246,37 +269,65 @@ namespace {
             return idx;
         }
 
-        int build(const Conn& c)
+        int build(Scope& sc, const Conn& c)
         {
-            auto key = std::make_pair(c.layer, c.node);
+            auto key = std::make_tuple(c.layer, c.node, c.tensor);
+            auto& memo = sc.memo;
             auto it = memo.find(key);
             if (it != memo.end())
                 return it->second;
-            auto lit = layers.find(c.layer);
-            if (lit == layers.end())
+            auto lit = sc.layers.find(c.layer);
+            if (lit == sc.layers.end())
                 throw FormatError("dangling connection to layer " + c.layer);
             const Value& L = *lit->second;
             const std::string cls = L.at("class_name").str();
             const Value& cfg = L.at("config");
             if (cls == "InputLayer") {
-                auto io = input_ops.find(c.layer);
-                if (io == input_ops.end())
+                auto io = sc.input_ops.find(c.layer);
+                if (io == sc.input_ops.end())
                     throw FormatError("input layer " + c.layer + " is not listed in input_layers");
                 return memo[key] = io->second;
             }
-            if (c.tensor != 0)
+            const bool nested = cls == "Functional" || cls == "Model";
+            if (c.tensor != 0 && !nested)
                 throw Unsupported("layers with several output tensors are not supported: " + c.layer);
             auto nodes = inbound_nodes(L);
-            if (c.node < 0 || c.node >= (int)nodes.size())
+            // a nested model counts its own construction as node 0 (layers/model_layer.hpp:36-44)
+            const int node = nested && c.node >= 1 ? c.node - 1 : c.node;
+            if (node < 0 || node >= (int)nodes.size())
                 throw FormatError("invalid node index for layer " + c.layer);
             std::vector<int> ins;
-            for (const auto& ic : nodes[c.node])
-                ins.push_back(build(ic));
+            for (const auto& ic : nodes[node])
+                ins.push_back(build(sc, ic));
             if (ins.empty())
                 throw FormatError("layer without inputs: " + c.layer);
+            if (nested) {
+                scopes.emplace_back(new Scope);
+                Scope& inner = *scopes.back();
+                inner.prefix = sc.prefix + c.layer + "_";
+                index_layers(inner, cfg.at("layers"));
+                const auto inner_in = model_connections(cfg.at("input_layers"));
+                const auto inner_out = model_connections(cfg.at("output_layers"));
+                if (inner_in.size() != ins.size())
+                    throw FormatError("invalid number of input tensors for this model: " + std::to_string(inner_in.size())
+                        + " required but " + std::to_string(ins.size()) + " provided");
+                for (size_t i = 0; i < ins.size(); ++i)
+                    inner.input_ops[inner_in[i].layer] = ins[i];
+                if (c.tensor < 0 || c.tensor >= (int)inner_out.size())
+                    throw FormatError("invalid tensor index for nested model " + c.layer);
+                // every output of this application is built now so they share the inner operands
+                int chosen = -1;
+                for (size_t t = 0; t < inner_out.size(); ++t) {
+                    const int r = build(inner, inner_out[t]);
+                    sc.memo[std::make_tuple(c.layer, c.node, (int)t)] = r;
+                    if ((int)t == c.tensor)
+                        chosen = r;
+                }
+                return chosen;
+            }
 
             Op op;
-            op.name = c.layer;
+            op.name = sc.prefix + c.layer;
             op.cls = cls;
             op.in = ins;
             int result;
@@ -291,9 +342,9 @@ namespace {
                 pair_from(cfg.at("kernel_size"), op.kh, op.kw);
                 op.cout = (int)cfg.at("filters").integer();
                 op.hw.resize(2);
-                op.hw[0] = decode_floats(param(c.layer, "weights"));
+                op.hw[0] = decode_floats(param(sc, c.layer, "weights"));
                 if (cfg.at("use_bias").boolean())
-                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
                 else
                     op.hw[1].assign(op.cout, 0.f);
                 if ((int)op.hw[1].size() != op.cout)
@@ -308,7 +359,7 @@ namespace {
                 pair_from(cfg.at("strides"), op.sy, op.sx);
                 pair_from(cfg.at("dilation_rate"), op.dy, op.dx);
                 pair_from(cfg.at("kernel_size"), op.kh, op.kw);
-                std::vector<float> sw = decode_floats(param(c.layer, "slice_weights"));
+                std::vector<float> sw = decode_floats(param(sc, c.layer, "slice_weights"));
                 if (sw.size() % ((size_t)op.kh * op.kw) != 0)
                     throw FormatError("invalid number of weights");
                 const int ch = (int)(sw.size() / ((size_t)op.kh * op.kw));
@@ -319,7 +370,7 @@ namespace {
                     for (int t = 0; t < op.kh * op.kw; ++t)
                         op.hw[0][(size_t)t * ch + z] = sw[(size_t)z * op.kh * op.kw + t];
                 if (cfg.at("use_bias").boolean())
-                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
                 else
                     op.hw[1].assign(ch, 0.f);
                 if ((int)op.hw[1].size() != ch)
@@ -328,10 +379,10 @@ namespace {
             } else if (cls == "Dense") {
                 op.kind = OpKind::Dense;
                 op.units = (int)cfg.at("units").integer();
-                std::vector<float> w = decode_floats(param(c.layer, "weights"));
+                std::vector<float> w = decode_floats(param(sc, c.layer, "weights"));
                 op.hw.resize(2);
                 if (cfg.at("use_bias").boolean())
-                    op.hw[1] = decode_floats(param(c.layer, "bias"));
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
                 else
                     op.hw[1].assign(op.units, 0.f);
                 if ((int)op.hw[1].size() != op.units || op.units == 0 || w.size() % (size_t)op.units != 0)
@@ -344,13 +395,13 @@ namespace {
                 result = with_fused_activation(add_op(std::move(op)), cfg);
             } else if (cls == "BatchNormalization") {
                 op.kind = OpKind::Affine;
-                std::vector<float> mean = decode_floats(param(c.layer, "moving_mean"));
-                std::vector<float> var = decode_floats(param(c.layer, "moving_variance"));
+                std::vector<float> mean = decode_floats(param(sc, c.layer, "moving_mean"));
+                std::vector<float> var = decode_floats(param(sc, c.layer, "moving_variance"));
                 std::vector<float> gamma, beta;
                 if (cfg.at("scale").boolean())
-                    gamma = decode_floats(param(c.layer, "gamma"));
+                    gamma = decode_floats(param(sc, c.layer, "gamma"));
                 if (cfg.at("center").boolean())
-                    beta = decode_floats(param(c.layer, "beta"));
+                    beta = decode_floats(param(sc, c.layer, "beta"));
                 const Value& ax = cfg.at("axis");
                 if (ax.is_array() && ax.size() != 1)
                     throw FormatError("invalid axis configuration");
@@ -374,10 +425,13 @@ namespace {
                 op.kind = OpKind::LayerNorm;
                 op.hw.resize(2);
                 if (cfg.at("scale").boolean())
-                    op.hw[0] = decode_floats(param(c.layer, "gamma"));
+                    op.hw[0] = decode_floats(param(sc, c.layer, "gamma"));
                 if (cfg.at("center").boolean())
-                    op.hw[1] = decode_floats(param(c.layer, "beta"));
+                    op.hw[1] = decode_floats(param(sc, c.layer, "beta"));
                 op.eps = (float)cfg.at("epsilon").number();
+                if (!op.hw[0].empty() && !op.hw[1].empty() && op.hw[0].size() != op.hw[1].size())
+                    throw FormatError("LayerNormalization: gamma and beta differ in size");
+                op.cout = (int)std::max(op.hw[0].size(), op.hw[1].size());
                 const Value& ax = cfg.at("axis");
                 op.target_shape.clear();
                 if (ax.is_array())
@@ -433,12 +487,73 @@ namespace {
             } else if (cls == "Add") {
                 op.kind = OpKind::Add;
                 result = add_op(std::move(op));
+            } else if (cls == "Concatenate") {
+                op.kind = OpKind::Concat;
+                op.axis = (int)cfg.at("axis").integer();
+                result = add_op(std::move(op));
+            } else if (cls == "EinsumDense") {
+                // import_model.hpp:820-848
+                op.kind = OpKind::Einsum;
+                op.equation = cfg.at("equation").str();
+                const Value* ba = cfg.find("bias_axes");
+                op.bias_axes = ba && ba->is_string() ? ba->str() : "";
+                op.full_out.push_back(-1); // batch slot
+                if (const Value* os = cfg.find("output_shape")) {
+                    if (os->is_array())
+                        for (const auto& d : os->arr)
+                            op.full_out.push_back(d.is_null() ? -1 : d.integer());
+                    else if (!os->is_null())
+                        op.full_out.push_back(os->integer());
+                }
+                for (const auto& d : param(sc, c.layer, "kernel_shape").arr)
+                    op.kernel_dims.push_back(d.integer());
+                op.hw.resize(2);
+                op.hw[0] = decode_floats(param(sc, c.layer, "kernel"));
+                if ((int64_t)op.hw[0].size() != volume(op.kernel_dims))
+                    throw FormatError("EinsumDense: kernel values do not fill kernel_shape");
+                EinsumSpec spec;
+                std::string err;
+                if (!spec.parse(op.equation, op.bias_axes, err))
+                    throw FormatError(err);
+                if (!op.bias_axes.empty())
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
+                std::string n_chars;
+                if (spec.gemm_form(&n_chars) && spec.ker.size() == op.kernel_dims.size()) {
+                    // kernel [K][N] -> [N][K]; bias spread over the N characters
+                    for (size_t i = 0; i < spec.ker.size(); ++i)
+                        spec.size[spec.ker[i]] = op.kernel_dims[i];
+                    const int64_t K = spec.volume_of(spec.summed), N = spec.volume_of(n_chars);
+                    std::vector<float> t(op.hw[0].size());
+                    for (int64_t k = 0; k < K; ++k)
+                        for (int64_t n = 0; n < N; ++n)
+                            t[(size_t)(n * K + k)] = op.hw[0][(size_t)(k * N + n)];
+                    op.hw[0].swap(t);
+                    std::vector<float> b((size_t)N, 0.f);
+                    if (!spec.bias_chars.empty()) {
+                        if ((int64_t)op.hw[1].size() != spec.volume_of(spec.bias_chars))
+                            throw FormatError("EinsumDense: bias size does not match bias_axes");
+                        for (int64_t n = 0; n < N; ++n) {
+                            int64_t rem = n, off = 0;
+                            for (size_t i = n_chars.size(); i-- > 0;) {
+                                const int64_t ext = spec.size.at(n_chars[i]);
+                                off += (rem % ext) * spec.stride_in(spec.bias_chars, n_chars[i]);
+                                rem /= ext;
+                            }
+                            b[(size_t)n] = op.hw[1][(size_t)off];
+                        }
+                    }
+                    op.hw[1].swap(b);
+                    op.gemm = true;
+                    op.n_in = (int)K;
+                    op.units = (int)N;
+                }
+                result = with_fused_activation(add_op(std::move(op)), cfg);
             } else if (cls == "Embedding") {
                 op.kind = OpKind::Embedding;
                 op.input_dim = (int)cfg.at("input_dim").integer();
                 op.output_dim = (int)cfg.at("output_dim").integer();
                 op.hw.resize(1);
-                op.hw[0] = decode_floats(param(c.layer, "weights"));
+                op.hw[0] = decode_floats(param(sc, c.layer, "weights"));
                 if (op.hw[0].size() != (size_t)op.input_dim * op.output_dim)
                     throw FormatError("embedding weight size does not match input_dim * output_dim");
                 m.has_embedding = true;
@@ -451,8 +566,8 @@ namespace {
                 op.use_bias = cfg.at("use_bias").boolean();
                 if (ins.size() != 2 && ins.size() != 3)
                     throw FormatError("Invalid number of inputs for MultiHeadAttention layer.");
-                const Value& shapes = param(c.layer, "weight_shapes");
-                const Value& vals = param(c.layer, "weights");
+                const Value& shapes = param(sc, c.layer, "weight_shapes");
+                const Value& vals = param(sc, c.layer, "weights");
                 const size_t expect = op.use_bias ? 8 : 4;
                 if (!shapes.is_array() || !vals.is_array() || shapes.size() != expect || vals.size() != expect)
                     throw FormatError("MultiHeadAttention expects q/k/v/output kernels (and biases)");
@@ -513,7 +628,7 @@ namespace {
             } else {
                 throw Unsupported("unknown layer type: " + cls);
             }
-            return memo[key] = result;
+            return sc.memo[key] = result;
         }
     };
 
@@ -632,7 +747,8 @@ namespace {
             if (a.dead || a.kind != OpKind::Act)
                 continue;
             Op& p = m.ops[a.in[0]];
-            const bool ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D || p.kind == OpKind::Add || p.kind == OpKind::Affine)
+            const bool ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D || p.kind == OpKind::Add || p.kind == OpKind::Affine
+                                || p.kind == OpKind::Einsum)
                 && p.act.kind == FDX_ACT_NONE && !p.softmax && p.consumers == 1;
             if (!ok)
                 continue;
@@ -770,21 +886,54 @@ namespace {
                     out = { in0->back() };
                 break;
             case OpKind::Add: {
+                // tensor.hpp:642-660: right-aligned axes must be equal or 1; the result has the larger rank
                 out = *in0;
                 for (size_t k = 1; k < o.in.size(); ++k) {
                     const Shape& b = shapes[o.in[k]];
                     if (b == out)
                         continue;
-                    // size-1 broadcasting is supported when the smaller operand, leading ones dropped, equals
-                    // the trailing dimensions of the larger one (it then repeats as a contiguous block)
-                    const Shape& big = volume(b) > volume(out) ? b : out;
-                    Shape small = volume(b) > volume(out) ? out : b;
-                    while (!small.empty() && small.front() == 1)
-                        small.erase(small.begin());
-                    bool ok = small.size() <= big.size() && std::equal(small.begin(), small.end(), big.end() - (long)small.size());
-                    FDX_REQUIRE(ok, "%s: unsupported broadcast in Add", o.name.c_str());
-                    out = Shape(big);
+                    Shape r(std::max(out.size(), b.size()), 1);
+                    for (size_t d = 0; d < r.size(); ++d) {
+                        const int64_t x = d < out.size() ? out[out.size() - 1 - d] : 1, y = d < b.size() ? b[b.size() - 1 - d] : 1;
+                        FDX_REQUIRE(x == y || x == 1 || y == 1, "Invalid shapes for combining tensors.");
+                        r[r.size() - 1 - d] = std::max(x, y);
+                    }
+                    out = r;
                 }
+                break;
+            }
+            case OpKind::Concat: {
+                // tensor.hpp:459-483: the axis counts from the first input's rank
+                const int rank = (int)in0->size();
+                int axis = o.axis < 0 ? o.axis + rank + 1 : o.axis;
+                FDX_REQUIRE(axis >= 1 && axis <= rank, "Invalid axis (%d) for tensor concatenation.", o.axis);
+                out = *in0;
+                for (size_t k = 1; k < o.in.size(); ++k) {
+                    const Shape& b = shapes[o.in[k]];
+                    FDX_REQUIRE(b.size() == out.size(), "%s: Concatenate inputs differ in rank", o.name.c_str());
+                    for (int d = 0; d < rank; ++d)
+                        FDX_REQUIRE(d == axis - 1 || b[(size_t)d] == out[(size_t)d], "%s: Concatenate inputs differ off the axis",
+                            o.name.c_str());
+                    out[(size_t)axis - 1] += b[(size_t)axis - 1];
+                }
+                break;
+            }
+            case OpKind::Einsum: {
+                EinsumSpec spec;
+                std::string err;
+                Shape dims = *in0;
+                if (!spec.parse(o.equation, o.bias_axes, err) || !(dims.size() < spec.lhs.size())) {
+                    set_error("%s: %s", o.name.c_str(), err.empty() ? "EinsumDense: input rank exceeds lhs char count." : err.c_str());
+                    return FDX_ERR_INVALID;
+                }
+                if (!spec.derive_sizes(o.kernel_dims, dims, o.full_out, err)) {
+                    set_error("%s: %s", o.name.c_str(), err.c_str());
+                    return FDX_ERR_INVALID;
+                }
+                out.clear();
+                for (size_t i = 1; i < spec.rhs.size(); ++i)
+                    out.push_back(spec.size.at(spec.rhs[i]));
+                FDX_REQUIRE(out.size() <= 5, "%s: EinsumDense output rank above 5", o.name.c_str());
                 break;
             }
             case OpKind::Embedding:
@@ -828,6 +977,7 @@ namespace {
         switch (o.kind) {
         case OpKind::Conv2D: return 2.0 * batch * volume(out) * o.kh * o.kw * o.n_in;
         case OpKind::Dense: return 2.0 * batch * volume(out) * o.n_in;
+        case OpKind::Einsum: return o.gemm ? 2.0 * batch * volume(out) * o.n_in : 0.0;
         case OpKind::MHA: {
             const double t = (double)shapes[o.in[0]][0], s = (double)shapes[o.in[1]][0];
             return 2.0 * batch * (t * o.d_in * o.heads * o.dk + s * o.d_in * o.heads * (o.dk + o.dv)
@@ -975,20 +1125,24 @@ namespace {
             break;
         }
         case OpKind::LayerNorm: {
+            // axes are 1-based positions in the sample's own rank (negative from the end)
             const int rank = (int)is->size();
-            std::vector<int64_t> axes = o.target_shape;
-            for (auto& a : axes)
+            int64_t dims5[5] = { 1, 1, 1, 1, 1 };
+            for (int k = 0; k < rank; ++k)
+                dims5[5 - rank + k] = (*is)[(size_t)k];
+            unsigned mask = 0;
+            int64_t count = 1;
+            for (int64_t a : o.target_shape) {
                 a = a < 0 ? a + rank + 1 : a;
-            std::sort(axes.begin(), axes.end());
-            int64_t depth = 1;
-            for (size_t k = 0; k < axes.size(); ++k) {
-                if (axes[k] != rank - (int64_t)axes.size() + 1 + (int64_t)k) {
-                    set_error("%s: LayerNormalization is supported over trailing axes only", o.name.c_str());
-                    return FDX_ERR_UNSUPPORTED;
-                }
-                depth *= (*is)[(size_t)axes[k] - 1];
+                FDX_REQUIRE(a >= 1 && a <= rank, "%s: LayerNormalization axis out of range", o.name.c_str());
+                const int pos = 5 - rank + (int)a - 1;
+                if (!((mask >> pos) & 1u))
+                    count *= dims5[pos];
+                mask |= 1u << pos;
             }
-            st = fdx_layernorm_f32(in0, (int64_t)B * volume(*is) / depth, (int)depth, o.dw[0], o.dw[1], o.eps, out);
+            FDX_REQUIRE(o.cout == 0 || o.cout == count, "%s: gamma / beta do not match the normalised axes",
+                o.name.c_str());
+            st = fdx_layernorm_axes_f32(in0, B, dims5, mask, o.dw[0], o.dw[1], o.eps, out);
             break;
         }
         case OpKind::Act:
@@ -1012,29 +1166,82 @@ namespace {
         case OpKind::Add: {
             // left fold (tensor.hpp:677-680); the last step carries the fused activation
             const float* acc = in0;
-            int64_t acc_vol = volume(*is);
+            Shape acc_shape = *is;
             for (size_t k = 1; k < o.in.size() && st == FDX_OK; ++k) {
                 const float* b = p.out[o.in[k]];
-                const int64_t bv = volume(p.shapes[o.in[k]]);
+                const Shape& bs = p.shapes[o.in[k]];
                 const fdx_act* a = k + 1 == o.in.size() ? actp : nullptr;
-                if (bv == acc_vol || B == 1) {
-                    const size_t big = (size_t)B * (size_t)std::max(acc_vol, bv), small = (size_t)B * (size_t)std::min(acc_vol, bv);
-                    st = fdx_eltwise_add_f32(acc_vol >= bv ? acc : b, acc_vol >= bv ? b : acc, big, small, a, out);
+                if (bs == acc_shape) {
+                    const size_t n = (size_t)B * (size_t)volume(bs);
+                    st = fdx_eltwise_add_f32(acc, b, n, n, a, out);
                 } else {
-                    // broadcast inside each sample: run sample by sample so the smaller operand repeats per sample
-                    const int64_t big = std::max(acc_vol, bv), small = std::min(acc_vol, bv);
-                    for (int s = 0; s < B && st == FDX_OK; ++s) {
-                        const float* pa = acc + (size_t)s * (size_t)acc_vol;
-                        const float* pb = b + (size_t)s * (size_t)bv;
-                        st = fdx_eltwise_add_f32(acc_vol >= bv ? pa : pb, acc_vol >= bv ? pb : pa, (size_t)big, (size_t)small, a,
-                            out + (size_t)s * (size_t)big);
+                    int64_t ad[5] = { 1, 1, 1, 1, 1 }, bd[5] = { 1, 1, 1, 1, 1 }, od[5];
+                    for (size_t d = 0; d < acc_shape.size(); ++d)
+                        ad[5 - acc_shape.size() + d] = acc_shape[d];
+                    for (size_t d = 0; d < bs.size(); ++d)
+                        bd[5 - bs.size() + d] = bs[d];
+                    // the running sum may already live in `out`; it is only read in place when it has the output's shape
+                    if (acc == out) {
+                        bool same = true;
+                        for (int d = 0; d < 5; ++d)
+                            same = same && ad[d] >= bd[d];
+                        FDX_REQUIRE(same, "%s: this chain of broadcasts needs a temporary", o.name.c_str());
                     }
+                    st = fdx_broadcast_add_f32(acc, ad, b, bd, B, a, out, od);
+                    Shape r(std::max(acc_shape.size(), bs.size()));
+                    for (size_t d = 0; d < r.size(); ++d)
+                        r[d] = od[5 - r.size() + d];
+                    acc_shape = r;
                 }
                 acc = out;
-                acc_vol = std::max(acc_vol, bv);
             }
             if (o.in.size() == 1)
-                st = fdx_activation_f32(in0, (size_t)B * (size_t)acc_vol, actp, out);
+                st = fdx_activation_f32(in0, (size_t)B * (size_t)volume(*is), actp, out);
+            break;
+        }
+        case OpKind::Concat: {
+            const int rank = (int)is->size();
+            const int axis = (o.axis < 0 ? o.axis + rank + 1 : o.axis) - 1;
+            int64_t outer = B;
+            for (int d = 0; d < axis; ++d)
+                outer *= (*is)[(size_t)d];
+            std::vector<const float*> ptrs;
+            std::vector<int64_t> inner;
+            for (int i : o.in) {
+                const Shape& s = p.shapes[i];
+                int64_t v = 1;
+                for (int d = axis; d < rank; ++d)
+                    v *= s[(size_t)d];
+                ptrs.push_back(p.out[i]);
+                inner.push_back(v);
+            }
+            st = fdx_concat_f32(ptrs.data(), (int)ptrs.size(), inner.data(), outer, out);
+            if (st == FDX_OK && actp)
+                st = fdx_activation_f32(out, (size_t)B * (size_t)volume(os), actp, out);
+            break;
+        }
+        case OpKind::Einsum: {
+            if (o.gemm) {
+                const int64_t rows = (int64_t)B * volume(*is) / o.n_in;
+                FDX_REQUIRE(rows < (1LL << 31), "%s: too many rows", o.name.c_str());
+                st = fdx_gemm_bias_act_f32(in0, o.n_in, o.dw[0], o.n_in, (int)rows, o.units, o.n_in, 1.0f, o.dw[1], 0, res, actp, out,
+                    o.units, nullptr);
+            } else {
+                // the leading lhs character is the batch: `B` samples back to back
+                EinsumSpec spec;
+                std::string err;
+                spec.parse(o.equation, o.bias_axes, err);
+                Shape dims = *is;
+                while (dims.size() + 1 < spec.lhs.size())
+                    dims.insert(dims.begin(), 1);
+                dims.insert(dims.begin(), B);
+                Shape full = o.full_out;
+                if (!spec.derive_sizes(o.kernel_dims, dims, full, err)) {
+                    set_error("%s: %s", o.name.c_str(), err.c_str());
+                    return FDX_ERR_INVALID;
+                }
+                st = einsum_launch(spec, in0, o.dw[0], o.dw[1], o.act, out);
+            }
             break;
         }
         case OpKind::Embedding:
@@ -1285,16 +1492,10 @@ extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int ve
             throw FormatError("missing layers array");
         static const Value empty_params = [] { Value v; v.type = Value::Object; return v; }();
         const Value* tp = root.find("trainable_params");
-        Builder b { *m, tp ? *tp : empty_params, {}, {}, {} };
-        for (const auto& l : layers.arr) {
-            const std::string name = l.at("name").str();
-            if (b.layers.count(name))
-                throw FormatError("layer names must be unique: " + name);
-            const std::string cls = l.at("class_name").str();
-            if (cls == "Functional" || cls == "Model" || cls == "Sequential")
-                throw Unsupported("nested models are not supported yet: " + name);
-            b.layers[name] = &l;
-        }
+        Builder b { *m, tp ? *tp : empty_params, {} };
+        b.scopes.emplace_back(new Scope);
+        Scope& top = *b.scopes.back();
+        Builder::index_layers(top, layers);
         for (const auto& s : root.at("input_shapes").arr)
             m->in_decl.push_back(decl_shape(s));
         for (const auto& s : root.at("output_shapes").arr)
@@ -1304,8 +1505,8 @@ extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int ve
         if (ins.size() != m->in_decl.size())
             throw FormatError("input_shapes does not match input_layers");
         for (size_t i = 0; i < ins.size(); ++i) {
-            auto lit = b.layers.find(ins[i].layer);
-            if (lit == b.layers.end() || lit->second->at("class_name").str() != "InputLayer")
+            auto lit = top.layers.find(ins[i].layer);
+            if (lit == top.layers.end() || lit->second->at("class_name").str() != "InputLayer")
                 throw FormatError("input_layers must name InputLayer layers");
             const Value* nodes = lit->second->find("inbound_nodes");
             if (nodes && nodes->size() != 0)
@@ -1317,10 +1518,10 @@ extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int ve
             op.input_index = (int)i;
             m->ops.push_back(std::move(op));
             m->inputs.push_back((int)m->ops.size() - 1);
-            b.input_ops[ins[i].layer] = m->inputs.back();
+            top.input_ops[ins[i].layer] = m->inputs.back();
         }
         for (const auto& o : outs)
-            m->outputs.push_back(b.build(o));
+            m->outputs.push_back(b.build(top, o));
         fuse(*m);
         fdx_status st = upload(*m);
         if (st != FDX_OK)

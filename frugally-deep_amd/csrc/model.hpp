@@ -8,11 +8,12 @@
 #include <vector>
 
 #include "common.hpp"
+#include "einsum.hpp"
 
 namespace fdx {
 
 enum class OpKind {
-    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View
+    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat
 };
 
 using Shape = std::vector<int64_t>; // dims of one sample, no batch axis
@@ -48,6 +49,10 @@ struct Op {
     Shape target_shape;
     bool flatten = false;
     int input_index = -1;
+    std::string equation, bias_axes; // EinsumDense
+    Shape kernel_dims, full_out;     // EinsumDense: kernel extents as stored, output_shape with the batch slot
+    bool gemm = false;               // EinsumDense that is one row-major GEMM (kernel stored transposed)
+    int axis = -1;                   // Concatenate
 
     // host weights (released after upload)
     std::vector<std::vector<float>> hw;
@@ -101,5 +106,6 @@ fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, con
     const float* v, int64_t ldv, int64_t v_batch, int batch, int t, int s, int heads, int dk, int dv, int causal,
     float* out, int64_t ldo, int64_t o_batch, void* scratch_dev);
 fdx_status argmax_launch(const float* x, int64_t rows, int depth, int32_t* out_idx, float* out_val, float* out_idx_f);
+fdx_status einsum_launch(EinsumSpec& spec, const float* in, const float* kernel, const float* bias, const Act& act, float* out);
 fdx_status gather_rows_launch(const float* in, int64_t rows, int depth, int64_t row_stride, int64_t offset, float* out);
 }

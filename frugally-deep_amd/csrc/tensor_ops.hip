@@ -1,0 +1,321 @@
+// Strided tensor kernels for the layer forms that are not a plain row-major pass: EinsumDense
+// with an arbitrary equation, element-wise Add with size-1 broadcasting on any axis,
+// Concatenate, and LayerNormalization over axes that are not the trailing ones.  They are
+// index-decoding kernels (one output element, or one normalisation group, per lane / wave) and
+// HBM-bound; the regular cases of the same layers take the contiguous kernels instead.
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+#include "einsum.hpp"
+
+namespace fdx {
+
+struct EinsumDesc {
+    int n_out, n_sum;
+    int64_t od[6], oi[6], ok[6], ob[6]; // per output char: extent, stride in input / kernel / bias
+    int64_t sd[4], si[4], sk[4];        // per summed char: extent, stride in input / kernel
+};
+
+// out[rhs] = sum over summed chars of in[lhs] * kernel[...] (+ bias), one output element per lane;
+// the summed characters advance like an odometer so the inner loop has no divisions.
+// include/fdeep/layers/einsum_dense_layer.hpp:169-196, 223-250
+__global__ void einsum_kernel(const float* __restrict__ in, const float* __restrict__ kernel, const float* __restrict__ bias,
+    float* __restrict__ out, EinsumDesc d, size_t total, Act act)
+{
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = o;
+        int64_t bi = 0, bk = 0, bb = 0;
+        for (int i = d.n_out - 1; i >= 0; --i) {
+            const int64_t c = (int64_t)(rem % (size_t)d.od[i]);
+            rem /= (size_t)d.od[i];
+            bi += c * d.oi[i];
+            bk += c * d.ok[i];
+            bb += c * d.ob[i];
+        }
+        float acc = 0.f;
+        int64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+        const int64_t e0 = d.n_sum > 0 ? d.sd[0] : 1, e1 = d.n_sum > 1 ? d.sd[1] : 1, e2 = d.n_sum > 2 ? d.sd[2] : 1,
+                      e3 = d.n_sum > 3 ? d.sd[3] : 1;
+        for (c0 = 0; c0 < e0; ++c0)
+            for (c1 = 0; c1 < e1; ++c1)
+                for (c2 = 0; c2 < e2; ++c2) {
+                    const int64_t pi = bi + c0 * d.si[0] + c1 * d.si[1] + c2 * d.si[2];
+                    const int64_t pk = bk + c0 * d.sk[0] + c1 * d.sk[1] + c2 * d.sk[2];
+                    for (c3 = 0; c3 < e3; ++c3)
+                        acc += in[pi + c3 * d.si[3]] * kernel[pk + c3 * d.sk[3]];
+                }
+        if (bias)
+            acc += bias[bb];
+        out[o] = apply_act(acc, act);
+    }
+}
+
+struct BcastDesc {
+    int64_t dims[6], sa[6], sb[6]; // output extents (batch first), operand strides (0 = repeated)
+};
+
+// include/fdeep/tensor.hpp:642-660: every axis of the two operands is equal or 1; the size-1 side repeats
+__global__ void bcast_add_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+    BcastDesc d, size_t total, Act act)
+{
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = o;
+        int64_t pa = 0, pb = 0;
+#pragma unroll
+        for (int i = 5; i >= 0; --i) {
+            const int64_t c = (int64_t)(rem % (size_t)d.dims[i]);
+            rem /= (size_t)d.dims[i];
+            pa += c * d.sa[i];
+            pb += c * d.sb[i];
+        }
+        out[o] = apply_act(a[pa] + b[pb], act);
+    }
+}
+
+// rows of `cols` floats copied into a wider row-major destination (row pitch ld_out)
+__global__ void copy_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t rows, int64_t cols, int64_t ld_out)
+{
+    const size_t total = (size_t)rows * (size_t)cols;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / (size_t)cols, c = i % (size_t)cols;
+        out[r * (size_t)ld_out + c] = in[i];
+    }
+}
+
+struct NormDesc {
+    int n_keep, n_norm;
+    int64_t kd[6], ks[6]; // kept axes (batch first): extent, stride
+    int64_t nd[5], ns[5]; // normalised axes in storage order: extent, stride
+};
+
+// One wave per group (= one position on the kept axes).  Mean, then the biased variance as the
+// mean of squared differences, then x * inv + (beta - mean * inv) with inv = gamma / sqrt(var + eps)
+// (include/fdeep/tensor.hpp:758-793, layers/layer_normalization_layer.hpp:37-61); gamma / beta are
+// indexed by the position on the normalised axes.
+__global__ __launch_bounds__(256) void layernorm_axes_kernel(const float* __restrict__ x, float* __restrict__ out, NormDesc d,
+    int64_t groups, int64_t count, const float* __restrict__ gamma, const float* __restrict__ beta, float eps)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (g >= groups)
+        return;
+    int64_t base = 0;
+    {
+        int64_t rem = g;
+        for (int i = d.n_keep - 1; i >= 0; --i) {
+            base += (rem % d.kd[i]) * d.ks[i];
+            rem /= d.kd[i];
+        }
+    }
+    auto offset = [&](int64_t e) {
+        int64_t off = base;
+        for (int i = d.n_norm - 1; i >= 0; --i) {
+            off += (e % d.nd[i]) * d.ns[i];
+            e /= d.nd[i];
+        }
+        return off;
+    };
+    float s = 0.f;
+    for (int64_t e = lane; e < count; e += 64)
+        s += x[offset(e)];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        s += __shfl_xor(s, o, 64);
+    const float mean = s / (float)count;
+    float v = 0.f;
+    for (int64_t e = lane; e < count; e += 64) {
+        const float df = x[offset(e)] - mean;
+        v += df * df;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    const float rstd = 1.0f / sqrtf(v / (float)count + eps);
+    for (int64_t e = lane; e < count; e += 64) {
+        const int64_t off = offset(e);
+        const float inv = (gamma ? gamma[e] : 1.0f) * rstd;
+        out[off] = x[off] * inv + ((beta ? beta[e] : 0.0f) - mean * inv);
+    }
+}
+
+static int grid_of(size_t work_items, int block)
+{
+    size_t g = (work_items + block - 1) / block;
+    const size_t cap = 256 * 16;
+    return (int)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+// Shared by the C entry point and the model executor.  in_dims: extents of the trailing lhs
+// characters (the batch is simply the first of them); the kernel keeps the layout of the file.
+fdx_status einsum_launch(EinsumSpec& spec, const float* in, const float* kernel, const float* bias, const Act& act, float* out)
+{
+    EinsumDesc d {};
+    d.n_out = (int)spec.rhs.size();
+    d.n_sum = (int)spec.summed.size();
+    for (int i = 0; i < d.n_out; ++i) {
+        const char c = spec.rhs[(size_t)i];
+        d.od[i] = spec.size.at(c);
+        d.oi[i] = spec.stride_in(spec.lhs, c);
+        d.ok[i] = spec.stride_in(spec.ker, c);
+        d.ob[i] = spec.stride_in(spec.bias_chars, c);
+    }
+    for (int i = 0; i < 4; ++i) {
+        d.sd[i] = 1;
+        d.si[i] = d.sk[i] = 0;
+    }
+    // the longest summed axis goes innermost only by position: keep the equation's order
+    for (int i = 0; i < d.n_sum; ++i) {
+        const char c = spec.summed[(size_t)i];
+        const int slot = 4 - d.n_sum + i; // right-aligned so the innermost loop is the last summed char
+        d.sd[slot] = spec.size.at(c);
+        d.si[slot] = spec.stride_in(spec.lhs, c);
+        d.sk[slot] = spec.stride_in(spec.ker, c);
+    }
+    d.n_sum = 4;
+    const int64_t total = spec.volume_of(spec.rhs), sum_vol = spec.volume_of(spec.summed);
+    FDX_REQUIRE(total > 0 && sum_vol > 0, "einsum_dense: empty operand");
+    profile_begin();
+    hipLaunchKernelGGL(einsum_kernel, dim3(grid_of((size_t)total, 256)), dim3(256), 0, stream(), in, kernel,
+        spec.bias_chars.empty() ? nullptr : bias, out, d, (size_t)total, act);
+    profile_end("einsum_dense_f32", 2.0 * (double)total * (double)sum_vol,
+        4.0 * ((double)spec.volume_of(spec.lhs) + (double)spec.volume_of(spec.ker) + (double)total));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+} // namespace fdx
+
+using namespace fdx;
+
+extern "C" fdx_status fdx_einsum_dense_f32(const char* equation, const char* bias_axes, const float* in, int in_rank,
+    const int64_t* in_dims, const float* kernel, int kernel_rank, const int64_t* kernel_dims, const float* bias,
+    const int64_t* full_output_shape, const fdx_act* act, float* out, int* out_rank, int64_t* out_dims)
+{
+    FDX_REQUIRE(equation && in && in_dims && kernel && kernel_dims && out, "einsum_dense: null argument");
+    FDX_REQUIRE(in_rank >= 1 && in_rank <= 6 && kernel_rank >= 1 && kernel_rank <= 6, "einsum_dense: ranks must be 1..6");
+    EinsumSpec spec;
+    std::string err;
+    if (!spec.parse(equation, bias_axes ? bias_axes : "", err)) {
+        set_error("%s", err.c_str());
+        return FDX_ERR_INVALID;
+    }
+    std::vector<int64_t> full;
+    if (full_output_shape)
+        full.assign(full_output_shape, full_output_shape + spec.rhs.size());
+    if (!spec.derive_sizes(std::vector<int64_t>(kernel_dims, kernel_dims + kernel_rank),
+            std::vector<int64_t>(in_dims, in_dims + in_rank), full, err)) {
+        set_error("%s", err.c_str());
+        return FDX_ERR_INVALID;
+    }
+    FDX_REQUIRE(spec.bias_chars.empty() || bias, "einsum_dense: bias_axes given without a bias");
+    if (out_rank)
+        *out_rank = (int)spec.rhs.size();
+    if (out_dims)
+        for (size_t i = 0; i < spec.rhs.size(); ++i)
+            out_dims[i] = spec.size.at(spec.rhs[i]);
+    return einsum_launch(spec, in, kernel, bias, make_act(act), out);
+}
+
+extern "C" fdx_status fdx_broadcast_add_f32(const float* a, const int64_t* a_dims5, const float* b, const int64_t* b_dims5,
+    int batch, const fdx_act* act, float* out, int64_t* out_dims5)
+{
+    FDX_REQUIRE(a && b && a_dims5 && b_dims5 && out && batch > 0, "broadcast_add: bad arguments");
+    BcastDesc d {};
+    int64_t va = 1, vb = 1, vo = 1;
+    for (int i = 0; i < 5; ++i) {
+        const int64_t x = a_dims5[i], y = b_dims5[i];
+        FDX_REQUIRE(x > 0 && y > 0 && (x == y || x == 1 || y == 1), "Invalid shapes for combining tensors.");
+        d.dims[i + 1] = std::max(x, y);
+        va *= x;
+        vb *= y;
+        vo *= d.dims[i + 1];
+        if (out_dims5)
+            out_dims5[i] = d.dims[i + 1];
+    }
+    int64_t sa = 1, sb = 1;
+    for (int i = 4; i >= 0; --i) {
+        d.sa[i + 1] = a_dims5[i] == 1 ? 0 : sa;
+        d.sb[i + 1] = b_dims5[i] == 1 ? 0 : sb;
+        sa *= a_dims5[i];
+        sb *= b_dims5[i];
+    }
+    d.dims[0] = batch;
+    d.sa[0] = va;
+    d.sb[0] = vb;
+    const size_t total = (size_t)batch * (size_t)vo;
+    profile_begin();
+    hipLaunchKernelGGL(bcast_add_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), a, b, out, d, total, make_act(act));
+    profile_end("broadcast_add_f32", 0.0, 4.0 * ((double)batch * (va + vb) + (double)total));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_concat_f32(const float* const* ins, int n_inputs, const int64_t* inner, int64_t outer, float* out)
+{
+    FDX_REQUIRE(ins && inner && out && n_inputs > 0 && outer > 0, "concat: bad arguments");
+    int64_t ld = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        FDX_REQUIRE(ins[i] && inner[i] > 0, "concat: bad input %d", i);
+        ld += inner[i];
+    }
+    int64_t off = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        const size_t total = (size_t)outer * (size_t)inner[i];
+        profile_begin();
+        hipLaunchKernelGGL(copy_rows_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), ins[i], out + off, outer, inner[i], ld);
+        profile_end("concat_f32", 0.0, 8.0 * (double)total);
+        FDX_LAUNCH_CHECK();
+        off += inner[i];
+    }
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
+    const float* beta, float eps, float* out)
+{
+    FDX_REQUIRE(x && dims5 && out && batch > 0 && axes_mask != 0 && axes_mask < 32, "layernorm_axes: bad arguments");
+    int64_t vol = 1;
+    for (int i = 0; i < 5; ++i) {
+        FDX_REQUIRE(dims5[i] > 0, "layernorm_axes: bad extent");
+        vol *= dims5[i];
+    }
+    // trailing axes (ignoring size-1 axes around them) are one contiguous row: the fast kernel
+    {
+        int64_t depth = 1;
+        int i = 4;
+        for (; i >= 0 && ((axes_mask >> i) & 1u || dims5[i] == 1); --i)
+            if ((axes_mask >> i) & 1u)
+                depth *= dims5[i];
+        bool rest_kept = true;
+        for (int j = i; j >= 0; --j)
+            if (((axes_mask >> j) & 1u) && dims5[j] != 1)
+                rest_kept = false;
+        if (rest_kept && depth < (1LL << 31))
+            return fdx_layernorm_f32(x, (int64_t)batch * vol / depth, (int)depth, gamma, beta, eps, out);
+    }
+    NormDesc d {};
+    d.kd[0] = batch;
+    d.ks[0] = vol;
+    d.n_keep = 1;
+    int64_t stride = vol, count = 1, groups = batch;
+    for (int i = 0; i < 5; ++i) {
+        stride /= dims5[i];
+        if ((axes_mask >> i) & 1u) {
+            d.nd[d.n_norm] = dims5[i];
+            d.ns[d.n_norm++] = stride;
+            count *= dims5[i];
+        } else {
+            d.kd[d.n_keep] = dims5[i];
+            d.ks[d.n_keep++] = stride;
+            groups *= dims5[i];
+        }
+    }
+    profile_begin();
+    hipLaunchKernelGGL(layernorm_axes_kernel, dim3((unsigned)((groups + 3) / 4)), dim3(256), 0, stream(), x, out, d, groups, count,
+        gamma, beta, eps);
+    profile_end("layernorm_axes_f32", 0.0, 8.0 * (double)batch * (double)vol);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}

@@ -56,7 +56,8 @@ class T:
 
 
 def _kt(t):
-    return {"class_name": "__keras_tensor__", "config": {"keras_history": [t.layer, 0, 0]}}
+    return {"class_name": "__keras_tensor__",
+            "config": {"keras_history": [t.layer, getattr(t, "node", 0), getattr(t, "tensor", 0)]}}
 
 
 class Builder:
@@ -173,8 +174,77 @@ class Builder:
         cls = "GlobalAveragePooling2D" if kind == "avg" else "GlobalMaxPooling2D"
         return self._add(cls, name, {"keepdims": False}, [x], (x.shape[-1],))
 
+    def layernorm_axes(self, x, name, axes, eps=1e-3, center=True, scale=True):
+        """LayerNormalization over arbitrary axes (1-based in the sample's rank, negative from the end);
+        gamma / beta are shaped like the normalised axes in storage order."""
+        rank = len(x.shape)
+        pos = sorted(set(a + rank + 1 if a < 0 else a for a in axes))
+        n = int(np.prod([x.shape[a - 1] for a in pos]))
+        p = {}
+        if scale:
+            p["gamma"] = (0.5 + self.rng.random(n)).astype(np.float32)
+        if center:
+            p["beta"] = self.normal((n,), 0.3)
+        self.params[name] = p
+        return self._add("LayerNormalization", name, {"axis": list(axes), "epsilon": eps, "center": center, "scale": scale},
+                         [x], x.shape)
+
     def add(self, xs, name):
-        return self._add("Add", name, {}, xs, xs[0].shape, merge=True)
+        rank = max(len(t.shape) for t in xs)
+        shape = [1] * rank
+        for t in xs:  # size-1 broadcasting on right-aligned axes
+            for i, d in enumerate(reversed(t.shape)):
+                cur = shape[rank - 1 - i]
+                shape[rank - 1 - i] = None if d is None or cur is None else max(cur, d)  # None = variable extent
+        return self._add("Add", name, {}, xs, tuple(shape), merge=True)
+
+    def concatenate(self, xs, name, axis=-1):
+        rank = len(xs[0].shape)
+        a = (axis + rank + 1 if axis < 0 else axis) - 1
+        shape = list(xs[0].shape)
+        shape[a] = sum(t.shape[a] for t in xs)
+        return self._add("Concatenate", name, {"axis": axis}, xs, tuple(shape), merge=True)
+
+    def einsum_dense(self, x, equation, kernel_shape, name, bias_axes=None, output_shape=None, activation=None, std=None):
+        """EinsumDense; the bias is stored over the bias axes in rhs order whatever the order of the
+        bias_axes string (include/fdeep/layers/einsum_dense_layer.hpp:197-222)."""
+        lhs, rest = equation.split(",")
+        ker, rhs = rest.split("->")
+        size = dict(zip(ker, kernel_shape))
+        for c, d in zip(lhs[len(lhs) - len(x.shape):], x.shape):
+            assert size.setdefault(c, d) == d, (equation, c)
+        summed = [c for c in lhs if c not in rhs and c in ker]
+        fan_in = int(np.prod([size[c] for c in summed])) if summed else 1
+        kernel = self.he(tuple(kernel_shape), fan_in) if std is None else self.normal(tuple(kernel_shape), std)
+        p = {"kernel": kernel, "kernel_shape": [int(v) for v in kernel_shape]}
+        if bias_axes:
+            bshape = [size[c] for c in rhs if c in bias_axes]
+            p["bias"] = self.normal(tuple(bshape), 0.5)
+            p["bias_shape"] = [int(v) for v in bshape]
+        self.params[name] = p
+        out_shape = tuple(size[c] for c in rhs[1:])
+        cfg = {"equation": equation, "bias_axes": bias_axes,
+               "output_shape": list(output_shape) if output_shape is not None else list(out_shape)}
+        if activation is not None:
+            cfg["activation"] = activation
+        return self._add("EinsumDense", name, cfg, [x], out_shape)
+
+    def nested(self, inner_spec, xs, name):
+        """Applies a finished model (Builder.finish) as one Functional layer; its parameters are stored under
+        "<name>_<inner layer>" (keras_export/convert_model.py:907-918).  Returns one tensor per inner output."""
+        arch = inner_spec["architecture"]
+        for lname, prm in inner_spec["trainable_params"].items():
+            self.params[name + "_" + lname] = prm
+        assert name not in self.names, name
+        self.names.add(name)
+        node = {"args": [_kt(t) for t in xs], "kwargs": {}}
+        self.layers.append({"class_name": "Functional", "name": name, "config": arch["config"], "inbound_nodes": [node]})
+        outs = []
+        for i, shp in enumerate(inner_spec["output_shapes"]):
+            t = T(name, shp)
+            t.node, t.tensor = 1, i  # Keras numbers the first outer call of a nested model as node 1
+            outs.append(t)
+        return outs
 
     def dense(self, x, units, name, activation=None, use_bias=True, init="he", bias_std=0.0):
         n_in = x.shape[-1]
@@ -223,7 +293,7 @@ class Builder:
             "architecture": {"class_name": "Functional", "config": {
                 "name": self.name, "layers": self.layers,
                 "input_layers": [[t.layer, 0, 0] for t in self.inputs],
-                "output_layers": [[t.layer, 0, 0] for t in outputs]}},
+                "output_layers": [[t.layer, getattr(t, "node", 0), getattr(t, "tensor", 0)] for t in outputs]}},
             "trainable_params": self.params,
             "hash": "",
         }

@@ -151,6 +151,33 @@ fdx_status fdx_zero_pad2d_nhwc_f32(const float* in, int n, int h, int w, int c, 
  * (include/fdeep/layers/layer_normalization_layer.hpp:37-63, tensor.hpp:758-793); gamma/beta may be NULL */
 fdx_status fdx_layernorm_f32(const float* x, int64_t rows, int depth, const float* gamma, const float* beta,
     float eps, float* out);
+/* LayerNormalization over any subset of the five right-aligned axes of each sample
+ * (layer_normalization_layer.hpp:37-61: moments over `axes`, gamma / beta shaped like the normalised
+ * axes).  dims5 = (dim5, dim4, height, width, depth); bit i of axes_mask selects dims5[i]; gamma / beta
+ * hold one value per position on the selected axes, in storage order.  Trailing axes take the
+ * row kernel above. */
+fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
+    const float* beta, float eps, float* out);
+/* out = act(a + b) with size-1 broadcasting on any of the five right-aligned axes, per sample
+ * (elem_wise_combine_tensors, include/fdeep/tensor.hpp:642-660); `batch` samples of each operand lie
+ * back to back; out_dims5 (may be NULL) receives the per-axis maximum */
+fdx_status fdx_broadcast_add_f32(const float* a, const int64_t* a_dims5, const float* b, const int64_t* b_dims5,
+    int batch, const fdx_act* act, float* out, int64_t* out_dims5);
+/* Concatenate along one axis (concatenate_tensors, include/fdeep/tensor.hpp:459-483): input i is
+ * `outer` rows of inner[i] floats (inner = extent on the axis times everything to its right, outer =
+ * batch times everything to its left); rows are laid side by side in `out` */
+fdx_status fdx_concat_f32(const float* const* ins, int n_inputs, const int64_t* inner, int64_t outer, float* out);
+/* EinsumDense, any equation "lhs,kernel->rhs" the reference evaluates
+ * (include/fdeep/layers/einsum_dense_layer.hpp:125-258): in_dims are the extents of the trailing
+ * in_rank characters of lhs (missing leading ones count as 1; with a batch the first lhs character
+ * simply has extent `batch`), kernel_dims those of the kernel as stored in the file, bias (NULL when
+ * bias_axes is NULL or empty) is laid out over the bias axes in rhs order (:197-222),
+ * full_output_shape (may be NULL) gives one extent per rhs character for characters that occur only
+ * in the output.  The output keeps every rhs character, the leading one included; out_rank /
+ * out_dims (up to 6 entries, may be NULL) receive its shape. */
+fdx_status fdx_einsum_dense_f32(const char* equation, const char* bias_axes, const float* in, int in_rank,
+    const int64_t* in_dims, const float* kernel, int kernel_rank, const int64_t* kernel_dims, const float* bias,
+    const int64_t* full_output_shape, const fdx_act* act, float* out, int* out_rank, int64_t* out_dims);
 /* softmax over the last axis in the reference's exp(x - m - log(sum)) form (tensor.hpp:1165-1192);
  * causal_period > 0 masks row r to its first (r % causal_period) + 1 + causal_offset entries
  * (the prefix identity of causal self-attention; no counterpart in the reference, which has no mask) */

@@ -142,6 +142,18 @@ def layernorm(x, gamma, beta, eps, n_axes=1):
     return out
 
 
+def layernorm_axes(x, axes, gamma, beta, eps):
+    """LayerNormalization over `axes` (1-based in x's rank, negative from the end): moments over those
+    axes, gamma / beta shaped like them in storage order (layers/layer_normalization_layer.hpp:37-61).
+    The axes are brought to the end, rows are normalised by the C routine, and the move is undone."""
+    x = _f32(x)
+    axes = sorted(set(a + x.ndim + 1 if a < 0 else a for a in axes))
+    src = [a - 1 for a in axes]
+    dst = list(range(x.ndim - len(axes), x.ndim))
+    xm = np.ascontiguousarray(np.moveaxis(x, src, dst))
+    return np.ascontiguousarray(np.moveaxis(layernorm(xm, gamma, beta, eps, len(axes)), dst, src))
+
+
 def batchnorm(x, mean, var, gamma, beta, eps):
     x = _f32(x)
     c = x.shape[-1]
@@ -397,10 +409,7 @@ class _Layer:
         elif cls == "LayerNormalization":
             x = ins[0]
             axes = c["axis"] if isinstance(c["axis"], list) else [c["axis"]]
-            axes = sorted(a + x.ndim + 1 if a < 0 else a for a in axes)
-            if axes != list(range(x.ndim + 1 - len(axes), x.ndim + 1)):
-                raise RuntimeError("oracle: LayerNormalization over non-trailing axes not restated")
-            out = layernorm(x, p["gamma"], p["beta"], c["epsilon"], len(axes))
+            out = layernorm_axes(x, axes, p["gamma"], p["beta"], c["epsilon"])
         elif cls == "ReLU":
             out = _activation("relu", c, ins[0])
         elif cls == "Activation":
@@ -422,6 +431,14 @@ class _Layer:
             out = ins[0]
             for other in ins[1:]:  # left fold, tensor.hpp:677-680
                 out = add(out, other)
+        elif cls == "Concatenate":
+            # the axis counts from the first input's rank, batch axis = 0 (tensor.hpp:459-483)
+            axis = int(c["axis"])
+            rank = _f32(ins[0]).ndim
+            axis = axis + rank + 1 if axis < 0 else axis
+            if not 1 <= axis <= rank:
+                raise RuntimeError("Invalid axis (%d) for tensor concatenation." % axis)
+            out = np.concatenate([_f32(t) for t in ins], axis=axis - 1)
         elif cls == "Embedding":
             out = embedding(ins[0], p["w"], int(c["input_dim"]), int(c["output_dim"]))
         elif cls == "MultiHeadAttention":
@@ -443,6 +460,60 @@ class _Layer:
         return out
 
 
+class _Graph:
+    """One level of the layer graph: the model itself or a nested Functional model, whose layers
+    read their parameters under "<outer layer names>_<layer>" (import_model.hpp:397-424)."""
+
+    def __init__(self, config, get_param):
+        self.layers = {}
+        self.nested = {}
+        for ld in config["layers"]:
+            if ld["name"] in self.layers or ld["name"] in self.nested:
+                raise RuntimeError("layer names must be unique")
+            if ld["class_name"] in ("Functional", "Model"):
+                prefix = ld["name"] + "_"
+                inner = _Graph(ld["config"], lambda layer, key, pf=prefix: get_param(pf + layer, key))
+                inner.nodes = [_node_inputs(n) for n in ld.get("inbound_nodes", [])]
+                self.nested[ld["name"]] = inner
+            else:
+                self.layers[ld["name"]] = _Layer(ld, get_param)
+        self.inputs = _connections(config["input_layers"])
+        self.outputs = _connections(config["output_layers"])
+
+    def run(self, inputs, causal=False, taps=None):
+        if len(inputs) != len(self.inputs):
+            raise RuntimeError("invalid number of input tensors for this model: %d required but %d provided"
+                               % (len(self.inputs), len(inputs)))
+        memo = {}
+        for (lname, node, tidx), x in zip(self.inputs, inputs):
+            memo[(lname, node)] = [x]
+
+        def get(conn):
+            lname, node, tidx = conn
+            if lname in self.nested:
+                inner = self.nested[lname]
+                # a nested model counts its construction as node 0 (layers/model_layer.hpp:36-44)
+                node = node - 1 if node >= 1 else node
+                key = (lname, node)
+                if key not in memo:
+                    memo[key] = inner.run([get(cn) for cn in inner.nodes[node]], causal)
+                return memo[key][tidx]
+            key = (lname, node)
+            if key not in memo:
+                layer = self.layers[lname]
+                ins = [get(cn) for cn in layer.nodes[node]]
+                if causal and layer.cls == "MultiHeadAttention":
+                    memo[key] = [OracleModel._causal_mha(layer, ins)]
+                else:
+                    memo[key] = [layer.apply(ins)]
+            return memo[key][0]
+
+        outs = [get(cn) for cn in self.outputs]
+        if taps is not None:
+            taps.update({k: v[0] for k, v in memo.items()})
+        return outs
+
+
 class OracleModel:
     """One converted-JSON model evaluated sample by sample on the CPU."""
 
@@ -461,15 +532,10 @@ class OracleModel:
         params = data.get("trainable_params", {})
         get_param = lambda layer, key: params[layer][key]
         self.name = arch["config"]["name"]
-        self.layers = {}
-        for ld in arch["config"]["layers"]:
-            if ld["class_name"] in ("Functional", "Model", "Sequential"):
-                raise RuntimeError("oracle: nested models not restated")
-            if ld["name"] in self.layers:
-                raise RuntimeError("layer names must be unique")
-            self.layers[ld["name"]] = _Layer(ld, get_param)
-        self.inputs = _connections(arch["config"]["input_layers"])
-        self.outputs = _connections(arch["config"]["output_layers"])
+        self.graph = _Graph(arch["config"], get_param)
+        self.layers = self.graph.layers
+        self.inputs = self.graph.inputs
+        self.outputs = self.graph.outputs
         self.input_shapes = data["input_shapes"]
         self.output_shapes = data["output_shapes"]
 
@@ -482,29 +548,10 @@ class OracleModel:
 
     def predict(self, inputs, causal=False, taps=None):
         """inputs: list of arrays without batch dim.  taps: optional dict that receives
-        every intermediate (layer name, node) -> array."""
+        every intermediate (layer name, node) -> array of the top-level graph."""
         inputs = [_f32(x) for x in inputs]
         self._check_inputs(inputs)
-        memo = {}
-        for (lname, node, tidx), x in zip(self.inputs, inputs):
-            memo[(lname, node)] = x
-
-        def get(conn):
-            lname, node, tidx = conn
-            key = (lname, node)
-            if key not in memo:
-                layer = self.layers[lname]
-                ins = [get(cn) for cn in layer.nodes[node]]
-                if causal and layer.cls == "MultiHeadAttention":
-                    memo[key] = self._causal_mha(layer, ins)
-                else:
-                    memo[key] = layer.apply(ins)
-            return memo[key]
-
-        outs = [get(cn) for cn in self.outputs]
-        if taps is not None:
-            taps.update(memo)
-        return outs
+        return self.graph.run(inputs, causal, taps)
 
     @staticmethod
     def _causal_mha(layer, ins):

@@ -1,0 +1,182 @@
+"""GPU parity for the strided layer forms: EinsumDense with arbitrary equations, Add with size-1
+broadcasting, Concatenate, LayerNormalization over arbitrary axes, and models that nest a
+Functional model, against the CPU oracle.  Tolerance: max|gpu - ref| / max|ref| <= 1e-4 per tensor
+(fp32, summation order differs); pure data movement (Concatenate) must be bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+EINSUM = [
+    # equation, sample shape, kernel shape, bias_axes
+    ("abc,cd->abd", (7, 12), (12, 9), "d"),          # the three equations of the reference's test models
+    ("abc,cde->abde", (5, 8), (8, 3, 4), "de"),      # (keras_export/generate_test_models.py:573-585)
+    ("abc,cde->abde", (5, 8), (8, 3, 4), "ed"),      # bias stored in rhs order whatever the string says
+    ("abcd,cde->abe", (4, 3, 6), (3, 6, 5), "e"),
+    ("abc,cd->abd", (7, 12), (12, 9), "b"),          # bias over a row axis
+    ("abc,cd->abd", (7, 12), (12, 9), None),
+    ("abc,dc->abd", (6, 10), (11, 10), "d"),         # kernel stored transposed
+    ("abc,cd->adb", (6, 10), (10, 4), "d"),          # output permuted
+    ("abc,bcd->abd", (6, 10), (6, 10, 3), "bd"),     # a character shared by all three operands
+    ("abcd,bde->ace", (3, 4, 5), (3, 5, 7), "e"),    # two summed characters that are not adjacent in the input
+    ("ab,bc->ac", (33,), (33, 65), "c"),
+]
+
+
+@pytest.mark.parametrize("eq,xs,ks,bias_axes", EINSUM)
+def test_einsum_dense_kernel(fdx, oracle, eq, xs, ks, bias_axes):
+    say("einsum", eq, xs, ks, bias_axes)
+    r = np.random.default_rng(abs(hash((eq, bias_axes))) % 2**31)
+    batch = 3
+    x = r.standard_normal((batch,) + xs).astype(np.float32)
+    k = r.standard_normal(ks).astype(np.float32)
+    lhs, rest = eq.split(",")
+    ker, rhs = rest.split("->")
+    size = dict(zip(ker, ks))
+    size.update(zip(lhs[1:], xs))
+    bias = None
+    if bias_axes:
+        bias = r.standard_normal([size[c] for c in rhs if c in bias_axes]).astype(np.float32)
+    want = np.stack([oracle.einsum_dense(x[i], eq, k, list(ks), bias, bias_axes) for i in range(batch)])
+    got = fdx.einsum_dense(x, eq, k, bias, bias_axes)
+    assert rel(got, want) <= TOL
+
+
+def test_einsum_dense_errors(fdx):
+    x, k = np.zeros((1, 4, 5), np.float32), np.zeros((6, 3), np.float32)
+    with pytest.raises(RuntimeError, match="inconsistent char size"):
+        fdx.einsum_dense(x, "abc,cd->abd", k)
+    with pytest.raises(RuntimeError, match="neither summed nor in the output"):
+        fdx.einsum_dense(x, "abc,bd->ad", np.zeros((4, 3), np.float32))
+
+
+BCAST = [((4, 5, 6), (4, 5, 6)), ((4, 5, 6), (1, 1, 6)), ((4, 5, 6), (4, 1, 1)), ((4, 1, 6), (1, 5, 1)), ((5, 6), (3, 1, 6)),
+         ((2, 3, 4, 5, 6), (1, 3, 1, 5, 1)), ((7,), (9, 1))]
+
+
+@pytest.mark.parametrize("sa,sb", BCAST)
+def test_broadcast_add(fdx, oracle, sa, sb):
+    say("broadcast_add", sa, sb)
+    r = np.random.default_rng(5)
+    a = r.standard_normal((3,) + sa).astype(np.float32)
+    b = r.standard_normal((3,) + sb).astype(np.float32)
+    want = np.stack([oracle.add(a[i], b[i]) for i in range(3)])
+    got = fdx.broadcast_add(a, b)
+    assert got.shape == want.shape and np.array_equal(got, want)
+    got = fdx.broadcast_add(a, b, act=fdx.relu_act(1.5, 0.1, 0.2))
+    want = np.stack([oracle.relu(oracle.add(a[i], b[i]), 1.5, 0.1, 0.2) for i in range(3)])
+    assert rel(got, want) <= 1e-6
+
+
+def test_broadcast_add_rejects_mismatch(fdx):
+    with pytest.raises(RuntimeError, match="Invalid shapes for combining tensors"):
+        fdx.broadcast_add(np.zeros((1, 4, 5), np.float32), np.zeros((1, 3, 5), np.float32))
+
+
+@pytest.mark.parametrize("shapes,axis", [([(4, 5, 6), (4, 5, 2), (4, 5, 9)], -1), ([(4, 5, 6), (4, 1, 6)], 2),
+                                         ([(2, 5, 6), (4, 5, 6)], 1), ([(7,), (3,)], 1), ([(3, 4), (3, 5)], -1)])
+def test_concat(fdx, shapes, axis):
+    say("concat", shapes, axis)
+    r = np.random.default_rng(6)
+    xs = [r.standard_normal((2,) + s).astype(np.float32) for s in shapes]
+    rank = len(shapes[0])
+    a = axis + rank + 1 if axis < 0 else axis
+    assert np.array_equal(fdx.concat(xs, axis), np.concatenate(xs, axis=a))
+
+
+@pytest.mark.parametrize("shape,axes", [((6, 7, 8), [-1]), ((6, 7, 8), [1]), ((6, 7, 8), [2]), ((6, 7, 8), [1, 3]),
+                                        ((6, 7, 8), [2, 3]), ((6, 7, 8), [1, 2, 3]), ((5, 300), [1]), ((3, 4, 5, 6), [2, 4]),
+                                        ((9,), [1]), ((6, 1, 8), [1, 3])])
+def test_layernorm_axes(fdx, oracle, shape, axes):
+    say("layernorm_axes", shape, axes)
+    r = np.random.default_rng(7)
+    x = (r.standard_normal((3,) + shape) * 2 + 1).astype(np.float32)
+    rank = len(shape)
+    n = int(np.prod([shape[(a + rank + 1 if a < 0 else a) - 1] for a in axes]))
+    g, b = r.standard_normal(n).astype(np.float32), r.standard_normal(n).astype(np.float32)
+    for gamma, beta in ((g, b), (None, None)):
+        want = np.stack([oracle.layernorm_axes(x[i], axes, gamma, beta, 1e-3) for i in range(3)])
+        assert rel(fdx.layernorm_axes(x, axes, gamma, beta, 1e-3), want) <= TOL
+
+
+def mixed_model(modelgen, seed=21):
+    """EinsumDense in GEMM form and in permuted form, Concatenate, broadcasting Add, LayerNormalization over the
+    sequence axis, and a nested Functional model applied to two different tensors (shared weights)."""
+    inner = modelgen.Builder("inner_block", seed + 1)
+    u = inner.input((6, 16), "inner_in")
+    h = inner.dense(u, 24, "inner_fc1", activation="relu", bias_std=0.2)
+    h2 = inner.dense(h, 16, "inner_fc2", bias_std=0.2)
+    inner_spec = inner.finish([inner.add([h2, u], "inner_add"), h])
+
+    b = modelgen.Builder("mixed", seed)
+    x = b.input((6, 16), "tokens")
+    gate = b.input((1, 16), "gate")
+    e1 = b.einsum_dense(x, "abc,cde->abde", (16, 2, 8), "proj_heads", bias_axes="ed")     # one GEMM
+    e2 = b.einsum_dense(e1, "abde,dec->abc", (2, 8, 16), "merge_heads", bias_axes="c", activation="gelu")
+    e3 = b.einsum_dense(x, "abc,cd->adb", (16, 5), "permuted", bias_axes="d")               # (5, 6): strided kernel
+    n1, side = b.nested(inner_spec, [e2], "shared_block")
+    s = b.add([n1, gate], "gated")                                                            # (6,16) + (1,16)
+    ln = b.layernorm_axes(s, "ln_seq", [1], eps=1e-3)                                         # over the sequence axis
+    cat = b.concatenate([ln, x, side], "cat", axis=-1)                                        # (6, 16+16+24)
+    out = b.dense(cat, 10, "head", activation="softmax")
+    return b.finish([out, e3, cat])
+
+
+def test_model_with_einsum_concat_broadcast_nested(fdx, oracle, modelgen):
+    say("mixed model")
+    spec = mixed_model(modelgen)
+    r = np.random.default_rng(3)
+    x = r.standard_normal((5, 6, 16)).astype(np.float32)
+    gate = r.standard_normal((5, 1, 16)).astype(np.float32)
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([x[i], gate[i]]) for i in range(5)]
+    want = [np.stack([w[k] for w in want]) for k in range(3)]
+    got = fdx.Model(js).predict([x, gate])
+    errs = [rel(g, w) for g, w in zip(got, want)]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= TOL
+
+
+def test_nested_model_applied_twice(fdx, oracle, modelgen):
+    """The same nested model called on two tensors: both calls read one set of parameters; the second call is
+    Keras node 2 of the nested layer."""
+    say("nested twice")
+    inner = modelgen.Builder("tower", 31)
+    u = inner.input((8, 8, 4), "tower_in")
+    c = inner.conv2d(u, 8, 3, "tower_conv", padding="same", activation="relu", bias_std=0.1)
+    bn = inner.batchnorm(c, "tower_bn", random_stats=True)
+    inner_spec = inner.finish([inner.gap(bn, "tower_gap")])
+
+    b = modelgen.Builder("siamese", 30)
+    xa, xb = b.input((8, 8, 4), "left"), b.input((8, 8, 4), "right")
+    (fa,) = b.nested(inner_spec, [xa], "tower")
+    # second application of the same layer: one more inbound node, referenced as node 2
+    b.layers[-1]["inbound_nodes"].append({"args": [modelgen._kt(xb)], "kwargs": {}})
+    fb = modelgen.T("tower", fa.shape)
+    fb.node, fb.tensor = 2, 0
+    out = b.dense(b.concatenate([fa, fb], "both", axis=-1), 3, "cmp", bias_std=0.1)
+    spec = b.finish([out])
+    r = np.random.default_rng(4)
+    xs = [r.standard_normal((4, 8, 8, 4)).astype(np.float32) for _ in range(2)]
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = np.stack([ref.predict([xs[0][i], xs[1][i]])[0] for i in range(4)])
+    got = fdx.Model(js).predict(xs)[0]
+    assert rel(got, want) <= TOL
+    # swapping the two inputs swaps the halves the head sees: a shared tower gives f(left) == f(right) on equal inputs
+    same = fdx.Model(js).predict([xs[0], xs[0]])[0]
+    ref_same = np.stack([ref.predict([xs[0][i], xs[0][i]])[0] for i in range(4)])
+    assert rel(same, ref_same) <= TOL

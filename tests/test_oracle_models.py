@@ -1,0 +1,165 @@
+"""CPU checks that pin the model-level parts of the oracle without the reference: the file format
+(base64 chunks, connection forms, parameter prefixes of nested models), the definition of causal
+attention by the prefix identity against torch's scaled_dot_product_attention(is_causal=True),
+BatchNormalization against its folded form, LayerNormalization over arbitrary axes against a
+float64 numpy statement, and the graph walk (nested model == the same layers written inline)."""
+import base64
+import json
+
+import numpy as np
+import pytest
+import torch
+
+
+def rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def test_base64_chunks_match_stdlib(oracle, modelgen):
+    r = np.random.default_rng(0)
+    for n in (1, 2, 3, 191, 192, 193, 1000):
+        v = r.standard_normal(n).astype(np.float32)
+        chunks = modelgen.encode_floats(v)
+        assert all(len(c) <= 1024 for c in chunks)
+        # 1024 characters hold exactly 768 bytes = 192 floats, so every chunk decodes on its own
+        assert b"".join(base64.b64decode(c) for c in chunks) == v.astype("<f4").tobytes()
+        assert np.array_equal(oracle.decode_floats(chunks), v)
+    # url-safe alphabet and plain number arrays are accepted too (base64.hpp:65-108, import_model.hpp:274-297)
+    v = np.frombuffer(bytes([0xfb, 0xff, 0xbf, 0x3f]), "<f4")
+    std = base64.b64encode(v.tobytes()).decode()
+    assert "+" in std or "/" in std
+    assert np.array_equal(oracle.decode_floats([std.replace("+", "-").replace("/", "_")]), v)
+    assert np.array_equal(oracle.decode_floats([1.5, -2.0]), np.array([1.5, -2.0], np.float32))
+    with pytest.raises(RuntimeError):
+        oracle.decode_floats([base64.b64encode(b"abc").decode()])
+
+
+def test_single_connection_may_be_a_flat_triple(oracle, modelgen):
+    spec = modelgen.small_cnn()
+    x = np.random.default_rng(1).uniform(-1, 1, (32, 32, 3)).astype(np.float32)
+    want = oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0]
+    cfg = spec["architecture"]["config"]
+    cfg["input_layers"] = cfg["input_layers"][0]
+    cfg["output_layers"] = cfg["output_layers"][0]
+    got = oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0]
+    assert np.array_equal(got, want)
+
+
+def test_causal_prefix_identity_equals_sdpa_is_causal(oracle, modelgen):
+    """Row t of causal self-attention is MHA(query = x[t:t+1], value = x[0:t+1]); with identity-like projections
+    removed this must be torch's causal SDPA on the projected tensors."""
+    b = modelgen.Builder("causal_probe", 9)
+    T, D, H, dk = 9, 16, 2, 8
+    x_in = b.input((T, D), "x")
+    out = b.mha(x_in, x_in, "attn", heads=H, key_dim=dk, std=0.3, bias_std=0.2)
+    spec = b.finish([out])
+    x = np.random.default_rng(2).standard_normal((T, D)).astype(np.float32)
+    got = oracle.OracleModel(modelgen.dumps(spec)).predict([x], causal=True)[0]
+    w = [np.asarray(v, np.float64) for v in spec["trainable_params"]["attn"]["weights"]]
+    qw, qb, kw, kb, vw, vb, ow, ob = w
+    X = x.astype(np.float64)
+    q = np.einsum("td,dhk->htk", X, qw) + qb[:, None, :]
+    k = np.einsum("td,dhk->htk", X, kw) + kb[:, None, :]
+    v = np.einsum("td,dhk->htk", X, vw) + vb[:, None, :]
+    o = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v),
+                                                         is_causal=True).numpy()
+    want = np.einsum("htk,hkd->td", o, ow) + ob
+    assert rel(got, want) <= 2e-6
+    # and without the flag the same file is the reference's unmasked attention
+    o = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v)).numpy()
+    assert rel(oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0], np.einsum("htk,hkd->td", o, ow) + ob) <= 2e-6
+
+
+def test_batchnorm_equals_folded_convolution(oracle, modelgen):
+    """conv -> BN equals a convolution with W' = W * inv[n], b' = b * inv + beta - mean * inv (the load-time fold
+    the GPU path applies), to 1e-6."""
+    b = modelgen.Builder("bn_probe", 12)
+    x_in = b.input((9, 9, 5), "x")
+    c = b.conv2d(x_in, 7, 3, "conv", padding="same", bias_std=0.3)
+    spec = b.finish([b.batchnorm(c, "bn", random_stats=True)])
+    x = np.random.default_rng(3).standard_normal((9, 9, 5)).astype(np.float32)
+    want = oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0]
+    p = spec["trainable_params"]
+    eps = [l for l in spec["architecture"]["config"]["layers"] if l["name"] == "bn"][0]["config"]["epsilon"]
+    inv = p["bn"]["gamma"].astype(np.float64) / np.sqrt(p["bn"]["moving_variance"].astype(np.float64) + eps)
+    w = p["conv"]["weights"].reshape(7, 3, 3, 5).astype(np.float64) * inv[:, None, None, None]
+    bias = p["conv"]["bias"].astype(np.float64) * inv + p["bn"]["beta"] - p["bn"]["moving_mean"] * inv
+    xt = torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None]
+    y = torch.nn.functional.conv2d(xt, torch.from_numpy(w).permute(0, 3, 1, 2), torch.from_numpy(bias), padding=1)
+    assert rel(want, y[0].permute(1, 2, 0).numpy()) <= 1e-6
+
+
+@pytest.mark.parametrize("shape,axes", [((6, 7, 8), [-1]), ((6, 7, 8), [1]), ((6, 7, 8), [1, 3]), ((6, 7, 8), [2, 3]),
+                                        ((3, 4, 5, 6), [2, 4]), ((6, 7, 8), [1, 2, 3])])
+def test_layernorm_axes_vs_float64(oracle, shape, axes):
+    r = np.random.default_rng(4)
+    x = (r.standard_normal(shape) * 3 + 2).astype(np.float32)
+    rank = len(shape)
+    pos = sorted(a + rank + 1 if a < 0 else a for a in axes)
+    pshape = [shape[a - 1] if a in pos else 1 for a in range(1, rank + 1)]
+    n = int(np.prod(pshape))
+    g, b = r.standard_normal(n).astype(np.float32), r.standard_normal(n).astype(np.float32)
+    X = x.astype(np.float64)
+    ax = tuple(a - 1 for a in pos)
+    mean, var = X.mean(ax, keepdims=True), X.var(ax, keepdims=True)  # biased variance
+    want = (X - mean) / np.sqrt(var + 1e-3) * g.reshape(pshape) + b.reshape(pshape)
+    assert rel(oracle.layernorm_axes(x, axes, g, b, 1e-3), want) <= 2e-6
+    if pos == list(range(rank - len(pos) + 1, rank + 1)):  # trailing axes: torch's layer_norm is the same formula
+        t = torch.nn.functional.layer_norm(torch.from_numpy(X), [shape[a - 1] for a in pos],
+                                           torch.from_numpy(g.astype(np.float64)).reshape([shape[a - 1] for a in pos]),
+                                           torch.from_numpy(b.astype(np.float64)).reshape([shape[a - 1] for a in pos]), 1e-3)
+        assert rel(oracle.layernorm_axes(x, axes, g, b, 1e-3), t.numpy()) <= 2e-6
+
+
+def test_nested_model_equals_inline_layers(oracle, modelgen):
+    """A Functional model used as a layer computes what its layers compute when written into the outer model, and
+    reads its parameters under "<layer>_<inner layer>"."""
+    def body(b, x, prefix):
+        h = b.dense(x, 12, prefix + "fc1", activation="relu", bias_std=0.2)
+        return b.add([b.dense(h, 8, prefix + "fc2", bias_std=0.2), x], prefix + "res")
+
+    inner = modelgen.Builder("blk", 5)
+    inner_out = body(inner, inner.input((4, 8), "blk_in"), "")
+    inner_spec = inner.finish([inner_out])
+
+    outer = modelgen.Builder("outer", 6)
+    x_in = outer.input((4, 8), "x")
+    (y,) = outer.nested(inner_spec, [x_in], "blk")
+    spec_nested = outer.finish([outer.dense(y, 3, "head", bias_std=0.1)])
+    assert "blk_fc1" in spec_nested["trainable_params"] and "fc1" not in spec_nested["trainable_params"]
+
+    flat = modelgen.Builder("outer", 6)
+    xf = flat.input((4, 8), "x")
+    yf = body(flat, xf, "blk_")
+    spec_flat = flat.finish([flat.dense(yf, 3, "head", bias_std=0.1)])
+    for name, prm in spec_nested["trainable_params"].items():  # same numbers under the same names
+        spec_flat["trainable_params"][name] = prm
+    x = np.random.default_rng(7).standard_normal((4, 8)).astype(np.float32)
+    a = oracle.OracleModel(modelgen.dumps(spec_nested)).predict([x])[0]
+    b = oracle.OracleModel(modelgen.dumps(spec_flat)).predict([x])[0]
+    assert np.array_equal(a, b)
+
+
+def test_concatenate_axis_counts_from_first_rank(oracle, modelgen):
+    b = modelgen.Builder("cat_probe", 8)
+    p, q = b.input((3, 4), "p"), b.input((3, 2), "q")
+    spec = b.finish([b.concatenate([p, q], "cat", axis=2), b.concatenate([p, p], "cat0", axis=1)])
+    r = np.random.default_rng(8)
+    xp, xq = r.standard_normal((3, 4)).astype(np.float32), r.standard_normal((3, 2)).astype(np.float32)
+    a, c = oracle.OracleModel(modelgen.dumps(spec)).predict([xp, xq])
+    assert np.array_equal(a, np.concatenate([xp, xq], axis=1)) and np.array_equal(c, np.concatenate([xp, xp], axis=0))
+
+
+def test_embedded_tests_replay_and_detect_corruption(oracle, modelgen):
+    spec = modelgen.small_cnn()
+    x = np.random.default_rng(9).uniform(-1, 1, (32, 32, 3)).astype(np.float32)
+    y = oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0]
+    spec["tests"] = [{"inputs": [x], "outputs": [y]}]
+    assert oracle.OracleModel(modelgen.dumps(spec)).run_embedded_tests()
+    spec["tests"] = [{"inputs": [x], "outputs": [y + 1e-3]}]
+    with pytest.raises(RuntimeError, match="test failed"):
+        oracle.OracleModel(modelgen.dumps(spec)).run_embedded_tests()
+    # the file is plain JSON
+    assert json.loads(modelgen.dumps(spec))["image_data_format"] == "channels_last"
