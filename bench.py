@@ -206,6 +206,57 @@ def bench_gpt2(fdx, modelgen, args):
     return out
 
 
+def bench_gpt2_kernels(fdx, args):
+    """The decode step's dominant kernel (the weight-streaming Dense for 16 rows) alone, at the five GEMM shapes of
+    a GPT-2-small block, each against a ring of weight copies larger than the caches so every launch streams
+    from HBM.  Used for per-kernel roofline figures and counter runs; not part of the headline metric."""
+    m, reps = 16, max(4, args.steps)
+    shapes = [("qkv (LayerNorm folded)", 768, 2304, True, False), ("attention output + residual", 768, 768, False, True),
+              ("mlp fc (LayerNorm folded, gelu)", 768, 3072, True, False), ("mlp proj + residual", 3072, 768, False, True),
+              ("lm head (LayerNorm folded)", 768, 50257, True, False)]
+    rng = np.random.default_rng(5)
+    out = []
+    ms = ctypes.c_float()
+    for name, k, n, ln, res in shapes:
+        copies = max(2, int(600e6 // (4 * k * n)))
+        w = fdx.DevBuf(4 * k * n * copies)
+        host = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+        for c in range(copies):
+            fdx.check(fdx.lib.fdx_h2d(ctypes.c_void_p(w.ptr.value + 4 * k * n * c), host.ctypes.data_as(ctypes.c_void_p),
+                                      ctypes.c_size_t(host.nbytes)))
+        x = fdx.DevBuf.from_host(rng.standard_normal((m, k)).astype(np.float32))
+        bias = fdx.DevBuf.from_host(rng.standard_normal(n).astype(np.float32))
+        rsum = fdx.DevBuf.from_host(host.sum(1).astype(np.float32))
+        r = fdx.DevBuf.from_host(rng.standard_normal((m, n)).astype(np.float32)) if res else None
+        y = fdx.DevBuf(4 * m * n)
+        f32p = ctypes.POINTER(ctypes.c_float)
+
+        def launch(c):
+            wp = ctypes.cast(ctypes.c_void_p(w.ptr.value + 4 * k * n * c), f32p)
+            if ln:
+                fdx.check(fdx.lib.fdx_layernorm_dense_rows_f32(fdx._dp(x), m, k, ctypes.c_float(1e-5), wp, fdx._dp(rsum),
+                                                               fdx._dp(bias), n, None, None, fdx._dp(y)))
+            else:
+                fdx.check(fdx.lib.fdx_dense_rows_f32(fdx._dp(x), m, k, wp, fdx._dp(bias), n, fdx._dp(r), None, fdx._dp(y)))
+
+        for c in range(copies):
+            launch(c)
+        fdx.sync()
+        fdx.check(fdx.lib.fdx_timer_start())
+        for i in range(reps * copies):
+            launch(i % copies)
+        fdx.check(fdx.lib.fdx_timer_stop(ctypes.byref(ms)))
+        us = ms.value * 1e3 / (reps * copies)
+        nbytes = 4.0 * (k * n + n + m * k + m * n * (2 if res else 1))
+        out.append({"shape": name, "rows": m, "k": k, "n": n, "us_per_launch_back_to_back": round(us, 2),
+                    "algorithmic_bytes": int(nbytes), "GB_per_s": round(nbytes / us / 1e3, 1),
+                    "hbm_frac": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4)})
+        for b in (w, x, bias, rsum, y) + ((r,) if r else ()):
+            b.free()
+    return {"metric": "decode Dense kernel, 16 rows, weights streamed from HBM", "unit": "us per launch",
+            "n_gpus": 1, "kernels": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -213,16 +264,28 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--decode-reps", type=int, default=2)
-    ap.add_argument("--workload", choices=["all", "resnet50", "gpt2"], default="all")
+    ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels"], default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="also launch one plain device copy (act_kernel, no activation) of this many MiB, whose known "
+                         "traffic scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (samples are independent; more GPUs would each take a "
                  "slice of the batch with their own copy of the weights) -- use --gpus 1")
     fdx, modelgen = load_package()
+    if args.calibrate_copy_mib > 0:
+        n = args.calibrate_copy_mib * (1 << 20) // 4
+        src, dst = fdx.DevBuf(4 * n), fdx.DevBuf(4 * n)
+        fdx.check(fdx.lib.fdx_activation_f32(fdx._dp(src), ctypes.c_size_t(n), None, fdx._dp(dst)))
+        fdx.sync()
+        src.free()
+        dst.free()
     result = {}
     if args.workload in ("all", "resnet50"):
         result = bench_resnet(fdx, modelgen, args)
+    if args.workload == "gpt2_kernels":
+        result = bench_gpt2_kernels(fdx, args)
     if args.workload in ("all", "gpt2"):
         g = bench_gpt2(fdx, modelgen, args)
         if result:
