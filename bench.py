@@ -26,6 +26,10 @@ for _p in (ROOT, os.path.join(ROOT, "oracle")):
 
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
+# of this file and scaled by a plain copy of known size (a process cannot read these counters for itself; the
+# summaries under profiles/ give the commands and the raw readings).  Valid for the default configurations only.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 136.6e6, "skinny_gemm, GPT-2 decode b16": 10.9e6}
 
 
 def load_package():
@@ -134,7 +138,7 @@ def bench_resnet(fdx, modelgen, args):
             "flops_per_launch": round(mf_flops / max(mf_launches, 1), 1),
             "avg_launch_ms": round(mf_ms / max(mf_launches, 1), 5),
             "share_of_step_time": round(mf_ms / total_ms, 4) if total_ms else None,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["igemm, ResNet50 b64"] if batch == 64 else None,
         },
         "kernel_ms_per_step": {k: round(v["ms"] / prof_steps, 4) for k, v in sorted(fams.items())},
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
@@ -198,7 +202,8 @@ def bench_gpt2(fdx, modelgen, args):
         "prefill_ms": round(prefill_ms, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4), "bytes_per_step_mean": round(total_bytes / new),
-                     "traffic": None},
+                     "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 49 of the step's 64 launches)",
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
         "load_seconds": round(load_s, 2),
     }
     sess.close()

@@ -195,6 +195,8 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
         float* part = p.workspace + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256;
         if (t < 256)
             __hip_atomic_store(part + t, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // every lane's partials have left the CU before the ticket is taken
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (t == 0) {

@@ -303,12 +303,63 @@ static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStrea
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-static void launch_fast(int cfg, const GemmParams& q, bool conv, int batch, hipStream_t s)
+// library-owned scratch of the split-K variant: partial tiles and one ticket per output tile
+// (tickets are zero between launches: the last unit of a tile resets its ticket)
+static float* g_split_ws = nullptr;
+static int* g_split_tickets = nullptr;
+constexpr size_t kSplitWsBytes = 192u << 20;
+constexpr int kSplitTickets = 1 << 16;
+
+static bool split_prepare()
 {
+    if (g_split_ws && g_split_tickets)
+        return true;
+    if (hipMalloc(&g_split_ws, kSplitWsBytes) != hipSuccess)
+        return false;
+    if (hipMalloc(&g_split_tickets, sizeof(int) * kSplitTickets) != hipSuccess
+        || hipMemset(g_split_tickets, 0, sizeof(int) * kSplitTickets) != hipSuccess)
+        return false;
+    return true;
+}
+
+static void tile_of(int cfg, int& bm, int& bn, int& bk)
+{
+    switch (cfg) {
+    case 10: bm = 128; bn = 128; bk = 16; break;
+    case 11: bm = 128; bn = 64; bk = 16; break;
+    case 12: bm = 64; bn = 64; bk = 16; break;
+    case 13: bm = 128; bn = 128; bk = 32; break;
+    case 14: bm = 128; bn = 64; bk = 32; break;
+    default: bm = 64; bn = 64; bk = 32; break;
+    }
+}
+
+// whether `splits` K ranges per tile are possible for this configuration: enough slabs per range, and the
+// partial tiles and tickets fit the scratch
+static bool split_fits(int cfg, int splits, const GemmParams& q, int batch)
+{
+    int bm, bn, bk;
+    tile_of(cfg, bm, bn, bk);
+    const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
+    return splits >= 2 && q.K / bk >= 2 * splits && tiles <= kSplitTickets
+        && (size_t)tiles * splits * bm * bn * sizeof(float) <= kSplitWsBytes && tiles * splits < (1 << 30);
+}
+
+static void launch_fast(int cfg, int splits, const GemmParams& q0, bool conv, int batch, hipStream_t s)
+{
+    GemmParams q = q0;
+    q.splits = splits;
+    q.split_ws = g_split_ws;
+    q.split_tickets = g_split_tickets;
 #define FDX_FAST(BM_, BN_, BK_)                                                                                  \
     {                                                                                                            \
         const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
-        if (conv)                                                                                                \
+        if (splits > 1) {                                                                                        \
+            if (conv)                                                                                            \
+                launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles * splits, q, s);     \
+            else                                                                                                 \
+                launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles * splits, q, s);    \
+        } else if (conv)                                                                                         \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s);                        \
         else                                                                                                     \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s);                       \
@@ -327,18 +378,23 @@ static void launch_fast(int cfg, const GemmParams& q, bool conv, int batch, hipS
 // First sight of a problem shape on the fast path: time every tile configuration once on the
 // real operands (the launches are idempotent) and remember the winner.  Tile count versus
 // resident workgroups, K depth and output width interact too irregularly for a closed rule.
+// A choice is (configuration, K splits) packed as cfg + 100 * splits; splits are tried only where
+// a configuration has few tiles for the chip.
 struct TuneKey {
     int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
     bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }
 };
 static std::map<TuneKey, int> g_tuned;
 static int g_autotune = -1;
+static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range per tile
 
 static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s)
 {
     if (g_autotune < 0) {
         const char* e = std::getenv("FDX_AUTOTUNE");
         g_autotune = (e && e[0] == '0') ? 0 : 1;
+        const char* sp = std::getenv("FDX_SPLITK");
+        g_split_enabled = (sp && sp[0] == '0') ? 0 : 1;
     }
     if (!g_autotune)
         return -1;
@@ -354,20 +410,28 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
         return -1;
     int best = -1;
     float best_ms = 1e30f;
+    const bool can_split = g_split_enabled && split_prepare();
     for (int cfg = 10; cfg <= 15; ++cfg) {
         if (cfg >= 13 && unit % 32 != 0)
             continue;
-        launch_fast(cfg, q, conv, batch, s); // warm-up
-        (void)hipEventRecord(a, s);
-        for (int r = 0; r < 3; ++r)
-            launch_fast(cfg, q, conv, batch, s);
-        (void)hipEventRecord(b, s);
-        float ms = 1e30f;
-        if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
-            continue;
-        if (ms < best_ms) {
-            best_ms = ms;
-            best = cfg;
+        int bm, bn, bk;
+        tile_of(cfg, bm, bn, bk);
+        const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
+        for (int splits = 1; splits <= 4; ++splits) {
+            if (splits > 1 && !(can_split && tiles <= 1024 && split_fits(cfg, splits, q, batch)))
+                continue;
+            launch_fast(cfg, splits, q, conv, batch, s); // warm-up
+            (void)hipEventRecord(a, s);
+            for (int r = 0; r < 3; ++r)
+                launch_fast(cfg, splits, q, conv, batch, s);
+            (void)hipEventRecord(b, s);
+            float ms = 1e30f;
+            if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
+                continue;
+            if (ms < best_ms) {
+                best_ms = ms;
+                best = cfg + 100 * splits;
+            }
         }
     }
     (void)hipEventDestroy(a);
@@ -407,9 +471,20 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
     const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31);
     const int unit = conv ? p.Cin : p.K;
 
-    int cfg = g_forced_tile;
+    int cfg = g_forced_tile, splits = 1;
+    if (cfg >= 100) { // tests: configuration + 100 * splits
+        splits = cfg / 100;
+        cfg %= 100;
+    }
     if (cfg >= 10 && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
         cfg = -1;
+    if (cfg < 10)
+        splits = 1;
+    if (cfg >= 10 && splits > 1) {
+        GemmParams q = p;
+        if (!split_prepare() || !split_fits(cfg, splits, q, batch))
+            splits = 1;
+    }
     if (cfg < 0) {
         if (fast_ok && p.N >= 64 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
             GemmParams q = p;
@@ -418,6 +493,10 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             q.b_records = (uint32_t)b_bytes;
             q.batch = batch;
             cfg = autotune(q, conv, batch, unit, s);
+            if (cfg >= 100) {
+                splits = cfg / 100;
+                cfg %= 100;
+            }
         }
         if (cfg >= 10) {
         } else if (fast_ok && p.N >= 64) {
@@ -447,7 +526,7 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         q.a_records = (uint32_t)a_bytes;
         q.b_records = (uint32_t)b_bytes;
         q.batch = batch;
-        launch_fast(cfg, q, conv, batch, s);
+        launch_fast(cfg, splits, q, conv, batch, s);
     } else {
         switch (cfg) {
         case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;

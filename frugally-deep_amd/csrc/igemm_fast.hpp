@@ -17,9 +17,15 @@
 //    their epilogue together and the matrix cores idle while HBM drains).
 //  * The epilogue goes through LDS so that bias, residual and output move as 16-byte
 //    accesses along the channel axis.
+//  * SPLIT: a layer with too few output tiles for the chip (late stages of a CNN at small
+//    batch) cuts every tile's K range into `splits` units.  A unit leaves its accumulators in a
+//    workspace and takes a ticket on the tile; the last unit to arrive adds all partial tiles
+//    in split order (so the sum does not depend on arrival order) and runs the epilogue.
+//    Nothing waits on another workgroup.  Partials are written and read with agent-scope
+//    accesses, which pass the per-XCD L2s, instead of a fence that writes a whole L2 back.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false>
 __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
 {
     constexpr int NT = 256;
@@ -36,6 +42,7 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
     constexpr uint32_t OOB = 0x80000000u; // beyond any extent this path accepts: the load returns zeros
 
     __shared__ __attribute__((aligned(16))) float smem[2 * (BM + BN) * STRIDE];
+    __shared__ int last_flag;
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -44,7 +51,8 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
 
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     const int per_problem = tiles_m * tiles_n;
-    const int total = per_problem * p.batch;
+    const int S = SPLIT ? p.splits : 1;
+    const int total = per_problem * p.batch * S; // units: (tile, K range)
     // XCD x (workgroups with blockIdx % 8 == x) owns the contiguous tile range [lo, hi) so tiles
     // that share an A row block also share that XCD's L2; its workgroups stride through it.
     const int xcd = blockIdx.x & 7, wg_in_xcd = blockIdx.x >> 3;
@@ -58,8 +66,11 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
     __amdgpu_buffer_rsrc_t srd_a, srd_b;
     int tap, fx, fy, c0, soff_a, soff_b;
     f32x4 ra[A_LOADS], rb[B_LOADS];
+    const int KT = p.K / BKT;
+    int kt_n = KT; // slabs of the current unit
 
-    auto setup = [&](int tile, int& m0, int& n0, int64_t& c_off) {
+    auto setup = [&](int unit, int& m0, int& n0, int64_t& c_off) {
+        const int tile = SPLIT ? unit / S : unit, split = SPLIT ? unit - tile * S : 0;
         const int z = tile / per_problem, id = tile - z * per_problem;
         m0 = (id / tiles_n) * BM;
         n0 = (id % tiles_n) * BN;
@@ -103,6 +114,21 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
         }
         tap = fx = fy = c0 = 0;
         soff_a = soff_b = 0;
+        if (SPLIT) {
+            const int kt_lo = (int)((int64_t)split * KT / S);
+            kt_n = (int)((int64_t)(split + 1) * KT / S) - kt_lo;
+            const int k_start = kt_lo * BKT;
+            soff_b = k_start * 4;
+            if (CONV) {
+                tap = k_start / p.Cin;
+                c0 = k_start - tap * p.Cin;
+                fy = tap / p.kw;
+                fx = tap - fy * p.kw;
+                soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.Cin + c0) * 4;
+            } else {
+                soff_a = k_start * 4;
+            }
+        }
     };
     auto load_tiles = [&]() {
 #pragma unroll
@@ -140,7 +166,6 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
             *reinterpret_cast<f32x4*>(&bs[(r0 + i * RPP) * STRIDE + kq * 4]) = rb[i];
     };
 
-    const int KT = p.K / BKT;
     int tile = lo + wg_in_xcd;
     if (tile >= hi)
         return; // uniform per workgroup
@@ -161,9 +186,10 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
 
         store_tiles(0);
         __syncthreads();
-        for (int kt = 0; kt < KT; ++kt) {
+        const int kt_end = kt_n;
+        for (int kt = 0; kt < kt_end; ++kt) {
             const int buf = kt & 1;
-            if (kt + 1 < KT)
+            if (kt + 1 < kt_end)
                 load_tiles();
             const float* as = smem + buf * (BM + BN) * STRIDE;
             const float* bs = as + BM * STRIDE;
@@ -184,7 +210,7 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
                         for (int j = 0; j < TN; ++j)
                             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
             }
-            if (kt + 1 < KT)
+            if (kt + 1 < kt_end)
                 store_tiles(buf ^ 1);
             __syncthreads();
         }
@@ -193,11 +219,65 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
         const int em0 = m0, en0 = n0;
         float* __restrict__ C = p.C + c_off;
         const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
+        const int unit_done = tile;
         tile += wgs_in_xcd;
         const bool more = tile < hi;
         if (more) {
             setup(tile, m0, n0, c_off);
             load_tiles(); // in flight while this tile is written out
+        }
+
+        if (SPLIT && S > 1) {
+            constexpr int TILE_F = BM * BN;
+            const int out_tile = unit_done / S, my_split = unit_done - out_tile * S;
+            float* mine = p.split_ws + (int64_t)unit_done * TILE_F + t;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        __hip_atomic_store(mine + ((i * TN + j) * 16 + e) * NT, acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // every lane's partials have left the CU before the ticket is taken
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (t == 0) {
+                const int ticket = __hip_atomic_fetch_add(p.split_tickets + out_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int last = ticket == S - 1;
+                if (last)
+                    __hip_atomic_store(p.split_tickets + out_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // next launch
+                last_flag = last;
+            }
+            __syncthreads();
+            const bool is_last = last_flag != 0;
+            __syncthreads(); // last_flag is rewritten by the next unit
+            if (!is_last) {
+                if (!more)
+                    break;
+                continue;
+            }
+            f32x16 own[TM][TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    own[i][j] = acc[i][j];
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        acc[i][j][e] = 0.f;
+                }
+            for (int sp = 0; sp < S; ++sp) {
+                const float* part = p.split_ws + ((int64_t)out_tile * S + sp) * TILE_F + t;
+                const bool self = sp == my_split;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            acc[i][j][e] += self ? own[i][j][e]
+                                                 : __hip_atomic_load(part + ((i * TN + j) * 16 + e) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
 
         // ---- epilogue: accumulators -> per-wave LDS scratch [32][WTN] -> 16-byte row accesses

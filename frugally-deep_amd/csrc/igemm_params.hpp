@@ -25,6 +25,10 @@ struct GemmParams {
     // fast path only: byte extents of one problem's A (counted from the shifted base) and B operands
     uint32_t a_records, b_records;
     int batch; // number of independent problems folded into the persistent tile walk
+    // split-K variant of the fast path: K ranges per tile, partial-tile workspace, one ticket per tile (zero between launches)
+    int splits;
+    float* split_ws;
+    int* split_tickets;
 };
 
 

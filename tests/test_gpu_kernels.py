@@ -331,3 +331,55 @@ def test_layernorm_dense_rows_folded(fdx, oracle, m, k, n):
                                                    fdx._dp(bf), n, None, None, fdx._dp(out)))
     want = oracle.dense(oracle.layernorm(x, None, None, 1e-3), np.ascontiguousarray(w.T).reshape(-1), None, n)
     assert rel(out.to_host((m, n)), want) <= TOL
+
+
+SPLIT_CASES = [
+    # n, h, w, cin, cout, kh, kw, strides, padding
+    (2, 7, 7, 64, 64, 3, 3, (1, 1), "same"),     # K = 576: 3x3 taps cut inside a tap's channels
+    (3, 14, 14, 48, 96, 3, 3, (1, 1), "same"),   # cin a multiple of 16 only: BK 16 configurations
+    (2, 7, 7, 512, 128, 1, 1, (1, 1), "valid"),  # pointwise: plain GEMM path, K = 512
+    (1, 9, 9, 32, 40, 5, 5, (2, 2), "same"),     # strided, ragged M and N
+]
+
+
+@pytest.mark.parametrize("tile", [210, 310, 211, 412, 213, 314, 215, 415])
+@pytest.mark.parametrize("case", SPLIT_CASES)
+def test_conv2d_split_k(fdx, oracle, case, tile):
+    """The K range of every output tile cut into 2..4 units whose partial tiles the last arriving workgroup adds
+    (forced: configuration + 100 * splits); twice in a row, so the tickets must have been reset; with a residual and
+    ReLU in the epilogue, which only the adding workgroup may apply."""
+    n, h, w, cin, cout, kh, kw, strides, padding = case
+    say("conv2d split-K", case, "tile", tile)
+    r = rng_for("conv-split", case)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, kh, kw, cin)) / np.sqrt(kh * kw * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, kh, kw, cin)
+    conv = np.stack([oracle.conv2d(x[i], wo, b, cout, kh, kw, strides, (1, 1), padding) for i in range(n)])
+    res = r.standard_normal(conv.shape).astype(np.float32)
+    want = oracle.relu(oracle.add(res, conv))
+    fdx.lib.fdx_debug_force_tile(tile)
+    try:
+        first = fdx.conv2d(x, wj, b, strides, (1, 1), padding, residual=res, act=fdx.relu_act())
+        second = fdx.conv2d(x, wj, b, strides, (1, 1), padding, residual=res, act=fdx.relu_act())
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(first, want) <= TOL
+    assert np.array_equal(first, second)  # partials are added in split order: the result does not depend on arrival order
+
+
+@pytest.mark.parametrize("tile", [213, 415])
+def test_gemm_split_k_many_tiles(fdx, oracle, tile):
+    say("gemm split-K", tile)
+    r = rng_for("gemm-split", tile)
+    m, n, k = 1000, 384, 2048
+    a = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    b = r.standard_normal(n).astype(np.float32)
+    want = oracle.gelu(oracle.dense(a, w.reshape(-1), b, n))
+    fdx.lib.fdx_debug_force_tile(tile)
+    try:
+        got = fdx.gemm(a, w.T, b, act=fdx.gelu_act())
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(got, want) <= TOL
