@@ -49,6 +49,7 @@ def _load():
 
 lib = _load()
 lib.fdx_last_error.restype = ctypes.c_char_p
+lib.fdx_set_last_error.restype = None
 lib.fdx_mha_scratch_bytes.restype = ctypes.c_size_t
 
 
@@ -361,18 +362,93 @@ def mha_decode(q, k_cache, v_cache, heads, dk, dv, length):
 
 # ------------------------------------------------------------------ whole models
 
+_PARAM_GETTER = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_char_p,
+                                 ctypes.POINTER(ctypes.POINTER(ctypes.c_float)), ctypes.POINTER(ctypes.c_size_t))
+_CREATE_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_size_t, _PARAM_GETTER,
+                              ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p))
+_APPLY_FN = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.POINTER(ctypes.c_float)),
+                             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_float),
+                             ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64))
+_DESTROY_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+
+
+class _CustomLayerStruct(ctypes.Structure):
+    _fields_ = [("class_name", ctypes.c_char_p), ("create", _CREATE_FN), ("apply", _APPLY_FN), ("destroy", _DESTROY_FN),
+                ("user", ctypes.c_void_p)]
+
+
+class _CustomLayers:
+    """ctypes glue for fdx_custom_layer: `creators` maps a class name to creator(get_param, layer_dict, name) -> callable
+    that takes the list of input arrays (no batch axis) and returns one array."""
+
+    def __init__(self, creators):
+        import json as _json
+        self.instances = {}
+        self.keep = []
+        self.errors = []
+        structs = []
+        for cls_name, creator in creators.items():
+            def create(user, lname, cfg, cfg_len, getter, gctx, inst, creator=creator):
+                try:
+                    def get_param(layer, key):
+                        vals, cnt = ctypes.POINTER(ctypes.c_float)(), ctypes.c_size_t()
+                        check(getter(gctx, layer.encode(), key.encode(), ctypes.byref(vals), ctypes.byref(cnt)))
+                        return np.ctypeslib.as_array(vals, (cnt.value,)).copy()
+                    fn = creator(get_param, _json.loads(ctypes.string_at(cfg, cfg_len)), lname.decode())
+                    handle = len(self.instances) + 1
+                    self.instances[handle] = fn
+                    inst[0] = handle
+                    return 0
+                except Exception as e:  # noqa: BLE001 - reported through the status code
+                    self.errors.append(e)
+                    lib.fdx_set_last_error(str(e).encode())
+                    return 1
+
+            def apply(inst, n, ins, ranks, dims5, out, orank, odims):
+                try:
+                    arrs = []
+                    for i in range(n):
+                        shape = tuple(int(dims5[i * 5 + k]) for k in range(5 - ranks[i], 5))
+                        arrs.append(np.ctypeslib.as_array(ins[i], shape).copy())
+                    y = np.ascontiguousarray(self.instances[inst](arrs), np.float32)
+                    orank[0] = y.ndim
+                    for k in range(5):
+                        odims[k] = 1 if k < 5 - y.ndim else y.shape[k - (5 - y.ndim)]
+                    if out:
+                        ctypes.memmove(out, y.ctypes.data, y.nbytes)
+                    return 0
+                except Exception as e:  # noqa: BLE001
+                    self.errors.append(e)
+                    lib.fdx_set_last_error(str(e).encode())
+                    return 1
+
+            def destroy(inst):
+                self.instances.pop(inst, None)
+
+            fns = (_CREATE_FN(create), _APPLY_FN(apply), _DESTROY_FN(destroy))
+            self.keep.append(fns)
+            structs.append(_CustomLayerStruct(cls_name.encode(), fns[0], fns[1], fns[2], None))
+        self.array = (_CustomLayerStruct * len(structs))(*structs)
+        self.count = len(structs)
+
+
 class Model:
     """A converted-JSON model resident on the GPU (fdx_model_*).  `source` is the file's bytes or a path."""
 
-    def __init__(self, source, verify=True, verify_epsilon=1e-4):
+    def __init__(self, source, verify=True, verify_epsilon=1e-4, custom_layers=None):
         if isinstance(source, str):
             if not os.path.exists(source):
                 raise FdxError("Can not open " + source)
             with open(source, "rb") as f:
                 source = f.read()
         self._h = ctypes.c_void_p()
-        check(lib.fdx_model_create(source, ctypes.c_size_t(len(source)), int(verify), ctypes.c_float(verify_epsilon),
-                                   ctypes.byref(self._h)))
+        self._custom = _CustomLayers(custom_layers) if custom_layers else None
+        if self._custom:
+            check(lib.fdx_model_create_custom(source, ctypes.c_size_t(len(source)), int(verify), ctypes.c_float(verify_epsilon),
+                                              self._custom.array, self._custom.count, ctypes.byref(self._h)))
+        else:
+            check(lib.fdx_model_create(source, ctypes.c_size_t(len(source)), int(verify), ctypes.c_float(verify_epsilon),
+                                       ctypes.byref(self._h)))
         ni, no = ctypes.c_int(), ctypes.c_int()
         check(lib.fdx_model_io_count(self._h, ctypes.byref(ni), ctypes.byref(no)))
         self.n_inputs, self.n_outputs = ni.value, no.value

@@ -21,7 +21,7 @@ namespace json {
         enum Type { Null, Bool, Number, String, Array, Object } type = Null;
         bool b = false;
         double num = 0;
-        const char* s = nullptr; // raw string body (still escaped)
+        const char* s = nullptr; // String: raw body (still escaped); Object: the object's own text, braces included
         size_t slen = 0;
         bool has_escape = false;
         std::vector<Value> arr;
@@ -154,11 +154,13 @@ namespace json {
             Value v;
             const char c = *p_;
             if (c == '{') {
+                v.s = p_;
                 ++p_;
                 v.type = Value::Object;
                 ws();
                 if (p_ < end_ && *p_ == '}') {
                     ++p_;
+                    v.slen = (size_t)(p_ - v.s);
                     return v;
                 }
                 for (;;) {
@@ -178,6 +180,7 @@ namespace json {
                     }
                     if (p_ < end_ && *p_ == '}') {
                         ++p_;
+                        v.slen = (size_t)(p_ - v.s);
                         return v;
                     }
                     fail("expected ',' or '}'");

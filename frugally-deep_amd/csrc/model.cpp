@@ -224,6 +224,30 @@ namespace {
         fdx_model& m;
         const Value& params;
         std::vector<std::unique_ptr<Scope>> scopes;
+        const fdx_custom_layer* customs = nullptr;
+        int n_customs = 0;
+
+        // trainable_params lookup handed to a custom layer's factory; the decoded vectors live until it returns
+        struct ParamCtx {
+            Builder* b;
+            const Scope* sc;
+            std::vector<std::vector<float>> keep;
+        };
+        static fdx_status get_param_cb(void* ctx, const char* layer, const char* key, const float** values, size_t* count)
+        {
+            auto* pc = static_cast<ParamCtx*>(ctx);
+            try {
+                pc->keep.push_back(decode_floats(pc->b->param(*pc->sc, layer, key)));
+            } catch (const std::exception& e) {
+                set_error("%s", e.what());
+                return FDX_ERR_FORMAT;
+            }
+            if (values)
+                *values = pc->keep.back().data();
+            if (count)
+                *count = pc->keep.back().size();
+            return FDX_OK;
+        }
 
         const Value& param(const Scope& sc, const std::string& layer, const char* key)
         {
@@ -331,7 +355,24 @@ namespace {
             op.cls = cls;
             op.in = ins;
             int result;
-            if (kIdentity.count(cls)) {
+            const fdx_custom_layer* custom = nullptr;
+            for (int i = 0; i < n_customs && !custom; ++i)
+                if (customs[i].class_name && cls == customs[i].class_name)
+                    custom = &customs[i];
+            if (custom) {
+                // a registered class takes precedence over a built-in one (import_model.hpp:1944-1950)
+                if (!custom->create || !custom->apply)
+                    throw FormatError("custom layer " + cls + " lacks create / apply");
+                op.kind = OpKind::Host;
+                fdx_host_layer hl;
+                hl.vt = *custom;
+                ParamCtx pc { this, &sc, {} };
+                if (custom->create(custom->user, c.layer.c_str(), L.s, L.slen, &Builder::get_param_cb, &pc, &hl.instance) != FDX_OK)
+                    throw FormatError("custom layer " + c.layer + " could not be created: " + fdx_last_error());
+                m.host_layers.push_back(hl);
+                op.host_index = (int)m.host_layers.size() - 1;
+                result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (kIdentity.count(cls)) {
                 op.kind = OpKind::View;
                 result = add_op(std::move(op));
             } else if (cls == "Conv2D" || cls == "Conv1D") {
@@ -918,6 +959,34 @@ namespace {
                 }
                 break;
             }
+            case OpKind::Host: {
+                const fdx_host_layer& hl = m.host_layers[(size_t)o.host_index];
+                std::vector<int> ranks;
+                std::vector<int64_t> dims5;
+                std::vector<const float*> ptrs(o.in.size(), nullptr);
+                std::vector<std::vector<float>> zeros;
+                for (int i : o.in) {
+                    const Shape& s = shapes[i];
+                    FDX_REQUIRE(!s.empty() && s.size() <= 5, "%s: custom layer inputs must have rank 1..5", o.name.c_str());
+                    ranks.push_back((int)s.size());
+                    for (size_t k = 0; k < 5; ++k)
+                        dims5.push_back(k < 5 - s.size() ? 1 : s[k - (5 - s.size())]);
+                    zeros.emplace_back((size_t)volume(s), 0.f);
+                }
+                for (size_t i = 0; i < ptrs.size(); ++i)
+                    ptrs[i] = zeros[i].data();
+                int orank = 0;
+                int64_t od[5] = { 1, 1, 1, 1, 1 };
+                if (hl.vt.apply(hl.instance, (int)o.in.size(), ptrs.data(), ranks.data(), dims5.data(), nullptr, &orank, od) != FDX_OK) {
+                    set_error("%s: custom layer failed on the shape pass: %s", o.name.c_str(), fdx_last_error());
+                    return FDX_ERR_INVALID;
+                }
+                FDX_REQUIRE(orank >= 1 && orank <= 5, "%s: custom layer returned rank %d", o.name.c_str(), orank);
+                out.assign(od + 5 - orank, od + 5);
+                for (auto d : out)
+                    FDX_REQUIRE(d > 0, "%s: custom layer returned an empty shape", o.name.c_str());
+                break;
+            }
             case OpKind::Einsum: {
                 EinsumSpec spec;
                 std::string err;
@@ -1220,6 +1289,46 @@ namespace {
                 st = fdx_activation_f32(out, (size_t)B * (size_t)volume(os), actp, out);
             break;
         }
+        case OpKind::Host: {
+            // drain the stream, run the layer on the host sample by sample, hand the result back to the device
+            const fdx_host_layer& hl = m.host_layers[(size_t)o.host_index];
+            const size_t n_in = o.in.size();
+            std::vector<std::vector<float>> hin(n_in);
+            std::vector<int> ranks;
+            std::vector<int64_t> dims5;
+            std::vector<int64_t> vols;
+            for (size_t i = 0; i < n_in; ++i) {
+                const Shape& s = p.shapes[o.in[i]];
+                vols.push_back(volume(s));
+                hin[i].resize((size_t)B * (size_t)vols[i]);
+                FDX_HIP(hipMemcpyAsync(hin[i].data(), p.out[o.in[i]], hin[i].size() * sizeof(float), hipMemcpyDeviceToHost, stream()));
+                ranks.push_back((int)s.size());
+                for (size_t k = 0; k < 5; ++k)
+                    dims5.push_back(k < 5 - s.size() ? 1 : s[k - (5 - s.size())]);
+            }
+            FDX_HIP(hipStreamSynchronize(stream()));
+            const int64_t ovol = volume(os);
+            std::vector<float> hout((size_t)B * (size_t)ovol);
+            std::vector<const float*> ptrs(n_in);
+            for (int b = 0; b < B; ++b) {
+                for (size_t i = 0; i < n_in; ++i)
+                    ptrs[i] = hin[i].data() + (size_t)b * (size_t)vols[i];
+                int orank = 0;
+                int64_t od[5] = { 1, 1, 1, 1, 1 };
+                if (hl.vt.apply(hl.instance, (int)n_in, ptrs.data(), ranks.data(), dims5.data(), hout.data() + (size_t)b * (size_t)ovol,
+                        &orank, od) != FDX_OK) {
+                    set_error("%s: custom layer failed: %s", o.name.c_str(), fdx_last_error());
+                    return FDX_ERR_INVALID;
+                }
+                FDX_REQUIRE(orank == (int)os.size() && Shape(od + 5 - orank, od + 5) == os,
+                    "%s: custom layer changed its output shape between calls", o.name.c_str());
+            }
+            FDX_HIP(hipMemcpyAsync(out, hout.data(), hout.size() * sizeof(float), hipMemcpyHostToDevice, stream()));
+            FDX_HIP(hipStreamSynchronize(stream()));
+            if (actp)
+                st = fdx_activation_f32(out, (size_t)B * (size_t)ovol, actp, out);
+            break;
+        }
         case OpKind::Einsum: {
             if (o.gemm) {
                 const int64_t rows = (int64_t)B * volume(*is) / o.n_in;
@@ -1461,6 +1570,9 @@ namespace {
 fdx_model::~fdx_model()
 {
     (void)hipStreamSynchronize(fdx::stream());
+    for (auto& hl : host_layers)
+        if (hl.vt.destroy && hl.instance)
+            hl.vt.destroy(hl.instance);
     plan.reset();
     for (float* p : device_allocs)
         (void)hipFree(p);
@@ -1470,7 +1582,14 @@ fdx_model::~fdx_model()
 
 extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int verify, float verify_epsilon, fdx_model** out)
 {
+    return fdx_model_create_custom(json_text, len, verify, verify_epsilon, nullptr, 0, out);
+}
+
+extern "C" fdx_status fdx_model_create_custom(const char* json_text, size_t len, int verify, float verify_epsilon,
+    const fdx_custom_layer* custom_layers, int n_custom_layers, fdx_model** out)
+{
     FDX_REQUIRE(json_text && out, "model_create: null argument");
+    FDX_REQUIRE(n_custom_layers >= 0 && (n_custom_layers == 0 || custom_layers), "model_create: bad custom layer list");
     *out = nullptr;
     if (fdx_sync() != FDX_OK)
         return FDX_ERR_HIP;
@@ -1493,6 +1612,8 @@ extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int ve
         static const Value empty_params = [] { Value v; v.type = Value::Object; return v; }();
         const Value* tp = root.find("trainable_params");
         Builder b { *m, tp ? *tp : empty_params, {} };
+        b.customs = custom_layers;
+        b.n_customs = n_custom_layers;
         b.scopes.emplace_back(new Scope);
         Scope& top = *b.scopes.back();
         Builder::index_layers(top, layers);

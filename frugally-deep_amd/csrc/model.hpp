@@ -13,7 +13,7 @@
 namespace fdx {
 
 enum class OpKind {
-    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat
+    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat, Host
 };
 
 using Shape = std::vector<int64_t>; // dims of one sample, no batch axis
@@ -53,6 +53,7 @@ struct Op {
     Shape kernel_dims, full_out;     // EinsumDense: kernel extents as stored, output_shape with the batch slot
     bool gemm = false;               // EinsumDense that is one row-major GEMM (kernel stored transposed)
     int axis = -1;                   // Concatenate
+    int host_index = -1;             // Host: index into fdx_model::host_layers
 
     // host weights (released after upload)
     std::vector<std::vector<float>> hw;
@@ -82,8 +83,15 @@ struct Plan {
 
 } // namespace fdx
 
+// one custom layer object created through fdx_custom_layer::create
+struct fdx_host_layer {
+    fdx_custom_layer vt;
+    void* instance = nullptr;
+};
+
 struct fdx_model {
     std::string name, hash;
+    std::vector<fdx_host_layer> host_layers;
     std::vector<fdx::Op> ops;
     std::vector<int> inputs, outputs;   // op indices
     std::vector<fdx::Shape> in_decl, out_decl; // declared shapes, -1 = variable

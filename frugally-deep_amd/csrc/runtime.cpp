@@ -126,6 +126,11 @@ fdx_status ensure_init()
 
 using namespace fdx;
 
+extern "C" void fdx_set_last_error(const char* text)
+{
+    fdx::set_error("%s", text ? text : "");
+}
+
 extern "C" const char* fdx_last_error(void) { return g_error.c_str(); }
 
 extern "C" fdx_status fdx_init(int device)

@@ -24,6 +24,7 @@
 #include <functional>
 #include <iostream>
 #include <iterator>
+#include <map>
 #include <memory>
 #include <sstream>
 #include <stdexcept>
@@ -297,6 +298,83 @@ inline std::vector<std::uint8_t> tensor_to_bytes(const tensor& t, float_type low
     return bytes;
 }
 
+namespace internal {
+    // Extension point for layer classes the device path does not know: a subclass of `layer` implements
+    // apply_impl on host tensors and is produced by a creator registered under the Keras class name
+    // (include/fdeep/layers/layer.hpp:32-88, include/fdeep/import_model.hpp:374-381).  The creator receives
+    // the layer's JSON text instead of a parsed nlohmann::json object, and get_param returns the decoded
+    // floats of one trainable_params entry.
+    class layer {
+    public:
+        explicit layer(const std::string& name)
+            : name_(name)
+        {
+        }
+        virtual ~layer() = default;
+        virtual tensors apply_impl(const tensors& inputs) const = 0;
+        std::string name_;
+    };
+    using layer_ptr = std::shared_ptr<layer>;
+    using get_param_f = std::function<float_vec(const std::string& layer_name, const std::string& param_name)>;
+    using layer_creator = std::function<layer_ptr(const get_param_f&, const std::string& layer_json, const std::string& name)>;
+    using layer_creators = std::map<std::string, layer_creator>;
+
+    inline fdx_status custom_create(void* user, const char* layer_name, const char* config_json, std::size_t config_len,
+        fdx_param_getter get_param, void* get_param_ctx, void** instance)
+    {
+        try {
+            const auto& creator = *static_cast<const layer_creator*>(user);
+            const get_param_f getter = [get_param, get_param_ctx](const std::string& l, const std::string& k) {
+                const float* values = nullptr;
+                std::size_t count = 0;
+                check(get_param(get_param_ctx, l.c_str(), k.c_str(), &values, &count));
+                return float_vec(values, values + count);
+            };
+            layer_ptr made = creator(getter, std::string(config_json, config_len), layer_name);
+            if (!made) {
+                fdx_set_last_error("custom layer creator returned no layer");
+                return FDX_ERR_INVALID;
+            }
+            *instance = new layer_ptr(std::move(made));
+            return FDX_OK;
+        } catch (const std::exception& e) {
+            fdx_set_last_error(e.what());
+            return FDX_ERR_INVALID;
+        }
+    }
+    inline fdx_status custom_apply(void* instance, int n_inputs, const float* const* inputs, const int* in_ranks,
+        const std::int64_t* in_dims5, float* output, int* out_rank, std::int64_t* out_dims5)
+    {
+        try {
+            tensors ins;
+            for (int i = 0; i < n_inputs; ++i) {
+                std::vector<std::size_t> dims;
+                for (int k = 5 - in_ranks[i]; k < 5; ++k)
+                    dims.push_back(static_cast<std::size_t>(in_dims5[i * 5 + k]));
+                const tensor_shape shape = create_tensor_shape_from_dims(dims);
+                ins.emplace_back(shape, float_vec(inputs[i], inputs[i] + shape.volume()));
+            }
+            const tensors outs = (*static_cast<layer_ptr*>(instance))->apply_impl(ins);
+            if (outs.size() != 1) {
+                fdx_set_last_error("a custom layer must return exactly one tensor");
+                return FDX_ERR_INVALID;
+            }
+            const tensor_shape& os = outs[0].shape();
+            *out_rank = static_cast<int>(os.rank());
+            const auto d = os.dimensions();
+            for (std::size_t k = 0; k < 5; ++k)
+                out_dims5[k] = static_cast<std::int64_t>(d[k]);
+            if (output)
+                std::copy(outs[0].as_vector()->begin(), outs[0].as_vector()->end(), output);
+            return FDX_OK;
+        } catch (const std::exception& e) {
+            fdx_set_last_error(e.what());
+            return FDX_ERR_INVALID;
+        }
+    }
+    inline void custom_destroy(void* instance) { delete static_cast<layer_ptr*>(instance); }
+}
+
 inline void cout_logger(const std::string& str) { std::cout << str << std::flush; }
 inline void dev_null_logger(const std::string&) {}
 
@@ -431,7 +509,8 @@ private:
             r.push_back(predict_multi({ ins }, false).front());
         return r;
     }
-    friend model read_model_from_string(const std::string&, bool, const std::function<void(std::string)>&, float_type);
+    friend model read_model_from_string(const std::string&, bool, const std::function<void(std::string)>&, float_type,
+        const internal::layer_creators&);
     std::shared_ptr<fdx_model> handle_;
     std::vector<tensor_shape_variable> input_shapes_, output_shapes_;
     std::string name_, hash_;
@@ -439,7 +518,8 @@ private:
 
 // Loads a converted-JSON model held in memory.  include/fdeep/model.hpp:271-281 (and 198-267 for the steps logged)
 inline model read_model_from_string(const std::string& content, bool verify = true,
-    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001))
+    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001),
+    const internal::layer_creators& custom_layer_creators = internal::layer_creators())
 {
     const auto log = [&logger](const std::string& msg) {
         if (logger)
@@ -448,7 +528,12 @@ inline model read_model_from_string(const std::string& content, bool verify = tr
     const auto t0 = std::chrono::steady_clock::now();
     log(std::string("Loading json, building model and uploading weights") + (verify ? ", running embedded tests" : "") + " ... ");
     fdx_model* raw = nullptr;
-    internal::check(fdx_model_create(content.data(), content.size(), verify ? 1 : 0, verify_epsilon, &raw));
+    std::vector<fdx_custom_layer> customs;
+    for (const auto& kv : custom_layer_creators)
+        customs.push_back(fdx_custom_layer { kv.first.c_str(), &internal::custom_create, &internal::custom_apply,
+            &internal::custom_destroy, const_cast<internal::layer_creator*>(&kv.second) });
+    internal::check(fdx_model_create_custom(content.data(), content.size(), verify ? 1 : 0, verify_epsilon, customs.data(),
+        static_cast<int>(customs.size()), &raw));
     model m;
     m.handle_ = std::shared_ptr<fdx_model>(raw, [](fdx_model* p) { fdx_model_destroy(p); });
     int n_in = 0, n_out = 0;
@@ -469,21 +554,23 @@ inline model read_model_from_string(const std::string& content, bool verify = tr
 }
 
 inline model read_model(std::istream& model_file_stream, bool verify = true,
-    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001))
+    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001),
+    const internal::layer_creators& custom_layer_creators = internal::layer_creators())
 {
     const std::string content((std::istreambuf_iterator<char>(model_file_stream)), std::istreambuf_iterator<char>());
-    return read_model_from_string(content, verify, logger, verify_epsilon);
+    return read_model_from_string(content, verify, logger, verify_epsilon, custom_layer_creators);
 }
 
 // include/fdeep/model.hpp:285-301
 inline model load_model(const std::string& file_path, bool verify = true,
-    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001))
+    const std::function<void(std::string)>& logger = cout_logger, float_type verify_epsilon = static_cast<float_type>(0.0001),
+    const internal::layer_creators& custom_layer_creators = internal::layer_creators())
 {
     std::ifstream in_stream(file_path, std::ios::binary);
     internal::assertion(in_stream.good(), "Can not open " + file_path);
     if (logger)
         logger("Loading model " + file_path + "\n");
-    return read_model(in_stream, verify, logger, verify_epsilon);
+    return read_model(in_stream, verify, logger, verify_epsilon, custom_layer_creators);
 }
 
 } // namespace fdeep

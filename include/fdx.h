@@ -36,6 +36,8 @@ typedef struct fdx_act {
 } fdx_act;
 
 const char* fdx_last_error(void);
+/* lets a callback (custom layer) leave the text that fdx_last_error() reports for its failure */
+void fdx_set_last_error(const char* text);
 fdx_status fdx_init(int device);
 
 /* ---- device memory plumbing for callers that do not link HIP themselves ---- */
@@ -223,6 +225,30 @@ typedef struct fdx_session fdx_session;
  * test cases with absolute tolerance verify_epsilon (model.hpp:254-267, import_model.hpp:1990-2021).
  */
 fdx_status fdx_model_create(const char* json, size_t len, int verify, float verify_epsilon, fdx_model** out);
+/* ---- host fallback for layer classes the device path does not implement ----
+ * The counterpart of the reference's extension point: internal::layer_creators, a map from class name
+ * to a factory of layer objects whose apply_impl runs on host tensors
+ * (include/fdeep/import_model.hpp:374-381, 1944-1950; include/fdeep/layers/layer.hpp:32-88).  A class
+ * registered here takes precedence over a built-in one, as in the reference's map_union.  The layer
+ * runs on the host, one sample at a time, between device segments: the stream is drained, the inputs
+ * are copied to host memory, `apply` is called per sample, and the output is copied back. */
+typedef fdx_status (*fdx_param_getter)(void* ctx, const char* layer_name, const char* param_name,
+    const float** values, size_t* count); /* decoded trainable_params entry; valid until `create` returns */
+typedef struct fdx_custom_layer {
+    const char* class_name;
+    /* once per layer of this class while the model is built; config_json is the layer's JSON object */
+    fdx_status (*create)(void* user, const char* layer_name, const char* config_json, size_t config_len,
+        fdx_param_getter get_param, void* get_param_ctx, void** instance);
+    /* one sample: n_inputs host tensors, each with a rank and five right-aligned extents; writes the output's
+     * rank and extents, and its values unless `output` is NULL (the shape pass at plan time) */
+    fdx_status (*apply)(void* instance, int n_inputs, const float* const* inputs, const int* in_ranks,
+        const int64_t* in_dims5, float* output, int* out_rank, int64_t* out_dims5);
+    void (*destroy)(void* instance);
+    void* user;
+} fdx_custom_layer;
+/* fdx_model_create with custom layers (load_model's custom_layer_creators argument, model.hpp:285-301) */
+fdx_status fdx_model_create_custom(const char* json_text, size_t len, int verify, float verify_epsilon,
+    const fdx_custom_layer* custom_layers, int n_custom_layers, fdx_model** out);
 fdx_status fdx_model_destroy(fdx_model* m);
 fdx_status fdx_model_name(const fdx_model* m, const char** name, const char** hash);
 /* number of inputs/outputs and their shapes: rank and dims (-1 = variable), model.hpp:66-96 */

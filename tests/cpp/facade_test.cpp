@@ -91,6 +91,42 @@ int main(int argc, char** argv)
     for (int i = 0; i < 6; ++i)
         EXPECT(back[static_cast<std::size_t>(i)] == px[i]);
     EXPECT(fdeep::show_tensor_shape(t.shape()) == "3(1, 2, 3)");
+
+    // custom layer: a class the device path does not know, created through custom_layer_creators
+    // (the reference's FAQ example shape: a layer subclass with apply_impl, registered by class name)
+    if (argc > 3) {
+        class scale_shift_layer : public fdeep::internal::layer {
+        public:
+            scale_shift_layer(const std::string& name, const fdeep::float_vec& offset)
+                : layer(name)
+                , offset_(offset)
+            {
+            }
+            fdeep::tensors apply_impl(const fdeep::tensors& inputs) const override
+            {
+                fdeep::float_vec v = *inputs.at(0).as_vector();
+                for (std::size_t i = 0; i < v.size(); ++i)
+                    v[i] = 2.0f * v[i] + offset_[i % offset_.size()];
+                return { fdeep::tensor(inputs[0].shape(), std::move(v)) };
+            }
+            fdeep::float_vec offset_;
+        };
+        int created = 0;
+        const fdeep::internal::layer_creators creators = { { "ScaleShift",
+            [&created](const fdeep::internal::get_param_f& get_param, const std::string& layer_json, const std::string& name) {
+                ++created;
+                if (layer_json.find("\"ScaleShift\"") == std::string::npos)
+                    throw std::runtime_error("layer json not passed");
+                return std::make_shared<scale_shift_layer>(name, get_param(name, "offset"));
+            } } };
+        EXPECT(throws_with([&] { fdeep::load_model(argv[3], true, fdeep::dev_null_logger); }, "unknown layer type: ScaleShift"));
+        // the file's embedded test (written by the oracle with the same layer semantics) is replayed on load
+        const auto custom = fdeep::load_model(argv[3], true, fdeep::dev_null_logger, static_cast<fdeep::float_type>(0.00001), creators);
+        EXPECT(created == 1);
+        const std::vector<fdeep::tensors> batch(3, custom.generate_dummy_inputs());
+        const auto outs = custom.predict_multi(batch, true);
+        EXPECT(outs.size() == 3 && outs[0][0].to_vector() == outs[2][0].to_vector());
+    }
     std::printf("facade_test ok\n");
     return 0;
 }

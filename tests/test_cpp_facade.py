@@ -40,6 +40,20 @@ def test_facade_runs_reference_style_checks(fdx, oracle, modelgen, tmp_path):
     idx = np.arange(32 * 32 * 3, dtype=np.float32)
     probe = np.sin(np.float32(0.37) * idx).astype(np.float32).reshape(32, 32, 3)
     want = oracle.argmax(ref.predict([probe])[0])
-    out = subprocess.run([EXE, str(path), str(want)], capture_output=True, text=True, timeout=120)
+    # a model with a layer class only a custom creator knows: Dense -> ScaleShift (2x + offset[c]) -> Dense
+    b = modelgen.Builder("with_custom", 77)
+    t_in = b.input((5, 8), "x")
+    h = b.dense(t_in, 6, "fc1", activation="relu", bias_std=0.2)
+    b.params["scale_shift"] = {"offset": np.arange(6, dtype=np.float32) / 4}
+    c = b._add("ScaleShift", "scale_shift", {"name": "scale_shift"}, [h], h.shape)
+    cspec = b.finish([b.dense(c, 3, "fc2", bias_std=0.2)])
+    xc = np.random.default_rng(42).standard_normal((5, 8)).astype(np.float32)
+    p = cspec["trainable_params"]
+    hid = oracle.relu(oracle.dense(xc, p["fc1"]["weights"].reshape(-1), p["fc1"]["bias"], 6))
+    hid = (2.0 * hid + p["scale_shift"]["offset"]).astype(np.float32)
+    cspec["tests"] = [{"inputs": [xc], "outputs": [oracle.dense(hid, p["fc2"]["weights"].reshape(-1), p["fc2"]["bias"], 3)]}]
+    cpath = tmp_path / "with_custom.json"
+    cpath.write_bytes(modelgen.dumps(cspec))
+    out = subprocess.run([EXE, str(path), str(want), str(cpath)], capture_output=True, text=True, timeout=120)
     print(out.stdout, out.stderr, flush=True)
     assert out.returncode == 0 and "facade_test ok" in out.stdout

@@ -180,3 +180,48 @@ def test_nested_model_applied_twice(fdx, oracle, modelgen):
     same = fdx.Model(js).predict([xs[0], xs[0]])[0]
     ref_same = np.stack([ref.predict([xs[0][i], xs[0][i]])[0] for i in range(4)])
     assert rel(same, ref_same) <= TOL
+
+
+def test_custom_layer_runs_on_host_between_device_segments(fdx, oracle, modelgen):
+    """A layer class the device path does not implement, supplied by the caller: it sees one sample at a time as
+    host arrays, receives its trainable_params through get_param and its JSON through the creator, may change the
+    shape, and its fused `activation` is applied afterwards like for any other layer."""
+    say("custom layer")
+    b = modelgen.Builder("custom_host", 55)
+    x_in = b.input((6, 8), "x")
+    h = b.dense(x_in, 12, "fc1", activation="relu", bias_std=0.2)
+    b.params["pairs"] = {"scale": np.linspace(0.5, 1.5, 6).astype(np.float32)}
+    c = b._add("PairSum", "pairs", {"name": "pairs", "activation": "relu", "shift": -0.25}, [h], (6, 6))
+    spec = b.finish([b.dense(c, 4, "fc2", bias_std=0.2), c])
+    seen = []
+
+    def creator(get_param, layer, name):
+        scale = get_param(name, "scale")
+        shift = layer["config"]["shift"]
+        seen.append((name, layer["class_name"]))
+        return lambda ins: (ins[0][:, 0::2] + ins[0][:, 1::2]) * scale + shift  # (6, 12) -> (6, 6)
+
+    r = np.random.default_rng(8)
+    x = r.standard_normal((5, 6, 8)).astype(np.float32)
+    p = spec["trainable_params"]
+    hid = np.stack([oracle.relu(oracle.dense(x[i], p["fc1"]["weights"].reshape(-1), p["fc1"]["bias"], 12)) for i in range(5)])
+    mid = oracle.relu(((hid[:, :, 0::2] + hid[:, :, 1::2]) * p["pairs"]["scale"] - 0.25).astype(np.float32))
+    want = np.stack([oracle.dense(mid[i], p["fc2"]["weights"].reshape(-1), p["fc2"]["bias"], 4) for i in range(5)])
+    js = modelgen.dumps(spec)
+    with pytest.raises(fdx.FdxError, match="unknown layer type: PairSum"):
+        fdx.Model(js)
+    model = fdx.Model(js, custom_layers={"PairSum": creator})
+    assert seen == [("pairs", "PairSum")]
+    got = model.predict([x])
+    assert rel(got[1], mid) <= 1e-6 and rel(got[0], want) <= TOL
+    # a registered class overrides a built-in one
+    const = lambda gp, layer, name: (lambda ins: np.full((6, 12 if name == "fc1" else 4), 7.0, np.float32))
+    over = fdx.Model(js, custom_layers={"PairSum": creator, "Dense": const})
+    assert np.all(over.predict([x])[0] == 7)
+    # a failing layer surfaces as an error with its message
+    def broken(get_param, layer, name):
+        def run(ins):
+            raise ValueError("boom in " + name)
+        return run
+    with pytest.raises(fdx.FdxError, match="custom layer failed.*boom in pairs"):
+        fdx.Model(js, custom_layers={"PairSum": broken}).predict([x])
