@@ -154,6 +154,55 @@ def bench_resnet(fdx, modelgen, args):
     return result
 
 
+def bench_secondary(fdx, modelgen, name, spec, batch, inputs, steps, warmup):
+    """Secondary configurations (MobileNetV2 b128, transformer encoder b32): samples / second of one batched predict
+    with inputs resident, and per kernel family the HIP-event time with its own roofline (TFLOP/s against the fp32
+    MFMA peak for the GEMM families, algorithmic GB/s against HBM for the memory-bound ones)."""
+    js = modelgen.dumps(spec)
+    model = fdx.Model(js, verify=False)
+    shapes = [tuple(x.shape[1:]) for x in inputs]
+    d_in = [fdx.DevBuf.from_host(x) for x in inputs]
+    out_shapes = model.infer_shapes(shapes)
+    d_out = [fdx.DevBuf(4 * batch * int(np.prod(s))) for s in out_shapes]
+    for _ in range(warmup):
+        model.predict_dev(batch, d_in, shapes, d_out)
+    fdx.sync()
+    ms = ctypes.c_float()
+    fdx.check(fdx.lib.fdx_timer_start())
+    for _ in range(steps):
+        model.predict_dev(batch, d_in, shapes, d_out)
+    fdx.check(fdx.lib.fdx_timer_stop(ctypes.byref(ms)))
+    flops = model.last_flops()
+    y = d_out[0].to_host((batch,) + tuple(out_shapes[0]))
+    assert np.isfinite(y).all()
+    fdx.check(fdx.lib.fdx_profile_enable(1))
+    fdx.check(fdx.lib.fdx_profile_reset())
+    prof_steps = 3
+    for _ in range(prof_steps):
+        model.predict_dev(batch, d_in, shapes, d_out)
+    fdx.sync()
+    fams = profile_families(fdx)
+    fdx.check(fdx.lib.fdx_profile_enable(0))
+    per_family = {}
+    for k, v in sorted(fams.items()):
+        e = {"ms_per_step": round(v["ms"] / prof_steps, 4), "launches_per_step": v["launches"] // prof_steps}
+        if v["flops"] > 0:
+            tf = v["flops"] / (v["ms"] / 1e3) / 1e12
+            e.update(TFLOP_s=round(tf, 2), mfma_frac=round(tf / PEAK_FP32_MFMA_TFLOPS, 4))
+        elif v["bytes"] > 0:
+            gb = v["bytes"] / (v["ms"] / 1e3) / 1e9
+            e.update(GB_s=round(gb, 1), hbm_frac=round(gb / PEAK_HBM_GBS, 4))
+        per_family[k] = e
+    sec = ms.value / 1e3 / steps
+    res = {"workload": name, "batch": batch, "value": round(batch / sec, 1), "unit": "samples/s", "ms_per_step": round(sec * 1e3, 4),
+           "gflop_per_sample": round(flops / batch / 1e9, 4),
+           "model_mfma_frac": round(flops / sec / (PEAK_FP32_MFMA_TFLOPS * 1e12), 4), "kernels": per_family}
+    model.close()
+    for b in d_in + d_out:
+        b.free()
+    return res
+
+
 def gpt2_step_bytes(L, batch=16, layers=12, d=768, ffn=3072, vocab=50257):
     """Bytes one decode step must stream at context length L (keys visible incl. the new token)."""
     w_layers = layers * (4 * d * d + 4 * d + 2 * d * ffn + ffn + d + 4 * d) * 4
@@ -269,7 +318,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--decode-reps", type=int, default=2)
-    ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels"], default="all")
+    ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels", "mobilenet_v2", "encoder"], default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also launch one plain device copy (act_kernel, no activation) of this many MiB, whose known "
@@ -297,6 +346,22 @@ def main():
             result["gpt2_decode"] = g
         else:
             result = g
+    rng = np.random.default_rng(77)
+    secondary = {}
+    if args.workload in ("all", "mobilenet_v2"):
+        x = rng.uniform(0, 1, (128, 224, 224, 3)).astype(np.float32)
+        secondary["mobilenet_v2"] = bench_secondary(fdx, modelgen, "MobileNetV2 alpha 1.0 architecture, 224x224x3, batch 128",
+                                                    modelgen.mobilenet_v2(), 128, [x], max(3, args.steps // 2), 3)
+    if args.workload in ("all", "encoder"):
+        x = rng.standard_normal((32, 256, 512)).astype(np.float32)
+        secondary["encoder"] = bench_secondary(fdx, modelgen, "6-layer pre-LN transformer encoder, seq 256, d 512, 8 heads, "
+                                               "ffn 2048 (erf-GELU), batch 32", modelgen.encoder(), 32, [x],
+                                               max(3, args.steps // 2), 3)
+    if secondary:
+        if result:
+            result["secondary"] = secondary
+        else:
+            result = {"metric": "secondary configurations", "n_gpus": 1, "secondary": secondary}
     print(json.dumps(result), flush=True)
 
 

@@ -100,6 +100,71 @@ __global__ void dwconv_kernel(const float* __restrict__ in, const float* __restr
     }
 }
 
+
+// 3x3, dilation 1, four channels per lane and TX consecutive output columns per thread: the nine
+// filter vectors stay in registers and each input row segment is loaded once for all TX outputs
+// (the plain kernel above issues 18 loads per output vector, which caps it well below HBM speed).
+template <int STRIDE, int TX>
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(const float* __restrict__ in, const float* __restrict__ wts,
+    const float* __restrict__ bias, float* __restrict__ out, int n, int h, int w, int c, int pad_top, int pad_left,
+    int oh, int ow, Act act)
+{
+    constexpr int COLS = (TX - 1) * STRIDE + 3;
+    const int cv = c / 4, xt = (ow + TX - 1) / TX;
+    const int64_t total = (int64_t)n * oh * xt * cv;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int cq = (int)(idx % cv);
+        int64_t rest = idx / cv;
+        const int ox0 = (int)(rest % xt) * TX;
+        rest /= xt;
+        const int oy = (int)(rest % oh);
+        const int img = (int)(rest / oh);
+        const int c0 = cq * 4;
+        f32x4 wv[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+            wv[t] = *reinterpret_cast<const f32x4*>(wts + (int64_t)t * c + c0);
+        f32x4 acc[TX];
+        const f32x4 b4 = bias ? *reinterpret_cast<const f32x4*>(bias + c0) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+        for (int j = 0; j < TX; ++j)
+            acc[j] = b4;
+        const float* ib = in + (int64_t)img * h * w * c + c0;
+        const int ix0 = ox0 * STRIDE - pad_left;
+#pragma unroll
+        for (int fy = 0; fy < 3; ++fy) {
+            const int iy = oy * STRIDE - pad_top + fy;
+            if (iy < 0 || iy >= h)
+                continue;
+            const float* row = ib + (int64_t)iy * w * c;
+            f32x4 col[COLS];
+#pragma unroll
+            for (int k = 0; k < COLS; ++k) {
+                const int ix = ix0 + k;
+                col[k] = (ix >= 0 && ix < w) ? *reinterpret_cast<const f32x4*>(row + (int64_t)ix * c) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+            }
+#pragma unroll
+            for (int j = 0; j < TX; ++j)
+#pragma unroll
+                for (int fx = 0; fx < 3; ++fx)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        acc[j][v] += col[j * STRIDE + fx][v] * wv[fy * 3 + fx][v];
+        }
+        float* op = out + (((int64_t)img * oh + oy) * ow + ox0) * c + c0;
+#pragma unroll
+        for (int j = 0; j < TX; ++j)
+            if (ox0 + j < ow) {
+                f32x4 r;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    r[v] = apply_act(acc[j][v], act);
+                *reinterpret_cast<f32x4*>(op + (int64_t)j * c) = r;
+            }
+    }
+}
+
 // ------------------------------------------------------------------ pooling
 __global__ void pool2d_kernel(const float* __restrict__ in, float* __restrict__ out, int n, int h, int w, int c,
     int ph, int pw, int sy, int sx, int pad_top, int pad_left, int zt, int zl, int zb, int zr, int oh, int ow, int mode)
@@ -453,7 +518,14 @@ extern "C" fdx_status fdx_dwconv2d_nhwc_f32(const float* in, int n, int h, int w
     const bool vec = c % 4 == 0 && al16(in) && al16(weights_hwc) && al16(out);
     const size_t items = (size_t)n * out_h * out_w * (vec ? c / 4 : c);
     profile_begin();
-    if (vec)
+    const bool k3 = vec && kh == 3 && kw == 3 && dy == 1 && dx == 1 && sy == sx && (sy == 1 || sy == 2) && (!bias || al16(bias));
+    if (k3 && sy == 1)
+        hipLaunchKernelGGL((dwconv3x3_kernel<1, 8>), dim3(grid_for((size_t)n * out_h * ((out_w + 7) / 8) * (c / 4), 256)), dim3(256), 0,
+            stream(), in, weights_hwc, bias, out, n, h, w, c, pad_top, pad_left, out_h, out_w, a);
+    else if (k3)
+        hipLaunchKernelGGL((dwconv3x3_kernel<2, 4>), dim3(grid_for((size_t)n * out_h * ((out_w + 3) / 4) * (c / 4), 256)), dim3(256), 0,
+            stream(), in, weights_hwc, bias, out, n, h, w, c, pad_top, pad_left, out_h, out_w, a);
+    else if (vec)
         hipLaunchKernelGGL(dwconv_kernel<4>, dim3(grid_for(items, 256)), dim3(256), 0, stream(), in, weights_hwc, bias,
             out, n, h, w, c, kh, kw, sy, sx, dy, dx, pad_top, pad_left, out_h, out_w, a);
     else

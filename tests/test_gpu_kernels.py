@@ -109,7 +109,10 @@ def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
 @pytest.mark.parametrize("case", [
     (2, 9, 8, 8, 3, 3, (1, 1), (1, 1), "same"), (2, 9, 8, 6, 3, 3, (2, 2), (1, 1), "same"),
     (1, 10, 11, 5, 3, 3, (2, 2), (1, 1), "valid"), (2, 12, 12, 4, 3, 3, (1, 1), (2, 2), "same"),
-    (3, 28, 28, 96, 3, 3, (2, 2), (1, 1), "valid"), (2, 14, 14, 144, 3, 3, (1, 1), (1, 1), "same")])
+    (3, 28, 28, 96, 3, 3, (2, 2), (1, 1), "valid"), (2, 14, 14, 144, 3, 3, (1, 1), (1, 1), "same"),
+    # the column-tiled 3x3 kernel: widths that are not a multiple of its four-column tile, one-column images, same / valid
+    (2, 7, 7, 32, 3, 3, (1, 1), (1, 1), "same"), (1, 5, 1, 8, 3, 3, (1, 1), (1, 1), "same"), (2, 9, 13, 16, 3, 3, (2, 2), (1, 1), "same"),
+    (1, 8, 10, 12, 3, 3, (1, 1), (1, 1), "valid"), (1, 3, 3, 4, 3, 3, (2, 2), (1, 1), "valid"), (2, 6, 5, 8, 5, 5, (1, 1), (1, 1), "same")])
 def test_dwconv_vs_oracle(fdx, oracle, case):
     n, h, w, c, kh, kw, strides, dilation, padding = case
     say("dwconv", case)
