@@ -17,6 +17,11 @@ c_float_p = ctypes.POINTER(ctypes.c_float)
 c_void_pp = ctypes.POINTER(ctypes.c_void_p)
 
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+# config name -> FDX_ACT_* (include/fdx.h)
+ACT_KINDS = {"tanh": 3, "sigmoid": 4, "swish": 5, "silu": 5, "hard_sigmoid": 6, "selu": 7, "elu": 8, "celu": 8, "exponential": 9,
+             "softsign": 10, "softplus": 11, "leaky_relu": 12, "hard_shrink": 13, "soft_shrink": 14, "sparse_plus": 15,
+             "squareplus": 16, "tanh_shrink": 17, "threshold": 18, "log_sigmoid": 19, "hard_tanh": 20, "log": 21}
+COMBINE = {"add": 0, "mul": 1, "sub": 2, "max": 3, "min": 4, "prelu": 5}
 FLT_MAX = float(np.finfo(np.float32).max)
 PAD = {"valid": 0, "same": 1, "causal": 2}
 
@@ -60,6 +65,21 @@ def check(status):
 
 def relu_act(max_value=None, negative_slope=0.0, threshold=0.0):
     return Act(ACT_RELU, FLT_MAX if max_value is None else max_value, negative_slope, threshold)
+
+
+def named_act(name, p0=0.0, p1=0.0):
+    """fdx_act for an activation by its config name; p0 / p1 as the oracle's activation(): alpha, slope, threshold, b,
+    (threshold, default value)."""
+    kind = ACT_KINDS[name]
+    if name in ("elu", "celu", "leaky_relu"):
+        return Act(kind, FLT_MAX, p0, 0.0)
+    if name in ("hard_shrink", "soft_shrink"):
+        return Act(kind, FLT_MAX, 0.0, p0)
+    if name == "squareplus":
+        return Act(kind, p0, 0.0, 0.0)
+    if name == "threshold":
+        return Act(kind, p1, 0.0, p0)
+    return Act(kind, FLT_MAX, 0.0, 0.0)
 
 
 def gelu_act():
@@ -267,6 +287,21 @@ def broadcast_add(a, b, act=None):
                                     _dp(out), od))
     got = tuple(od)[5 - rank:]
     return out.to_host((batch,) + got)
+
+
+def broadcast_combine(op, a, b, b_shared=False, scale=1.0, act=None):
+    """a: (batch, ...); b: (batch, ...) or, with b_shared, one tensor without a batch axis used for every sample."""
+    a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+    batch = a.shape[0]
+    bs = b.shape if b_shared else b.shape[1:]
+    rank = max(a.ndim - 1, len(bs))
+    pa, pb = (1,) * (rank - a.ndim + 1) + a.shape[1:], (1,) * (rank - len(bs)) + tuple(bs)
+    od = (ctypes.c_int64 * 5)()
+    out = DevBuf(4 * batch * int(np.prod([max(x, y) for x, y in zip(pa, pb)])))
+    da, db = DevBuf.from_host(a), DevBuf.from_host(b)
+    check(lib.fdx_broadcast_combine_f32(COMBINE[op], _dp(da), _dims5(a.shape[1:]), _dp(db), _dims5(bs), int(b_shared), batch,
+                                        ctypes.c_float(scale), _act_ref(act), _dp(out), od))
+    return out.to_host((batch,) + tuple(od)[5 - rank:])
 
 
 def concat(xs, axis):

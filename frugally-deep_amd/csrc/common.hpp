@@ -51,7 +51,52 @@ __device__ __forceinline__ float apply_act(float x, const Act& a)
     return x;
 }
 
+// every activation kind (stand-alone activation kernel only; the epilogues keep the two-way switch above
+// so that the GEMM kernels do not carry transcendental code they never run)
+__device__ __forceinline__ float apply_act_full(float x, const Act& a)
+{
+    switch (a.kind) {
+    case FDX_ACT_NONE: return x;
+    case FDX_ACT_RELU:
+    case FDX_ACT_GELU: return apply_act(x, a);
+    case FDX_ACT_TANH: return tanhf(x);
+    case FDX_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
+    case FDX_ACT_SWISH: return x / (1.0f + expf(-x));
+    case FDX_ACT_HARD_SIGMOID: return x < -3.0f ? 0.0f : (x > 3.0f ? 1.0f : x / 6.0f + 0.5f);
+    case FDX_ACT_SELU: return 1.0507009873554804934193349852946f * (x >= 0.0f ? x : 1.6732632423543772848170429916717f * (expf(x) - 1.0f));
+    case FDX_ACT_ELU: return x >= 0.0f ? x : a.negative_slope * (expf(x) - 1.0f);
+    case FDX_ACT_EXPONENTIAL: return expf(x);
+    case FDX_ACT_SOFTSIGN: return x / (fabsf(x) + 1.0f);
+    case FDX_ACT_SOFTPLUS: {
+        const float thr = -13.942385f; // log(FLT_EPSILON) + 2
+        return x > -thr ? x : (x < thr ? expf(x) : log1pf(expf(x)));
+    }
+    case FDX_ACT_LEAKY_RELU: return x > 0.0f ? x : a.negative_slope * x;
+    case FDX_ACT_HARD_SHRINK: return fabsf(x) > a.threshold ? x : 0.0f;
+    case FDX_ACT_SOFT_SHRINK: return x > a.threshold ? x - a.threshold : (x < -a.threshold ? x + a.threshold : 0.0f);
+    case FDX_ACT_SPARSE_PLUS: return x <= -1.0f ? 0.0f : (x < 1.0f ? 0.25f * (x + 1.0f) * (x + 1.0f) : x);
+    case FDX_ACT_SQUARE_PLUS: return (x + sqrtf(x * x + a.max_value)) / 2.0f;
+    case FDX_ACT_TANH_SHRINK: return x - tanhf(x);
+    case FDX_ACT_THRESHOLD: return x > a.threshold ? x : a.max_value;
+    case FDX_ACT_LOG_SIGMOID: return logf(1.0f / (1.0f + expf(-x)));
+    case FDX_ACT_HARD_TANH: return x < -1.0f ? -1.0f : (x > 1.0f ? 1.0f : x);
+    case FDX_ACT_LOG: return logf(x);
+    default: return x;
+    }
+}
+
+// activations an epilogue can carry
+inline bool epilogue_act_ok(const fdx_act* a) { return !a || a->kind == FDX_ACT_NONE || a->kind == FDX_ACT_RELU || a->kind == FDX_ACT_GELU; }
+
 } // namespace fdx
+
+#define FDX_REQUIRE_EPILOGUE_ACT(act)                                                                     \
+    do {                                                                                                  \
+        if (!fdx::epilogue_act_ok(act)) {                                                                 \
+            fdx::set_error("this launcher fuses only NONE / RELU / GELU; run other activations through fdx_activation_f32"); \
+            return FDX_ERR_UNSUPPORTED;                                                                   \
+        }                                                                                                 \
+    } while (0)
 
 #define FDX_HIP(expr)                                                                                     \
     do {                                                                                                  \

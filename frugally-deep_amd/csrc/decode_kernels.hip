@@ -631,6 +631,7 @@ extern "C" fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const flo
     fdx::SkinnyParams p;
     std::memset(&p, 0, sizeof p);
     p.X = x; p.ldx = k; p.W = w_nk; p.ldw = k; p.M = m; p.N = n; p.K = k; p.bias = bias; p.residual = residual; p.ldr = n;
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     p.act = fdx::make_act(act);
     p.n_seg = 1;
     p.seg[0] = { out, n, 0, 0 };
@@ -650,6 +651,7 @@ extern "C" fdx_status fdx_layernorm_dense_rows_f32(const float* x, int m, int k,
     fdx::SkinnyParams p;
     std::memset(&p, 0, sizeof p);
     p.X = x; p.ldx = k; p.W = w_folded; p.ldw = k; p.M = m; p.N = n; p.K = k; p.bias = bias_folded; p.residual = residual; p.ldr = n;
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     p.act = fdx::make_act(act);
     p.ln = 1; p.ln_eps = ln_eps; p.w_rowsum = w_rowsum;
     p.n_seg = 1;

@@ -557,6 +557,7 @@ extern "C" fdx_status fdx_conv2d_nhwc_f32(const float* in, int n, int h, int w, 
     const float* residual, const fdx_act* act, float* out)
 {
     FDX_REQUIRE(in && weights && out, "conv2d: null pointer");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     FDX_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0 && kh > 0 && kw > 0, "conv2d: bad shape");
     FDX_REQUIRE(sy > 0 && sx > 0 && dy > 0 && dx > 0 && out_h > 0 && out_w > 0, "conv2d: bad stride/dilation/output");
     FDX_REQUIRE(pad_top >= 0 && pad_left >= 0, "conv2d: negative padding");
@@ -586,6 +587,7 @@ extern "C" fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const f
     const float* residual, const fdx_act* act, float* c, int64_t ldc, const fdx_gemm_batch* batch)
 {
     FDX_REQUIRE(a && b_nk && c, "gemm: null pointer");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     FDX_REQUIRE(m > 0 && n > 0 && k > 0 && lda >= k && ldb >= k && ldc >= n, "gemm: bad shape m=%d n=%d k=%d", m, n, k);
     GemmParams p {};
     p.A = a; p.B = b_nk; p.C = c; p.bias = bias; p.residual = residual;

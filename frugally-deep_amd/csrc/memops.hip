@@ -261,10 +261,10 @@ __global__ void act_kernel(const float* __restrict__ x, float* __restrict__ out,
             f32x4 r;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                r[e] = apply_act(v[e], act);
+                r[e] = apply_act_full(v[e], act);
             reinterpret_cast<f32x4*>(out)[i] = r;
         } else {
-            out[i] = apply_act(x[i], act);
+            out[i] = apply_act_full(x[i], act);
         }
     }
 }
@@ -514,6 +514,7 @@ extern "C" fdx_status fdx_dwconv2d_nhwc_f32(const float* in, int n, int h, int w
     FDX_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && kh > 0 && kw > 0 && sy > 0 && sx > 0 && dy > 0 && dx > 0
             && out_h > 0 && out_w > 0 && pad_top >= 0 && pad_left >= 0,
         "dwconv2d: bad shape");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     const Act a = make_act(act);
     const bool vec = c % 4 == 0 && al16(in) && al16(weights_hwc) && al16(out);
     const size_t items = (size_t)n * out_h * out_w * (vec ? c / 4 : c);
@@ -568,6 +569,7 @@ extern "C" fdx_status fdx_eltwise_add_f32(const float* a, const float* b, size_t
     const fdx_act* act, float* out)
 {
     FDX_REQUIRE(a && b && out && count > 0 && b_count > 0 && count % b_count == 0, "eltwise_add: bad arguments");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     const Act ac = make_act(act);
     const bool vec = count % 4 == 0 && b_count % 4 == 0 && al16(a) && al16(b) && al16(out);
     profile_begin();
@@ -583,6 +585,7 @@ extern "C" fdx_status fdx_eltwise_add_f32(const float* a, const float* b, size_t
 extern "C" fdx_status fdx_activation_f32(const float* x, size_t count, const fdx_act* act, float* out)
 {
     FDX_REQUIRE(x && out && count > 0, "activation: bad arguments");
+    FDX_REQUIRE(!act || (act->kind >= 0 && act->kind < FDX_ACT_COUNT), "activation: unknown kind %d", act ? act->kind : 0);
     const Act ac = make_act(act);
     const bool vec = count % 4 == 0 && al16(x) && al16(out);
     profile_begin();
@@ -599,6 +602,7 @@ extern "C" fdx_status fdx_channel_affine_f32(const float* x, size_t positions, i
     const float* shift, const fdx_act* act, float* out)
 {
     FDX_REQUIRE(x && out && scale && shift && positions > 0 && c > 0, "channel_affine: bad arguments");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     const size_t count = positions * (size_t)c;
     profile_begin();
     hipLaunchKernelGGL(affine_kernel, dim3(grid_for(count, 256)), dim3(256), 0, stream(), x, out, count, c, scale, shift,

@@ -179,17 +179,30 @@ namespace {
 
     // Sets an activation by name; returns false for "softmax" (caller schedules the softmax kernel).
     // import_model.hpp:1649-1700; relu parameters only when max_value is present and non-null (:1289-1302).
-    enum class ActParse { Epilogue, Softmax, Linear };
+    enum class ActParse { Epilogue, Softmax, Linear, Standalone, LogSoftmax };
+    float cfg_float(const Value* cfg, const char* key, float dflt)
+    {
+        const Value* v = cfg ? cfg->find(key) : nullptr;
+        return v && v->is_number() ? (float)v->number() : dflt;
+    }
+    // import_model.hpp:1649-1700 (names), :1200-1385 (parameters and their defaults)
     ActParse parse_activation(const std::string& type, const Value* cfg, Act& act)
     {
+        const float big = 3.402823466e+38f;
+        auto plain = [&](int kind) {
+            act = { kind, big, 0.f, 0.f };
+            return ActParse::Standalone;
+        };
         if (type == "linear")
             return ActParse::Linear;
         if (type == "softmax")
             return ActParse::Softmax;
+        if (type == "log_softmax")
+            return ActParse::LogSoftmax;
         if (type == "relu") {
-            act = { FDX_ACT_RELU, 3.402823466e+38f, 0.f, 0.f };
+            act = { FDX_ACT_RELU, big, 0.f, 0.f };
             const Value* mv = cfg ? cfg->find("max_value") : nullptr;
-            if (mv && !mv->is_null()) {
+            if (mv && !mv->is_null()) { // parameters only when max_value is present and non-null (:1289-1302)
                 act.max_value = (float)mv->number();
                 act.negative_slope = (float)cfg->at("negative_slope").number();
                 act.threshold = (float)cfg->at("threshold").number();
@@ -204,11 +217,56 @@ namespace {
             const Value* ap = cfg ? cfg->find("approximate") : nullptr;
             if (ap && !ap->is_null() && ap->boolean())
                 throw FormatError("Gelu with approximate = True is not supported.");
-            act = { FDX_ACT_GELU, 3.402823466e+38f, 0.f, 0.f };
+            act = { FDX_ACT_GELU, big, 0.f, 0.f };
             return ActParse::Epilogue;
+        }
+        if (type == "tanh") return plain(FDX_ACT_TANH);
+        if (type == "sigmoid") return plain(FDX_ACT_SIGMOID);
+        if (type == "swish" || type == "silu") return plain(FDX_ACT_SWISH);
+        if (type == "hard_sigmoid") return plain(FDX_ACT_HARD_SIGMOID);
+        if (type == "selu") return plain(FDX_ACT_SELU);
+        if (type == "exponential") return plain(FDX_ACT_EXPONENTIAL);
+        if (type == "softsign") return plain(FDX_ACT_SOFTSIGN);
+        if (type == "softplus") return plain(FDX_ACT_SOFTPLUS);
+        if (type == "sparse_plus") return plain(FDX_ACT_SPARSE_PLUS);
+        if (type == "tanh_shrink") return plain(FDX_ACT_TANH_SHRINK);
+        if (type == "log_sigmoid") return plain(FDX_ACT_LOG_SIGMOID);
+        if (type == "hard_tanh") return plain(FDX_ACT_HARD_TANH);
+        if (type == "elu" || type == "celu") {
+            act = { FDX_ACT_ELU, big, cfg_float(cfg, "alpha", 1.0f), 0.f };
+            return ActParse::Standalone;
+        }
+        if (type == "leaky_relu") {
+            act = { FDX_ACT_LEAKY_RELU, big, cfg_float(cfg, "negative_slope", 0.2f), 0.f };
+            return ActParse::Standalone;
+        }
+        if (type == "hard_shrink" || type == "soft_shrink") {
+            if (!cfg || !cfg->find("threshold"))
+                throw FormatError(type + " needs a threshold");
+            act = { type[0] == 'h' ? FDX_ACT_HARD_SHRINK : FDX_ACT_SOFT_SHRINK, big, 0.f, (float)cfg->at("threshold").number() };
+            return ActParse::Standalone;
+        }
+        if (type == "squareplus") {
+            act = { FDX_ACT_SQUARE_PLUS, cfg_float(cfg, "b", 4.0f), 0.f, 0.f };
+            return ActParse::Standalone;
+        }
+        if (type == "threshold") { // Keras renamed threshold_value -> threshold, value -> default_value (:1277-1287)
+            const float thr = cfg && cfg->find("threshold") ? cfg_float(cfg, "threshold", 0.f) : cfg_float(cfg, "threshold_value", 0.f);
+            const float dv = cfg && cfg->find("default_value") ? cfg_float(cfg, "default_value", 0.f) : cfg_float(cfg, "value", 0.f);
+            act = { FDX_ACT_THRESHOLD, dv, 0.f, thr };
+            return ActParse::Standalone;
         }
         throw Unsupported("unknown activation type: " + type);
     }
+
+    // layer classes that are one element-wise activation (import_model.hpp:1839-1865)
+    const std::map<std::string, std::string> kActivationLayers = { { "LeakyReLU", "leaky_relu" }, { "LeakyRelu", "leaky_relu" },
+        { "ELU", "elu" }, { "Elu", "elu" }, { "Celu", "celu" }, { "ReLU", "relu" }, { "Relu6", "relu6" }, { "Exp", "exponential" },
+        { "Gelu", "gelu" }, { "Selu", "selu" }, { "Silu", "silu" }, { "Tanh", "tanh" }, { "TanhShrink", "tanh_shrink" },
+        { "Threshold", "threshold" }, { "Sigmoid", "sigmoid" }, { "HardShrink", "hard_shrink" }, { "HardSigmoid", "hard_sigmoid" },
+        { "HardTanh", "hard_tanh" }, { "SoftShrink", "soft_shrink" }, { "Softplus", "softplus" }, { "Softsign", "softsign" },
+        { "SparsePlus", "sparse_plus" }, { "Squareplus", "squareplus" }, { "LogSigmoid", "log_sigmoid" }, { "LogSoftmax", "log_softmax" },
+        { "Softmax", "softmax" } };
 
     // One level of the layer graph: the top-level model or one application of a nested
     // Functional model (create_model_layer, import_model.hpp:397-424).  A nested level reads its
@@ -276,7 +334,25 @@ namespace {
             return (int)m.ops.size() - 1;
         }
 
-        // applies config["activation"] after the op (import_model.hpp:1953-1962)
+        // an element-wise activation (or softmax / log_softmax) as an op of its own after `in`
+        int activation_op(const std::string& name, const std::string& type, const Value* cfg, int in)
+        {
+            Op op;
+            op.name = name;
+            op.cls = "Activation";
+            op.in = { in };
+            switch (parse_activation(type, cfg, op.act)) {
+            case ActParse::Linear: op.kind = OpKind::View; break;
+            case ActParse::Softmax: op.kind = OpKind::Softmax; break;
+            case ActParse::LogSoftmax: op.kind = OpKind::Softmax; op.log_after = true; break;
+            case ActParse::Epilogue:
+            case ActParse::Standalone: op.kind = OpKind::Act; break;
+            }
+            return add_op(std::move(op));
+        }
+
+        // applies config["activation"] after the op (import_model.hpp:1953-1962): ReLU / GELU ride in the producer's
+        // epilogue, softmax is flagged on the producer, everything else becomes an activation op of its own
         int with_fused_activation(int idx, const Value& cfg)
         {
             const Value* a = cfg.find("activation");
@@ -289,6 +365,8 @@ namespace {
             case ActParse::Linear: return idx;
             case ActParse::Softmax: m.ops[idx].softmax = true; return idx;
             case ActParse::Epilogue: m.ops[idx].act = act; return idx;
+            case ActParse::Standalone:
+            case ActParse::LogSoftmax: return activation_op(m.ops[idx].name + "_activation", a->str(), nullptr, idx);
             }
             return idx;
         }
@@ -481,20 +559,19 @@ namespace {
                 else
                     op.target_shape.push_back(ax.integer());
                 result = add_op(std::move(op));
-            } else if (cls == "ReLU") {
-                op.kind = OpKind::Act;
-                parse_activation("relu", &cfg, op.act);
-                result = add_op(std::move(op));
             } else if (cls == "Activation") {
-                const std::string type = cfg.at("activation").str();
-                switch (parse_activation(type, &cfg, op.act)) {
-                case ActParse::Linear: op.kind = OpKind::View; break;
-                case ActParse::Softmax: op.kind = OpKind::Softmax; break;
-                case ActParse::Epilogue: op.kind = OpKind::Act; break;
-                }
-                result = add_op(std::move(op));
-            } else if (cls == "Softmax") {
-                op.kind = OpKind::Softmax;
+                result = activation_op(op.name, cfg.at("activation").str(), &cfg, ins[0]);
+            } else if (kActivationLayers.count(cls)) {
+                result = activation_op(op.name, kActivationLayers.at(cls), &cfg, ins[0]);
+            } else if (cls == "PReLU") {
+                op.kind = OpKind::PReLU;
+                op.hw.resize(1);
+                op.hw[0] = decode_floats(param(sc, c.layer, "alpha"));
+                op.cout = (int)op.hw[0].size();
+                if (const Value* sa = cfg.find("shared_axes"))
+                    if (sa->is_array())
+                        for (const auto& a : sa->arr)
+                            op.shared_axes.push_back(a.integer());
                 result = add_op(std::move(op));
             } else if (cls == "ZeroPadding2D") {
                 op.kind = OpKind::ZeroPad;
@@ -525,8 +602,17 @@ namespace {
                 const Value* kd = cfg.find("keepdims");
                 op.keepdims = kd && kd->is_bool() && kd->boolean();
                 result = add_op(std::move(op));
-            } else if (cls == "Add") {
+            } else if (cls == "Add" || cls == "Multiply" || cls == "Subtract" || cls == "Average" || cls == "Maximum"
+                || cls == "Minimum") {
                 op.kind = OpKind::Add;
+                op.combine = cls == "Multiply" ? FDX_COMBINE_MUL : cls == "Subtract" ? FDX_COMBINE_SUB
+                    : cls == "Maximum"         ? FDX_COMBINE_MAX
+                    : cls == "Minimum"         ? FDX_COMBINE_MIN
+                                               : FDX_COMBINE_ADD;
+                if (cls == "Subtract" && ins.size() != 2)
+                    throw FormatError("subtract layer needs exactly two input tensors");
+                if (cls == "Average")
+                    op.scale = 1.0f / (float)ins.size(); // average_tensors: the sum times 1 / n (tensor.hpp:886-891)
                 result = add_op(std::move(op));
             } else if (cls == "Concatenate") {
                 op.kind = OpKind::Concat;
@@ -785,7 +871,7 @@ namespace {
         // 2. stand-alone ReLU / GELU into the producer's epilogue
         for (size_t i = 0; i < m.ops.size(); ++i) {
             Op& a = m.ops[i];
-            if (a.dead || a.kind != OpKind::Act)
+            if (a.dead || a.kind != OpKind::Act || !(a.act.kind == FDX_ACT_RELU || a.act.kind == FDX_ACT_GELU))
                 continue;
             Op& p = m.ops[a.in[0]];
             const bool ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D || p.kind == OpKind::Add || p.kind == OpKind::Affine
@@ -815,7 +901,8 @@ namespace {
         // 4. two-input equal-shape Add into the epilogue of the convolution / dense that feeds it
         for (size_t i = 0; i < m.ops.size() && have_shapes; ++i) {
             Op& add = m.ops[i];
-            if (add.dead || add.kind != OpKind::Add || add.in.size() != 2 || add.in[0] == add.in[1])
+            if (add.dead || add.kind != OpKind::Add || add.in.size() != 2 || add.in[0] == add.in[1] || add.combine != FDX_COMBINE_ADD
+                || add.scale != 1.0f)
                 continue;
             if (shapes[add.in[0]] != shapes[add.in[1]])
                 continue;
@@ -905,6 +992,7 @@ namespace {
             case OpKind::Act:
             case OpKind::Softmax:
             case OpKind::LayerNorm:
+            case OpKind::PReLU:
                 out = *in0;
                 break;
             case OpKind::ZeroPad:
@@ -1219,7 +1307,33 @@ namespace {
             break;
         case OpKind::Softmax:
             st = fdx_softmax_f32(in0, (int64_t)B * volume(*is) / is->back(), (int)is->back(), 0, 0, out);
+            if (st == FDX_OK && o.log_after) { // log_softmax = log(softmax(x)) (layers/log_softmax_layer.hpp)
+                const fdx_act lg = { FDX_ACT_LOG, 0.f, 0.f, 0.f };
+                st = fdx_activation_f32(out, (size_t)B * (size_t)volume(*is), &lg, out);
+            }
             break;
+        case OpKind::PReLU: {
+            // layers/prelu_layer.hpp:29-70: alpha is laid out over (height, width, depth) with the shared axes collapsed;
+            // shared axis numbers shift up when the sample has no height (and no width) axis of its own
+            FDX_REQUIRE(is->size() <= 3, "%s: PReLU needs rank <= 3", o.name.c_str());
+            int64_t xd[5] = { 1, 1, 1, 1, 1 };
+            for (size_t d = 0; d < is->size(); ++d)
+                xd[5 - is->size() + d] = (*is)[d];
+            bool shared[4] = { false, false, false, false };
+            int64_t shift = 0;
+            for (int64_t a : o.shared_axes) {
+                if ((a == 1 && xd[2] == 1) || (a == 2 && xd[3] == 1))
+                    ++shift;
+                const int64_t ax = a + shift;
+                if (ax >= 1 && ax <= 3)
+                    shared[ax] = true;
+            }
+            int64_t ad[5] = { 1, 1, shared[1] ? 1 : xd[2], shared[2] ? 1 : xd[3], shared[3] ? 1 : xd[4] };
+            FDX_REQUIRE(ad[2] * ad[3] * ad[4] <= o.cout, "%s: PReLU alpha holds %d values, the input needs %lld", o.name.c_str(), o.cout,
+                (long long)(ad[2] * ad[3] * ad[4]));
+            st = fdx_broadcast_combine_f32(FDX_COMBINE_PRELU, in0, xd, o.dw[0], ad, 1, B, 1.0f, actp, out, nullptr);
+            break;
+        }
         case OpKind::ZeroPad:
             st = fdx_zero_pad2d_nhwc_f32(in0, B, (int)(*is)[0], (int)(*is)[1], (int)(*is)[2], o.zp[0], o.zp[1], o.zp[2], o.zp[3], out);
             break;
@@ -1233,14 +1347,20 @@ namespace {
             st = fdx_global_pool_f32(in0, B, (int)(volume(*is) / is->back()), (int)is->back(), o.pool_mode, out);
             break;
         case OpKind::Add: {
-            // left fold (tensor.hpp:677-680); the last step carries the fused activation
+            // left fold of the layer's operation (tensor.hpp:677-690); the last step carries the scale of Average and
+            // the fused activation
             const float* acc = in0;
             Shape acc_shape = *is;
+            if (o.combine == FDX_COMBINE_MAX || o.combine == FDX_COMBINE_MIN)
+                for (int i : o.in)
+                    FDX_REQUIRE(p.shapes[i] == *is, "all tensors must have the same size");
             for (size_t k = 1; k < o.in.size() && st == FDX_OK; ++k) {
                 const float* b = p.out[o.in[k]];
                 const Shape& bs = p.shapes[o.in[k]];
-                const fdx_act* a = k + 1 == o.in.size() ? actp : nullptr;
-                if (bs == acc_shape) {
+                const bool last = k + 1 == o.in.size();
+                const fdx_act* a = last ? actp : nullptr;
+                const float scale = last ? o.scale : 1.0f;
+                if (bs == acc_shape && o.combine == FDX_COMBINE_ADD && scale == 1.0f) {
                     const size_t n = (size_t)B * (size_t)volume(bs);
                     st = fdx_eltwise_add_f32(acc, b, n, n, a, out);
                 } else {
@@ -1249,14 +1369,14 @@ namespace {
                         ad[5 - acc_shape.size() + d] = acc_shape[d];
                     for (size_t d = 0; d < bs.size(); ++d)
                         bd[5 - bs.size() + d] = bs[d];
-                    // the running sum may already live in `out`; it is only read in place when it has the output's shape
+                    // the running result may already live in `out`; it is only read in place when it has the output's shape
                     if (acc == out) {
                         bool same = true;
                         for (int d = 0; d < 5; ++d)
                             same = same && ad[d] >= bd[d];
                         FDX_REQUIRE(same, "%s: this chain of broadcasts needs a temporary", o.name.c_str());
                     }
-                    st = fdx_broadcast_add_f32(acc, ad, b, bd, B, a, out, od);
+                    st = fdx_broadcast_combine_f32(o.combine, acc, ad, b, bd, 0, B, scale, a, out, od);
                     Shape r(std::max(acc_shape.size(), bs.size()));
                     for (size_t d = 0; d < r.size(); ++d)
                         r[d] = od[5 - r.size() + d];

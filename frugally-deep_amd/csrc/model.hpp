@@ -13,7 +13,7 @@
 namespace fdx {
 
 enum class OpKind {
-    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat, Host
+    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat, Host, PReLU
 };
 
 using Shape = std::vector<int64_t>; // dims of one sample, no batch axis
@@ -54,6 +54,10 @@ struct Op {
     bool gemm = false;               // EinsumDense that is one row-major GEMM (kernel stored transposed)
     int axis = -1;                   // Concatenate
     int host_index = -1;             // Host: index into fdx_model::host_layers
+    int combine = 0;                 // Add-like merges: FDX_COMBINE_* operation
+    float scale = 1.0f;              // Average: 1 / number of inputs
+    bool log_after = false;          // Softmax op that is a log_softmax
+    std::vector<int64_t> shared_axes; // PReLU
 
     // host weights (released after upload)
     std::vector<std::vector<float>> hw;

@@ -57,8 +57,22 @@ struct BcastDesc {
 };
 
 // include/fdeep/tensor.hpp:642-660: every axis of the two operands is equal or 1; the size-1 side repeats
-__global__ void bcast_add_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
-    BcastDesc d, size_t total, Act act)
+template <int OP>
+__device__ __forceinline__ float combine(float x, float y)
+{
+    switch (OP) {
+    case FDX_COMBINE_MUL: return x * y;
+    case FDX_COMBINE_SUB: return x - y;
+    case FDX_COMBINE_MAX: return fmaxf(x, y);
+    case FDX_COMBINE_MIN: return fminf(x, y);
+    case FDX_COMBINE_PRELU: return x > 0.0f ? x : y * x;
+    default: return x + y;
+    }
+}
+
+template <int OP>
+__global__ void bcast_combine_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out,
+    BcastDesc d, size_t total, float scale, Act act)
 {
     for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
         size_t rem = o;
@@ -70,7 +84,7 @@ __global__ void bcast_add_kernel(const float* __restrict__ a, const float* __res
             pa += c * d.sa[i];
             pb += c * d.sb[i];
         }
-        out[o] = apply_act(a[pa] + b[pb], act);
+        out[o] = apply_act(scale * combine<OP>(a[pa], b[pb]), act);
     }
 }
 
@@ -194,6 +208,7 @@ extern "C" fdx_status fdx_einsum_dense_f32(const char* equation, const char* bia
     const int64_t* full_output_shape, const fdx_act* act, float* out, int* out_rank, int64_t* out_dims)
 {
     FDX_REQUIRE(equation && in && in_dims && kernel && kernel_dims && out, "einsum_dense: null argument");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     FDX_REQUIRE(in_rank >= 1 && in_rank <= 6 && kernel_rank >= 1 && kernel_rank <= 6, "einsum_dense: ranks must be 1..6");
     EinsumSpec spec;
     std::string err;
@@ -221,7 +236,15 @@ extern "C" fdx_status fdx_einsum_dense_f32(const char* equation, const char* bia
 extern "C" fdx_status fdx_broadcast_add_f32(const float* a, const int64_t* a_dims5, const float* b, const int64_t* b_dims5,
     int batch, const fdx_act* act, float* out, int64_t* out_dims5)
 {
-    FDX_REQUIRE(a && b && a_dims5 && b_dims5 && out && batch > 0, "broadcast_add: bad arguments");
+    return fdx_broadcast_combine_f32(FDX_COMBINE_ADD, a, a_dims5, b, b_dims5, 0, batch, 1.0f, act, out, out_dims5);
+}
+
+extern "C" fdx_status fdx_broadcast_combine_f32(int op, const float* a, const int64_t* a_dims5, const float* b,
+    const int64_t* b_dims5, int b_shared, int batch, float scale, const fdx_act* act, float* out, int64_t* out_dims5)
+{
+    FDX_REQUIRE(a && b && a_dims5 && b_dims5 && out && batch > 0, "broadcast_combine: bad arguments");
+    FDX_REQUIRE(op >= FDX_COMBINE_ADD && op <= FDX_COMBINE_PRELU, "broadcast_combine: unknown operation %d", op);
+    FDX_REQUIRE_EPILOGUE_ACT(act);
     BcastDesc d {};
     int64_t va = 1, vb = 1, vo = 1;
     for (int i = 0; i < 5; ++i) {
@@ -243,11 +266,20 @@ extern "C" fdx_status fdx_broadcast_add_f32(const float* a, const int64_t* a_dim
     }
     d.dims[0] = batch;
     d.sa[0] = va;
-    d.sb[0] = vb;
+    d.sb[0] = b_shared ? 0 : vb;
     const size_t total = (size_t)batch * (size_t)vo;
+    const Act ac = make_act(act);
+    const dim3 grid(grid_of(total, 256)), block(256);
     profile_begin();
-    hipLaunchKernelGGL(bcast_add_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), a, b, out, d, total, make_act(act));
-    profile_end("broadcast_add_f32", 0.0, 4.0 * ((double)batch * (va + vb) + (double)total));
+    switch (op) {
+    case FDX_COMBINE_MUL: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_MUL>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    case FDX_COMBINE_SUB: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_SUB>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    case FDX_COMBINE_MAX: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_MAX>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    case FDX_COMBINE_MIN: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_MIN>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    case FDX_COMBINE_PRELU: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_PRELU>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    default: hipLaunchKernelGGL(bcast_combine_kernel<FDX_COMBINE_ADD>, grid, block, 0, stream(), a, b, out, d, total, scale, ac); break;
+    }
+    profile_end("broadcast_combine_f32", 0.0, 4.0 * ((double)batch * va + (double)(b_shared ? 1 : batch) * vb + (double)total));
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }

@@ -159,6 +159,21 @@ class Builder:
     def activation(self, x, name, kind):
         return self._add("Activation", name, {"activation": kind}, [x], x.shape)
 
+    def activation_layer(self, x, cls, name, cfg=None):
+        """A layer class that is one element-wise activation (LeakyReLU, ELU, Softmax, Threshold, ...)."""
+        return self._add(cls, name, dict(cfg or {}), [x], x.shape)
+
+    def prelu(self, x, name, shared_axes=None):
+        dims = [1 if (shared_axes and a + 1 in shared_axes) else d for a, d in enumerate(x.shape)]
+        self.params[name] = {"alpha": self.rng.uniform(-0.5, 0.9, int(np.prod(dims))).astype(np.float32)}
+        return self._add("PReLU", name, {"shared_axes": list(shared_axes) if shared_axes else None}, [x], x.shape)
+
+    def merge(self, xs, cls, name):
+        """Multiply / Subtract / Average / Maximum / Minimum (same shape rules as Add)."""
+        t = self.add(xs, name)
+        self.layers[-1]["class_name"] = cls
+        return t
+
     def zero_pad(self, x, name, pad):
         (pt, pb), (pl, pr) = pad
         h, w, c = x.shape

@@ -26,14 +26,35 @@ extern "C" {
 typedef int fdx_status;
 enum { FDX_OK = 0, FDX_ERR_INVALID = 1, FDX_ERR_HIP = 2, FDX_ERR_FORMAT = 3, FDX_ERR_UNSUPPORTED = 4 };
 
-/* activation fused into a producer's epilogue or applied stand-alone */
-enum { FDX_ACT_NONE = 0, FDX_ACT_RELU = 1, FDX_ACT_GELU = 2 };
+/* Activations.  NONE / RELU / GELU may be fused into any producer's epilogue; the others run through
+ * fdx_activation_f32 (the launchers that take an epilogue activation reject them).  Formulas as in
+ * include/fdeep/recurrent_ops.hpp:24-86 and include/fdeep/layers/<name>_layer.hpp; the three float fields
+ * carry each kind's parameters:
+ *   RELU         max_value, negative_slope, threshold            (relu_layer.hpp:40-46)
+ *   ELU / CELU   negative_slope = alpha: x >= 0 ? x : alpha * (e^x - 1)
+ *   LEAKY_RELU   negative_slope: x > 0 ? x : slope * x
+ *   HARD_SHRINK  threshold: |x| > thr ? x : 0          SOFT_SHRINK  threshold: x -+ thr or 0
+ *   SQUARE_PLUS  max_value = b: (x + sqrt(x^2 + b)) / 2
+ *   THRESHOLD    threshold, max_value = default value: x > thr ? x : default
+ *   LOG          natural logarithm (second half of log_softmax = log(softmax(x)), log_softmax_layer.hpp) */
+enum {
+    FDX_ACT_NONE = 0, FDX_ACT_RELU = 1, FDX_ACT_GELU = 2,
+    FDX_ACT_TANH = 3, FDX_ACT_SIGMOID = 4, FDX_ACT_SWISH = 5, FDX_ACT_HARD_SIGMOID = 6, FDX_ACT_SELU = 7, FDX_ACT_ELU = 8,
+    FDX_ACT_EXPONENTIAL = 9, FDX_ACT_SOFTSIGN = 10, FDX_ACT_SOFTPLUS = 11, FDX_ACT_LEAKY_RELU = 12, FDX_ACT_HARD_SHRINK = 13,
+    FDX_ACT_SOFT_SHRINK = 14, FDX_ACT_SPARSE_PLUS = 15, FDX_ACT_SQUARE_PLUS = 16, FDX_ACT_TANH_SHRINK = 17,
+    FDX_ACT_THRESHOLD = 18, FDX_ACT_LOG_SIGMOID = 19, FDX_ACT_HARD_TANH = 20, FDX_ACT_LOG = 21, FDX_ACT_COUNT = 22
+};
 typedef struct fdx_act {
     int kind;             /* FDX_ACT_*                                              */
-    float max_value;      /* relu family: x >= max -> max            (relu_layer.hpp:40-46) */
-    float negative_slope; /*              x < threshold -> slope * (x - threshold)  */
+    float max_value;
+    float negative_slope;
     float threshold;
 } fdx_act;
+
+/* element-wise combinations of two operands with size-1 broadcasting (fdx_broadcast_combine_f32):
+ * add_tensors / mult_tensors / subtract_tensors (include/fdeep/tensor.hpp:662-675), max_tensors / min_tensors
+ * (:893-929), and PReLU's a > 0 ? a : b * a with b the learned slopes (layers/prelu_layer.hpp:29-70) */
+enum { FDX_COMBINE_ADD = 0, FDX_COMBINE_MUL = 1, FDX_COMBINE_SUB = 2, FDX_COMBINE_MAX = 3, FDX_COMBINE_MIN = 4, FDX_COMBINE_PRELU = 5 };
 
 const char* fdx_last_error(void);
 /* lets a callback (custom layer) leave the text that fdx_last_error() reports for its failure */
@@ -165,6 +186,10 @@ fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims
  * back to back; out_dims5 (may be NULL) receives the per-axis maximum */
 fdx_status fdx_broadcast_add_f32(const float* a, const int64_t* a_dims5, const float* b, const int64_t* b_dims5,
     int batch, const fdx_act* act, float* out, int64_t* out_dims5);
+/* the same with any FDX_COMBINE_* operation, then out = act(scale * combine(a, b)) (scale serves
+ * average_tensors, tensor.hpp:886-891); b_shared != 0: one b for all samples (learned parameters) */
+fdx_status fdx_broadcast_combine_f32(int op, const float* a, const int64_t* a_dims5, const float* b, const int64_t* b_dims5,
+    int b_shared, int batch, float scale, const fdx_act* act, float* out, int64_t* out_dims5);
 /* Concatenate along one axis (concatenate_tensors, include/fdeep/tensor.hpp:459-483): input i is
  * `outer` rows of inner[i] floats (inner = extent on the axis times everything to its right, outer =
  * batch times everything to its left); rows are laid side by side in `out` */

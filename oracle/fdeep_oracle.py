@@ -181,6 +181,39 @@ def gelu(x):
     return out
 
 
+def activation(name, x, p0=0.0, p1=0.0):
+    """Any of the reference's element-wise activations by its config name (import_model.hpp:1649-1700)."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    if lib().fdo_activation(name.encode(), ctypes.c_float(p0), ctypes.c_float(p1), _p(x), ctypes.c_size_t(x.size), _p(out)) != 0:
+        raise RuntimeError("unknown activation type: " + name)
+    return out
+
+
+def combine(op, a, b):
+    """mul / sub / max / min of two tensors; size-1 axes are expanded first (tensor.hpp:642-660)."""
+    a, b = np.broadcast_arrays(_f32(a), _f32(b)) if np.shape(a) != np.shape(b) else (_f32(a), _f32(b))
+    a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+    out = np.empty_like(a)
+    lib().fdo_combine({"mul": 1, "sub": 2, "max": 3, "min": 4}[op], _p(a), _p(b), ctypes.c_size_t(a.size), _p(out))
+    return out
+
+
+def prelu(x, alpha, shared_axes):
+    """layers/prelu_layer.hpp:29-70, including the shift of the shared axis numbers for samples without a height
+    (and width) axis of their own."""
+    x = _f32(x)
+    h, w, c = ((1, 1, 1) + x.shape)[-3:]
+    shifted, shift = [], 0
+    for a in shared_axes:
+        if (a == 1 and h == 1) or (a == 2 and w == 1):
+            shift += 1
+        shifted.append(a + shift)
+    out = np.empty_like(x)
+    lib().fdo_prelu(_p(x), h, w, c, _p(_f32(alpha)), int(1 in shifted), int(2 in shifted), int(3 in shifted), _p(out))
+    return out
+
+
 def pool2d(x, pool_size, strides, padding, mode):
     x = _f32(x)
     h, w, c = x.shape
@@ -334,7 +367,31 @@ def _activation(name, cfg, x):
         return gelu(x)
     if name == "softmax":
         return softmax(x)
-    raise RuntimeError("unknown activation type: " + name)
+    if name == "log_softmax":
+        return activation("log", softmax(x))
+    # parameters and their defaults: import_model.hpp:1200-1385
+    if name in ("elu", "celu"):
+        return activation(name, x, cfg.get("alpha", 1.0))
+    if name == "leaky_relu":
+        return activation(name, x, cfg.get("negative_slope", 0.2))
+    if name in ("hard_shrink", "soft_shrink"):
+        return activation(name, x, cfg["threshold"])
+    if name == "squareplus":
+        b = cfg.get("b")
+        return activation(name, x, 4.0 if b is None else b)
+    if name == "threshold":
+        thr = cfg["threshold"] if "threshold" in cfg else cfg["threshold_value"]
+        dv = cfg["default_value"] if "default_value" in cfg else cfg["value"]
+        return activation(name, x, thr, dv)
+    return activation(name, x)
+
+
+ACTIVATION_LAYERS = {"LeakyReLU": "leaky_relu", "LeakyRelu": "leaky_relu", "ELU": "elu", "Elu": "elu", "Celu": "celu",
+                     "Relu6": "relu6", "Exp": "exponential", "Gelu": "gelu", "Selu": "selu", "Silu": "silu", "Tanh": "tanh",
+                     "TanhShrink": "tanh_shrink", "Threshold": "threshold", "Sigmoid": "sigmoid", "HardShrink": "hard_shrink",
+                     "HardSigmoid": "hard_sigmoid", "HardTanh": "hard_tanh", "SoftShrink": "soft_shrink", "Softplus": "softplus",
+                     "Softsign": "softsign", "SparsePlus": "sparse_plus", "Squareplus": "squareplus",
+                     "LogSigmoid": "log_sigmoid", "LogSoftmax": "log_softmax"}  # import_model.hpp:1839-1865
 
 
 class _Layer:
@@ -376,6 +433,8 @@ class _Layer:
             vals = [decode_floats(v) for v in get_param(name, "weights")]
             assert len(shapes) == len(vals)
             self.p["w"] = vals
+        elif cls == "PReLU":
+            self.p["alpha"] = decode_floats(get_param(name, "alpha"))
         elif cls == "EinsumDense":
             self.p["kernel"] = decode_floats(get_param(name, "kernel"))
             self.p["kernel_shape"] = [int(v) for v in get_param(name, "kernel_shape")]
@@ -414,6 +473,10 @@ class _Layer:
             out = _activation("relu", c, ins[0])
         elif cls == "Activation":
             return _activation(c["activation"], c, ins[0])
+        elif cls in ACTIVATION_LAYERS:
+            return _activation(ACTIVATION_LAYERS[cls], c, ins[0])
+        elif cls == "PReLU":
+            out = prelu(ins[0], p["alpha"], c.get("shared_axes") or [])
         elif cls == "Softmax":
             out = softmax(ins[0])
         elif cls == "ZeroPadding2D":
@@ -431,6 +494,19 @@ class _Layer:
             out = ins[0]
             for other in ins[1:]:  # left fold, tensor.hpp:677-680
                 out = add(out, other)
+        elif cls in ("Multiply", "Maximum", "Minimum"):
+            out = ins[0]
+            for other in ins[1:]:  # left folds (tensor.hpp:687-690, 893-929)
+                out = combine({"Multiply": "mul", "Maximum": "max", "Minimum": "min"}[cls], out, other)
+        elif cls == "Subtract":
+            if len(ins) != 2:
+                raise RuntimeError("subtract layer needs exactly two input tensors")
+            out = combine("sub", ins[0], ins[1])
+        elif cls == "Average":
+            out = ins[0]
+            for other in ins[1:]:
+                out = add(out, other)
+            out = (out * np.float32(1.0 / len(ins))).astype(np.float32)  # sum times 1 / n, tensor.hpp:886-891
         elif cls == "Concatenate":
             # the axis counts from the first input's rank, batch axis = 0 (tensor.hpp:459-483)
             axis = int(c["axis"])

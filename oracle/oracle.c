@@ -382,6 +382,72 @@ void fdo_gelu(const float* x, size_t n, float* y)
 }
 
 /*
+ * The other element-wise activations, one name each as the reference dispatches them
+ * (include/fdeep/import_model.hpp:1649-1700); formulas from include/fdeep/recurrent_ops.hpp:24-86 and
+ * include/fdeep/layers/<name>_layer.hpp.  p0 / p1 are the layer's parameters where it has any:
+ * elu / celu alpha, leaky_relu slope, hard_shrink / soft_shrink threshold, squareplus b,
+ * threshold (threshold, default value).  Returns -1 for a name the reference does not know.
+ */
+int fdo_activation(const char* name, float p0, float p1, const float* x, size_t n, float* y)
+{
+#define FDO_MAP(expr)                  \
+    do {                               \
+        for (size_t i = 0; i < n; ++i) { \
+            const float v = x[i];      \
+            y[i] = (expr);             \
+        }                              \
+        return 0;                      \
+    } while (0)
+    if (!strcmp(name, "tanh")) FDO_MAP(tanhf(v));
+    if (!strcmp(name, "sigmoid")) FDO_MAP(1 / (1 + expf(-v)));
+    if (!strcmp(name, "swish") || !strcmp(name, "silu")) FDO_MAP(v / (1 + expf(-v)));
+    if (!strcmp(name, "hard_sigmoid")) FDO_MAP(v < -3 ? 0.0f : (v > 3 ? 1.0f : v / 6.0f + 0.5f));
+    if (!strcmp(name, "selu"))
+        FDO_MAP(1.0507009873554804934193349852946f * (v >= 0 ? v : 1.6732632423543772848170429916717f * (expf(v) - 1)));
+    if (!strcmp(name, "elu") || !strcmp(name, "celu")) FDO_MAP(v >= 0 ? v : p0 * (expf(v) - 1));
+    if (!strcmp(name, "exponential")) FDO_MAP(expf(v));
+    if (!strcmp(name, "softsign")) FDO_MAP(v / (fabsf(v) + 1.0f));
+    if (!strcmp(name, "softplus")) {
+        const float threshold = logf(FLT_EPSILON) + 2; /* layers/softplus_layer.hpp */
+        FDO_MAP(v > -threshold ? v : (v < threshold ? expf(v) : log1pf(expf(v))));
+    }
+    if (!strcmp(name, "leaky_relu")) FDO_MAP(v > 0 ? v : p0 * v);
+    if (!strcmp(name, "hard_shrink")) FDO_MAP(fabsf(v) > p0 ? v : 0.0f);
+    if (!strcmp(name, "soft_shrink")) FDO_MAP(v > p0 ? v - p0 : (v < -p0 ? v + p0 : 0.0f));
+    if (!strcmp(name, "sparse_plus")) FDO_MAP(v <= -1 ? 0.0f : (v < 1 ? 0.25f * (v + 1.0f) * (v + 1.0f) : v));
+    if (!strcmp(name, "squareplus")) FDO_MAP((v + sqrtf(v * v + p0)) / 2.0f);
+    if (!strcmp(name, "tanh_shrink")) FDO_MAP(v - tanhf(v));
+    if (!strcmp(name, "threshold")) FDO_MAP(v > p0 ? v : p1);
+    if (!strcmp(name, "log_sigmoid")) FDO_MAP(logf(1 / (1 + expf(-v))));
+    if (!strcmp(name, "hard_tanh")) FDO_MAP(v < -1 ? -1.0f : (v > 1 ? 1.0f : v));
+    if (!strcmp(name, "log")) FDO_MAP(logf(v)); /* second half of log_softmax = log(softmax(x)) */
+#undef FDO_MAP
+    return -1;
+}
+
+/* element-wise merges of equal-shaped tensors: mult / subtract (include/fdeep/tensor.hpp:667-675),
+ * max_tensors / min_tensors (:893-929); op 1 mul, 2 sub, 3 max, 4 min */
+void fdo_combine(int op, const float* a, const float* b, size_t n, float* y)
+{
+    for (size_t i = 0; i < n; ++i)
+        y[i] = op == 1 ? a[i] * b[i] : op == 2 ? a[i] - b[i] : op == 3 ? (a[i] > b[i] ? a[i] : b[i]) : (a[i] < b[i] ? a[i] : b[i]);
+}
+
+/* PReLU on a (h, w, c) sample: x > 0 ? x : alpha[pos] * x with alpha laid out over the axes that are not shared
+ * (include/fdeep/layers/prelu_layer.hpp:46-66) */
+void fdo_prelu(const float* x, int h, int w, int c, const float* alpha, int h_shared, int w_shared, int c_shared, float* y)
+{
+    const int aw = w_shared ? 1 : w, ac = c_shared ? 1 : c;
+    for (int yy = 0; yy < h; ++yy)
+        for (int xx = 0; xx < w; ++xx)
+            for (int z = 0; z < c; ++z) {
+                const size_t i = ((size_t)yy * w + xx) * c + z;
+                const size_t pos = (size_t)(h_shared ? 0 : yy) * aw * ac + (size_t)(w_shared ? 0 : xx) * ac + (c_shared ? 0 : z);
+                y[i] = x[i] > 0 ? x[i] : alpha[pos] * x[i];
+            }
+}
+
+/*
  * Max / average 2-D pooling with TF padding; padded taps carry the lowest()
  * sentinel: ignored by max and left out of the average's divisor.
  * include/fdeep/layers/pooling_3d_layer.hpp:44-79, max_pooling_3d_layer.hpp:17-38,

@@ -225,3 +225,83 @@ def test_custom_layer_runs_on_host_between_device_segments(fdx, oracle, modelgen
         return run
     with pytest.raises(fdx.FdxError, match="custom layer failed.*boom in pairs"):
         fdx.Model(js, custom_layers={"PairSum": broken}).predict([x])
+
+
+ACTS = [("tanh", ()), ("sigmoid", ()), ("swish", ()), ("hard_sigmoid", ()), ("selu", ()), ("elu", (0.7,)), ("celu", (1.0,)),
+        ("exponential", ()), ("softsign", ()), ("softplus", ()), ("leaky_relu", (0.2,)), ("hard_shrink", (0.5,)),
+        ("soft_shrink", (0.5,)), ("sparse_plus", ()), ("squareplus", (4.0,)), ("tanh_shrink", ()), ("threshold", (0.25, -2.0)),
+        ("log_sigmoid", ()), ("hard_tanh", ())]
+
+
+@pytest.mark.parametrize("name,params", ACTS, ids=[a[0] for a in ACTS])
+def test_activation_kinds(fdx, oracle, name, params):
+    say("activation", name)
+    r = np.random.default_rng(12)
+    x = np.concatenate([r.standard_normal(1021) * 3, [-20.0, -14.0, -13.5, -3.0, -1.0, -0.5, 0.0, 0.25, 0.5, 1.0, 3.0, 13.5, 14.0, 20.0]])
+    x = x.astype(np.float32)
+    want = oracle.activation(name, x, *params)
+    got = fdx.activation(x, fdx.named_act(name, *params))
+    assert (np.abs(got - want) / np.maximum(np.abs(want), 1.0)).max() <= 2e-6
+
+
+def test_epilogue_launchers_reject_other_activations(fdx):
+    x = np.zeros((2, 4, 4, 8), np.float32)
+    with pytest.raises(fdx.FdxError, match="fuses only NONE / RELU / GELU"):
+        fdx.conv2d(x, np.zeros((8, 1, 1, 8), np.float32), None, act=fdx.named_act("tanh"))
+
+
+@pytest.mark.parametrize("op", ["mul", "sub", "max", "min"])
+def test_broadcast_combine(fdx, oracle, op):
+    say("combine", op)
+    r = np.random.default_rng(13)
+    a = r.standard_normal((3, 4, 5, 6)).astype(np.float32)
+    for bshape in ((4, 5, 6), (1, 5, 1), (4, 1, 6)):
+        b = r.standard_normal((3,) + bshape).astype(np.float32)
+        want = np.stack([oracle.combine(op, a[i], b[i]) for i in range(3)])
+        assert np.array_equal(fdx.broadcast_combine(op, a, b), want)
+    got = fdx.broadcast_combine("add", a, a[::-1].copy(), scale=0.5)   # Average of two
+    assert np.array_equal(got, ((a + a[::-1]) * np.float32(0.5)).astype(np.float32))
+
+
+def test_prelu_kernel(fdx, oracle):
+    r = np.random.default_rng(14)
+    x = r.standard_normal((3, 5, 6, 8)).astype(np.float32)
+    for shared, ashape in (([1, 2], (1, 1, 8)), ([], (5, 6, 8)), ([3], (5, 6, 1)), ([2], (5, 1, 8))):
+        alpha = r.uniform(-1, 1, ashape).astype(np.float32)
+        want = np.stack([oracle.prelu(x[i], alpha.reshape(-1), shared) for i in range(3)])
+        assert np.array_equal(fdx.broadcast_combine("prelu", x, alpha, b_shared=True), want)
+
+
+def test_model_with_activations_and_merges(fdx, oracle, modelgen):
+    """Stand-alone activation layers, activations named in a layer's config (fused or not), PReLU, log_softmax, and the
+    Multiply / Subtract / Average / Maximum / Minimum merges, against the oracle."""
+    say("activation / merge model")
+    b = modelgen.Builder("acts", 61)
+    x = b.input((6, 6, 8), "x")
+    c1 = b.conv2d(x, 8, 3, "c1", padding="same", activation="swish", bias_std=0.2)
+    c2 = b.conv2d(x, 8, 1, "c2", activation="tanh", bias_std=0.2)
+    l1 = b.activation_layer(c1, "LeakyReLU", "leaky", {"negative_slope": 0.3})
+    e1 = b.activation_layer(c2, "ELU", "elu", {"alpha": 0.5})
+    p1 = b.prelu(l1, "prelu", shared_axes=[1, 2])
+    mul = b.merge([p1, e1], "Multiply", "mul")
+    sub = b.merge([mul, c1], "Subtract", "sub")
+    avg = b.merge([sub, c2, x], "Average", "avg")
+    mx = b.merge([avg, p1], "Maximum", "mx")
+    mn = b.merge([mx, e1], "Minimum", "mn")
+    sp = b.activation(mn, "softplus_act", "softplus")
+    hs = b.activation_layer(sp, "HardSigmoid", "hsig")
+    th = b.activation_layer(hs, "Threshold", "thr", {"threshold": 0.55, "default_value": -1.0})
+    g = b.gap(th, "gap")
+    d = b.dense(g, 5, "fc", activation="log_softmax", bias_std=0.2)
+    spec = b.finish([d, mn, th])
+    xs = np.random.default_rng(15).standard_normal((4, 6, 6, 8)).astype(np.float32)
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([xs[i]]) for i in range(4)]
+    want = [np.stack([w[k] for w in want]) for k in range(3)]
+    got = fdx.Model(js).predict([xs])
+    # the threshold layer is discontinuous: an input within rounding of the threshold may fall on either side
+    errs = [rel(got[0], want[0]), rel(got[1], want[1])]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= TOL
+    assert (np.abs(got[2] - want[2]) > 1e-4).mean() < 0.01

@@ -6,6 +6,8 @@ import math
 
 import numpy as np
 import pytest
+import torch
+from scipy import special
 
 TOL = 2e-5
 
@@ -323,3 +325,61 @@ def test_einsum_dense_vs_numpy(oracle, eq, xs, ks, bias_axes):
     got = oracle.einsum_dense(x, eq, k, list(ks), bias, bias_axes)
     assert got.shape == want.shape[1:]
     assert rel(got, want[0]) < TOL
+
+
+ACTIVATION_PINS = [
+    # name, oracle parameters, independent float64 statement (torch / numpy / scipy, none of them the reference)
+    ("tanh", (), lambda x: np.tanh(x)),
+    ("sigmoid", (), lambda x: special.expit(x)),
+    ("swish", (), lambda x: torch.nn.functional.silu(torch.from_numpy(x)).numpy()),
+    ("silu", (), lambda x: x * special.expit(x)),
+    ("hard_sigmoid", (), lambda x: torch.nn.functional.hardsigmoid(torch.from_numpy(x)).numpy()),
+    ("selu", (), lambda x: torch.nn.functional.selu(torch.from_numpy(x)).numpy()),
+    ("elu", (0.7,), lambda x: torch.nn.functional.elu(torch.from_numpy(x), 0.7).numpy()),
+    ("celu", (1.0,), lambda x: torch.nn.functional.celu(torch.from_numpy(x), 1.0).numpy()),
+    ("exponential", (), lambda x: np.exp(x)),
+    ("softsign", (), lambda x: torch.nn.functional.softsign(torch.from_numpy(x)).numpy()),
+    ("softplus", (), lambda x: np.logaddexp(0.0, x)),
+    ("leaky_relu", (0.2,), lambda x: torch.nn.functional.leaky_relu(torch.from_numpy(x), 0.2).numpy()),
+    ("hard_shrink", (0.5,), lambda x: torch.nn.functional.hardshrink(torch.from_numpy(x), 0.5).numpy()),
+    ("soft_shrink", (0.5,), lambda x: torch.nn.functional.softshrink(torch.from_numpy(x), 0.5).numpy()),
+    ("sparse_plus", (), lambda x: np.where(x <= -1, 0.0, np.where(x < 1, 0.25 * (x + 1) ** 2, x))),
+    ("squareplus", (4.0,), lambda x: (x + np.sqrt(x * x + 4.0)) / 2),
+    ("tanh_shrink", (), lambda x: torch.nn.functional.tanhshrink(torch.from_numpy(x)).numpy()),
+    ("threshold", (0.25, -2.0), lambda x: torch.nn.functional.threshold(torch.from_numpy(x), 0.25, -2.0).numpy()),
+    ("log_sigmoid", (), lambda x: torch.nn.functional.logsigmoid(torch.from_numpy(x)).numpy()),
+    ("hard_tanh", (), lambda x: torch.nn.functional.hardtanh(torch.from_numpy(x)).numpy()),
+]
+
+
+@pytest.mark.parametrize("name,params,ref", ACTIVATION_PINS, ids=[a[0] for a in ACTIVATION_PINS])
+def test_activation_vs_float64(oracle, name, params, ref):
+    r = np.random.default_rng(3)
+    x = np.concatenate([r.standard_normal(500) * 3, [-20.0, -14.0, -13.5, -3.0, -1.0, -0.5, 0.0, 0.25, 0.5, 1.0, 3.0, 13.5, 14.0, 20.0]])  # thresholds exact in float
+    x = x.astype(np.float32)
+    want = ref(x.astype(np.float64))
+    got = oracle.activation(name, x, *params)
+    scale = np.maximum(np.abs(want), 1.0)
+    assert (np.abs(got - want) / scale).max() <= 3e-6
+    with pytest.raises(RuntimeError, match="unknown activation type"):
+        oracle.activation("no_such_activation", x)
+
+
+def test_log_softmax_prelu_and_merges(oracle):
+    r = np.random.default_rng(4)
+    x = r.standard_normal((5, 7, 6)).astype(np.float32)
+    got = oracle._activation("log_softmax", {}, x)
+    assert np.abs(got - special.log_softmax(x.astype(np.float64), axis=-1)).max() <= 2e-6
+    y = r.standard_normal((5, 7, 6)).astype(np.float32)
+    for op, f in (("mul", np.multiply), ("sub", np.subtract), ("max", np.maximum), ("min", np.minimum)):
+        assert np.array_equal(oracle.combine(op, x, y), f(x, y))
+    assert np.array_equal(oracle.combine("mul", x, y[:, :1, :]), x * y[:, :1, :])  # size-1 broadcasting
+    # PReLU: alpha over the axes that are not shared; torch's prelu covers the channel-only case
+    alpha = r.uniform(-1, 1, 6).astype(np.float32)
+    want = torch.nn.functional.prelu(torch.from_numpy(x).permute(2, 0, 1)[None], torch.from_numpy(alpha))[0].permute(1, 2, 0).numpy()
+    assert np.array_equal(oracle.prelu(x, alpha, [1, 2]), want)
+    full = r.uniform(-1, 1, x.size).astype(np.float32)
+    assert np.array_equal(oracle.prelu(x, full, []), np.where(x > 0, x, full.reshape(x.shape) * x))
+    # a (T, D) sample has no height axis: Keras' shared axis 1 (the sequence) is the reference's width axis
+    seq = r.standard_normal((7, 6)).astype(np.float32)
+    assert np.array_equal(oracle.prelu(seq, alpha, [1]), np.where(seq > 0, seq, alpha[None, :] * seq))
