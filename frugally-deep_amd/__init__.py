@@ -274,6 +274,20 @@ def layernorm_axes(x, axes, gamma, beta, eps):
     return out.to_host(x.shape)
 
 
+def rmsnorm_axes(x, axes, scale, eps):
+    x = np.ascontiguousarray(x, np.float32)
+    rank = x.ndim - 1
+    mask = 0
+    for a in axes:
+        a = a + rank + 1 if a < 0 else a
+        mask |= 1 << (5 - rank + a - 1)
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    ds = None if scale is None else DevBuf.from_host(scale)
+    check(lib.fdx_rmsnorm_axes_f32(_dp(dx), x.shape[0], _dims5(x.shape[1:]), ctypes.c_uint(mask), _dp(ds), ctypes.c_float(eps),
+                                   _dp(out)))
+    return out.to_host(x.shape)
+
+
 def broadcast_add(a, b, act=None):
     """a, b: (batch, ...sample dims) with right-aligned size-1 broadcasting between the samples."""
     a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)

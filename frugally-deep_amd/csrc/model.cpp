@@ -540,6 +540,141 @@ namespace {
                 }
                 op.cout = (int)mean.size();
                 result = add_op(std::move(op));
+            } else if (cls == "SeparableConv2D" || cls == "SeparableConv1D") {
+                // depthwise part without bias or activation, then a 1x1 valid convolution that carries the bias and the
+                // layer's activation (layers/separable_conv_2d_layer.hpp:26-55, import_model.hpp:558-592)
+                Op dw;
+                dw.kind = OpKind::DWConv2D;
+                dw.name = op.name + "_depthwise_part";
+                dw.cls = cls;
+                dw.in = ins;
+                dw.padding = padding_from(cfg.at("padding").str());
+                pair_from(cfg.at("strides"), dw.sy, dw.sx);
+                pair_from(cfg.at("dilation_rate"), dw.dy, dw.dx);
+                pair_from(cfg.at("kernel_size"), dw.kh, dw.kw);
+                std::vector<float> sw = decode_floats(param(sc, c.layer, "slice_weights"));
+                if (sw.size() % ((size_t)dw.kh * dw.kw) != 0)
+                    throw FormatError("invalid number of weights");
+                const int ch = (int)(sw.size() / ((size_t)dw.kh * dw.kw));
+                dw.cout = dw.n_in = ch;
+                dw.hw.resize(2);
+                dw.hw[0].resize(sw.size()); // [c][kh][kw] -> [kh][kw][c]
+                for (int z = 0; z < ch; ++z)
+                    for (int t = 0; t < dw.kh * dw.kw; ++t)
+                        dw.hw[0][(size_t)t * ch + z] = sw[(size_t)z * dw.kh * dw.kw + t];
+                dw.hw[1].assign(ch, 0.f);
+                const int dwi = add_op(std::move(dw));
+                op.kind = OpKind::Conv2D;
+                op.in = { dwi };
+                op.cout = (int)cfg.at("filters").integer();
+                op.n_in = ch;
+                op.hw.resize(2);
+                op.hw[0] = decode_floats(param(sc, c.layer, "stack_weights")); // [cout][1][1][cin]
+                if (op.hw[0].size() != (size_t)op.cout * ch)
+                    throw FormatError("invalid weights sizes");
+                if (cfg.at("use_bias").boolean())
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
+                else
+                    op.hw[1].assign(op.cout, 0.f);
+                if ((int)op.hw[1].size() != op.cout)
+                    throw FormatError("size of bias does not match");
+                result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (cls == "RMSNormalization") {
+                op.kind = OpKind::LayerNorm;
+                op.rms = true;
+                op.hw.resize(2);
+                op.hw[0] = decode_floats(param(sc, c.layer, "scale"));
+                op.cout = (int)op.hw[0].size();
+                op.eps = (float)cfg.at("epsilon").number();
+                const Value& ax = cfg.at("axis");
+                if (ax.is_array())
+                    for (const auto& a : ax.arr)
+                        op.target_shape.push_back(a.integer());
+                else
+                    op.target_shape.push_back(ax.integer());
+                result = add_op(std::move(op));
+            } else if (cls == "GroupQueryAttention" || cls == "GroupedQueryAttention") {
+                // import_model.hpp:1445-1466, layers/group_query_attention_layer.hpp.  Runs on the attention op of
+                // MultiHeadAttention with the key / value kernels repeated once per query head of their group.
+                op.kind = OpKind::MHA;
+                const int hd = (int)cfg.at("head_dim").integer(), hq = (int)cfg.at("num_query_heads").integer(),
+                          hkv = (int)cfg.at("num_key_value_heads").integer();
+                op.use_bias = cfg.at("use_bias").boolean();
+                const Value* ug = cfg.find("use_gate");
+                op.gate = ug && ug->is_bool() && ug->boolean();
+                if (hkv <= 0)
+                    throw FormatError("num_key_value_heads must be > 0.");
+                if (hq % hkv != 0)
+                    throw FormatError("num_query_heads must be divisible by num_key_value_heads.");
+                if (ins.size() != 2 && ins.size() != 3)
+                    throw FormatError("GroupQueryAttention requires 2 or 3 inputs (query, value[, key]).");
+                const Value& vals = param(sc, c.layer, "weights");
+                const size_t step = op.use_bias ? 2 : 1, n_proj = op.gate ? 5 : 4;
+                if (!vals.is_array() || vals.size() != step * n_proj)
+                    throw FormatError("GroupQueryAttention: unexpected number of weights");
+                std::vector<std::vector<float>> w;
+                for (const auto& v : vals.arr)
+                    w.push_back(decode_floats(v));
+                op.heads = hq;
+                op.dk = op.dv = hd;
+                const int group = hq / hkv;
+                int d_in = -1;
+                // (D, heads, hd) -> [hq*hd][D], head h of the result read from head h / rep of the file
+                auto kernel_t = [&](const std::vector<float>& k, int heads, int rep) {
+                    if (k.size() % ((size_t)heads * hd) != 0)
+                        throw FormatError("GroupQueryAttention: kernel size does not match the head layout");
+                    const int d = (int)(k.size() / ((size_t)heads * hd));
+                    if (d_in >= 0 && d != d_in)
+                        throw FormatError("GroupQueryAttention kernels disagree on the input depth");
+                    d_in = d;
+                    std::vector<float> t((size_t)heads * rep * hd * d);
+                    for (int h = 0; h < heads * rep; ++h)
+                        for (int cc = 0; cc < hd; ++cc)
+                            for (int i = 0; i < d; ++i)
+                                t[((size_t)h * hd + cc) * d + i] = k[((size_t)i * heads + h / rep) * hd + cc];
+                    return t;
+                };
+                auto bias_of = [&](size_t proj, int heads, int rep) {
+                    std::vector<float> b((size_t)heads * rep * hd, 0.f);
+                    if (op.use_bias) {
+                        const std::vector<float>& src = w[proj * step + 1];
+                        if (src.size() != (size_t)heads * hd)
+                            throw FormatError("GroupQueryAttention: bias size does not match the head layout");
+                        for (int h = 0; h < heads * rep; ++h)
+                            for (int cc = 0; cc < hd; ++cc)
+                                b[(size_t)h * hd + cc] = src[(size_t)(h / rep) * hd + cc];
+                    }
+                    return b;
+                };
+                const size_t vi = op.gate ? 3 : 2, oi = op.gate ? 4 : 3;
+                op.hw.resize(op.gate ? 10 : 8);
+                op.hw[0] = kernel_t(w[0], hq, 1);
+                op.hw[1] = bias_of(0, hq, 1);
+                op.hw[2] = kernel_t(w[step], hkv, group);
+                op.hw[3] = bias_of(1, hkv, group);
+                op.hw[4] = kernel_t(w[vi * step], hkv, group);
+                op.hw[5] = bias_of(vi, hkv, group);
+                op.d_in = d_in;
+                const std::vector<float>& ow = w[oi * step]; // (hq, hd, Dout) -> [Dout][hq*hd]
+                const int kin = hq * hd;
+                if (ow.size() % (size_t)kin != 0)
+                    throw FormatError("Invalid output kernel shape for GroupQueryAttention");
+                op.dout = (int)(ow.size() / (size_t)kin);
+                op.hw[6].resize(ow.size());
+                for (int i = 0; i < kin; ++i)
+                    for (int o2 = 0; o2 < op.dout; ++o2)
+                        op.hw[6][(size_t)o2 * kin + i] = ow[(size_t)i * op.dout + o2];
+                op.hw[7].assign((size_t)op.dout, 0.f);
+                if (op.use_bias) {
+                    if (w[oi * step + 1].size() != (size_t)op.dout)
+                        throw FormatError("GroupQueryAttention: output bias size");
+                    op.hw[7] = w[oi * step + 1];
+                }
+                if (op.gate) {
+                    op.hw[8] = kernel_t(w[2 * step], hq, 1);
+                    op.hw[9] = bias_of(2, hq, 1);
+                }
+                result = add_op(std::move(op));
             } else if (cls == "LayerNormalization") {
                 op.kind = OpKind::LayerNorm;
                 op.hw.resize(2);
@@ -1199,8 +1334,8 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
         if (o.kind == OpKind::MHA) { // per-op scratch: placed while inputs and output are live, free again afterwards
             const int64_t T = p->shapes[o.in[0]][0], S = p->shapes[o.in[1]][0];
             const size_t nk = (size_t)o.heads * o.dk, nv = (size_t)o.heads * o.dv, fb = sizeof(float) * (size_t)batch;
-            const size_t sizes[5] = { fb * T * nk, fb * S * nk, fb * S * nv, fb * T * nv,
-                fdx_mha_scratch_bytes(batch, o.heads, (int)T, (int)S, o.dv) };
+            const size_t sizes[6] = { fb * T * nk, fb * S * nk, fb * S * nv, fb * T * nv,
+                fdx_mha_scratch_bytes(batch, o.heads, (int)T, (int)S, o.dv), o.gate ? fb * T * nv : (size_t)256 };
             std::vector<int> held;
             for (size_t sz : sizes) {
                 int b = -1;
@@ -1299,7 +1434,8 @@ namespace {
             }
             FDX_REQUIRE(o.cout == 0 || o.cout == count, "%s: gamma / beta do not match the normalised axes",
                 o.name.c_str());
-            st = fdx_layernorm_axes_f32(in0, B, dims5, mask, o.dw[0], o.dw[1], o.eps, out);
+            st = o.rms ? fdx_rmsnorm_axes_f32(in0, B, dims5, mask, o.dw[0], o.eps, out)
+                       : fdx_layernorm_axes_f32(in0, B, dims5, mask, o.dw[0], o.dw[1], o.eps, out);
             break;
         }
         case OpKind::Act:
@@ -1494,6 +1630,16 @@ namespace {
                 return st;
             if ((st = fdx_mha_prefill_f32(q, k, v, B, T, S, H, o.dk, o.dv, 0, merged, scratch)) != FDX_OK)
                 return st;
+            if (o.gate) { // attention output times sigmoid(gate projection of the query) (group_query_attention_layer.hpp:157-164)
+                float* gbuf = tmp[5];
+                const fdx_act sg = { FDX_ACT_SIGMOID, 0.f, 0.f, 0.f };
+                const size_t n = (size_t)B * (size_t)T * (size_t)nv;
+                int64_t flat[5] = { 1, 1, 1, 1, (int64_t)n };
+                if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[8], D, B * T, (int)nv, D, 1.f, o.dw[9], 0, nullptr, nullptr, gbuf, nv, nullptr)) != FDX_OK
+                    || (st = fdx_activation_f32(gbuf, n, &sg, gbuf)) != FDX_OK
+                    || (st = fdx_broadcast_combine_f32(FDX_COMBINE_MUL, merged, flat, gbuf, flat, 0, 1, 1.0f, nullptr, merged, nullptr)) != FDX_OK)
+                    return st;
+            }
             st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, B * T, o.dout, (int)nv, 1.f, o.dw[7], 0, nullptr, nullptr, out,
                 o.dout, nullptr);
             break;

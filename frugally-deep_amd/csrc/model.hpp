@@ -57,6 +57,8 @@ struct Op {
     int combine = 0;                 // Add-like merges: FDX_COMBINE_* operation
     float scale = 1.0f;              // Average: 1 / number of inputs
     bool log_after = false;          // Softmax op that is a log_softmax
+    bool rms = false;                // LayerNorm op that is an RMSNormalization
+    bool gate = false;               // attention with a sigmoid gate on its output (GroupQueryAttention use_gate)
     std::vector<int64_t> shared_axes; // PReLU
 
     // host weights (released after upload)

@@ -693,6 +693,13 @@ extern "C" fdx_status fdx_session_create(fdx_model* m, int batch, int max_len, f
         const Op& o = m->ops[s->order[p]];
         if (o.dead)
             continue;
+        // layer variants the cached step does not implement
+        if ((o.kind == OpKind::LayerNorm && o.rms) || (o.kind == OpKind::Add && (o.combine != FDX_COMBINE_ADD || o.scale != 1.0f))
+            || (o.kind == OpKind::Softmax && o.log_after) || (o.kind == OpKind::MHA && o.gate)
+            || (o.kind == OpKind::Act && !(o.act.kind == FDX_ACT_RELU || o.act.kind == FDX_ACT_GELU || o.act.kind == FDX_ACT_NONE))) {
+            set_error("session_create: layer %s (%s) is not supported inside a decode session", o.name.c_str(), o.cls.c_str());
+            return FDX_ERR_UNSUPPORTED;
+        }
         switch (o.kind) {
         case OpKind::Input: case OpKind::Embedding: case OpKind::Add: case OpKind::LayerNorm: case OpKind::Act:
         case OpKind::Softmax: case OpKind::Dense: case OpKind::View:

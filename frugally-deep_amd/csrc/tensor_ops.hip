@@ -108,6 +108,8 @@ struct NormDesc {
 // mean of squared differences, then x * inv + (beta - mean * inv) with inv = gamma / sqrt(var + eps)
 // (include/fdeep/tensor.hpp:758-793, layers/layer_normalization_layer.hpp:37-61); gamma / beta are
 // indexed by the position on the normalised axes.
+// RMS: no mean, x / sqrt(mean(x^2) + eps) * gamma (include/fdeep/layers/rms_normalization_layer.hpp:37-69).
+template <bool RMS>
 __global__ __launch_bounds__(256) void layernorm_axes_kernel(const float* __restrict__ x, float* __restrict__ out, NormDesc d,
     int64_t groups, int64_t count, const float* __restrict__ gamma, const float* __restrict__ beta, float eps)
 {
@@ -132,12 +134,13 @@ __global__ __launch_bounds__(256) void layernorm_axes_kernel(const float* __rest
         return off;
     };
     float s = 0.f;
-    for (int64_t e = lane; e < count; e += 64)
-        s += x[offset(e)];
+    if (!RMS)
+        for (int64_t e = lane; e < count; e += 64)
+            s += x[offset(e)];
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1)
         s += __shfl_xor(s, o, 64);
-    const float mean = s / (float)count;
+    const float mean = RMS ? 0.f : s / (float)count;
     float v = 0.f;
     for (int64_t e = lane; e < count; e += 64) {
         const float df = x[offset(e)] - mean;
@@ -304,8 +307,8 @@ extern "C" fdx_status fdx_concat_f32(const float* const* ins, int n_inputs, cons
     return FDX_OK;
 }
 
-extern "C" fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
-    const float* beta, float eps, float* out)
+static fdx_status norm_axes(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
+    const float* beta, float eps, float* out, bool rms)
 {
     FDX_REQUIRE(x && dims5 && out && batch > 0 && axes_mask != 0 && axes_mask < 32, "layernorm_axes: bad arguments");
     int64_t vol = 1;
@@ -324,7 +327,7 @@ extern "C" fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const in
         for (int j = i; j >= 0; --j)
             if (((axes_mask >> j) & 1u) && dims5[j] != 1)
                 rest_kept = false;
-        if (rest_kept && depth < (1LL << 31))
+        if (!rms && rest_kept && depth < (1LL << 31))
             return fdx_layernorm_f32(x, (int64_t)batch * vol / depth, (int)depth, gamma, beta, eps, out);
     }
     NormDesc d {};
@@ -345,9 +348,25 @@ extern "C" fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const in
         }
     }
     profile_begin();
-    hipLaunchKernelGGL(layernorm_axes_kernel, dim3((unsigned)((groups + 3) / 4)), dim3(256), 0, stream(), x, out, d, groups, count,
-        gamma, beta, eps);
-    profile_end("layernorm_axes_f32", 0.0, 8.0 * (double)batch * (double)vol);
+    if (rms)
+        hipLaunchKernelGGL(layernorm_axes_kernel<true>, dim3((unsigned)((groups + 3) / 4)), dim3(256), 0, stream(), x, out, d, groups,
+            count, gamma, nullptr, eps);
+    else
+        hipLaunchKernelGGL(layernorm_axes_kernel<false>, dim3((unsigned)((groups + 3) / 4)), dim3(256), 0, stream(), x, out, d, groups,
+            count, gamma, beta, eps);
+    profile_end(rms ? "rmsnorm_axes_f32" : "layernorm_axes_f32", 0.0, 8.0 * (double)batch * (double)vol);
     FDX_LAUNCH_CHECK();
     return FDX_OK;
+}
+
+extern "C" fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
+    const float* beta, float eps, float* out)
+{
+    return norm_axes(x, batch, dims5, axes_mask, gamma, beta, eps, out, false);
+}
+
+extern "C" fdx_status fdx_rmsnorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* scale,
+    float eps, float* out)
+{
+    return norm_axes(x, batch, dims5, axes_mask, scale, nullptr, eps, out, true);
 }

@@ -159,6 +159,48 @@ class Builder:
     def activation(self, x, name, kind):
         return self._add("Activation", name, {"activation": kind}, [x], x.shape)
 
+    def separable_conv2d(self, x, filters, k, name, strides=1, padding="valid", use_bias=True, activation=None, dilation=1):
+        h, w, cin = x.shape
+        self.params[name] = {"slice_weights": self.he((cin, k, k), k * k), "stack_weights": self.he((filters, 1, 1, cin), cin)}
+        if use_bias:
+            self.params[name]["bias"] = self.normal((filters,), 0.2)
+        cfg = {"filters": filters, "kernel_size": [k, k], "strides": [strides, strides], "dilation_rate": [dilation, dilation],
+               "padding": padding, "use_bias": use_bias}
+        if activation is not None:
+            cfg["activation"] = activation
+        ek = (k - 1) * dilation + 1
+        return self._add("SeparableConv2D", name, cfg, [x], (self._win(h, ek, strides, padding), self._win(w, ek, strides, padding), filters))
+
+    def rmsnorm(self, x, name, axes=(-1,), eps=1e-6):
+        rank = len(x.shape)
+        pos = sorted(set(a + rank + 1 if a < 0 else a for a in axes))
+        n = int(np.prod([x.shape[a - 1] for a in pos]))
+        self.params[name] = {"scale": (0.5 + self.rng.random(n)).astype(np.float32)}
+        return self._add("RMSNormalization", name, {"axis": list(axes), "epsilon": eps}, [x], x.shape)
+
+    def gqa(self, q, v, name, head_dim, num_query_heads, num_kv_heads, use_bias=True, use_gate=False, k=None, std=0.2):
+        """GroupQueryAttention; weights in Keras order Q, K, [Gate], V, Out, each bias right after its kernel."""
+        d = q.shape[-1]
+        shapes, vals = [], []
+
+        def put(kshape, bshape):
+            shapes.append(list(kshape))
+            vals.append(self.normal(kshape, std))
+            if use_bias:
+                shapes.append(list(bshape))
+                vals.append(self.normal(bshape, 0.2))
+
+        put((d, num_query_heads, head_dim), (num_query_heads, head_dim))
+        put((d, num_kv_heads, head_dim), (num_kv_heads, head_dim))
+        if use_gate:
+            put((d, num_query_heads, head_dim), (num_query_heads, head_dim))
+        put((d, num_kv_heads, head_dim), (num_kv_heads, head_dim))
+        put((num_query_heads, head_dim, d), (d,))
+        self.params[name] = {"weight_shapes": shapes, "weights": vals}
+        cfg = {"head_dim": head_dim, "num_query_heads": num_query_heads, "num_key_value_heads": num_kv_heads,
+               "use_bias": use_bias, "use_gate": use_gate}
+        return self._add("GroupedQueryAttention", name, cfg, [q, v] + ([k] if k is not None else []), q.shape[:-1] + (d,))
+
     def activation_layer(self, x, cls, name, cfg=None):
         """A layer class that is one element-wise activation (LeakyReLU, ELU, Softmax, Threshold, ...)."""
         return self._add(cls, name, dict(cfg or {}), [x], x.shape)

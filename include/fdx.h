@@ -181,6 +181,10 @@ fdx_status fdx_layernorm_f32(const float* x, int64_t rows, int depth, const floa
  * row kernel above. */
 fdx_status fdx_layernorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* gamma,
     const float* beta, float eps, float* out);
+/* RMSNormalization over the selected axes: x / sqrt(mean(x^2) + eps) * scale
+ * (include/fdeep/layers/rms_normalization_layer.hpp:37-69); arguments as fdx_layernorm_axes_f32 */
+fdx_status fdx_rmsnorm_axes_f32(const float* x, int batch, const int64_t* dims5, unsigned axes_mask, const float* scale,
+    float eps, float* out);
 /* out = act(a + b) with size-1 broadcasting on any of the five right-aligned axes, per sample
  * (elem_wise_combine_tensors, include/fdeep/tensor.hpp:642-660); `batch` samples of each operand lie
  * back to back; out_dims5 (may be NULL) receives the per-axis maximum */

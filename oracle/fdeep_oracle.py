@@ -282,6 +282,41 @@ def mha(query, value, key, heads, dk, dv, weights, use_bias):
     return out
 
 
+def gqa(query, value, key, head_dim, hq, hkv, weights, use_bias, use_gate):
+    """GroupQueryAttention; weights in Keras order Q, K, [Gate], V, Out with each bias right after its kernel
+    (include/fdeep/layers/group_query_attention_layer.hpp:45-60)."""
+    q, v = _f32(query), _f32(value)
+    k = v if key is None else _f32(key)
+    step = 2 if use_bias else 1
+    w = [_f32(a).reshape(-1) for a in weights]
+    def kern(i):
+        return w[i * step]
+    def bias(i):
+        return w[i * step + 1] if use_bias else None
+    vi, oi = (3, 4) if use_gate else (2, 3)
+    dout = kern(oi).size // (hq * head_dim)
+    out = np.empty((q.shape[0], dout), np.float32)
+    rc = lib().fdo_gqa(_p(q), q.shape[0], _p(v), _p(k), v.shape[0], q.shape[1], head_dim, hq, hkv, _p(kern(0)), _p(bias(0)),
+                       _p(kern(1)), _p(bias(1)), _p(kern(2)) if use_gate else None, _p(bias(2)) if use_gate else None,
+                       _p(kern(vi)), _p(bias(vi)), _p(kern(oi)), _p(bias(oi)), dout, _p(out))
+    if rc != 0:
+        raise RuntimeError("num_query_heads must be divisible by num_key_value_heads.")
+    return out
+
+
+def rmsnorm_axes(x, axes, scale, eps):
+    """RMSNormalization over `axes` (1-based, negative from the end), scale shaped like those axes
+    (layers/rms_normalization_layer.hpp:37-69); the axes are brought to the end around the row routine."""
+    x = _f32(x)
+    axes = sorted(set(a + x.ndim + 1 if a < 0 else a for a in axes))
+    src, dst = [a - 1 for a in axes], list(range(x.ndim - len(axes), x.ndim))
+    xm = np.ascontiguousarray(np.moveaxis(x, src, dst))
+    depth = int(np.prod(xm.shape[xm.ndim - len(axes):]))
+    out = np.empty_like(xm)
+    lib().fdo_rmsnorm(_p(xm), ctypes.c_size_t(xm.size // depth), depth, _p(scale), ctypes.c_float(eps), _p(out))
+    return np.ascontiguousarray(np.moveaxis(out, dst, src))
+
+
 def einsum_dense(x, equation, kernel, kernel_shape, bias, bias_axes):
     """EinsumDense on one sample; x excludes the batch dim (size-1 batch char is re-added)."""
     x = _f32(x)
@@ -435,6 +470,16 @@ class _Layer:
             self.p["w"] = vals
         elif cls == "PReLU":
             self.p["alpha"] = decode_floats(get_param(name, "alpha"))
+        elif cls in ("SeparableConv2D", "SeparableConv1D"):
+            self.kh, self.kw = c["kernel_size"] if len(c["kernel_size"]) == 2 else (1, c["kernel_size"][0])
+            self.p["slice"] = decode_floats(get_param(name, "slice_weights"))
+            self.p["stack"] = decode_floats(get_param(name, "stack_weights"))
+            self.cout = int(c["filters"])
+            self.p["b"] = decode_floats(get_param(name, "bias")) if c["use_bias"] else np.zeros(self.cout, np.float32)
+        elif cls == "RMSNormalization":
+            self.p["scale"] = decode_floats(get_param(name, "scale"))
+        elif cls in ("GroupQueryAttention", "GroupedQueryAttention"):
+            self.p["w"] = [decode_floats(v) for v in get_param(name, "weights")]
         elif cls == "EinsumDense":
             self.p["kernel"] = decode_floats(get_param(name, "kernel"))
             self.p["kernel_shape"] = [int(v) for v in get_param(name, "kernel_shape")]
@@ -521,6 +566,18 @@ class _Layer:
             key = ins[2] if len(ins) > 2 else None
             out = mha(ins[0], ins[1], key, int(c["num_heads"]), int(c["key_dim"]), int(c["value_dim"]),
                       p["w"], bool(c["use_bias"]))
+        elif cls in ("SeparableConv2D", "SeparableConv1D"):
+            # depthwise part without bias, then a 1x1 valid convolution (layers/separable_conv_2d_layer.hpp:26-55)
+            ch = p["slice"].size // (self.kh * self.kw)
+            tmp = depthwise_conv2d(ins[0], p["slice"], np.zeros(ch, np.float32), self.kh, self.kw, c["strides"],
+                                   c["dilation_rate"], c["padding"])
+            out = conv2d(tmp, conv2d_prepare(p["stack"], self.cout, 1, 1, ch), p["b"], self.cout, 1, 1, (1, 1), (1, 1), "valid")
+        elif cls == "RMSNormalization":
+            axes = c["axis"] if isinstance(c["axis"], list) else [c["axis"]]
+            out = rmsnorm_axes(ins[0], axes, p["scale"] if p["scale"].size else None, c["epsilon"])
+        elif cls in ("GroupQueryAttention", "GroupedQueryAttention"):
+            out = gqa(ins[0], ins[1], ins[2] if len(ins) > 2 else None, int(c["head_dim"]), int(c["num_query_heads"]),
+                      int(c["num_key_value_heads"]), p["w"], bool(c["use_bias"]), bool(c.get("use_gate", False)))
         elif cls == "EinsumDense":
             out = einsum_dense(ins[0], c["equation"], p["kernel"], p["kernel_shape"], p["bias"],
                                c.get("bias_axes"))

@@ -604,6 +604,103 @@ int fdo_mha(const float* query, int t, const float* value, const float* key, int
 }
 
 /*
+ * GroupQueryAttention: Q projected to hq heads, K / V to hkv heads (kernels (D, heads, hd), biases
+ * (heads, hd)); query head h reads key/value head h / (hq / hkv); scores scaled by 1/sqrt(hd) in
+ * float, softmax as exp(s - max) / sum; optional sigmoid gate (a second projection of the query)
+ * multiplied onto the attention output; output kernel (hq, hd, dout).
+ * include/fdeep/layers/group_query_attention_layer.hpp:62-220.  Biases / gate may be NULL.
+ */
+int fdo_gqa(const float* query, int t, const float* value, const float* key, int s, int d, int hd, int hq, int hkv,
+    const float* qw, const float* qb, const float* kw, const float* kb, const float* gw, const float* gb,
+    const float* vw, const float* vb, const float* ow, const float* ob, int dout, float* out)
+{
+    if (hkv <= 0 || hq % hkv != 0)
+        return -1;
+    const int group = hq / hkv;
+    float* q = (float*)malloc(sizeof(float) * (size_t)t * hq * hd);
+    float* g = gw ? (float*)malloc(sizeof(float) * (size_t)t * hq * hd) : NULL;
+    float* k = (float*)malloc(sizeof(float) * (size_t)s * hkv * hd);
+    float* v = (float*)malloc(sizeof(float) * (size_t)s * hkv * hd);
+    float* attn = (float*)malloc(sizeof(float) * (size_t)t * hq * hd);
+    float* sc = (float*)malloc(sizeof(float) * (size_t)s);
+#define FDO_PROJECT(dst, src, rows, heads, w, b)                                  \
+    for (int r = 0; r < rows; ++r)                                                \
+        for (int h = 0; h < heads; ++h)                                           \
+            for (int c = 0; c < hd; ++c) {                                        \
+                float acc = 0;                                                    \
+                for (int i = 0; i < d; ++i)                                       \
+                    acc += src[(size_t)r * d + i] * w[((size_t)i * heads + h) * hd + c]; \
+                if (b)                                                            \
+                    acc += b[h * hd + c];                                         \
+                dst[((size_t)r * heads + h) * hd + c] = acc;                      \
+            }
+    FDO_PROJECT(q, query, t, hq, qw, qb)
+    FDO_PROJECT(k, key, s, hkv, kw, kb)
+    FDO_PROJECT(v, value, s, hkv, vw, vb)
+    if (gw)
+        FDO_PROJECT(g, query, t, hq, gw, gb)
+#undef FDO_PROJECT
+    const float inv_sqrt = 1.0f / sqrtf((float)hd);
+    for (int h = 0; h < hq; ++h) {
+        const int hk = h / group;
+        for (int tq = 0; tq < t; ++tq) {
+            float mx = -INFINITY;
+            for (int tk = 0; tk < s; ++tk) {
+                float a = 0;
+                for (int c = 0; c < hd; ++c)
+                    a += q[((size_t)tq * hq + h) * hd + c] * k[((size_t)tk * hkv + hk) * hd + c];
+                a *= inv_sqrt;
+                sc[tk] = a;
+                if (a > mx)
+                    mx = a;
+            }
+            float sum = 0;
+            for (int tk = 0; tk < s; ++tk) {
+                sc[tk] = expf(sc[tk] - mx);
+                sum += sc[tk];
+            }
+            for (int tk = 0; tk < s; ++tk)
+                sc[tk] /= sum;
+            for (int c = 0; c < hd; ++c) {
+                float a = 0;
+                for (int tk = 0; tk < s; ++tk)
+                    a += sc[tk] * v[((size_t)tk * hkv + hk) * hd + c];
+                attn[((size_t)tq * hq + h) * hd + c] = a;
+            }
+        }
+    }
+    if (g)
+        for (size_t i = 0; i < (size_t)t * hq * hd; ++i)
+            attn[i] *= 1.0f / (1.0f + expf(-g[i]));
+    for (int r = 0; r < t; ++r)
+        for (int o = 0; o < dout; ++o) {
+            float a = 0;
+            for (int i = 0; i < hq * hd; ++i)
+                a += attn[(size_t)r * hq * hd + i] * ow[(size_t)i * dout + o];
+            if (ob)
+                a += ob[o];
+            out[(size_t)r * dout + o] = a;
+        }
+    free(q); free(g); free(k); free(v); free(attn); free(sc);
+    return 0;
+}
+
+/* RMSNormalization over the last `depth` elements of each row: x / sqrt(mean(x^2) + eps) * scale
+ * (include/fdeep/layers/rms_normalization_layer.hpp:37-69); scale may be NULL */
+void fdo_rmsnorm(const float* x, size_t rows, int depth, const float* scale, float eps, float* y)
+{
+    for (size_t r = 0; r < rows; ++r) {
+        const float* xr = x + r * (size_t)depth;
+        float ss = 0;
+        for (int i = 0; i < depth; ++i)
+            ss += xr[i] * xr[i];
+        const float inv = 1.0f / sqrtf(ss / (float)depth + eps);
+        for (int i = 0; i < depth; ++i)
+            y[r * (size_t)depth + i] = xr[i] * inv * (scale ? scale[i] : 1.0f);
+    }
+}
+
+/*
  * EinsumDense restricted to one contraction of the form used by the reference's
  * tests: out[rhs] = sum over summed chars of in[lhs] * kernel[rhs_kernel] (+ bias
  * laid out in rhs-char order over the chars named by bias_axes).  The leading

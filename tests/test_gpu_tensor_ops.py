@@ -305,3 +305,46 @@ def test_model_with_activations_and_merges(fdx, oracle, modelgen):
     say("  rel errors:", ["%.2e" % e for e in errs])
     assert max(errs) <= TOL
     assert (np.abs(got[2] - want[2]) > 1e-4).mean() < 0.01
+
+
+@pytest.mark.parametrize("shape,axes", [((6, 7, 8), [-1]), ((6, 7, 8), [1]), ((6, 7, 8), [1, 3]), ((5, 300), [2]), ((9,), [1])])
+def test_rmsnorm_axes(fdx, oracle, shape, axes):
+    say("rmsnorm", shape, axes)
+    r = np.random.default_rng(16)
+    x = (r.standard_normal((3,) + shape) * 2 + 1).astype(np.float32)
+    rank = len(shape)
+    n = int(np.prod([shape[(a + rank + 1 if a < 0 else a) - 1] for a in axes]))
+    scale = r.standard_normal(n).astype(np.float32)
+    for sc in (scale, None):
+        want = np.stack([oracle.rmsnorm_axes(x[i], axes, sc, 1e-6) for i in range(3)])
+        assert rel(fdx.rmsnorm_axes(x, axes, sc, 1e-6), want) <= TOL
+
+
+def test_model_with_separable_conv_rmsnorm_gqa(fdx, oracle, modelgen):
+    """SeparableConv2D (depthwise + pointwise), RMSNormalization, GroupedQueryAttention with and without the sigmoid
+    gate and with a separate key input, against the oracle."""
+    say("separable / rmsnorm / gqa model")
+    b = modelgen.Builder("next_rows", 71)
+    img = b.input((10, 9, 6), "img")
+    s1 = b.separable_conv2d(img, 12, 3, "sep1", strides=2, padding="same", activation="relu")
+    s2 = b.separable_conv2d(s1, 16, 3, "sep2", padding="valid", use_bias=False, dilation=1)
+    seq = b._add("Reshape", "to_seq", {"target_shape": [9, 16]}, [s2], (9, 16))
+    n1 = b.rmsnorm(seq, "rms1")
+    a1 = b.gqa(n1, n1, "gqa_self", head_dim=8, num_query_heads=4, num_kv_heads=2, use_gate=True)
+    r1 = b.add([seq, a1], "res1")
+    n2 = b.rmsnorm(r1, "rms2", axes=(1,))
+    mem = b.input((5, 16), "memory")
+    a2 = b.gqa(n2, mem, "gqa_cross", head_dim=4, num_query_heads=6, num_kv_heads=1, use_bias=False, k=mem)
+    out = b.dense(b.add([r1, a2], "res2"), 7, "head", bias_std=0.1)
+    spec = b.finish([out, s2, a1])
+    r = np.random.default_rng(17)
+    xi = r.standard_normal((4, 10, 9, 6)).astype(np.float32)
+    xm = r.standard_normal((4, 5, 16)).astype(np.float32)
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([xi[i], xm[i]]) for i in range(4)]
+    want = [np.stack([w[k] for w in want]) for k in range(3)]
+    got = fdx.Model(js).predict([xi, xm])
+    errs = [rel(g, w) for g, w in zip(got, want)]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= TOL

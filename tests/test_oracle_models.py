@@ -9,6 +9,7 @@ import json
 import numpy as np
 import pytest
 import torch
+from scipy import special
 
 
 def rel(a, b):
@@ -163,3 +164,72 @@ def test_embedded_tests_replay_and_detect_corruption(oracle, modelgen):
         oracle.OracleModel(modelgen.dumps(spec)).run_embedded_tests()
     # the file is plain JSON
     assert json.loads(modelgen.dumps(spec))["image_data_format"] == "channels_last"
+
+
+def test_gqa_vs_float64_and_reduction_to_mha(oracle, modelgen):
+    """GroupQueryAttention against an explicit float64 statement (query head h reads kv head h // group, sigmoid gate),
+    and with as many kv heads as query heads and no gate it must equal MultiHeadAttention on the same kernels."""
+    r = np.random.default_rng(21)
+    T, S, D, hd, hq, hkv = 5, 7, 12, 4, 6, 2
+    q, v = r.standard_normal((T, D)).astype(np.float32), r.standard_normal((S, D)).astype(np.float32)
+    def mk(*shape):
+        return (r.standard_normal(shape) * 0.4).astype(np.float32)
+    for use_bias in (True, False):
+        for use_gate in (True, False):
+            w = []
+            def put(kshape, bshape):
+                w.append(mk(*kshape))
+                if use_bias:
+                    w.append(mk(*bshape))
+            put((D, hq, hd), (hq, hd)); put((D, hkv, hd), (hkv, hd))
+            if use_gate:
+                put((D, hq, hd), (hq, hd))
+            put((D, hkv, hd), (hkv, hd)); put((hq, hd, D), (D,))
+            got = oracle.gqa(q, v, None, hd, hq, hkv, w, use_bias, use_gate)
+            W = [a.astype(np.float64) for a in w]
+            step = 2 if use_bias else 1
+            kern = lambda i: W[i * step]
+            bias = lambda i: W[i * step + 1] if use_bias else 0.0
+            vi, oi = (3, 4) if use_gate else (2, 3)
+            Q = np.einsum("td,dhc->thc", q.astype(np.float64), kern(0)) + bias(0)
+            K = np.einsum("sd,dhc->shc", v.astype(np.float64), kern(1)) + bias(1)
+            V = np.einsum("sd,dhc->shc", v.astype(np.float64), kern(vi)) + bias(vi)
+            K, V = np.repeat(K, hq // hkv, axis=1), np.repeat(V, hq // hkv, axis=1)
+            P = special.softmax(np.einsum("thc,shc->hts", Q, K) / np.sqrt(hd), axis=-1)
+            A = np.einsum("hts,shc->thc", P, V)
+            if use_gate:
+                A = A * special.expit(np.einsum("td,dhc->thc", q.astype(np.float64), kern(2)) + bias(2))
+            want = np.einsum("thc,hcd->td", A, kern(oi)) + bias(oi)
+            assert rel(got, want) <= 3e-6
+    # hkv == hq, no gate: the MultiHeadAttention layer with key_dim = value_dim = head_dim
+    w = [mk(D, hq, hd), mk(hq, hd), mk(D, hq, hd), mk(hq, hd), mk(D, hq, hd), mk(hq, hd), mk(hq, hd, D), mk(D)]
+    a = oracle.gqa(q, v, None, hd, hq, hq, w, True, False)
+    b = oracle.mha(q, v, None, hq, hd, hd, w, True)
+    assert rel(a, b) <= 2e-6
+
+
+def test_rmsnorm_and_separable_conv(oracle, modelgen):
+    r = np.random.default_rng(22)
+    x = (r.standard_normal((6, 7, 8)) * 2 + 1).astype(np.float32)
+    for axes in ([-1], [1], [1, 3]):
+        pos = sorted(a + 4 if a < 0 else a for a in axes)
+        pshape = [x.shape[a - 1] if a in pos else 1 for a in (1, 2, 3)]
+        scale = r.standard_normal(int(np.prod(pshape))).astype(np.float32)
+        X = x.astype(np.float64)
+        want = X / np.sqrt((X * X).mean(tuple(a - 1 for a in pos), keepdims=True) + 1e-6) * scale.reshape(pshape)
+        assert rel(oracle.rmsnorm_axes(x, axes, scale, 1e-6), want) <= 2e-6
+    t = torch.nn.functional.rms_norm(torch.from_numpy(x.astype(np.float64)), [8], eps=1e-6).numpy()
+    assert rel(oracle.rmsnorm_axes(x, [-1], None, 1e-6), t) <= 2e-6
+    # SeparableConv2D = grouped 3x3 convolution without bias, then a 1x1 convolution with bias (torch, float64)
+    b = modelgen.Builder("sep_probe", 23)
+    x_in = b.input((9, 10, 6), "x")
+    spec = b.finish([b.separable_conv2d(x_in, 5, 3, "sep", strides=2, padding="same")])
+    xs = r.standard_normal((9, 10, 6)).astype(np.float32)
+    got = oracle.OracleModel(modelgen.dumps(spec)).predict([xs])[0]
+    p = spec["trainable_params"]["sep"]
+    xt = torch.from_numpy(xs.astype(np.float64)).permute(2, 0, 1)[None]
+    xt = torch.nn.functional.pad(xt, (0, 1, 1, 1))  # TF same, k3 s2: height 9 -> pad (1, 1), width 10 -> pad (0, 1)
+    dw = torch.nn.functional.conv2d(xt, torch.from_numpy(p["slice_weights"].astype(np.float64))[:, None], stride=2, groups=6)
+    pw = torch.nn.functional.conv2d(dw, torch.from_numpy(p["stack_weights"].astype(np.float64)).permute(0, 3, 1, 2),
+                                    torch.from_numpy(p["bias"].astype(np.float64)))
+    assert rel(got, pw[0].permute(1, 2, 0).numpy()) <= 3e-6
