@@ -288,6 +288,33 @@ def rmsnorm_axes(x, axes, scale, eps):
     return out.to_host(x.shape)
 
 
+def permute(x, dims):
+    """x: (batch, ...); dims: the Permute layer's 1-based axis list."""
+    x = np.ascontiguousarray(x, np.float32)
+    rank = x.ndim - 1
+    d = (ctypes.c_int64 * rank)(*x.shape[1:])
+    perm = (ctypes.c_int * rank)(*[v - 1 for v in dims])
+    dx, out = DevBuf.from_host(x), DevBuf(x.nbytes)
+    check(lib.fdx_permute_f32(_dp(dx), x.shape[0], rank, d, perm, _dp(out)))
+    return out.to_host((x.shape[0],) + tuple(x.shape[v] for v in dims))
+
+
+def crop2d(x, top, bottom, left, right):
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    dx, out = DevBuf.from_host(x), DevBuf(4 * n * (h - top - bottom) * (w - left - right) * c)
+    check(lib.fdx_crop2d_nhwc_f32(_dp(dx), n, h, w, c, top, bottom, left, right, _dp(out)))
+    return out.to_host((n, h - top - bottom, w - left - right, c))
+
+
+def upsample2d(x, factor_y, factor_x, bilinear=False):
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    dx, out = DevBuf.from_host(x), DevBuf(4 * x.size * factor_y * factor_x)
+    check(lib.fdx_upsample2d_nhwc_f32(_dp(dx), n, h, w, c, factor_y, factor_x, int(bilinear), _dp(out)))
+    return out.to_host((n, h * factor_y, w * factor_x, c))
+
+
 def broadcast_add(a, b, act=None):
     """a, b: (batch, ...sample dims) with right-aligned size-1 broadcasting between the samples."""
     a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)

@@ -166,8 +166,9 @@ namespace {
         } else if (v.is_array() && v.size() == 1) { // 1-D layers: width only
             a = 1;
             b = (int)v.at((size_t)0).integer();
-        } else {
-            a = b = (int)v.integer();
+        } else { // a bare number is a width (create_shape2, import_model.hpp:229-242)
+            a = 1;
+            b = (int)v.integer();
         }
     }
 
@@ -708,6 +709,55 @@ namespace {
                         for (const auto& a : sa->arr)
                             op.shared_axes.push_back(a.integer());
                 result = add_op(std::move(op));
+            } else if (cls == "UpSampling2D" || cls == "UpSampling1D") {
+                op.kind = OpKind::Resize;
+                if (cls == "UpSampling1D") {
+                    op.kh = 1;
+                    op.kw = (int)cfg.at("size").integer();
+                } else {
+                    pair_from(cfg.at("size"), op.kh, op.kw);
+                    const std::string ip = cfg.at("interpolation").str();
+                    if (ip != "nearest" && ip != "bilinear")
+                        throw FormatError("Invalid interpolation method: " + ip);
+                    op.bilinear = ip == "bilinear";
+                }
+                if (op.kh < 1 || op.kw < 1)
+                    throw FormatError("invalid upsampling factor");
+                result = add_op(std::move(op));
+            } else if (cls == "Cropping2D" || cls == "Cropping1D") {
+                // import_model.hpp:1075-1115: ((top, bottom), (left, right)), or for 1-D (left, right)
+                op.kind = OpKind::Crop;
+                const Value& cr = cfg.at("cropping");
+                if (!cr.is_array() || cr.size() != 2)
+                    throw FormatError("invalid cropping format");
+                if (cr.arr[0].is_array()) {
+                    if (cr.arr[0].size() != 2 || cr.arr[1].size() != 2)
+                        throw FormatError("invalid cropping format");
+                    op.zp[0] = (int)cr.arr[0].at((size_t)0).integer();
+                    op.zp[1] = (int)cr.arr[0].at(1).integer();
+                    op.zp[2] = (int)cr.arr[1].at((size_t)0).integer();
+                    op.zp[3] = (int)cr.arr[1].at(1).integer();
+                } else {
+                    op.zp[2] = (int)cr.at((size_t)0).integer();
+                    op.zp[3] = (int)cr.at(1).integer();
+                }
+                result = add_op(std::move(op));
+            } else if (cls == "Permute") {
+                op.kind = OpKind::Permute;
+                for (const auto& d : cfg.at("dims").arr)
+                    op.target_shape.push_back(d.integer());
+                result = add_op(std::move(op));
+            } else if (cls == "ZeroPadding1D") {
+                op.kind = OpKind::ZeroPad;
+                const Value& p = cfg.at("padding");
+                if (p.is_array() && p.size() == 2) {
+                    op.zp[2] = (int)p.at((size_t)0).integer();
+                    op.zp[3] = (int)p.at(1).integer();
+                } else if (p.is_number()) {
+                    op.zp[2] = op.zp[3] = (int)p.integer();
+                } else
+                    throw FormatError("invalid padding format");
+                result = add_op(std::move(op));
             } else if (cls == "ZeroPadding2D") {
                 op.kind = OpKind::ZeroPad;
                 const Value& p = cfg.at("padding");
@@ -718,7 +768,7 @@ namespace {
                 op.zp[2] = (int)p.arr[1].at((size_t)0).integer();
                 op.zp[3] = (int)p.arr[1].at(1).integer();
                 result = add_op(std::move(op));
-            } else if (cls == "MaxPooling2D" || cls == "AveragePooling2D") {
+            } else if (cls == "MaxPooling2D" || cls == "AveragePooling2D" || cls == "MaxPooling1D" || cls == "AveragePooling1D") {
                 op.kind = OpKind::Pool;
                 op.pool_mode = cls[0] == 'M' ? 0 : 1;
                 pair_from(cfg.at("pool_size"), op.kh, op.kw);
@@ -1081,6 +1131,16 @@ namespace {
         return FDX_OK;
     }
 
+    // (height, width, depth) view of a rank-3 sample, or of a rank-2 (width, depth) one with height 1; empty otherwise
+    Shape hwc(const Shape& s)
+    {
+        if (s.size() == 3)
+            return s;
+        if (s.size() == 2)
+            return { 1, s[0], s[1] };
+        return {};
+    }
+
     fdx_status window(int h, int w, const Op& o, bool dilated, int* g)
     {
         const int ekh = dilated ? (o.kh - 1) * o.dy + 1 : o.kh, ekw = dilated ? (o.kw - 1) * o.dx + 1 : o.kw;
@@ -1130,17 +1190,53 @@ namespace {
             case OpKind::PReLU:
                 out = *in0;
                 break;
-            case OpKind::ZeroPad:
-                FDX_REQUIRE(in0->size() == 3, "%s: ZeroPadding2D needs a rank-3 input", o.name.c_str());
-                out = { (*in0)[0] + o.zp[0] + o.zp[1], (*in0)[1] + o.zp[2] + o.zp[3], (*in0)[2] };
+            case OpKind::ZeroPad: {
+                const Shape s3 = hwc(*in0);
+                FDX_REQUIRE(!s3.empty(), "%s: zero padding needs a rank-2 or rank-3 input", o.name.c_str());
+                out = { s3[0] + o.zp[0] + o.zp[1], s3[1] + o.zp[2] + o.zp[3], s3[2] };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
                 break;
-            case OpKind::Pool:
-                FDX_REQUIRE(in0->size() == 3, "%s: pooling needs a rank-3 input", o.name.c_str());
-                if (window((int)(*in0)[0], (int)(*in0)[1], o, false, g) != FDX_OK)
+            }
+            case OpKind::Pool: {
+                const Shape s3 = hwc(*in0);
+                FDX_REQUIRE(!s3.empty(), "%s: pooling needs a rank-2 or rank-3 input", o.name.c_str());
+                if (window((int)s3[0], (int)s3[1], o, false, g) != FDX_OK)
                     return FDX_ERR_INVALID;
                 FDX_REQUIRE(g[4] > 0 && g[5] > 0, "%s: empty pooling output", o.name.c_str());
-                out = { g[4], g[5], (*in0)[2] };
+                out = { g[4], g[5], s3[2] };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
                 break;
+            }
+            case OpKind::Resize: {
+                const Shape s3 = hwc(*in0);
+                FDX_REQUIRE(!s3.empty(), "%s: upsampling needs a rank-2 or rank-3 input", o.name.c_str());
+                out = { s3[0] * o.kh, s3[1] * o.kw, s3[2] };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
+                break;
+            }
+            case OpKind::Crop: {
+                const Shape s3 = hwc(*in0);
+                FDX_REQUIRE(!s3.empty(), "%s: cropping needs a rank-2 or rank-3 input", o.name.c_str());
+                FDX_REQUIRE(o.zp[0] + o.zp[1] < s3[0] && o.zp[2] + o.zp[3] < s3[1], "%s: cropping removes the whole tensor", o.name.c_str());
+                out = { s3[0] - o.zp[0] - o.zp[1], s3[1] - o.zp[2] - o.zp[3], s3[2] };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
+                break;
+            }
+            case OpKind::Permute: {
+                FDX_REQUIRE(o.target_shape.size() == in0->size(), "%s: Permute dims do not match the input rank", o.name.c_str());
+                out.clear();
+                std::vector<char> seen(in0->size(), 0);
+                for (int64_t d : o.target_shape) {
+                    FDX_REQUIRE(d >= 1 && d <= (int64_t)in0->size() && !seen[(size_t)d - 1], "Invalid dims for permute.");
+                    seen[(size_t)d - 1] = 1;
+                    out.push_back((*in0)[(size_t)d - 1]);
+                }
+                break;
+            }
             case OpKind::GlobalPool:
                 FDX_REQUIRE(in0->size() >= 2, "%s: global pooling needs rank >= 2", o.name.c_str());
                 if (o.keepdims) {
@@ -1470,15 +1566,36 @@ namespace {
             st = fdx_broadcast_combine_f32(FDX_COMBINE_PRELU, in0, xd, o.dw[0], ad, 1, B, 1.0f, actp, out, nullptr);
             break;
         }
-        case OpKind::ZeroPad:
-            st = fdx_zero_pad2d_nhwc_f32(in0, B, (int)(*is)[0], (int)(*is)[1], (int)(*is)[2], o.zp[0], o.zp[1], o.zp[2], o.zp[3], out);
+        case OpKind::ZeroPad: {
+            const Shape s3 = hwc(*is);
+            st = fdx_zero_pad2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.zp[0], o.zp[1], o.zp[2], o.zp[3], out);
             break;
-        case OpKind::Pool:
-            if ((st = window((int)(*is)[0], (int)(*is)[1], o, false, g)) != FDX_OK)
+        }
+        case OpKind::Pool: {
+            const Shape s3 = hwc(*is);
+            if ((st = window((int)s3[0], (int)s3[1], o, false, g)) != FDX_OK)
                 return st;
-            st = fdx_pool2d_nhwc_f32(in0, B, (int)(*is)[0], (int)(*is)[1], (int)(*is)[2], o.kh, o.kw, o.sy, o.sx, g[0] + o.zp[0],
+            st = fdx_pool2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.kh, o.kw, o.sy, o.sx, g[0] + o.zp[0],
                 g[2] + o.zp[2], o.zp[0], o.zp[2], o.zp[1], o.zp[3], g[4], g[5], o.pool_mode, out);
             break;
+        }
+        case OpKind::Resize: {
+            const Shape s3 = hwc(*is);
+            st = fdx_upsample2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.kh, o.kw, o.bilinear ? 1 : 0, out);
+            break;
+        }
+        case OpKind::Crop: {
+            const Shape s3 = hwc(*is);
+            st = fdx_crop2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.zp[0], o.zp[1], o.zp[2], o.zp[3], out);
+            break;
+        }
+        case OpKind::Permute: {
+            int perm[5];
+            for (size_t d = 0; d < o.target_shape.size(); ++d)
+                perm[d] = (int)o.target_shape[d] - 1;
+            st = fdx_permute_f32(in0, B, (int)is->size(), is->data(), perm, out);
+            break;
+        }
         case OpKind::GlobalPool:
             st = fdx_global_pool_f32(in0, B, (int)(volume(*is) / is->back()), (int)is->back(), o.pool_mode, out);
             break;

@@ -157,6 +157,72 @@ __global__ __launch_bounds__(256) void layernorm_axes_kernel(const float* __rest
     }
 }
 
+struct PermuteDesc {
+    int64_t od[6], is[6]; // output extents (batch first) and, per output axis, the stride of its source axis
+};
+
+// permute_tensor (include/fdeep/tensor.hpp:526-549): output axis i is input axis dims[i] - 1
+__global__ void permute_kernel(const float* __restrict__ in, float* __restrict__ out, PermuteDesc d, size_t total)
+{
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = o;
+        int64_t pi = 0;
+#pragma unroll
+        for (int i = 5; i >= 0; --i) {
+            pi += (int64_t)(rem % (size_t)d.od[i]) * d.is[i];
+            rem /= (size_t)d.od[i];
+        }
+        out[o] = in[pi];
+    }
+}
+
+// crop_tensor (include/fdeep/tensor.hpp:586-610) on [n][h][w][c]
+__global__ void crop2d_kernel(const float* __restrict__ in, float* __restrict__ out, int h, int w, int c, int top, int left,
+    int oh, int ow, size_t total)
+{
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        const int z = (int)(o % (size_t)c);
+        size_t rest = o / (size_t)c;
+        const int x = (int)(rest % (size_t)ow);
+        rest /= (size_t)ow;
+        const int y = (int)(rest % (size_t)oh);
+        const size_t img = rest / (size_t)oh;
+        out[o] = in[((img * h + (y + top)) * (size_t)w + (x + left)) * c + z];
+    }
+}
+
+// resize2d_nearest / resize2d_bilinear for integer factors (include/fdeep/tensor.hpp:959-974, 997-1035): source
+// coordinate (y + 0.5) / factor - 0.5; nearest rounds it (= y / factor for integer factors), bilinear clamps it to
+// [0, extent] and blends the four neighbours, the lower / right one clamped to the last row / column
+template <bool BILINEAR>
+__global__ void resize2d_kernel(const float* __restrict__ in, float* __restrict__ out, int h, int w, int c, int fy, int fx,
+    size_t total)
+{
+    const int oh = h * fy, ow = w * fx;
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        const int z = (int)(o % (size_t)c);
+        size_t rest = o / (size_t)c;
+        const int x = (int)(rest % (size_t)ow);
+        rest /= (size_t)ow;
+        const int y = (int)(rest % (size_t)oh);
+        const float* img = in + (rest / (size_t)oh) * (size_t)h * w * c;
+        if (!BILINEAR) {
+            out[o] = img[((size_t)(y / fy) * w + (x / fx)) * c + z];
+        } else {
+            float yi = ((float)y + 0.5f) / (float)fy - 0.5f, xi = ((float)x + 0.5f) / (float)fx - 0.5f;
+            yi = fminf(fmaxf(yi, 0.f), (float)h);
+            xi = fminf(fmaxf(xi, 0.f), (float)w);
+            const int yt = (int)floorf(yi), xl = (int)floorf(xi);
+            const int yb = min(h - 1, yt + 1), xr = min(w - 1, xl + 1);
+            const int ytc = min(yt, h - 1), xlc = min(xl, w - 1);
+            const double ft = (double)((float)yb - yi), fb = 1.0 - ft, fl = (double)((float)xr - xi), fr = 1.0 - fl;
+            const double v = ft * fl * img[((size_t)ytc * w + xlc) * c + z] + ft * fr * img[((size_t)ytc * w + xr) * c + z]
+                + fb * fl * img[((size_t)yb * w + xlc) * c + z] + fb * fr * img[((size_t)yb * w + xr) * c + z];
+            out[o] = (float)v;
+        }
+    }
+}
+
 static int grid_of(size_t work_items, int block)
 {
     size_t g = (work_items + block - 1) / block;
@@ -369,4 +435,67 @@ extern "C" fdx_status fdx_rmsnorm_axes_f32(const float* x, int batch, const int6
     float eps, float* out)
 {
     return norm_axes(x, batch, dims5, axes_mask, scale, nullptr, eps, out, true);
+}
+
+extern "C" fdx_status fdx_permute_f32(const float* in, int batch, int rank, const int64_t* dims, const int* perm, float* out)
+{
+    FDX_REQUIRE(in && dims && perm && out && batch > 0 && rank >= 1 && rank <= 5, "permute: bad arguments");
+    int64_t istride[5], vol = 1;
+    bool seen[5] = { false, false, false, false, false };
+    for (int i = rank - 1; i >= 0; --i) {
+        FDX_REQUIRE(dims[i] > 0, "permute: bad extent");
+        istride[i] = vol;
+        vol *= dims[i];
+    }
+    PermuteDesc d {};
+    for (int i = 0; i < 6; ++i) {
+        d.od[i] = 1;
+        d.is[i] = 0;
+    }
+    d.od[0] = batch;
+    d.is[0] = vol;
+    for (int i = 0; i < rank; ++i) {
+        FDX_REQUIRE(perm[i] >= 0 && perm[i] < rank && !seen[perm[i]], "Invalid dims for permute.");
+        seen[perm[i]] = true;
+        d.od[6 - rank + i] = dims[perm[i]];
+        d.is[6 - rank + i] = istride[perm[i]];
+    }
+    const size_t total = (size_t)batch * (size_t)vol;
+    profile_begin();
+    hipLaunchKernelGGL(permute_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, d, total);
+    profile_end("permute_f32", 0.0, 8.0 * (double)total);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_crop2d_nhwc_f32(const float* in, int n, int h, int w, int c, int top, int bottom, int left, int right,
+    float* out)
+{
+    FDX_REQUIRE(in && out && n > 0 && h > 0 && w > 0 && c > 0 && top >= 0 && bottom >= 0 && left >= 0 && right >= 0
+            && top + bottom < h && left + right < w,
+        "crop2d: bad arguments");
+    const int oh = h - top - bottom, ow = w - left - right;
+    const size_t total = (size_t)n * oh * ow * c;
+    profile_begin();
+    hipLaunchKernelGGL(crop2d_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, h, w, c, top, left, oh, ow, total);
+    profile_end("crop2d_f32", 0.0, 8.0 * (double)total);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_upsample2d_nhwc_f32(const float* in, int n, int h, int w, int c, int factor_y, int factor_x, int bilinear,
+    float* out)
+{
+    FDX_REQUIRE(in && out && n > 0 && h > 0 && w > 0 && c > 0 && factor_y > 0 && factor_x > 0, "upsample2d: bad arguments");
+    const size_t total = (size_t)n * h * factor_y * w * factor_x * c;
+    profile_begin();
+    if (bilinear)
+        hipLaunchKernelGGL(resize2d_kernel<true>, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, h, w, c, factor_y,
+            factor_x, total);
+    else
+        hipLaunchKernelGGL(resize2d_kernel<false>, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, h, w, c, factor_y,
+            factor_x, total);
+    profile_end("upsample2d_f32", 0.0, 4.0 * ((double)total + (double)n * h * w * c));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
 }

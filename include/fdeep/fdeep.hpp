@@ -11,9 +11,9 @@
 //   model, load_model, read_model, read_model_from_string, loggers
 //                           include/fdeep/model.hpp:20-301
 // Errors are std::runtime_error, as raised by include/fdeep/common.hpp:42-57.
-// Custom layer creators (import_model.hpp:374-381) are not supported: the GPU plan only
-// runs layer types the library knows; an unknown type fails at load with the reference's
-// "unknown layer type: X" message.
+// Custom layer creators (import_model.hpp:374-381): supported through internal::layer_creators below; such
+// layers run on the host between device segments.  A layer type nobody knows fails at load with the
+// reference's "unknown layer type: X" message.
 #pragma once
 
 #include <algorithm>
@@ -79,7 +79,14 @@ public:
     }
     void shrink_rank() { rank_ = minimal_rank(); }
     void maximize_rank() { rank_ = 5; }
-    std::vector<std::size_t> dimensions() const { return { size_dim_5_, size_dim_4_, height_, width_, depth_ }; }
+    // the extents the rank covers, outermost first (include/fdeep/tensor_shape.hpp:153-164)
+    std::vector<std::size_t> dimensions() const
+    {
+        const std::vector<std::size_t> all = dimensions5();
+        return std::vector<std::size_t>(all.end() - static_cast<std::ptrdiff_t>(rank_), all.end());
+    }
+    // all five right-aligned extents
+    std::vector<std::size_t> dimensions5() const { return { size_dim_5_, size_dim_4_, height_, width_, depth_ }; }
 
     std::size_t rank_;
     std::size_t size_dim_5_;
@@ -91,7 +98,7 @@ public:
 
 inline bool operator==(const tensor_shape& a, const tensor_shape& b)
 {
-    return a.rank() == b.rank() && a.dimensions() == b.dimensions();
+    return a.rank() == b.rank() && a.dimensions5() == b.dimensions5();
 }
 inline bool operator!=(const tensor_shape& a, const tensor_shape& b) { return !(a == b); }
 
@@ -109,7 +116,7 @@ inline tensor_shape create_tensor_shape_from_dims(const std::vector<std::size_t>
 
 inline std::string show_tensor_shape(const tensor_shape& s)
 {
-    const auto d = s.dimensions();
+    const auto d = s.dimensions5();
     std::string r = std::to_string(s.rank()) + "(";
     for (std::size_t i = 5 - s.rank(); i < 5; ++i)
         r += std::to_string(d[i]) + (i + 1 < 5 ? ", " : "");
@@ -154,7 +161,7 @@ namespace internal {
     // fills unknown dimensions from `def`, right-aligned (include/fdeep/tensor_shape.hpp, make_tensor_shape_with)
     inline tensor_shape make_tensor_shape_with(const tensor_shape& def, const tensor_shape_variable& s)
     {
-        const auto dd = def.dimensions();
+        const auto dd = def.dimensions5();
         std::vector<std::size_t> dims;
         for (std::size_t i = 5 - s.rank(); i < 5; ++i)
             dims.push_back(s.fixed(i) ? static_cast<std::size_t>(s.dim(i)) : dd[i]);
@@ -175,7 +182,12 @@ public:
     tensor_pos(std::size_t pos_dim_5, std::size_t pos_dim_4, std::size_t y, std::size_t x, std::size_t z)
         : rank_(5), pos_dim_5_(pos_dim_5), pos_dim_4_(pos_dim_4), y_(y), x_(x), z_(z) {}
     std::size_t rank() const { return rank_; }
-    std::vector<std::size_t> dimensions() const { return { pos_dim_5_, pos_dim_4_, y_, x_, z_ }; }
+    // the coordinates the rank covers, outermost first (include/fdeep/tensor_pos.hpp)
+    std::vector<std::size_t> dimensions() const
+    {
+        const std::vector<std::size_t> all = { pos_dim_5_, pos_dim_4_, y_, x_, z_ };
+        return std::vector<std::size_t>(all.end() - static_cast<std::ptrdiff_t>(rank_), all.end());
+    }
     std::size_t rank_;
     std::size_t pos_dim_5_;
     std::size_t pos_dim_4_;
@@ -361,7 +373,7 @@ namespace internal {
             }
             const tensor_shape& os = outs[0].shape();
             *out_rank = static_cast<int>(os.rank());
-            const auto d = os.dimensions();
+            const auto d = os.dimensions5();
             for (std::size_t k = 0; k < 5; ++k)
                 out_dims5[k] = static_cast<std::int64_t>(d[k]);
             if (output)
@@ -404,7 +416,7 @@ public:
         std::vector<int> in_ranks(n_in);
         for (std::size_t i = 0; i < n_in; ++i) {
             const tensor_shape& s = inputs_vec.front()[i].shape();
-            const auto d = s.dimensions();
+            const auto d = s.dimensions5();
             for (int k = 0; k < 5; ++k)
                 in_dims[i * 5 + k] = static_cast<std::int64_t>(d[k]);
             in_ranks[i] = static_cast<int>(s.rank());

@@ -198,6 +198,15 @@ fdx_status fdx_broadcast_combine_f32(int op, const float* a, const int64_t* a_di
  * `outer` rows of inner[i] floats (inner = extent on the axis times everything to its right, outer =
  * batch times everything to its left); rows are laid side by side in `out` */
 fdx_status fdx_concat_f32(const float* const* ins, int n_inputs, const int64_t* inner, int64_t outer, float* out);
+/* Permute (permute_tensor, include/fdeep/tensor.hpp:526-549): output axis i of each sample is input axis perm[i]
+ * (0-based; the layer's `dims` minus one); dims = the sample's `rank` extents */
+fdx_status fdx_permute_f32(const float* in, int batch, int rank, const int64_t* dims, const int* perm, float* out);
+/* Cropping1D / Cropping2D (crop_tensor, include/fdeep/tensor.hpp:586-610) */
+fdx_status fdx_crop2d_nhwc_f32(const float* in, int n, int h, int w, int c, int top, int bottom, int left, int right, float* out);
+/* UpSampling1D / UpSampling2D by integer factors, nearest or bilinear (resize2d_nearest / resize2d_bilinear,
+ * include/fdeep/tensor.hpp:959-974, 997-1035; layers/upsampling_2d_layer.hpp) */
+fdx_status fdx_upsample2d_nhwc_f32(const float* in, int n, int h, int w, int c, int factor_y, int factor_x, int bilinear,
+    float* out);
 /* EinsumDense, any equation "lhs,kernel->rhs" the reference evaluates
  * (include/fdeep/layers/einsum_dense_layer.hpp:125-258): in_dims are the extents of the trailing
  * in_rank characters of lhs (missing leading ones count as 1; with a batch the first lhs character

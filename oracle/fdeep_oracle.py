@@ -317,6 +317,15 @@ def rmsnorm_axes(x, axes, scale, eps):
     return np.ascontiguousarray(np.moveaxis(out, dst, src))
 
 
+def upsample2d(x, factor_y, factor_x, bilinear=False):
+    """UpSampling2D on an (h, w, c) sample by integer factors (layers/upsampling_2d_layer.hpp)."""
+    x = _f32(x)
+    h, w, c = x.shape
+    out = np.empty((h * factor_y, w * factor_x, c), np.float32)
+    lib().fdo_upsample2d(_p(x), h, w, c, int(factor_y), int(factor_x), int(bool(bilinear)), _p(out))
+    return out
+
+
 def einsum_dense(x, equation, kernel, kernel_shape, bias, bias_axes):
     """EinsumDense on one sample; x excludes the batch dim (size-1 batch char is re-added)."""
     x = _f32(x)
@@ -429,6 +438,13 @@ ACTIVATION_LAYERS = {"LeakyReLU": "leaky_relu", "LeakyRelu": "leaky_relu", "ELU"
                      "LogSigmoid": "log_sigmoid", "LogSoftmax": "log_softmax"}  # import_model.hpp:1839-1865
 
 
+def _pair(v):
+    """create_shape2 (import_model.hpp): two values, or one value for the width of a 1-D layer (height 1)."""
+    if isinstance(v, (list, tuple)):
+        return (int(v[0]), int(v[1])) if len(v) == 2 else (1, int(v[0]))
+    return (1, int(v))  # a bare number is a width
+
+
 class _Layer:
     def __init__(self, data, get_param):
         self.name = data["name"]
@@ -437,8 +453,8 @@ class _Layer:
         self.nodes = [_node_inputs(n) for n in data.get("inbound_nodes", [])]
         self.p = {}
         c, cls, name = self.cfg, self.cls, self.name
-        if cls in ("Conv2D",):
-            self.kh, self.kw = c["kernel_size"]
+        if cls in ("Conv2D", "Conv1D"):
+            self.kh, self.kw = _pair(c["kernel_size"])
             self.cout = int(c["filters"])
             w = decode_floats(get_param(name, "weights"))
             self.cin = w.size // (self.kh * self.kw * self.cout)
@@ -491,9 +507,12 @@ class _Layer:
             raise AssertionError("input layers are seeded, never applied")
         if cls in IDENTITY_LAYERS:
             out = ins[0]
-        elif cls == "Conv2D":
-            out = conv2d(ins[0], p["w"], p["b"], self.cout, self.kh, self.kw, c["strides"],
-                         c["dilation_rate"], c["padding"])
+        elif cls in ("Conv2D", "Conv1D"):
+            x = _f32(ins[0])
+            one_d = x.ndim == 2  # a (width, depth) sequence is a height-1 image
+            out = conv2d(x[None] if one_d else x, p["w"], p["b"], self.cout, self.kh, self.kw, _pair(c["strides"]),
+                         _pair(c["dilation_rate"]), c["padding"])
+            out = out[0] if one_d else out
         elif cls == "DepthwiseConv2D":
             out = depthwise_conv2d(ins[0], p["w"], p["b"], self.kh, self.kw, c["strides"],
                                    c["dilation_rate"], c["padding"])
@@ -533,6 +552,34 @@ class _Layer:
         elif cls in ("MaxPooling2D", "AveragePooling2D"):
             strides = c["strides"] if c.get("strides") is not None else c["pool_size"]
             out = pool2d(ins[0], c["pool_size"], strides, c["padding"], "max" if cls[0] == "M" else "avg")
+        elif cls in ("MaxPooling1D", "AveragePooling1D"):
+            # the 1-D layers are the 2-D ones on a height-1 tensor (import_model.hpp:866-905)
+            size = c["pool_size"][0] if isinstance(c["pool_size"], list) else c["pool_size"]
+            st = c["strides"] if c.get("strides") is not None else size
+            st = st[0] if isinstance(st, list) else st
+            out = pool2d(_f32(ins[0])[None], (1, size), (1, st), c["padding"], "max" if cls[0] == "M" else "avg")[0]
+        elif cls == "ZeroPadding1D":
+            pad = c["padding"]
+            left, right = (pad, pad) if isinstance(pad, int) else pad
+            x = _f32(ins[0])
+            out = np.zeros((x.shape[0] + left + right, x.shape[1]), np.float32)
+            out[left:left + x.shape[0]] = x
+        elif cls in ("Cropping2D", "Cropping1D"):
+            cr = c["cropping"]  # crop_tensor, tensor.hpp:586-610
+            x = _f32(ins[0])
+            if isinstance(cr[0], list):
+                (t, b), (l, r) = cr
+                out = np.ascontiguousarray(x[t:x.shape[0] - b, l:x.shape[1] - r])
+            else:
+                out = np.ascontiguousarray(x[cr[0]:x.shape[0] - cr[1]])
+        elif cls == "UpSampling2D":
+            if c["interpolation"] not in ("nearest", "bilinear"):
+                raise RuntimeError("Invalid interpolation method: " + c["interpolation"])
+            out = upsample2d(ins[0], c["size"][0], c["size"][1], c["interpolation"] == "bilinear")
+        elif cls == "UpSampling1D":
+            out = upsample2d(_f32(ins[0])[None], 1, c["size"])[0]  # x_in = x / size, layers/upsampling_1d_layer.hpp
+        elif cls == "Permute":
+            out = np.ascontiguousarray(np.transpose(_f32(ins[0]), [d - 1 for d in c["dims"]]))  # tensor.hpp:526-549
         elif cls in ("GlobalAveragePooling2D", "GlobalMaxPooling2D", "GlobalAveragePooling1D", "GlobalMaxPooling1D"):
             out = global_pool(ins[0], "max" if "Max" in cls else "avg", bool(c.get("keepdims", False)))
         elif cls == "Add":

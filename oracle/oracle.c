@@ -604,6 +604,42 @@ int fdo_mha(const float* query, int t, const float* value, const float* key, int
 }
 
 /*
+ * UpSampling2D by integer factors (layers/upsampling_2d_layer.hpp; resize2d_nearest / resize2d_bilinear,
+ * include/fdeep/tensor.hpp:959-974, 997-1035).  Source coordinate of output row y: (y + 0.5) / scale - 0.5 with
+ * scale = out / in in float.  Nearest rounds it to the closest index; for an integer factor f that coordinate lies
+ * strictly inside (q - 0.5, q + 0.5) for y = q f + r, so every round-to-nearest rule (the reference calls
+ * FunctionalPlus' round) gives q = y / f.  Bilinear clamps the coordinate to [0, extent], takes floor and floor + 1
+ * (the latter clamped to the last index) and blends with weights formed as in the reference: the upper / left weight
+ * in float, its complement and the products in double.
+ */
+void fdo_upsample2d(const float* in, int h, int w, int c, int fy, int fx, int bilinear, float* out)
+{
+    const int oh = h * fy, ow = w * fx;
+    const float scale_y = (float)oh / (float)h, scale_x = (float)ow / (float)w;
+    for (int y = 0; y < oh; ++y)
+        for (int x = 0; x < ow; ++x)
+            for (int z = 0; z < c; ++z) {
+                float* dst = out + ((size_t)y * ow + x) * c + z;
+                if (!bilinear) {
+                    *dst = in[((size_t)(y / fy) * w + (x / fx)) * c + z];
+                    continue;
+                }
+                float yi = ((float)y + 0.5f) / scale_y - 0.5f, xi = ((float)x + 0.5f) / scale_x - 0.5f;
+                yi = yi < 0 ? 0 : yi;
+                xi = xi < 0 ? 0 : xi;
+                yi = yi > (float)h ? (float)h : yi;
+                xi = xi > (float)w ? (float)w : xi;
+                const int yt = (int)floorf(yi), xl = (int)floorf(xi);
+                const int yb = yt + 1 < h - 1 ? yt + 1 : h - 1, xr = xl + 1 < w - 1 ? xl + 1 : w - 1;
+                const int ytc = yt < h - 1 ? yt : h - 1, xlc = xl < w - 1 ? xl : w - 1; /* the coordinate stays below the extent, so this clamp never acts; it only guards the read */
+                const float ft = (float)yb - yi, fl = (float)xr - xi;
+                const double fb = 1.0 - ft, fr = 1.0 - fl;
+                *dst = (float)(ft * fl * in[((size_t)ytc * w + xlc) * c + z] + ft * fr * in[((size_t)ytc * w + xr) * c + z]
+                    + fb * fl * in[((size_t)yb * w + xlc) * c + z] + fb * fr * in[((size_t)yb * w + xr) * c + z]);
+            }
+}
+
+/*
  * GroupQueryAttention: Q projected to hq heads, K / V to hkv heads (kernels (D, heads, hd), biases
  * (heads, hd)); query head h reads key/value head h / (hq / hkv); scores scaled by 1/sqrt(hd) in
  * float, softmax as exp(s - max) / sum; optional sigmoid gate (a second projection of the query)

@@ -91,6 +91,9 @@ int main(int argc, char** argv)
     for (int i = 0; i < 6; ++i)
         EXPECT(back[static_cast<std::size_t>(i)] == px[i]);
     EXPECT(fdeep::show_tensor_shape(t.shape()) == "3(1, 2, 3)");
+    // dimensions() covers the rank only (include/fdeep/tensor_shape.hpp:153-164)
+    EXPECT((fdeep::tensor_shape(7, 5).dimensions() == std::vector<std::size_t> { 7, 5 }));
+    EXPECT((fdeep::tensor_pos(1, 2, 3).dimensions() == std::vector<std::size_t> { 1, 2, 3 }));
 
     // custom layer: a class the device path does not know, created through custom_layer_creators
     // (the reference's FAQ example shape: a layer subclass with apply_impl, registered by class name)

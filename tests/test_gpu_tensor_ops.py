@@ -348,3 +348,55 @@ def test_model_with_separable_conv_rmsnorm_gqa(fdx, oracle, modelgen):
     errs = [rel(g, w) for g, w in zip(got, want)]
     say("  rel errors:", ["%.2e" % e for e in errs])
     assert max(errs) <= TOL
+
+
+def test_permute_crop_upsample_kernels(fdx, oracle):
+    say("permute / crop / upsample kernels")
+    r = np.random.default_rng(18)
+    x = r.standard_normal((3, 4, 5, 6)).astype(np.float32)
+    for dims in ([1, 2, 3], [3, 1, 2], [2, 1, 3], [3, 2, 1]):
+        assert np.array_equal(fdx.permute(x, dims), np.transpose(x, [0] + dims))
+    assert np.array_equal(fdx.permute(x[:, 0], [2, 1]), np.transpose(x[:, 0], [0, 2, 1]))
+    assert np.array_equal(fdx.crop2d(x, 1, 0, 2, 1), x[:, 1:, 2:4])
+    for fy, fx in ((2, 2), (3, 1), (1, 4)):
+        assert np.array_equal(fdx.upsample2d(x, fy, fx), np.stack([oracle.upsample2d(x[i], fy, fx) for i in range(3)]))
+        want = np.stack([oracle.upsample2d(x[i], fy, fx, True) for i in range(3)])
+        assert rel(fdx.upsample2d(x, fy, fx, True), want) <= 1e-6
+
+
+def test_model_with_resampling_layers(fdx, oracle, modelgen):
+    """An encoder / decoder shaped model: Conv, MaxPooling, UpSampling2D (nearest and bilinear), Cropping2D, Concatenate
+    skip connection, Permute, and the 1-D forms (Conv1D, ZeroPadding1D, MaxPooling1D, AveragePooling1D, UpSampling1D,
+    Cropping1D) on a sequence."""
+    say("resampling model")
+    b = modelgen.Builder("unet_like", 81)
+    img = b.input((12, 12, 3), "img")
+    e1 = b.conv2d(img, 8, 3, "enc1", padding="same", activation="relu", bias_std=0.1)
+    p1 = b.pool(e1, "pool1", 2, 2)
+    e2 = b.conv2d(p1, 12, 3, "enc2", padding="same", activation="relu", bias_std=0.1)
+    u1 = b._add("UpSampling2D", "up_nearest", {"size": [2, 2], "interpolation": "nearest"}, [e2], (12, 12, 12))
+    cat = b.concatenate([u1, e1], "skip", axis=-1)
+    d1 = b.conv2d(cat, 6, 3, "dec1", padding="same", bias_std=0.1)
+    u2 = b._add("UpSampling2D", "up_bilinear", {"size": [2, 3], "interpolation": "bilinear"}, [d1], (24, 36, 6))
+    cr = b._add("Cropping2D", "crop", {"cropping": [[2, 1], [0, 5]]}, [u2], (21, 31, 6))
+    pm = b._add("Permute", "perm", {"dims": [2, 1, 3]}, [cr], (31, 21, 6))
+    seq = b.input((10, 4), "seq")
+    z1 = b._add("ZeroPadding1D", "pad1d", {"padding": [2, 1]}, [seq], (13, 4))
+    c1 = b._add("Conv1D", "conv1d", {"filters": 6, "kernel_size": [3], "strides": [1], "dilation_rate": [1], "padding": "valid",
+                                      "use_bias": True}, [z1], (11, 6))
+    b.params["conv1d"] = {"weights": b.he((6, 1, 3, 4), 12), "bias": b.normal((6,), 0.1)}
+    m1 = b._add("MaxPooling1D", "mp1d", {"pool_size": [2], "strides": [2], "padding": "valid"}, [c1], (5, 6))
+    a1 = b._add("AveragePooling1D", "ap1d", {"pool_size": [2], "strides": [1], "padding": "same"}, [m1], (5, 6))
+    us = b._add("UpSampling1D", "up1d", {"size": 3}, [a1], (15, 6))
+    c1d = b._add("Cropping1D", "crop1d", {"cropping": [2, 4]}, [us], (9, 6))
+    spec = b.finish([pm, c1d, u1])
+    r = np.random.default_rng(19)
+    xi, xs = r.standard_normal((3, 12, 12, 3)).astype(np.float32), r.standard_normal((3, 10, 4)).astype(np.float32)
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([xi[i], xs[i]]) for i in range(3)]
+    want = [np.stack([w[k] for w in want]) for k in range(3)]
+    got = fdx.Model(js).predict([xi, xs])
+    errs = [rel(g, w) for g, w in zip(got, want)]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= TOL

@@ -233,3 +233,16 @@ def test_rmsnorm_and_separable_conv(oracle, modelgen):
     pw = torch.nn.functional.conv2d(dw, torch.from_numpy(p["stack_weights"].astype(np.float64)).permute(0, 3, 1, 2),
                                     torch.from_numpy(p["bias"].astype(np.float64)))
     assert rel(got, pw[0].permute(1, 2, 0).numpy()) <= 3e-6
+
+
+def test_upsampling_vs_torch_interpolate(oracle):
+    """Nearest and bilinear upsampling by integer factors equal torch's interpolate (half-pixel centres,
+    align_corners=False), which is the coordinate rule the reference states."""
+    r = np.random.default_rng(31)
+    x = r.standard_normal((5, 6, 3)).astype(np.float32)
+    xt = torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None]
+    for fy, fx in ((2, 2), (3, 1), (1, 4), (2, 3)):
+        near = torch.nn.functional.interpolate(xt, scale_factor=(fy, fx), mode="nearest")[0].permute(1, 2, 0).numpy()
+        assert np.array_equal(oracle.upsample2d(x, fy, fx), near.astype(np.float32))
+        bil = torch.nn.functional.interpolate(xt, scale_factor=(fy, fx), mode="bilinear", align_corners=False)[0]
+        assert rel(oracle.upsample2d(x, fy, fx, bilinear=True), bil.permute(1, 2, 0).numpy()) <= 2e-6
