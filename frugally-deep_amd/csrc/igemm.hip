@@ -284,21 +284,28 @@ static void launch_cfg(const GemmParams& p, int a_mode, int b_vec, int batch, hi
 // kernel), or one per tile when there are fewer tiles than that.
 static int g_persist_scale = 0; // 0 = resident workgroups; tests and tuning may override the grid cap
 template <typename K>
-static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStream_t s)
+static int resident_workgroups(K kernel, int threads)
 {
     static int resident = 0; // one instance per kernel instantiation
     if (resident == 0) {
         int per_cu = 1, dev = 0;
         hipDeviceProp_t prop;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1)
             per_cu = 1;
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
             prop.multiProcessorCount = 256;
         resident = per_cu * prop.multiProcessorCount;
     }
+    return resident;
+}
+
+template <typename K>
+static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStream_t s, int threads = 256)
+{
+    const int resident = resident_workgroups(kernel, threads);
     const int cap = g_persist_scale > 0 ? g_persist_scale : resident;
     const int grid = tiles < cap ? tiles : cap;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, q);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), 0, s, q);
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -330,39 +337,69 @@ static void tile_of(int cfg, int& bm, int& bn, int& bk)
     case 12: bm = 64; bn = 64; bk = 16; break;
     case 13: bm = 128; bn = 128; bk = 32; break;
     case 14: bm = 128; bn = 64; bk = 32; break;
+    case 15: bm = 64; bn = 64; bk = 32; break;
+    case 16: bm = 128; bn = 128; bk = 32; break;
+    case 17: bm = 128; bn = 128; bk = 32; break;
+    case 18: bm = 256; bn = 128; bk = 32; break;
     default: bm = 64; bn = 64; bk = 32; break;
     }
 }
 
-// whether `splits` K ranges per tile are possible for this configuration: enough slabs per range, and the
-// partial tiles and tickets fit the scratch
-static bool split_fits(int cfg, int splits, const GemmParams& q, int batch)
+// whether `splits` K ranges per tile are possible for `split_tiles` tiles of this configuration: enough slabs per
+// range, and the partial tiles and tickets fit the scratch
+static bool split_fits(int cfg, int splits, int64_t split_tiles, const GemmParams& q)
 {
     int bm, bn, bk;
     tile_of(cfg, bm, bn, bk);
-    const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
-    return splits >= 2 && q.K / bk >= 2 * splits && tiles <= kSplitTickets
-        && (size_t)tiles * splits * bm * bn * sizeof(float) <= kSplitWsBytes && tiles * splits < (1 << 30);
+    return splits >= 2 && q.K / bk >= 2 * splits && split_tiles <= kSplitTickets
+        && (size_t)split_tiles * splits * bm * bn * sizeof(float) <= kSplitWsBytes && split_tiles * splits < (1 << 30);
 }
 
-static void launch_fast(int cfg, int splits, const GemmParams& q0, bool conv, int batch, hipStream_t s)
+// One launch of the split variant.  hybrid: the tiles that fill whole rounds of resident workgroups are computed
+// whole and only the last, partial round is cut into K ranges, so that every workgroup ends at about the same time;
+// otherwise every tile is cut.  Returns false when the cut does not fit the scratch.
+template <typename K>
+static bool launch_split(K kernel, int tiles, int splits, bool hybrid, int cfg, GemmParams& q, hipStream_t s)
+{
+    const int resident = g_persist_scale > 0 ? g_persist_scale : resident_workgroups(kernel, 256);
+    const int dp = hybrid ? (tiles / resident) * resident : 0;
+    if (tiles - dp > 0 && !split_fits(cfg, splits, tiles - dp, q))
+        return false;
+    q.split_dp_tiles = dp;
+    launch_persistent(kernel, dp + (tiles - dp) * splits, q, s);
+    return true;
+}
+
+static bool launch_fast(int cfg, int splits, bool hybrid, const GemmParams& q0, bool conv, int batch, hipStream_t s)
 {
     GemmParams q = q0;
     q.splits = splits;
+    q.split_dp_tiles = 0;
     q.split_ws = g_split_ws;
     q.split_tickets = g_split_tickets;
+    bool ok = true;
 #define FDX_FAST(BM_, BN_, BK_)                                                                                  \
     {                                                                                                            \
         const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
         if (splits > 1) {                                                                                        \
             if (conv)                                                                                            \
-                launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles * splits, q, s);     \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles, splits, hybrid, cfg, q, s); \
             else                                                                                                 \
-                launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles * splits, q, s);    \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles, splits, hybrid, cfg, q, s); \
         } else if (conv)                                                                                         \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s);                        \
         else                                                                                                     \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s);                       \
+    }
+        // eight-wave variants: more waves per SIMD to cover LDS and global latency, or a 256-row tile that halves the
+        // operand traffic per FLOP
+#define FDX_FAST8(BM_, BN_, WM_, WN_)                                                                            \
+    {                                                                                                            \
+        const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
+        if (conv)                                                                                                \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, true>, tiles, q, s, 512);                \
+        else                                                                                                     \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, false>, tiles, q, s, 512);               \
     }
         switch (cfg) {
         case 10: FDX_FAST(128, 128, 16) break;
@@ -370,16 +407,22 @@ static void launch_fast(int cfg, int splits, const GemmParams& q0, bool conv, in
         case 12: FDX_FAST(64, 64, 16) break;
         case 13: FDX_FAST(128, 128, 32) break;
         case 14: FDX_FAST(128, 64, 32) break;
+        case 16: FDX_FAST8(128, 128, 2, 4) break;
+        case 17: FDX_FAST8(128, 128, 4, 2) break;
+        case 18: FDX_FAST8(256, 128, 4, 2) break;
         default: FDX_FAST(64, 64, 32) break;
         }
 #undef FDX_FAST
+#undef FDX_FAST8
+    return ok;
 }
 
 // First sight of a problem shape on the fast path: time every tile configuration once on the
 // real operands (the launches are idempotent) and remember the winner.  Tile count versus
 // resident workgroups, K depth and output width interact too irregularly for a closed rule.
-// A choice is (configuration, K splits) packed as cfg + 100 * splits; splits are tried only where
-// a configuration has few tiles for the chip.
+// A choice is (configuration, K splits, hybrid) packed as cfg + 100 * splits + 10000 * hybrid.  Cutting every tile
+// is tried only where a configuration has few tiles for the chip; the hybrid cut of the last partial round wherever
+// there is one.
 struct TuneKey {
     int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
     bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }
@@ -411,26 +454,34 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     int best = -1;
     float best_ms = 1e30f;
     const bool can_split = g_split_enabled && split_prepare();
-    for (int cfg = 10; cfg <= 15; ++cfg) {
+    for (int cfg = 10; cfg <= 18; ++cfg) {
         if (cfg >= 13 && unit % 32 != 0)
             continue;
         int bm, bn, bk;
         tile_of(cfg, bm, bn, bk);
         const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
-        for (int splits = 1; splits <= 4; ++splits) {
-            if (splits > 1 && !(can_split && tiles <= 1024 && split_fits(cfg, splits, q, batch)))
+        static const int kChoices[][2] = { { 1, 0 }, { 2, 0 }, { 3, 0 }, { 4, 0 }, { 2, 1 }, { 3, 1 }, { 4, 1 }, { 6, 1 }, { 8, 1 } };
+        for (const auto& ch : kChoices) {
+            const int splits = ch[0];
+            const bool hybrid = ch[1] != 0;
+            if (splits > 1 && !(can_split && cfg <= 15))
                 continue;
-            launch_fast(cfg, splits, q, conv, batch, s); // warm-up
+            if (splits > 1 && !hybrid && !(tiles <= 1024 && split_fits(cfg, splits, tiles, q)))
+                continue;
+            if (hybrid && tiles > 16384)
+                continue;
+            if (!launch_fast(cfg, splits, hybrid, q, conv, batch, s)) // warm-up; false = the cut does not fit
+                continue;
             (void)hipEventRecord(a, s);
             for (int r = 0; r < 3; ++r)
-                launch_fast(cfg, splits, q, conv, batch, s);
+                launch_fast(cfg, splits, hybrid, q, conv, batch, s);
             (void)hipEventRecord(b, s);
             float ms = 1e30f;
             if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
                 continue;
             if (ms < best_ms) {
                 best_ms = ms;
-                best = cfg + 100 * splits;
+                best = cfg + 100 * splits + (hybrid ? 10000 : 0);
             }
         }
     }
@@ -472,19 +523,20 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
     const int unit = conv ? p.Cin : p.K;
 
     int cfg = g_forced_tile, splits = 1;
-    if (cfg >= 100) { // tests: configuration + 100 * splits
-        splits = cfg / 100;
+    bool hybrid = false;
+    auto unpack = [&]() { // configuration + 100 * splits + 10000 * hybrid
+        hybrid = cfg >= 10000;
+        splits = std::max(1, (cfg % 10000) / 100);
         cfg %= 100;
-    }
+    };
+    if (cfg >= 100)
+        unpack();
     if (cfg >= 10 && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
         cfg = -1;
     if (cfg < 10)
         splits = 1;
-    if (cfg >= 10 && splits > 1) {
-        GemmParams q = p;
-        if (!split_prepare() || !split_fits(cfg, splits, q, batch))
-            splits = 1;
-    }
+    if (cfg >= 10 && splits > 1 && (cfg > 15 || !split_prepare()))
+        splits = 1;
     if (cfg < 0) {
         if (fast_ok && p.N >= 64 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
             GemmParams q = p;
@@ -493,10 +545,8 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             q.b_records = (uint32_t)b_bytes;
             q.batch = batch;
             cfg = autotune(q, conv, batch, unit, s);
-            if (cfg >= 100) {
-                splits = cfg / 100;
-                cfg %= 100;
-            }
+            if (cfg >= 100)
+                unpack();
         }
         if (cfg >= 10) {
         } else if (fast_ok && p.N >= 64) {
@@ -526,7 +576,8 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         q.a_records = (uint32_t)a_bytes;
         q.b_records = (uint32_t)b_bytes;
         q.batch = batch;
-        launch_fast(cfg, splits, q, conv, batch, s);
+        if (!launch_fast(cfg, splits, hybrid, q, conv, batch, s))
+            launch_fast(cfg, 1, false, q, conv, batch, s); // the requested cut does not fit the scratch
     } else {
         switch (cfg) {
         case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
@@ -548,6 +599,14 @@ using namespace fdx;
 extern "C" fdx_status fdx_debug_force_tile(int cfg)
 {
     fdx::g_forced_tile = cfg;
+    return FDX_OK;
+}
+
+// tests: caps the persistent grid (0 = as many workgroups as are resident on the chip)
+extern "C" fdx_status fdx_debug_persist_cap(int workgroups)
+{
+    // the tile walk hands every eighth workgroup one eighth of the tiles, so a capped grid keeps at least eight
+    fdx::g_persist_scale = workgroups > 0 && workgroups < 8 ? 8 : workgroups;
     return FDX_OK;
 }
 

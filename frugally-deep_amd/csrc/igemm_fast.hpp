@@ -26,10 +26,10 @@
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false>
-__global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(GemmParams p)
 {
-    constexpr int NT = 256;
-    static_assert(WAVES_M * WAVES_N == 4, "256 threads");
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
+    static_assert(NT == 256 || NT == 512, "four or eight waves");
     constexpr int STRIDE = BKT + 4;
     constexpr int CPR = BKT / 4;  // 16-byte chunks per tile row
     constexpr int RPP = NT / CPR; // tile rows filled per loader pass
@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int OSTRIDE = WTN + 4; // epilogue scratch row
-    static_assert(2 * (BM + BN) * STRIDE >= 4 * 32 * OSTRIDE, "epilogue scratch must fit in the operand buffers");
+    static_assert(2 * (BM + BN) * STRIDE >= WAVES_M * WAVES_N * 32 * OSTRIDE, "epilogue scratch must fit in the operand buffers");
     constexpr uint32_t OOB = 0x80000000u; // beyond any extent this path accepts: the load returns zeros
 
     __shared__ __attribute__((aligned(16))) float smem[2 * (BM + BN) * STRIDE];
@@ -52,13 +52,17 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     const int per_problem = tiles_m * tiles_n;
     const int S = SPLIT ? p.splits : 1;
-    const int total = per_problem * p.batch * S; // units: (tile, K range)
-    // XCD x (workgroups with blockIdx % 8 == x) owns the contiguous tile range [lo, hi) so tiles
-    // that share an A row block also share that XCD's L2; its workgroups stride through it.
+    const int all_tiles = per_problem * p.batch;
+    // Units of work: the first n_dp tiles are computed whole; every later tile is cut into S K ranges ("split
+    // units").  XCD x (workgroups with blockIdx % 8 == x) owns a contiguous range of the whole tiles and one of the
+    // split units, so tiles that share an A row block also share that XCD's L2 and both kinds of work are spread
+    // evenly; its workgroups stride through the two ranges one after the other.
+    const int n_dp = SPLIT ? p.split_dp_tiles : all_tiles, n_su = SPLIT ? (all_tiles - n_dp) * S : 0;
     const int xcd = blockIdx.x & 7, wg_in_xcd = blockIdx.x >> 3;
     const int wgs_in_xcd = ((int)gridDim.x - xcd + 7) >> 3;
-    const int per = total >> 3, rem = total & 7;
-    const int lo = xcd * per + (xcd < rem ? xcd : rem), hi = lo + per + (xcd < rem ? 1 : 0);
+    const int alo = xcd * (n_dp >> 3) + (xcd < (n_dp & 7) ? xcd : (n_dp & 7)), na = (n_dp >> 3) + (xcd < (n_dp & 7) ? 1 : 0);
+    const int blo = xcd * (n_su >> 3) + (xcd < (n_su & 7) ? xcd : (n_su & 7)), nb = (n_su >> 3) + (xcd < (n_su & 7) ? 1 : 0);
+    const int hi = na + nb; // local unit indices [0, hi)
 
     // ---- per-tile loader state
     uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
@@ -69,8 +73,15 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
     const int KT = p.K / BKT;
     int kt_n = KT; // slabs of the current unit
 
-    auto setup = [&](int unit, int& m0, int& n0, int64_t& c_off) {
-        const int tile = SPLIT ? unit / S : unit, split = SPLIT ? unit - tile * S : 0;
+    int cur_su = -1; // split unit of the current work item, -1 for a whole tile
+    auto setup = [&](int local, int& m0, int& n0, int64_t& c_off) {
+        int tile = alo + local, split = 0;
+        cur_su = -1;
+        if (SPLIT && local >= na) {
+            cur_su = blo + (local - na);
+            tile = n_dp + cur_su / S;
+            split = cur_su - (cur_su / S) * S;
+        }
         const int z = tile / per_problem, id = tile - z * per_problem;
         m0 = (id / tiles_n) * BM;
         n0 = (id % tiles_n) * BN;
@@ -114,7 +125,8 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
         }
         tap = fx = fy = c0 = 0;
         soff_a = soff_b = 0;
-        if (SPLIT) {
+        kt_n = KT;
+        if (SPLIT && cur_su >= 0) {
             const int kt_lo = (int)((int64_t)split * KT / S);
             kt_n = (int)((int64_t)(split + 1) * KT / S) - kt_lo;
             const int k_start = kt_lo * BKT;
@@ -166,7 +178,7 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
             *reinterpret_cast<f32x4*>(&bs[(r0 + i * RPP) * STRIDE + kq * 4]) = rb[i];
     };
 
-    int tile = lo + wg_in_xcd;
+    int tile = wg_in_xcd; // local unit index
     if (tile >= hi)
         return; // uniform per workgroup
     int m0, n0;
@@ -219,7 +231,7 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
         const int em0 = m0, en0 = n0;
         float* __restrict__ C = p.C + c_off;
         const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
-        const int unit_done = tile;
+        const int su_done = cur_su;
         tile += wgs_in_xcd;
         const bool more = tile < hi;
         if (more) {
@@ -227,10 +239,10 @@ __global__ __launch_bounds__(256) void igemm_fast_kernel(GemmParams p)
             load_tiles(); // in flight while this tile is written out
         }
 
-        if (SPLIT && S > 1) {
+        if (SPLIT && su_done >= 0) {
             constexpr int TILE_F = BM * BN;
-            const int out_tile = unit_done / S, my_split = unit_done - out_tile * S;
-            float* mine = p.split_ws + (int64_t)unit_done * TILE_F + t;
+            const int out_tile = su_done / S, my_split = su_done - out_tile * S; // out_tile counts from the first split tile
+            float* mine = p.split_ws + (int64_t)su_done * TILE_F + t;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll

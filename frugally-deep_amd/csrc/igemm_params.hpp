@@ -27,6 +27,7 @@ struct GemmParams {
     int batch; // number of independent problems folded into the persistent tile walk
     // split-K variant of the fast path: K ranges per tile, partial-tile workspace, one ticket per tile (zero between launches)
     int splits;
+    int split_dp_tiles; // leading tiles that are computed whole (one unit each); the rest are cut into `splits` K ranges
     float* split_ws;
     int* split_tickets;
 };

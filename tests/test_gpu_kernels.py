@@ -41,7 +41,7 @@ CONV_CASES = [
 ]
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 17, 18])
 @pytest.mark.parametrize("case", CONV_CASES)
 def test_conv2d_vs_oracle(fdx, oracle, case, tile):
     n, h, w, cin, cout, kh, kw, strides, dilation, padding = case
@@ -84,7 +84,7 @@ GEMM_CASES = [(1, 10, 32), (16, 768, 768), (37, 50, 29), (256, 2048, 512), (130,
               (300, 96, 100)]
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 17, 18])
 @pytest.mark.parametrize("m,n,k", GEMM_CASES)
 def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
     say("gemm", m, n, k, "tile", tile)
@@ -386,3 +386,29 @@ def test_gemm_split_k_many_tiles(fdx, oracle, tile):
     finally:
         fdx.lib.fdx_debug_force_tile(-1)
     assert rel(got, want) <= TOL
+
+
+@pytest.mark.parametrize("tile,cap", [(10215, 24), (10315, 24), (10413, 8), (10214, 16), (10612, 40), (10815, 9)])
+def test_conv2d_hybrid_whole_tiles_plus_split_remainder(fdx, oracle, tile, cap):
+    """Persistent grid capped to `cap` workgroups: the tiles that fill whole rounds run as whole tiles, the last partial
+    round is cut into K ranges (configuration + 100 * splits + 10000); result equals the oracle and repeats bit for bit."""
+    say("conv2d hybrid", tile, cap)
+    n, h, w, cin, cout = 3, 20, 19, 64, 96
+    r = rng_for("conv-hybrid", tile)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, 3, 3, cin)) / np.sqrt(9 * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, 3, 3, cin)
+    conv = np.stack([oracle.conv2d(x[i], wo, b, cout, 3, 3, (1, 1), (1, 1), "same") for i in range(n)])
+    res = r.standard_normal(conv.shape).astype(np.float32)
+    want = oracle.relu(oracle.add(res, conv))
+    fdx.lib.fdx_debug_force_tile(tile)
+    fdx.lib.fdx_debug_persist_cap(cap)
+    try:
+        first = fdx.conv2d(x, wj, b, (1, 1), (1, 1), "same", residual=res, act=fdx.relu_act())
+        second = fdx.conv2d(x, wj, b, (1, 1), (1, 1), "same", residual=res, act=fdx.relu_act())
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+        fdx.lib.fdx_debug_persist_cap(0)
+    assert rel(first, want) <= TOL
+    assert np.array_equal(first, second)
