@@ -304,6 +304,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
             bias4 = *reinterpret_cast<const f32x4*>(p.bias + n);
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
+            // the residual rows of this 32-row band are requested before the accumulators go through LDS, so their
+            // latency is covered by the transposition instead of stalling every store
+            f32x4 rr[32 / RPS];
+#pragma unroll
+            for (int ps = 0; ps < 32 / RPS; ++ps) {
+                const int m = em0 + wm * WTM + i * 32 + ps * RPS + srow;
+                rr[ps] = f32x4 { 0.f, 0.f, 0.f, 0.f };
+                if (R && m < p.M && n_ok)
+                    rr[ps] = *reinterpret_cast<const f32x4*>(R + (int64_t)m * p.ldc + n);
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -317,12 +327,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                 if (m < p.M && n_ok) {
                     f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
                     const int64_t off = (int64_t)m * p.ldc + n;
-                    f32x4 r = { 0.f, 0.f, 0.f, 0.f };
-                    if (R)
-                        r = *reinterpret_cast<const f32x4*>(R + off);
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        v[e] = apply_act(v[e] * p.alpha + bias4[e] + r[e], p.act);
+                        v[e] = apply_act(v[e] * p.alpha + bias4[e] + rr[ps][e], p.act);
                     *reinterpret_cast<f32x4*>(C + off) = v;
                 }
             }

@@ -166,40 +166,61 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const float* __restrict_
 }
 
 // ------------------------------------------------------------------ pooling
+// One lane per (output pixel, VEC channels); VEC = 4 moves 16 bytes per access.
+template <int VEC>
 __global__ void pool2d_kernel(const float* __restrict__ in, float* __restrict__ out, int n, int h, int w, int c,
     int ph, int pw, int sy, int sx, int pad_top, int pad_left, int zt, int zl, int zb, int zr, int oh, int ow, int mode)
 {
-    const int64_t total = (int64_t)n * oh * ow * c;
+    const int cv = c / VEC;
+    const int64_t total = (int64_t)n * oh * ow * cv;
     for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
          idx += (int64_t)gridDim.x * blockDim.x) {
-        const int ch = (int)(idx % c);
-        int64_t pix = idx / c;
+        const int ch = (int)(idx % cv) * VEC;
+        int64_t pix = idx / cv;
         const int ox = (int)(pix % ow);
         pix /= ow;
         const int oy = (int)(pix % oh);
         const int img = (int)(pix / oh);
-        float val = mode == 0 ? -FLT_MAX : 0.f;
+        float val[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+            val[v] = mode == 0 ? -FLT_MAX : 0.f;
         int div = 0;
         for (int fy = 0; fy < ph; ++fy) {
             const int iy = oy * sy + fy - pad_top;
             for (int fx = 0; fx < pw; ++fx) {
                 const int ix = ox * sx + fx - pad_left;
-                float cur;
-                if (iy >= 0 && iy < h && ix >= 0 && ix < w)
-                    cur = in[(((int64_t)img * h + iy) * w + ix) * c + ch];
-                else if (iy >= -zt && iy < h + zb && ix >= -zl && ix < w + zr)
-                    cur = 0.f; // inside a folded explicit zero-padding frame: a real zero
-                else
+                float cur[VEC];
+                if (iy >= 0 && iy < h && ix >= 0 && ix < w) {
+                    const float* src = in + (((int64_t)img * h + iy) * w + ix) * c + ch;
+                    if (VEC == 4) {
+                        const f32x4 t = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v)
+                            cur[v] = t[v];
+                    } else
+                        cur[0] = src[0];
+                } else if (iy >= -zt && iy < h + zb && ix >= -zl && ix < w + zr) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v)
+                        cur[v] = 0.f; // inside a folded explicit zero-padding frame: a real zero
+                } else
                     continue; // TF padding: ignored by max, excluded from the average
-                if (mode == 0)
-                    val = fmaxf(val, cur);
-                else {
-                    val += cur;
-                    ++div;
-                }
+#pragma unroll
+                for (int v = 0; v < VEC; ++v)
+                    val[v] = mode == 0 ? fmaxf(val[v], cur[v]) : val[v] + cur[v];
+                ++div;
             }
         }
-        out[idx] = mode == 0 ? val : val / (float)div;
+        float* dst = out + (((int64_t)img * oh + oy) * ow + ox) * c + ch;
+        if (VEC == 4) {
+            f32x4 r;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                r[v] = mode == 0 ? val[v] : val[v] / (float)div;
+            *reinterpret_cast<f32x4*>(dst) = r;
+        } else
+            dst[0] = mode == 0 ? val[0] : val[0] / (float)div;
     }
 }
 
@@ -547,8 +568,12 @@ extern "C" fdx_status fdx_pool2d_nhwc_f32(const float* in, int n, int h, int w, 
     FDX_REQUIRE(mode == 0 || mode == 1, "pool2d: mode must be 0 (max) or 1 (average)");
     const size_t items = (size_t)n * out_h * out_w * c;
     profile_begin();
-    hipLaunchKernelGGL(pool2d_kernel, dim3(grid_for(items, 256)), dim3(256), 0, stream(), in, out, n, h, w, c, ph, pw,
-        sy, sx, pad_top, pad_left, zero_top, zero_left, zero_bottom, zero_right, out_h, out_w, mode);
+    if (c % 4 == 0 && al16(in) && al16(out))
+        hipLaunchKernelGGL(pool2d_kernel<4>, dim3(grid_for(items / 4, 256)), dim3(256), 0, stream(), in, out, n, h, w, c, ph, pw,
+            sy, sx, pad_top, pad_left, zero_top, zero_left, zero_bottom, zero_right, out_h, out_w, mode);
+    else
+        hipLaunchKernelGGL(pool2d_kernel<1>, dim3(grid_for(items, 256)), dim3(256), 0, stream(), in, out, n, h, w, c, ph, pw,
+            sy, sx, pad_top, pad_left, zero_top, zero_left, zero_bottom, zero_right, out_h, out_w, mode);
     profile_end("pool2d_f32", 0.0, 4.0 * ((double)n * h * w * c + (double)items));
     FDX_LAUNCH_CHECK();
     return FDX_OK;
