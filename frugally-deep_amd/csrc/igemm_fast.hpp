@@ -319,7 +319,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     scratch[(8 * (e >> 2) + 4 * fh + (e & 3)) * OSTRIDE + j * 32 + fr] = acc[i][j][e];
-            __syncthreads();
+            // the scratch band is private to this wave and a wave's LDS accesses complete in order: no workgroup barrier
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
             for (int ps = 0; ps < 32 / RPS; ++ps) {
                 const int row = ps * RPS + srow;
@@ -333,9 +336,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                     *reinterpret_cast<f32x4*>(C + off) = v;
                 }
             }
-            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
         if (!more)
             break;
+        __syncthreads(); // every wave is done with its scratch before the next tile's operands overwrite it
     }
 }
