@@ -288,6 +288,30 @@ def rmsnorm_axes(x, axes, scale, eps):
     return out.to_host(x.shape)
 
 
+def conv2d_s2d(x, w, bias, padding="valid", residual=None, act=None, extra_pad=(0, 0)):
+    """Stride-2 stem convolution through the space-to-depth path; x [n,h,w,c], w [cout,k,k,c]; extra_pad = (top, left)
+    zero rows / columns of a folded ZeroPadding2D."""
+    x, w = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(w, np.float32)
+    n, h, wd, cin = x.shape
+    cout, k = w.shape[0], w.shape[1]
+    if not lib.fdx_conv2d_s2d_eligible(cin, k, w.shape[2], 2, 2, 1, 1, cout):
+        raise FdxError("shape not eligible for the space-to-depth path")
+    g = window_geometry(h + 2 * extra_pad[0], wd + 2 * extra_pad[1], k, k, 2, 2, padding)
+    lib.fdx_conv2d_s2d_weight_floats.restype = ctypes.c_size_t
+    lib.fdx_conv2d_s2d_scratch_bytes.restype = ctypes.c_size_t
+    w2 = np.empty(lib.fdx_conv2d_s2d_weight_floats(cout, cin, k), np.float32)
+    check(lib.fdx_conv2d_s2d_prepare(w.ctypes.data_as(c_float_p), cout, cin, k, w2.ctypes.data_as(c_float_p)))
+    dx, dw = DevBuf.from_host(x), DevBuf.from_host(w2)
+    db = None if bias is None else DevBuf.from_host(np.ascontiguousarray(bias, np.float32))
+    dr = None if residual is None else DevBuf.from_host(np.ascontiguousarray(residual, np.float32))
+    oh, ow = g["out_h"], g["out_w"]
+    scratch = DevBuf(lib.fdx_conv2d_s2d_scratch_bytes(n, oh, ow, cin, k))
+    out = DevBuf(4 * n * oh * ow * cout)
+    check(lib.fdx_conv2d_s2d_nhwc_f32(_dp(dx), n, h, wd, cin, _dp(dw), _dp(db), cout, k, g["pad_top"] + extra_pad[0], g["pad_left"] + extra_pad[1],
+                                      oh, ow, _dp(dr), _act_ref(act), _dp(scratch), _dp(out)))
+    return out.to_host((n, oh, ow, cout))
+
+
 def permute(x, dims):
     """x: (batch, ...); dims: the Permute layer's 1-based axis list."""
     x = np.ascontiguousarray(x, np.float32)

@@ -451,8 +451,8 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     hipEvent_t a, b;
     if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess)
         return -1;
-    int best = -1;
-    float best_ms = 1e30f;
+    int best = -1, best_split = -1;
+    float best_ms = 1e30f, best_split_ms = 1e30f;
     const bool can_split = g_split_enabled && split_prepare();
     for (int cfg = 10; cfg <= 18; ++cfg) {
         if (cfg >= 13 && unit % 32 != 0)
@@ -460,6 +460,8 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
         int bm, bn, bk;
         tile_of(cfg, bm, bn, bk);
         const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
+        if (bn > 64 && q.N <= bn / 2)
+            continue; // a tile at least twice as wide as the output only idles half of every MFMA
         static const int kChoices[][2] = { { 1, 0 }, { 2, 0 }, { 3, 0 }, { 4, 0 }, { 2, 1 }, { 3, 1 }, { 4, 1 }, { 6, 1 }, { 8, 1 } };
         for (const auto& ch : kChoices) {
             const int splits = ch[0];
@@ -479,19 +481,32 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
             float ms = 1e30f;
             if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
                 continue;
-            if (ms < best_ms) {
-                best_ms = ms;
-                best = cfg + 100 * splits + (hybrid ? 10000 : 0);
+            if (splits == 1) {
+                if (ms < best_ms) {
+                    best_ms = ms;
+                    best = cfg;
+                }
+            } else if (ms < best_split_ms) {
+                best_split_ms = ms;
+                best_split = cfg + 100 * splits + (hybrid ? 10000 : 0);
             }
         }
     }
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+    static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
+    if (log_picks)
+        std::fprintf(stderr, "[fdx tune] conv=%d M=%d N=%d K=%d Cin=%d k=%dx%d s=%d res=%d: plain %d %.1f us, split %d %.1f us\n", (int)conv,
+            q.M, q.N, q.K, q.Cin, q.kh, q.kw, q.sy, (int)(q.residual != nullptr), best, best_ms * 1e3f / 3, best_split, best_split_ms * 1e3f / 3);
+    if (best_split >= 0 && (best < 0 || best_split_ms < best_ms))
+        best = best_split;
+    if (log_picks)
+        std::fprintf(stderr, "[fdx tune]   -> %d\n", best);
     g_tuned[key] = best;
     return best;
 }
 
-static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* family)
+static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* family, double algorithmic_flops = 0.0)
 {
     int a_mode;
     if (conv)
@@ -511,9 +526,11 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
     const int64_t b_bytes = ((int64_t)(p.N - 1) * p.ldb + p.K) * 4;
     int64_t a_bytes, a_shift = 0;
     bool a_ok;
+    if (p.pix_stride == 0)
+        p.pix_stride = p.Cin;
     if (conv) {
-        a_shift = ((int64_t)p.pad_top * p.W + p.pad_left) * p.Cin;
-        a_bytes = ((int64_t)(p.M / (p.OH * p.OW)) * p.H * p.W * p.Cin + a_shift) * 4 + 64;
+        a_shift = ((int64_t)p.pad_top * p.W + p.pad_left) * p.pix_stride;
+        a_bytes = ((int64_t)(p.M / (p.OH * p.OW)) * p.H * p.W * p.pix_stride + a_shift) * 4 + 64;
         a_ok = a_mode == A_CONV_VEC && p.Cin % 16 == 0 && p.kh * p.kw <= 64;
     } else {
         a_bytes = ((int64_t)(p.M - 1) * p.lda + p.K) * 4;
@@ -569,6 +586,10 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             cfg = 3;
     }
 
+    if (cfg < 10 && conv && p.pix_stride != p.Cin) {
+        set_error("igemm: a strided-pixel view needs the fast path");
+        return FDX_ERR_INVALID;
+    }
     profile_begin();
     if (cfg >= 10) {
         GemmParams q = p;
@@ -586,15 +607,102 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
         }
     }
-    const double flops = 2.0 * p.M * (double)p.N * p.K * batch;
+    const double flops = algorithmic_flops > 0.0 ? algorithmic_flops : 2.0 * p.M * (double)p.N * p.K * batch;
     profile_end(family, flops, 0.0);
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }
 
+// ------------------------------------------------------------------ stem convolutions (few input channels, stride 2)
+// A k x k stride-2 convolution over c <= 4 channels is a (k'/2) x (k'/2) stride-1 convolution over the 2x2
+// space-to-depth image with 4c channels (k' = k rounded up to even, the extra filter row / column zero).  In that view
+// one filter row reads k'/2 neighbouring pixels = one contiguous run of 2 k' c floats, which the fast path walks as
+// Cin = run, kw = 1 with a pixel pitch of 4c floats -- instead of gathering c floats per tap through scalar loads.
+__global__ void s2d_kernel(const float* __restrict__ in, float* __restrict__ out, int h, int w, int c, int pad_top, int pad_left,
+    int h2, int w2, size_t total)
+{
+    const int c4 = 4 * c;
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        const int q = (int)(o % (size_t)c4);
+        size_t rest = o / (size_t)c4;
+        const int x2 = (int)(rest % (size_t)w2);
+        rest /= (size_t)w2;
+        const int y2 = (int)(rest % (size_t)h2);
+        const size_t img = rest / (size_t)h2;
+        const int dy = q / (2 * c), dx = (q / c) & 1, ch = q % c;
+        const int iy = 2 * y2 + dy - pad_top, ix = 2 * x2 + dx - pad_left;
+        out[o] = (iy >= 0 && iy < h && ix >= 0 && ix < w) ? in[((img * h + iy) * (size_t)w + ix) * c + ch] : 0.f;
+    }
+}
+
 } // namespace fdx
 
 using namespace fdx;
+
+extern "C" int fdx_conv2d_s2d_eligible(int cin, int kh, int kw, int sy, int sx, int dy, int dx, int cout)
+{
+    const int k8 = (kh + 1) & ~1;
+    return cin >= 1 && cin <= 4 && kh == kw && kh >= 2 && sy == 2 && sx == 2 && dy == 1 && dx == 1 && (k8 * 2 * cin) % 16 == 0
+        && cout % 4 == 0 && cout >= 64;
+}
+
+extern "C" size_t fdx_conv2d_s2d_scratch_bytes(int n, int out_h, int out_w, int cin, int k)
+{
+    const int k2 = ((k + 1) & ~1) / 2;
+    return sizeof(float) * (size_t)n * (size_t)(out_h + k2 - 1) * (size_t)(out_w + k2 - 1) * 4 * (size_t)cin + 256;
+}
+
+extern "C" size_t fdx_conv2d_s2d_weight_floats(int cout, int cin, int k)
+{
+    const int k2 = ((k + 1) & ~1) / 2;
+    return (size_t)cout * k2 * k2 * 4 * cin;
+}
+
+// host: weights [cout][k][k][cin] -> [cout][ky][kx][(dy, dx, c)] with w2 = w[2 ky + dy][2 kx + dx][c], zero beyond k
+extern "C" fdx_status fdx_conv2d_s2d_prepare(const float* weights, int cout, int cin, int k, float* weights_s2d)
+{
+    FDX_REQUIRE(weights && weights_s2d && cout > 0 && cin > 0 && k > 0, "conv2d_s2d_prepare: bad arguments");
+    const int k2 = ((k + 1) & ~1) / 2;
+    size_t o = 0;
+    for (int n = 0; n < cout; ++n)
+        for (int ky = 0; ky < k2; ++ky)
+            for (int kx = 0; kx < k2; ++kx)
+                for (int dy = 0; dy < 2; ++dy)
+                    for (int dx = 0; dx < 2; ++dx)
+                        for (int c = 0; c < cin; ++c) {
+                            const int fy = 2 * ky + dy, fx = 2 * kx + dx;
+                            weights_s2d[o++] = (fy < k && fx < k) ? weights[(((size_t)n * k + fy) * k + fx) * cin + c] : 0.f;
+                        }
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_conv2d_s2d_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* weights_s2d,
+    const float* bias, int cout, int k, int pad_top, int pad_left, int out_h, int out_w, const float* residual,
+    const fdx_act* act, float* scratch, float* out)
+{
+    FDX_REQUIRE(in && weights_s2d && scratch && out && n > 0 && h > 0 && w > 0 && out_h > 0 && out_w > 0, "conv2d_s2d: bad arguments");
+    FDX_REQUIRE(fdx_conv2d_s2d_eligible(cin, k, k, 2, 2, 1, 1, cout), "conv2d_s2d: shape not eligible");
+    FDX_REQUIRE(pad_top >= 0 && pad_left >= 0, "conv2d_s2d: negative padding");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    const int k2 = ((k + 1) & ~1) / 2, h2 = out_h + k2 - 1, w2 = out_w + k2 - 1, c4 = 4 * cin;
+    FDX_REQUIRE((int64_t)n * h2 * w2 * c4 < (1LL << 29) && (int64_t)n * out_h * out_w < (1LL << 31), "conv2d_s2d: dimension overflow");
+    const size_t total = (size_t)n * h2 * w2 * c4;
+    profile_begin();
+    hipLaunchKernelGGL(s2d_kernel, dim3((unsigned)std::min<size_t>((total + 255) / 256, 256 * 16)), dim3(256), 0, stream(), in, scratch, h, w,
+        cin, pad_top, pad_left, h2, w2, total);
+    profile_end("space_to_depth_f32", 0.0, 4.0 * ((double)n * h * w * cin + (double)total));
+    FDX_LAUNCH_CHECK();
+    GemmParams p {};
+    p.A = scratch; p.B = weights_s2d; p.C = out; p.bias = bias; p.residual = residual;
+    p.M = n * out_h * out_w; p.N = cout; p.K = k2 * k2 * c4;
+    p.lda = 0; p.ldb = p.K; p.ldc = cout;
+    p.alpha = 1.f; p.bias_per_row = 0; p.act = make_act(act);
+    p.inner = 1;
+    p.H = h2; p.W = w2; p.Cin = k2 * c4; p.pix_stride = c4; p.kh = k2; p.kw = 1; p.sy = 1; p.sx = 1; p.dy = 1; p.dx = 1;
+    p.pad_top = 0; p.pad_left = 0; p.OH = out_h; p.OW = out_w;
+    // the profile counts the layer's own multiply-adds, not the zero taps of the widened filter
+    return run_igemm(p, true, 1, "conv_igemm_f32", 2.0 * p.M * (double)cout * k * k * cin);
+}
 
 extern "C" fdx_status fdx_debug_force_tile(int cfg)
 {

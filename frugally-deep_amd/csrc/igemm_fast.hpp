@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                     const int oy = rm / p.OW, ox = rm - oy * p.OW;
                     const int iy0 = oy * p.sy - p.pad_top, ix0 = ox * p.sx - p.pad_left;
                     // byte offset from the shifted base (shift = (pad_top*W + pad_left)*Cin elements)
-                    a_voff[i] = (uint32_t)(((img * p.H + oy * p.sy) * p.W + ox * p.sx) * p.Cin) * 4u + kq * 16;
+                    a_voff[i] = (uint32_t)(((img * p.H + oy * p.sy) * p.W + ox * p.sx) * p.pix_stride) * 4u + kq * 16;
                     uint64_t mk = 0;
                     for (int y = 0; y < p.kh; ++y) {
                         const int iy = iy0 + y * p.dy;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                 c0 = k_start - tap * p.Cin;
                 fy = tap / p.kw;
                 fx = tap - fy * p.kw;
-                soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.Cin + c0) * 4;
+                soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.pix_stride + c0) * 4;
             } else {
                 soff_a = k_start * 4;
             }
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                     ++fy;
                 }
             }
-            soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.Cin + c0) * 4;
+            soff_a = ((fy * p.dy * p.W + fx * p.dx) * p.pix_stride + c0) * 4;
         } else {
             soff_a += BKT * 4;
         }

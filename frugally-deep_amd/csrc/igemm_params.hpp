@@ -22,6 +22,9 @@ struct GemmParams {
     int64_t a_outer, a_inner, b_outer, b_inner, c_outer, c_inner;
     // convolution view of A
     int H, W, Cin, kh, kw, sy, sx, dy, dx, pad_top, pad_left, OH, OW;
+    // fast path: floats between neighbouring input pixels (= Cin, except for the space-to-depth view of a stem
+    // convolution, where a filter row reads a run of Cin floats that spans several pixels)
+    int pix_stride;
     // fast path only: byte extents of one problem's A (counted from the shifted base) and B operands
     uint32_t a_records, b_records;
     int batch; // number of independent problems folded into the persistent tile walk

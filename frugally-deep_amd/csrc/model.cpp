@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <set>
@@ -1113,6 +1114,14 @@ namespace {
                 o.hw.clear();
                 continue;
             }
+            // stem convolutions get a third weight array: the filter in its space-to-depth layout
+            static const bool s2d_on = [] { const char* e = std::getenv("FDX_S2D"); return !(e && e[0] == '0'); }();
+            if (s2d_on && o.kind == OpKind::Conv2D && o.hw.size() == 2
+                && fdx_conv2d_s2d_eligible(o.n_in, o.kh, o.kw, o.sy, o.sx, o.dy, o.dx, o.cout)) {
+                o.hw.emplace_back(fdx_conv2d_s2d_weight_floats(o.cout, o.n_in, o.kh));
+                if (fdx_conv2d_s2d_prepare(o.hw[0].data(), o.cout, o.n_in, o.kh, o.hw[2].data()) != FDX_OK)
+                    return FDX_ERR_INVALID;
+            }
             o.dw.assign(o.hw.size(), nullptr);
             for (size_t i = 0; i < o.hw.size(); ++i) {
                 if (o.hw[i].empty())
@@ -1397,6 +1406,7 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->block_of.assign(n, -1);
     p->last_use.assign(n, -1);
     p->temps.assign(n, {});
+    std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
     for (int idx : p->order) {
@@ -1427,6 +1437,8 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
                 return FDX_ERR_HIP;
             }
         }
+        if (o.kind == OpKind::Conv2D && o.dw.size() > 2 && o.dw[2] && p->shapes[idx].size() == 3)
+            s2d_ops.push_back(idx); // scratch placed after the activations, see below
         if (o.kind == OpKind::MHA) { // per-op scratch: placed while inputs and output are live, free again afterwards
             const int64_t T = p->shapes[o.in[0]][0], S = p->shapes[o.in[1]][0];
             const size_t nk = (size_t)o.heads * o.dk, nv = (size_t)o.heads * o.dv, fb = sizeof(float) * (size_t)batch;
@@ -1454,6 +1466,20 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
                 p->blocks[p->block_of[q]].busy = false;
         if (p->last_use[idx] < 0 && p->block_of[idx] >= 0) // produced but never read
             p->blocks[p->block_of[idx]].busy = false;
+    }
+    // The space-to-depth scratch of stem convolutions gets blocks of its own, allocated last, so that it does not
+    // change which blocks the activations land in.
+    for (int idx : s2d_ops) {
+        const Op& o = m->ops[idx];
+        Block b;
+        b.bytes = fdx_conv2d_s2d_scratch_bytes(batch, (int)p->shapes[idx][0], (int)p->shapes[idx][1], o.n_in, o.kh);
+        if (hipMalloc(&b.p, b.bytes) != hipSuccess) {
+            set_error("out of device memory while planning %s", o.name.c_str());
+            return FDX_ERR_HIP;
+        }
+        b.busy = true;
+        p->blocks.push_back(b);
+        p->temps[idx].push_back(static_cast<float*>(b.p));
     }
     m->plan = std::move(p);
     *out = m->plan.get();
@@ -1487,7 +1513,10 @@ namespace {
             const int h = one_d ? 1 : (int)(*is)[0], w = (int)(*is)[one_d ? 0 : 1], c = (int)is->back();
             if ((st = window(h, w, o, true, g)) != FDX_OK)
                 return st;
-            if (o.kind == OpKind::Conv2D)
+            if (o.kind == OpKind::Conv2D && !p.temps[idx].empty())
+                st = fdx_conv2d_s2d_nhwc_f32(in0, B, h, w, c, o.dw[2], o.dw[1], o.cout, o.kh, g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5],
+                    res, actp, p.temps[idx][0], out);
+            else if (o.kind == OpKind::Conv2D)
                 st = fdx_conv2d_nhwc_f32(in0, B, h, w, c, o.dw[0], o.dw[1], o.cout, o.kh, o.kw, o.sy, o.sx, o.dy, o.dx,
                     g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5], res, actp, out);
             else

@@ -93,6 +93,21 @@ fdx_status fdx_conv2d_nhwc_f32(const float* in, int n, int h, int w, int cin,
     const float* residual, const fdx_act* act, float* out);
 
 /*
+ * The same Conv2D for stem layers (1..4 input channels, square kernel, stride 2, dilation 1, cout a multiple of 4
+ * and >= 64; fdx_conv2d_s2d_eligible says whether a layer qualifies): the input is first rewritten as its 2x2
+ * space-to-depth image (into `scratch`, fdx_conv2d_s2d_scratch_bytes) so that a filter row reads one contiguous
+ * run, then the implicit GEMM runs on that view.  weights_s2d comes from fdx_conv2d_s2d_prepare (host side, once
+ * per layer, fdx_conv2d_s2d_weight_floats values).  Results equal fdx_conv2d_nhwc_f32 up to summation order.
+ */
+int fdx_conv2d_s2d_eligible(int cin, int kh, int kw, int sy, int sx, int dy, int dx, int cout);
+size_t fdx_conv2d_s2d_scratch_bytes(int n, int out_h, int out_w, int cin, int k);
+size_t fdx_conv2d_s2d_weight_floats(int cout, int cin, int k);
+fdx_status fdx_conv2d_s2d_prepare(const float* weights, int cout, int cin, int k, float* weights_s2d);
+fdx_status fdx_conv2d_s2d_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* weights_s2d,
+    const float* bias, int cout, int k, int pad_top, int pad_left, int out_h, int out_w, const float* residual,
+    const fdx_act* act, float* scratch, float* out);
+
+/*
  * DepthwiseConv2D (depth multiplier 1); replaces depthwise_convolve
  * (include/fdeep/depthwise_convolution.hpp:21-99).  weights_hwc is [kh][kw][c]
  * (the converted-JSON slice_weights [c][kh][kw] transposed once at load).

@@ -412,3 +412,29 @@ def test_conv2d_hybrid_whole_tiles_plus_split_remainder(fdx, oracle, tile, cap):
         fdx.lib.fdx_debug_persist_cap(0)
     assert rel(first, want) <= TOL
     assert np.array_equal(first, second)
+
+
+@pytest.mark.parametrize("case", [
+    # n, h, w, cin, cout, k, padding, explicit zero frame (top/left = bottom/right)
+    (2, 30, 30, 3, 64, 7, "valid", 3),   # ResNet stem: ZeroPadding2D(3) then 7x7 / 2 valid
+    (2, 33, 29, 3, 64, 7, "same", 0),    # odd extents, TF same padding
+    (3, 17, 18, 4, 64, 3, "same", 0),    # four channels, 3x3 / 2
+    (1, 20, 20, 4, 128, 5, "valid", 1),
+    (2, 16, 16, 3, 96, 8, "valid", 0),   # even kernel
+])
+def test_conv2d_space_to_depth_stem(fdx, oracle, case):
+    """Stride-2 convolutions over 3 or 4 channels through the space-to-depth view against the oracle's Conv2D."""
+    n, h, w, cin, cout, k, padding, frame = case
+    say("conv2d s2d", case)
+    r = rng_for("conv-s2d", case)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, k, k, cin)) / np.sqrt(k * k * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, k, k, cin)
+    xp = np.pad(x, ((0, 0), (frame, frame), (frame, frame), (0, 0)))
+    want = oracle.relu(np.stack([oracle.conv2d(xp[i], wo, b, cout, k, k, (2, 2), (1, 1), padding) for i in range(n)]))
+    got = fdx.conv2d_s2d(x, wj, b, padding, act=fdx.relu_act(), extra_pad=(frame, frame))
+    assert rel(got, want) <= TOL
+    # and the general path on the same operands agrees
+    plain = fdx.conv2d(xp, wj, b, (2, 2), (1, 1), padding, act=fdx.relu_act())
+    assert rel(got, plain) <= TOL
