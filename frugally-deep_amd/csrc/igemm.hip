@@ -618,20 +618,26 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
 // space-to-depth image with 4c channels (k' = k rounded up to even, the extra filter row / column zero).  In that view
 // one filter row reads k'/2 neighbouring pixels = one contiguous run of 2 k' c floats, which the fast path walks as
 // Cin = run, kw = 1 with a pixel pitch of 4c floats -- instead of gathering c floats per tap through scalar loads.
+// one thread per (space-to-depth pixel, source row): 2c contiguous input floats become 2c contiguous output floats
 __global__ void s2d_kernel(const float* __restrict__ in, float* __restrict__ out, int h, int w, int c, int pad_top, int pad_left,
     int h2, int w2, size_t total)
 {
-    const int c4 = 4 * c;
+    const int run = 2 * c;
     for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
-        const int q = (int)(o % (size_t)c4);
-        size_t rest = o / (size_t)c4;
+        const int dy = (int)(o & 1);
+        size_t rest = o >> 1;
         const int x2 = (int)(rest % (size_t)w2);
         rest /= (size_t)w2;
         const int y2 = (int)(rest % (size_t)h2);
         const size_t img = rest / (size_t)h2;
-        const int dy = q / (2 * c), dx = (q / c) & 1, ch = q % c;
-        const int iy = 2 * y2 + dy - pad_top, ix = 2 * x2 + dx - pad_left;
-        out[o] = (iy >= 0 && iy < h && ix >= 0 && ix < w) ? in[((img * h + iy) * (size_t)w + ix) * c + ch] : 0.f;
+        const int iy = 2 * y2 + dy - pad_top, ix0 = 2 * x2 - pad_left;
+        float* dst = out + (o >> 1) * (size_t)(2 * run) + (size_t)dy * run;
+        const bool row_ok = iy >= 0 && iy < h;
+        const float* src = in + ((img * h + (row_ok ? iy : 0)) * (size_t)w) * c;
+        for (int q = 0; q < run; ++q) {
+            const int ix = ix0 + q / c;
+            dst[q] = (row_ok && ix >= 0 && ix < w) ? src[(size_t)ix * c + q % c] : 0.f;
+        }
     }
 }
 
@@ -686,10 +692,10 @@ extern "C" fdx_status fdx_conv2d_s2d_nhwc_f32(const float* in, int n, int h, int
     FDX_REQUIRE_EPILOGUE_ACT(act);
     const int k2 = ((k + 1) & ~1) / 2, h2 = out_h + k2 - 1, w2 = out_w + k2 - 1, c4 = 4 * cin;
     FDX_REQUIRE((int64_t)n * h2 * w2 * c4 < (1LL << 29) && (int64_t)n * out_h * out_w < (1LL << 31), "conv2d_s2d: dimension overflow");
-    const size_t total = (size_t)n * h2 * w2 * c4;
+    const size_t total = (size_t)n * h2 * w2 * c4, items = (size_t)n * h2 * w2 * 2;
     profile_begin();
-    hipLaunchKernelGGL(s2d_kernel, dim3((unsigned)std::min<size_t>((total + 255) / 256, 256 * 16)), dim3(256), 0, stream(), in, scratch, h, w,
-        cin, pad_top, pad_left, h2, w2, total);
+    hipLaunchKernelGGL(s2d_kernel, dim3((unsigned)std::min<size_t>((items + 255) / 256, 256 * 32)), dim3(256), 0, stream(), in, scratch, h, w,
+        cin, pad_top, pad_left, h2, w2, items);
     profile_end("space_to_depth_f32", 0.0, 4.0 * ((double)n * h * w * cin + (double)total));
     FDX_LAUNCH_CHECK();
     GemmParams p {};
