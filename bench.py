@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file and scaled by a plain copy of known size (a process cannot read these counters for itself; the
 # summaries under profiles/ give the commands and the raw readings).  Valid for the default configurations only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 136.6e6, "skinny_gemm, GPT-2 decode b16": 10.9e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 151.4e6, "skinny_gemm, GPT-2 decode b16": 10.9e6}
 
 
 def load_package():
@@ -130,7 +130,7 @@ def bench_resnet(fdx, modelgen, args):
         "model_roofline_frac": round(img_s * flops_per_image / (PEAK_FP32_MFMA_TFLOPS * 1e12), 4),
         "roofline": {
             "bound": "mfma",
-            "kernel": "igemm_kernel (implicit-GEMM Conv2D / GEMM, fp32 MFMA, all tile instantiations)",
+            "kernel": "igemm_fast_kernel (implicit-GEMM Conv2D / GEMM, fp32 MFMA, all tile instantiations)",
             "achieved": round(achieved, 3),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",

@@ -634,9 +634,12 @@ __global__ void s2d_kernel(const float* __restrict__ in, float* __restrict__ out
         float* dst = out + (o >> 1) * (size_t)(2 * run) + (size_t)dy * run;
         const bool row_ok = iy >= 0 && iy < h;
         const float* src = in + ((img * h + (row_ok ? iy : 0)) * (size_t)w) * c;
-        for (int q = 0; q < run; ++q) {
-            const int ix = ix0 + q / c;
-            dst[q] = (row_ok && ix >= 0 && ix < w) ? src[(size_t)ix * c + q % c] : 0.f;
+        for (int q = 0; q < run; q += 2) { // run = 2c is even and dst is 8-byte aligned: pairs keep the stores whole
+            const int ixa = ix0 + q / c, ixb = ix0 + (q + 1) / c;
+            float2 v;
+            v.x = (row_ok && ixa >= 0 && ixa < w) ? src[(size_t)ixa * c + q % c] : 0.f;
+            v.y = (row_ok && ixb >= 0 && ixb < w) ? src[(size_t)ixb * c + (q + 1) % c] : 0.f;
+            *reinterpret_cast<float2*>(dst + q) = v;
         }
     }
 }
