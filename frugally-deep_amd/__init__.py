@@ -339,6 +339,16 @@ def upsample2d(x, factor_y, factor_x, bilinear=False):
     return out.to_host((n, h * factor_y, w * factor_x, c))
 
 
+def dilate2d(x, rate_y, rate_x, trailing_zeros=False):
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    extra = (rate_y - 1, rate_x - 1) if trailing_zeros and (rate_y, rate_x) != (1, 1) else (0, 0)
+    oh, ow = (h - 1) * rate_y + 1 + extra[0], (w - 1) * rate_x + 1 + extra[1]
+    dx, out = DevBuf.from_host(x), DevBuf(4 * n * oh * ow * c)
+    check(lib.fdx_dilate2d_nhwc_f32(_dp(dx), n, h, w, c, rate_y, rate_x, int(trailing_zeros), _dp(out)))
+    return out.to_host((n, oh, ow, c))
+
+
 def broadcast_add(a, b, act=None):
     """a, b: (batch, ...sample dims) with right-aligned size-1 broadcasting between the samples."""
     a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)

@@ -474,6 +474,56 @@ namespace {
                     throw FormatError("invalid number of weights");
                 op.n_in = (int)(op.hw[0].size() / ((size_t)op.kh * op.kw * op.cout));
                 result = with_fused_activation(add_op(std::move(op)), cfg);
+            } else if (cls == "Conv2DTranspose" || cls == "Conv1DTranspose") {
+                // convolve_transposed (convolution.hpp:443-469, import_model.hpp:528-556): zeros between the input pixels,
+                // then a stride-1 convolution with the filter mirrored in height and width (filter.hpp:94-97). "valid"
+                // pads the zero-stuffed image by the inflated filter size minus one on every side, which is an explicit
+                // zero frame around a valid window; "same" is the ordinary stride-1 rule. "causal" cannot pass the
+                // reference's own output-width assertion (convolution.hpp:243) and is refused at load.
+                const int pad_mode = padding_from(cfg.at("padding").str());
+                if (pad_mode == 2)
+                    throw FormatError("output width does not match");
+                int ry = 1, rx = 1;
+                pair_from(cfg.at("strides"), ry, rx);
+                if (ry != 1 || rx != 1) {
+                    Op dil;
+                    dil.kind = OpKind::Dilate;
+                    dil.name = op.name + "_zero_insertion";
+                    dil.cls = cls;
+                    dil.in = ins;
+                    dil.kh = ry;
+                    dil.kw = rx;
+                    dil.trailing = pad_mode == 1;
+                    op.in = { add_op(std::move(dil)) };
+                }
+                op.kind = OpKind::Conv2D;
+                op.padding = pad_mode;
+                pair_from(cfg.at("dilation_rate"), op.dy, op.dx);
+                pair_from(cfg.at("kernel_size"), op.kh, op.kw);
+                op.cout = (int)cfg.at("filters").integer();
+                op.hw.resize(2);
+                std::vector<float> wj = decode_floats(param(sc, c.layer, "weights"));
+                if (cfg.at("use_bias").boolean())
+                    op.hw[1] = decode_floats(param(sc, c.layer, "bias"));
+                else
+                    op.hw[1].assign(op.cout, 0.f);
+                if ((int)op.hw[1].size() != op.cout)
+                    throw FormatError("size of bias does not match");
+                if (wj.empty() || wj.size() % ((size_t)op.kh * op.kw * op.cout) != 0)
+                    throw FormatError("invalid number of weights");
+                op.n_in = (int)(wj.size() / ((size_t)op.kh * op.kw * op.cout));
+                op.hw[0].resize(wj.size()); // [cout][kh][kw][cin], taps mirrored
+                for (int n = 0; n < op.cout; ++n)
+                    for (int y = 0; y < op.kh; ++y)
+                        for (int x = 0; x < op.kw; ++x)
+                            std::copy_n(&wj[(((size_t)n * op.kh + (op.kh - 1 - y)) * op.kw + (op.kw - 1 - x)) * op.n_in], op.n_in,
+                                &op.hw[0][(((size_t)n * op.kh + y) * op.kw + x) * op.n_in]);
+                if (pad_mode == 0) {
+                    const int ekh = (op.kh - 1) * op.dy + 1, ekw = (op.kw - 1) * op.dx + 1;
+                    op.zp[0] = op.zp[1] = ekh - 1;
+                    op.zp[2] = op.zp[3] = ekw - 1;
+                }
+                result = with_fused_activation(add_op(std::move(op)), cfg);
             } else if (cls == "DepthwiseConv2D" || cls == "DepthwiseConv1D") {
                 op.kind = OpKind::DWConv2D;
                 op.padding = padding_from(cfg.at("padding").str());
@@ -1079,7 +1129,7 @@ namespace {
             if (z.dead || z.kind != OpKind::ZeroPad || z.consumers != 1)
                 continue;
             for (int k = 0; k < 4; ++k)
-                c.zp[k] = z.zp[k];
+                c.zp[k] += z.zp[k];
             c.in[0] = z.in[0];
             z.dead = true;
             count_consumers(m);
@@ -1222,6 +1272,14 @@ namespace {
                 const Shape s3 = hwc(*in0);
                 FDX_REQUIRE(!s3.empty(), "%s: upsampling needs a rank-2 or rank-3 input", o.name.c_str());
                 out = { s3[0] * o.kh, s3[1] * o.kw, s3[2] };
+                if (in0->size() == 2)
+                    out.erase(out.begin());
+                break;
+            }
+            case OpKind::Dilate: {
+                const Shape s3 = hwc(*in0);
+                FDX_REQUIRE(!s3.empty(), "Invalid rank for dilation");
+                out = { (s3[0] - 1) * o.kh + 1 + (o.trailing ? o.kh - 1 : 0), (s3[1] - 1) * o.kw + 1 + (o.trailing ? o.kw - 1 : 0), s3[2] };
                 if (in0->size() == 2)
                     out.erase(out.begin());
                 break;
@@ -1611,6 +1669,11 @@ namespace {
         case OpKind::Resize: {
             const Shape s3 = hwc(*is);
             st = fdx_upsample2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.kh, o.kw, o.bilinear ? 1 : 0, out);
+            break;
+        }
+        case OpKind::Dilate: {
+            const Shape s3 = hwc(*is);
+            st = fdx_dilate2d_nhwc_f32(in0, B, (int)s3[0], (int)s3[1], (int)s3[2], o.kh, o.kw, o.trailing ? 1 : 0, out);
             break;
         }
         case OpKind::Crop: {

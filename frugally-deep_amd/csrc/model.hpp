@@ -13,7 +13,7 @@
 namespace fdx {
 
 enum class OpKind {
-    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat, Host, PReLU, Resize, Crop, Permute
+    Input, Conv2D, DWConv2D, Dense, Affine, LayerNorm, Act, Softmax, ZeroPad, Pool, GlobalPool, Add, Embedding, MHA, View, Einsum, Concat, Host, PReLU, Resize, Crop, Permute, Dilate
 };
 
 using Shape = std::vector<int64_t>; // dims of one sample, no batch axis
@@ -59,6 +59,7 @@ struct Op {
     bool log_after = false;          // Softmax op that is a log_softmax
     bool rms = false;                // LayerNorm op that is an RMSNormalization
     bool bilinear = false;           // Resize: interpolation (kh / kw hold the factors; Crop keeps its margins in zp)
+    bool trailing = false;           // Dilate: zero insertion in front of a "same" transposed convolution (kh / kw hold the rates)
     bool gate = false;               // attention with a sigmoid gate on its output (GroupQueryAttention use_gate)
     std::vector<int64_t> shared_axes; // PReLU
 

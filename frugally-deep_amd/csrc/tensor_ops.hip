@@ -191,6 +191,25 @@ __global__ void crop2d_kernel(const float* __restrict__ in, float* __restrict__ 
     }
 }
 
+// dilate_tensor (include/fdeep/tensor.hpp:612-640) on [n][h][w][c]: input pixel (y, x) lands on (y*ry + oy, x*rx + ox), every
+// other output pixel is zero; one thread per output element, so the zeros are written by the same pass
+__global__ void dilate2d_kernel(const float* __restrict__ in, float* __restrict__ out, int h, int w, int c, int ry, int rx, int oy,
+    int ox, int oh, int ow, size_t total)
+{
+    for (size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (size_t)gridDim.x * blockDim.x) {
+        const int z = (int)(o % (size_t)c);
+        size_t rest = o / (size_t)c;
+        const int x = (int)(rest % (size_t)ow) - ox;
+        rest /= (size_t)ow;
+        const int y = (int)(rest % (size_t)oh) - oy;
+        const size_t img = rest / (size_t)oh;
+        float v = 0.f;
+        if (y >= 0 && x >= 0 && y % ry == 0 && x % rx == 0 && y / ry < h && x / rx < w)
+            v = in[((img * h + (size_t)(y / ry)) * w + (size_t)(x / rx)) * c + z];
+        out[o] = v;
+    }
+}
+
 // resize2d_nearest / resize2d_bilinear for integer factors (include/fdeep/tensor.hpp:959-974, 997-1035): source
 // coordinate (y + 0.5) / factor - 0.5; nearest rounds it (= y / factor for integer factors), bilinear clamps it to
 // [0, extent] and blends the four neighbours, the lower / right one clamped to the last row / column
@@ -479,6 +498,22 @@ extern "C" fdx_status fdx_crop2d_nhwc_f32(const float* in, int n, int h, int w, 
     profile_begin();
     hipLaunchKernelGGL(crop2d_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, h, w, c, top, left, oh, ow, total);
     profile_end("crop2d_f32", 0.0, 8.0 * (double)total);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_dilate2d_nhwc_f32(const float* in, int n, int h, int w, int c, int rate_y, int rate_x, int trailing_zeros,
+    float* out)
+{
+    FDX_REQUIRE(in && out && n > 0 && h > 0 && w > 0 && c > 0 && rate_y > 0 && rate_x > 0, "dilate2d: bad arguments");
+    const bool unit = rate_y == 1 && rate_x == 1; // the reference returns the input itself for rate (1, 1)
+    const int ey = (trailing_zeros && !unit) ? rate_y - 1 : 0, ex = (trailing_zeros && !unit) ? rate_x - 1 : 0;
+    const int oh = (h - 1) * rate_y + 1 + ey, ow = (w - 1) * rate_x + 1 + ex;
+    const size_t total = (size_t)n * oh * ow * c;
+    profile_begin();
+    hipLaunchKernelGGL(dilate2d_kernel, dim3(grid_of(total, 256)), dim3(256), 0, stream(), in, out, h, w, c, rate_y, rate_x,
+        ey - ey / 2, ex - ex / 2, oh, ow, total);
+    profile_end("dilate2d_f32", 0.0, 4.0 * ((double)total + (double)n * h * w * c));
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }

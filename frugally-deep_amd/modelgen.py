@@ -116,6 +116,30 @@ class Builder:
         ow = self._win(w, (kw - 1) * dx + 1, sx, padding)
         return self._add("Conv2D", name, cfg, [x], (oh, ow, filters))
 
+    def conv2d_transpose(self, x, filters, k, name, strides=1, padding="valid", use_bias=True, activation=None, dilation=1,
+                         bias_std=0.2):
+        """Conv2DTranspose (Conv1DTranspose for a rank-2 input); weights in the exporter's [filters][kh][kw][cin] order."""
+        one_d = len(x.shape) == 2
+        kh, kw = (k, k) if isinstance(k, int) else k
+        sy, sx = (strides, strides) if isinstance(strides, int) else strides
+        dy, dx = (dilation, dilation) if isinstance(dilation, int) else dilation
+        h, w, cin = (1,) + tuple(x.shape) if one_d else x.shape
+        if one_d:
+            kh, sy, dy = 1, 1, 1
+        self.params[name] = {"weights": self.he((filters, kh, kw, cin), kh * kw * cin)}
+        if use_bias:
+            self.params[name]["bias"] = self.normal((filters,), bias_std)
+        cfg = {"filters": filters, "padding": padding, "use_bias": use_bias,
+               "kernel_size": [kw] if one_d else [kh, kw], "strides": [sx] if one_d else [sy, sx],
+               "dilation_rate": [dx] if one_d else [dy, dx]}
+        if activation is not None:
+            cfg["activation"] = activation
+        if padding == "same":
+            oh, ow = h * sy, w * sx
+        else:
+            oh, ow = (h - 1) * sy + (kh - 1) * dy + 1, (w - 1) * sx + (kw - 1) * dx + 1
+        return self._add("Conv1DTranspose" if one_d else "Conv2DTranspose", name, cfg, [x], (ow, filters) if one_d else (oh, ow, filters))
+
     def depthwise_conv2d(self, x, k, name, strides=1, padding="valid", use_bias=False, dilation=1, bias_std=0.0):
         kh, kw = (k, k) if isinstance(k, int) else k
         sy, sx = (strides, strides) if isinstance(strides, int) else strides

@@ -218,6 +218,12 @@ fdx_status fdx_concat_f32(const float* const* ins, int n_inputs, const int64_t* 
 fdx_status fdx_permute_f32(const float* in, int batch, int rank, const int64_t* dims, const int* perm, float* out);
 /* Cropping1D / Cropping2D (crop_tensor, include/fdeep/tensor.hpp:586-610) */
 fdx_status fdx_crop2d_nhwc_f32(const float* in, int n, int h, int w, int c, int top, int bottom, int left, int right, float* out);
+/* Zero insertion in front of a transposed convolution (dilate_tensor, include/fdeep/tensor.hpp:612-640, called by
+ * convolve_transposed, include/fdeep/convolution.hpp:443-469): the output has (h-1)*rate_y+1 by (w-1)*rate_x+1 pixels,
+ * plus rate-1 more with the larger half in front when trailing_zeros is set (the layer's "same" padding) and the
+ * rate is not (1, 1).  Conv2DTranspose = this, then fdx_conv2d_nhwc_f32 with stride 1 on the mirrored filter. */
+fdx_status fdx_dilate2d_nhwc_f32(const float* in, int n, int h, int w, int c, int rate_y, int rate_x, int trailing_zeros,
+    float* out);
 /* UpSampling1D / UpSampling2D by integer factors, nearest or bilinear (resize2d_nearest / resize2d_bilinear,
  * include/fdeep/tensor.hpp:959-974, 997-1035; layers/upsampling_2d_layer.hpp) */
 fdx_status fdx_upsample2d_nhwc_f32(const float* in, int n, int h, int w, int c, int factor_y, int factor_x, int bilinear,

@@ -46,7 +46,9 @@ IDENTITY_LAYERS = {
 def build(force=False):
     """Compile liboracle.so with the Makefile next to this file."""
     so = os.path.join(_HERE, "liboracle.so")
-    if force or not os.path.exists(so):
+    src = os.path.join(_HERE, "oracle.c")
+    stale = os.path.exists(so) and os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(so)
+    if force or stale or not os.path.exists(so):
         subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
     return so
 
@@ -99,6 +101,26 @@ def conv2d(x, w_hwio, bias, cout, kh, kw, strides=(1, 1), dilation=(1, 1), paddi
     out = np.empty((hw[0], hw[1], cout), np.float32)
     if lib().fdo_conv2d(_p(x), *args, _p(out), hw) != 0:
         raise RuntimeError("conv2d failed")
+    return out
+
+
+def conv2d_transpose_prepare(w_json, cout, kh, kw, cin):
+    """Filter of a transposed convolution: mirrored in height and width at load (filter.hpp:94-97)."""
+    w = _f32(w_json).reshape(cout, kh, kw, cin)[:, ::-1, ::-1, :]
+    return conv2d_prepare(np.ascontiguousarray(w), cout, kh, kw, cin)
+
+
+def conv2d_transpose(x, w_hwio_flipped, bias, cout, kh, kw, strides=(1, 1), dilation=(1, 1), padding="valid"):
+    x = _f32(x)
+    h, w, cin = x.shape
+    hw = (ctypes.c_int * 2)()
+    args = (h, w, cin, _p(w_hwio_flipped), _p(bias), cout, kh, kw, strides[0], strides[1],
+            dilation[0], dilation[1], PAD[padding])
+    if lib().fdo_conv2d_transpose(_p(x), *args, None, hw) != 0:
+        raise RuntimeError("transposed convolution: output width does not match")
+    out = np.empty((hw[0], hw[1], cout), np.float32)
+    if lib().fdo_conv2d_transpose(_p(x), *args, _p(out), hw) != 0:
+        raise RuntimeError("conv2d_transpose failed")
     return out
 
 
@@ -453,12 +475,13 @@ class _Layer:
         self.nodes = [_node_inputs(n) for n in data.get("inbound_nodes", [])]
         self.p = {}
         c, cls, name = self.cfg, self.cls, self.name
-        if cls in ("Conv2D", "Conv1D"):
+        if cls in ("Conv2D", "Conv1D", "Conv2DTranspose", "Conv1DTranspose"):
             self.kh, self.kw = _pair(c["kernel_size"])
             self.cout = int(c["filters"])
             w = decode_floats(get_param(name, "weights"))
             self.cin = w.size // (self.kh * self.kw * self.cout)
-            self.p["w"] = conv2d_prepare(w, self.cout, self.kh, self.kw, self.cin)
+            prepare = conv2d_transpose_prepare if cls.endswith("Transpose") else conv2d_prepare
+            self.p["w"] = prepare(w, self.cout, self.kh, self.kw, self.cin)
             self.p["b"] = decode_floats(get_param(name, "bias")) if c["use_bias"] else np.zeros(self.cout, np.float32)
         elif cls == "DepthwiseConv2D":
             self.kh, self.kw = c["kernel_size"]
@@ -512,6 +535,12 @@ class _Layer:
             one_d = x.ndim == 2  # a (width, depth) sequence is a height-1 image
             out = conv2d(x[None] if one_d else x, p["w"], p["b"], self.cout, self.kh, self.kw, _pair(c["strides"]),
                          _pair(c["dilation_rate"]), c["padding"])
+            out = out[0] if one_d else out
+        elif cls in ("Conv2DTranspose", "Conv1DTranspose"):
+            x = _f32(ins[0])
+            one_d = x.ndim == 2
+            out = conv2d_transpose(x[None] if one_d else x, p["w"], p["b"], self.cout, self.kh, self.kw,
+                                   _pair(c["strides"]), _pair(c["dilation_rate"]), c["padding"])
             out = out[0] if one_d else out
         elif cls == "DepthwiseConv2D":
             out = depthwise_conv2d(ins[0], p["w"], p["b"], self.kh, self.kw, c["strides"],

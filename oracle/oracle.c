@@ -207,6 +207,63 @@ int fdo_conv2d(const float* in, int h, int w, int cin, const float* w_hwio, cons
 }
 
 /*
+ * Conv2DTranspose / Conv1DTranspose layer.  The filter arrives in the converted-JSON order
+ * [Cout][kh][kw][Cin] (keras_export/convert_model.py:221-224) and is mirrored in height and
+ * width at load (include/fdeep/filter.hpp:94-97); w_hwio_flipped is that mirrored filter in
+ * [kh][kw][Cin][Cout] order (fdo_conv2d_prepare of the mirrored array).  Forward
+ * (include/fdeep/convolution.hpp:443-469): zeros are inserted between the input pixels
+ * (dilate_tensor, include/fdeep/tensor.hpp:612-640 -- with "same" padding sy-1 / sx-1
+ * further zeros are added, the larger half in front), the result is padded by the
+ * transposed branch of preprocess_convolution (convolution.hpp:320-396: kh-1 / kw-1 on every
+ * side for "valid", the stride-1 "same" split otherwise) and convolved with stride 1.
+ * Filter dilation is applied to the filter before mirroring (filter.hpp:93), so (dy, dx) act
+ * as an ordinary dilation of the mirrored filter and the window uses the inflated size.
+ * "causal" fails the reference's own output-width assertion (convolution.hpp:243) for any
+ * filter wider than one tap and is rejected here.
+ */
+int fdo_conv2d_transpose(const float* in, int h, int w, int cin, const float* w_hwio_flipped, const float* bias,
+    int cout, int kh, int kw, int sy, int sx, int dy, int dx, int pad_type,
+    float* out, int* out_hw)
+{
+    if (pad_type != 0 && pad_type != 1)
+        return -1;
+    const int same = pad_type == 1;
+    const int ekh = (kh - 1) * dy + 1, ekw = (kw - 1) * dx + 1;
+    const int exp_y = (same && !(sy == 1 && sx == 1)) ? sy - 1 : 0;
+    const int exp_x = (same && !(sy == 1 && sx == 1)) ? sx - 1 : 0;
+    const int dh = (h - 1) * sy + 1 + exp_y, dw = (w - 1) * sx + 1 + exp_x;
+    const int off_y = exp_y - exp_y / 2, off_x = exp_x - exp_x / 2;
+    int pt, pb, pl, pr, oh, ow;
+    if (same) {
+        /* stride 1: in % 1 == 0 -> pad_along = max(filter - 1, 0) */
+        oh = dh;
+        ow = dw;
+        pt = (ekh - 1) / 2; pb = (ekh - 1) - pt;
+        pl = (ekw - 1) / 2; pr = (ekw - 1) - pl;
+    } else {
+        oh = dh + ekh - 1;
+        ow = dw + ekw - 1;
+        pt = pb = ekh - 1;
+        pl = pr = ekw - 1;
+    }
+    out_hw[0] = oh;
+    out_hw[1] = ow;
+    if (!out)
+        return 0;
+    const int ph = dh + pt + pb, pw = dw + pl + pr;
+    float* padded = (float*)calloc((size_t)ph * pw * cin, sizeof(float));
+    if (!padded)
+        return -2;
+    for (int y = 0; y < h; ++y)
+        for (int x = 0; x < w; ++x)
+            memcpy(padded + ((size_t)(y * sy + off_y + pt) * pw + (x * sx + off_x + pl)) * cin,
+                in + ((size_t)y * w + x) * cin, sizeof(float) * (size_t)cin);
+    fdo_conv2d_padded(padded, ph, pw, cin, w_hwio_flipped, bias, cout, kh, kw, 1, 1, dy, dx, oh, ow, out);
+    free(padded);
+    return 0;
+}
+
+/*
  * DepthwiseConv2D (depth multiplier 1).  Filter arrives in converted-JSON order
  * [C][kh][kw] (keras_export/convert_model.py:203-206) and is inflated with zeros
  * for dilation at load (include/fdeep/filter.hpp:93,

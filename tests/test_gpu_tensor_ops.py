@@ -400,3 +400,72 @@ def test_model_with_resampling_layers(fdx, oracle, modelgen):
     errs = [rel(g, w) for g, w in zip(got, want)]
     say("  rel errors:", ["%.2e" % e for e in errs])
     assert max(errs) <= TOL
+
+
+def test_dilate_kernel(fdx):
+    say("dilate2d kernel")
+    r = np.random.default_rng(20)
+    x = r.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    for ry, rx, trailing in ((2, 2, False), (2, 2, True), (3, 2, True), (1, 4, True), (4, 1, False), (1, 1, True)):
+        ey, ex = ((ry - 1, rx - 1) if trailing and (ry, rx) != (1, 1) else (0, 0))
+        want = np.zeros((2, 2 * ry + 1 + ey, 3 * rx + 1 + ex, 5), np.float32)
+        want[:, ey - ey // 2::ry, ex - ex // 2::rx][:, :3, :4] = x
+        assert np.array_equal(fdx.dilate2d(x, ry, rx, trailing), want), (ry, rx, trailing)
+
+
+@pytest.mark.parametrize("case", [
+    # h, w, cin, cout, k, strides, padding, dilation, activation
+    (6, 7, 5, 8, 3, 2, "same", 1, "relu"),
+    (6, 7, 5, 8, 3, 2, "valid", 1, None),
+    (5, 5, 16, 32, (4, 2), (2, 3), "same", 1, None),
+    (5, 6, 16, 16, 3, 1, "valid", 1, "tanh"),
+    (5, 6, 3, 4, 3, 1, "same", 2, None),
+    (4, 4, 6, 5, 2, 3, "same", 1, None),   # kernel smaller than the stride
+    (4, 5, 6, 5, (3, 2), 2, "valid", (2, 1), "sigmoid"),
+])
+def test_conv2d_transpose_layer(fdx, oracle, modelgen, case):
+    h, w, cin, cout, k, strides, padding, dilation, activation = case
+    say("Conv2DTranspose", case)
+    b = modelgen.Builder("deconv", 90)
+    x = b.input((h, w, cin), "img")
+    y = b.conv2d_transpose(x, cout, k, "up", strides=strides, padding=padding, dilation=dilation, activation=activation)
+    js = modelgen.dumps(b.finish([y]))
+    r = np.random.default_rng(21)
+    xi = r.standard_normal((3, h, w, cin)).astype(np.float32)
+    ref = oracle.OracleModel(js)
+    want = np.stack([ref.predict([xi[i]])[0] for i in range(3)])
+    got = fdx.Model(js).predict([xi])[0]
+    assert got.shape == want.shape == (3,) + tuple(y.shape)
+    assert rel(got, want) <= TOL
+
+
+def test_decoder_model_with_transposed_convolutions(fdx, oracle, modelgen):
+    """Autoencoder shape: strided convolutions down, Conv2DTranspose up with a skip Add, BatchNormalization behind a
+    transposed convolution (folded at load), ZeroPadding2D in front of one, and Conv1DTranspose on a sequence."""
+    say("transposed-convolution decoder model")
+    b = modelgen.Builder("autoencoder", 91)
+    img = b.input((16, 16, 3), "img")
+    e1 = b.conv2d(img, 16, 3, "e1", strides=2, padding="same", activation="relu", bias_std=0.1)
+    e2 = b.conv2d(e1, 32, 3, "e2", strides=2, padding="same", activation="relu", bias_std=0.1)
+    d1 = b.conv2d_transpose(e2, 16, 3, "d1", strides=2, padding="same")
+    d1 = b.batchnorm(d1, "d1_bn", random_stats=True)
+    d1 = b.relu(d1, "d1_relu")
+    s1 = b.add([d1, e1], "skip")
+    d2 = b.conv2d_transpose(s1, 8, 4, "d2", strides=2, padding="same", activation="relu")
+    zp = b._add("ZeroPadding2D", "zp", {"padding": [[1, 0], [0, 2]]}, [d2], (17, 18, 8))
+    d3 = b.conv2d_transpose(zp, 3, 3, "d3", strides=1, padding="valid", activation="sigmoid")
+    seq = b.input((9, 4), "seq")
+    t1 = b.conv2d_transpose(seq, 6, 3, "t1", strides=2, padding="same", activation="relu")
+    t2 = b.conv2d_transpose(t1, 2, 2, "t2", strides=3, padding="valid")
+    spec = b.finish([d3, t2])
+    r = np.random.default_rng(22)
+    xi, xs = r.standard_normal((4, 16, 16, 3)).astype(np.float32), r.standard_normal((4, 9, 4)).astype(np.float32)
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([xi[i], xs[i]]) for i in range(4)]
+    want = [np.stack([w[k] for w in want]) for k in range(2)]
+    got = fdx.Model(js).predict([xi, xs])
+    assert got[0].shape == (4, 19, 20, 3) and got[1].shape == (4, 18 * 3 - 3 + 2, 2)
+    errs = [rel(g, w) for g, w in zip(got, want)]
+    say("  rel errors:", ["%.2e" % e for e in errs])
+    assert max(errs) <= TOL

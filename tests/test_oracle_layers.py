@@ -124,6 +124,100 @@ def test_conv2d_closed_forms(oracle):
     assert np.array_equal(got[:, :, 0], x1[0:4, 2:7, 0])
 
 
+def torch_conv_transpose_full(x, wj, b, strides, dilation):
+    """Scatter form in fp64: out[y*s + ky*d, x*s + kx*d, co] += in[y, x, ci] * K[co, ky, kx, ci] (+ bias)."""
+    import torch.nn.functional as F
+    xt = torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None]
+    wt = torch.from_numpy(wj.astype(np.float64)).permute(3, 0, 1, 2)  # [cin][cout][kh][kw]
+    y = F.conv_transpose2d(xt, wt, None if b is None else torch.from_numpy(b.astype(np.float64)),
+                           stride=strides, dilation=dilation)
+    return y[0].permute(1, 2, 0).numpy()
+
+
+TRANSPOSE_CASES = [
+    # h, w, cin, cout, kh, kw, strides, dilation
+    (5, 6, 3, 4, 3, 3, (1, 1), (1, 1)),
+    (5, 6, 3, 4, 3, 3, (2, 2), (1, 1)),
+    (4, 7, 2, 5, 4, 2, (2, 3), (1, 1)),
+    (6, 5, 4, 3, 5, 5, (3, 2), (1, 1)),
+    (5, 5, 2, 3, 3, 2, (2, 2), (2, 2)),
+    (1, 9, 3, 4, 1, 3, (1, 2), (1, 1)),   # Conv1DTranspose seen as a height-1 image
+    (4, 4, 3, 2, 1, 1, (3, 3), (1, 1)),
+    (4, 5, 3, 2, 2, 2, (3, 4), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSE_CASES)
+def test_conv2d_transpose_valid_vs_torch_fp64(oracle, case):
+    h, w, cin, cout, kh, kw, strides, dilation = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = rng.standard_normal((h, w, cin)).astype(np.float32)
+    wj = rng.standard_normal((cout, kh, kw, cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    got = oracle.conv2d_transpose(x, oracle.conv2d_transpose_prepare(wj, cout, kh, kw, cin), b, cout, kh, kw,
+                                  strides, dilation, "valid")
+    want = torch_conv_transpose_full(x, wj, b, strides, dilation)
+    assert got.shape == want.shape
+    assert rel(got, want) < TOL
+
+
+@pytest.mark.parametrize("case", [c for c in TRANSPOSE_CASES if c[7] == (1, 1) and c[4] >= c[6][0] and c[5] >= c[6][1]])
+def test_conv2d_transpose_same_is_input_gradient_of_same_conv(oracle, case):
+    # TensorFlow defines the layer as the input gradient of the strided "same" convolution whose output is x:
+    # an image of (h*sy, w*sx) pixels convolved with the same kernel (cin and cout swapped) gives (h, w).
+    import torch.nn.functional as F
+    h, w, cin, cout, kh, kw, strides, _ = case
+    rng = np.random.default_rng(hash(case) % 2**32 + 1)
+    x = rng.standard_normal((h, w, cin)).astype(np.float32)
+    wj = rng.standard_normal((cout, kh, kw, cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    got = oracle.conv2d_transpose(x, oracle.conv2d_transpose_prepare(wj, cout, kh, kw, cin), b, cout, kh, kw,
+                                  strides, (1, 1), "same")
+    big = torch.zeros(1, cout, h * strides[0], w * strides[1], dtype=torch.float64, requires_grad=True)
+    pads = []
+    for n, k, s in ((w * strides[1], kw, strides[1]), (h * strides[0], kh, strides[0])):
+        _, before, after = tf_geometry(n, k, s, "same")
+        pads += [before, after]
+    # forward filter of that convolution: [out = cin of the layer][in = cout of the layer][kh][kw]
+    fwd = torch.from_numpy(wj.astype(np.float64)).permute(3, 0, 1, 2)
+    y = F.conv2d(F.pad(big, pads), fwd, stride=strides)
+    assert tuple(y.shape[2:]) == (h, w)
+    (grad,) = torch.autograd.grad(y, big, torch.from_numpy(x.astype(np.float64)).permute(2, 0, 1)[None])
+    want = grad[0].permute(1, 2, 0).numpy() + b.astype(np.float64)
+    assert got.shape == want.shape
+    assert rel(got, want) < TOL
+
+
+@pytest.mark.parametrize("case", TRANSPOSE_CASES)
+def test_conv2d_transpose_same_is_a_window_of_the_full_result(oracle, case):
+    # "same" keeps h*sy x w*sx pixels of the full ("valid") result; the window starts where the reference's padding
+    # puts it (convolution.hpp:366-377 on the zero-stuffed input of tensor.hpp:619-626), which for kernels smaller
+    # than the stride lies one zero row / column before the full result.
+    h, w, cin, cout, kh, kw, strides, dilation = case
+    rng = np.random.default_rng(hash(case) % 2**32 + 2)
+    x = rng.standard_normal((h, w, cin)).astype(np.float32)
+    wj = rng.standard_normal((cout, kh, kw, cin)).astype(np.float32)
+    got = oracle.conv2d_transpose(x, oracle.conv2d_transpose_prepare(wj, cout, kh, kw, cin), None, cout, kh, kw,
+                                  strides, dilation, "same")
+    full = torch_conv_transpose_full(x, wj, None, strides, dilation)
+    assert got.shape == (h * strides[0], w * strides[1], cout)
+    starts = []
+    for k, d, s in ((kh, dilation[0], strides[0]), (kw, dilation[1], strides[1])):
+        ek = (k - 1) * d + 1
+        lead = 0 if strides == (1, 1) else (s - 1) - (s - 1) // 2
+        starts.append((ek - 1) - lead - (ek - 1) // 2)
+    big = np.zeros((full.shape[0] + 2 * 8, full.shape[1] + 2 * 8, cout))
+    big[8:8 + full.shape[0], 8:8 + full.shape[1]] = full
+    want = big[8 + starts[0]:8 + starts[0] + got.shape[0], 8 + starts[1]:8 + starts[1] + got.shape[1]]
+    assert rel(got, want) < TOL
+
+
+def test_conv2d_transpose_rejects_causal(oracle):
+    x = np.ones((4, 4, 1), np.float32)
+    with pytest.raises(RuntimeError):
+        oracle.conv2d_transpose(x, np.ones(4, np.float32), None, 1, 2, 2, (1, 1), (1, 1), "causal")
+
+
 @pytest.mark.parametrize("case", [
     (9, 8, 6, 3, 3, (1, 1), (1, 1), "same"), (9, 8, 6, 3, 3, (2, 2), (1, 1), "same"),
     (10, 11, 5, 3, 3, (2, 2), (1, 1), "valid"), (12, 12, 4, 3, 3, (1, 1), (2, 2), "same"),
