@@ -1446,12 +1446,18 @@ namespace {
 
 fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out)
 {
-    if (m->plan && m->plan->batch == batch && m->plan->in_shapes == in_shapes) {
-        *out = m->plan.get();
-        return FDX_OK;
+    for (size_t i = 0; i < m->plans.size(); ++i)
+        if (m->plans[i]->batch == batch && m->plans[i]->in_shapes == in_shapes) {
+            if (i != 0)
+                std::rotate(m->plans.begin(), m->plans.begin() + (std::ptrdiff_t)i, m->plans.begin() + (std::ptrdiff_t)i + 1);
+            *out = m->plans[0].get();
+            return FDX_OK;
+        }
+    if (m->plans.size() >= fdx_model::kMaxPlans) {
+        // the least recently used plan gives its buffers back before the new one asks for its own
+        FDX_HIP(hipStreamSynchronize(stream()));
+        m->plans.pop_back();
     }
-    FDX_HIP(hipStreamSynchronize(stream()));
-    m->plan.reset();
     std::unique_ptr<Plan> p(new Plan);
     p->batch = batch;
     p->in_shapes = in_shapes;
@@ -1539,8 +1545,8 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
         p->blocks.push_back(b);
         p->temps[idx].push_back(static_cast<float*>(b.p));
     }
-    m->plan = std::move(p);
-    *out = m->plan.get();
+    m->plans.insert(m->plans.begin(), std::move(p));
+    *out = m->plans[0].get();
     return FDX_OK;
 }
 
@@ -2048,7 +2054,7 @@ fdx_model::~fdx_model()
     for (auto& hl : host_layers)
         if (hl.vt.destroy && hl.instance)
             hl.vt.destroy(hl.instance);
-    plan.reset();
+    plans.clear();
     for (float* p : device_allocs)
         (void)hipFree(p);
     if (err_flag)

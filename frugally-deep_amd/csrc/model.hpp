@@ -106,7 +106,10 @@ struct fdx_model {
     std::vector<float*> device_allocs;
     int* err_flag = nullptr;
     bool has_embedding = false;
-    std::unique_ptr<fdx::Plan> plan;
+    // launch plans keyed by (batch, per-sample input shapes), most recently used first; a model fed alternating shapes
+    // (variable input dimensions, tensor_shape_variable.hpp) keeps up to kMaxPlans of them instead of re-planning
+    static constexpr size_t kMaxPlans = 4;
+    std::vector<std::unique_ptr<fdx::Plan>> plans;
     std::mutex mu;
     double last_flops = 0;
     ~fdx_model();

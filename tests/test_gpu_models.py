@@ -134,3 +134,36 @@ def test_input_shape_errors(fdx, modelgen):
     bad["architecture"]["config"]["layers"][1]["class_name"] = "Conv9D"
     with pytest.raises(fdx.FdxError, match="unknown layer type: Conv9D"):
         fdx.Model(modelgen.dumps(bad))
+
+
+def test_variable_input_size_cycles_through_more_shapes_than_cached_plans(fdx, oracle, modelgen):
+    """A fully convolutional model with variable height and width (input_shapes [null, null, 3]): every (batch, shape)
+    pair gets its own launch plan; a few recent ones are kept, so going round more shapes than that re-plans, and
+    coming back to a kept one reuses its buffers. Every call is checked against the oracle."""
+    say("variable-size fully convolutional model")
+    b = modelgen.Builder("fcn", 33)
+    x = b.input((16, 16, 3), "img")
+    y = b.conv2d(x, 8, 3, "c1", padding="same", activation="relu", bias_std=0.1)
+    y = b.pool(y, "p1", 2, 2)
+    y = b.conv2d(y, 16, 3, "c2", strides=2, padding="same", activation="relu", bias_std=0.1)
+    y = b.conv2d_transpose(y, 8, 3, "up", strides=2, padding="same", activation="relu")
+    y = b.conv2d(y, 4, 1, "head", bias_std=0.1)
+    spec = b.finish([y])
+    spec["input_shapes"] = [[None, None, 3]]
+    spec["output_shapes"] = [[None, None, 4]]
+    for layer in spec["architecture"]["config"]["layers"]:
+        if layer["class_name"] == "InputLayer":
+            layer["config"]["batch_shape"] = [None, None, None, 3]
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    model = fdx.Model(js)
+    r = np.random.default_rng(34)
+    sizes = [(16, 16), (12, 20), (9, 7), (24, 8), (31, 5), (10, 10)]
+    inputs = {s: r.standard_normal((2 + i % 2,) + s + (3,)).astype(np.float32) for i, s in enumerate(sizes)}
+    for s in sizes + sizes[::-1] + [sizes[0], sizes[0]]:
+        xi = inputs[s]
+        want = np.stack([ref.predict([xi[i]])[0] for i in range(xi.shape[0])])
+        got = model.predict([xi])[0]
+        assert rel(got, want) <= TOL, s
+    with pytest.raises(fdx.FdxError, match="Invalid inputs shape"):
+        model.predict([np.zeros((1, 8, 8, 4), np.float32)])
