@@ -1,12 +1,16 @@
 // MultiHeadAttention core on already projected q / k / v (gfx950).
 //
-// Prefill shape (many query rows): scores = scale * Q K^T as one batched NT GEMM over
-// (sequence, head) on fp32 MFMA, row softmax in the reference's log-sum form with an
-// optional causal prefix limit, then P V as a second batched NT GEMM against V^T.
+// Prefill shape (many query rows): one fused pass for head depths 32 / 64 / 128 (scores, softmax
+// and P V on fp32 MFMA with the probabilities kept in registers); any other depth runs as
+// scores = scale * Q K^T (one batched NT GEMM over (sequence, head)), row softmax in the
+// reference's log-sum form with an optional causal prefix limit, then P V as a second batched
+// NT GEMM against V^T.
 // Decode shape (one query row per sequence): a dedicated HBM-bound kernel that streams
 // the token-major key / value cache once.
 #include <cfloat>
 #include <cmath>
+#include <cstdint>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -94,6 +98,229 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(const float* __restrict
     }
 }
 
+// ---- fused prefill attention: scores, softmax and P V in one pass, nothing but the output written --------------------
+//
+// One workgroup = 128 query rows of one (sequence, head), one wave = 32 of them; keys / values pass through LDS in
+// tiles of 64.  The products are taken transposed on the 32x32x2 fp32 MFMA: S^T = K Q^T puts a query on a lane
+// (column) and keys on the accumulator registers, so the running maximum, the running sum and the rescaling of the
+// flash-attention recurrence are per-lane scalars, and the probabilities P^T are already laid out as the B operand of
+// O^T = V^T P^T -- they never leave the registers.  The contraction index of either product may be visited in any
+// order as long as both operands agree, which is what lets the accumulator layout (keys 8j + 4*half + i in register
+// 4j + i) feed the second product directly.
+//
+// Softmax as the reference takes it (include/fdeep/tensor.hpp:1165-1192) is exp(x - max - log(sum exp(x - max)));
+// here the running maximum replaces max and the division by the running sum comes last, which agrees to rounding.
+struct FlashParams {
+    const float* q; int64_t ldq, q_batch;
+    const float* k; int64_t ldk, k_batch;
+    const float* v; int64_t ldv, v_batch;
+    float* out; int64_t ldo, o_batch;
+    int t, s, heads, causal;
+    float scale;
+};
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void flash_prefill_kernel(FlashParams p)
+{
+    constexpr int KS = DK + 4;  // LDS row strides: 16-byte fragment reads along a key row stay conflict-free
+    constexpr int VS = DV + 8;  // lanes read along the depth; rows 4 apart (the two lane halves) fall on disjoint banks
+    constexpr int KL = DK / 16, VL = DV / 16; // 16-byte loads per thread for a 64-row tile
+    __shared__ __attribute__((aligned(16))) float ks[64 * KS];
+    __shared__ __attribute__((aligned(16))) float vs[64 * VS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 31, half = lane >> 5;
+    const int b = blockIdx.y / p.heads, h = blockIdx.y % p.heads;
+    const int q_first = blockIdx.x * 128;
+    const int query = q_first + wave * 32 + c;
+    const bool q_ok = query < p.t;
+    const int shift = p.s - p.t; // causal: query i sees keys 0 .. i + shift
+
+    // this lane's half of its query row: depth 8u + 4*half .. + 3, the same split the key fragments use
+    f32x4 qreg[DK / 8];
+    {
+        const float* qrow = p.q + (int64_t)b * p.q_batch + (int64_t)(q_ok ? query : 0) * p.ldq + h * DK + 4 * half;
+#pragma unroll
+        for (int u = 0; u < DK / 8; ++u)
+            qreg[u] = q_ok ? *reinterpret_cast<const f32x4*>(qrow + 8 * u) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+    }
+
+    // keys this workgroup needs: all of them, or up to the last one its last query may see
+    int s_end = p.s;
+    if (p.causal) {
+        const int q_last = (q_first + 128 < p.t ? q_first + 128 : p.t) - 1;
+        s_end = q_last + shift + 1 < p.s ? q_last + shift + 1 : p.s;
+    }
+    const int tiles = (s_end + 63) / 64;
+    const int wave_q_last = q_first + wave * 32 + 31;
+
+    const float* kbase = p.k + (int64_t)b * p.k_batch + h * DK;
+    const float* vbase = p.v + (int64_t)b * p.v_batch + h * DV;
+    f32x4 kst[KL], vst[VL];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int idx = tid + 256 * i, row = idx / (DK / 4), c4 = idx % (DK / 4);
+            kst[i] = j0 + row < p.s ? *reinterpret_cast<const f32x4*>(kbase + (int64_t)(j0 + row) * p.ldk + 4 * c4)
+                                     : f32x4 { 0.f, 0.f, 0.f, 0.f };
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int idx = tid + 256 * i, row = idx / (DV / 4), c4 = idx % (DV / 4);
+            vst[i] = j0 + row < p.s ? *reinterpret_cast<const f32x4*>(vbase + (int64_t)(j0 + row) * p.ldv + 4 * c4)
+                                     : f32x4 { 0.f, 0.f, 0.f, 0.f };
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int idx = tid + 256 * i, row = idx / (DK / 4), c4 = idx % (DK / 4);
+            *reinterpret_cast<f32x4*>(&ks[row * KS + 4 * c4]) = kst[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int idx = tid + 256 * i, row = idx / (DV / 4), c4 = idx % (DV / 4);
+            *reinterpret_cast<f32x4*>(&vs[row * VS + 4 * c4]) = vst[i];
+        }
+    };
+
+    f32x16 oacc[DV / 32];
+#pragma unroll
+    for (int d = 0; d < DV / 32; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            oacc[d][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    if (tiles > 0)
+        fetch(0);
+    for (int tile = 0; tile < tiles; ++tile) {
+        const int j0 = tile * 64;
+        __syncthreads(); // every wave is done with the previous tile
+        stage();
+        __syncthreads();
+        if (tile + 1 < tiles)
+            fetch(j0 + 64); // in flight while this tile is worked on
+        if (p.causal && j0 > wave_q_last + shift)
+            continue; // nothing in this tile is visible to any of this wave's queries (wave-uniform)
+
+        // S^T tile: 64 keys x 32 queries
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                sacc[kb][e] = 0.f;
+#pragma unroll
+            for (int u = 0; u < DK / 8; ++u) {
+                const f32x4 kf = *reinterpret_cast<const f32x4*>(&ks[(kb * 32 + c) * KS + 8 * u + 4 * half]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qreg[u][e], sacc[kb], 0, 0, 0);
+            }
+        }
+        // scale, mask, running maximum
+        const int key_limit = p.causal ? (query + shift < p.s - 1 ? query + shift : p.s - 1) : p.s - 1;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int key = j0 + kb * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                const float sv = key <= key_limit ? sacc[kb][e] * p.scale : -INFINITY;
+                sacc[kb][e] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        // a query that has seen no key yet (rows past the end of the sequence) keeps zeros instead of NaNs
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float corr = expf(m_run - m_use);
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float pv = expf(sacc[kb][e] - m_use);
+                sacc[kb][e] = pv;
+                rs += pv;
+            }
+        rs += __shfl_xor(rs, 32, 64);
+        l_run = l_run * corr + rs;
+        m_run = m_new;
+#pragma unroll
+        for (int d = 0; d < DV / 32; ++d)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                oacc[d][e] *= corr;
+        // O^T += V^T P^T
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float* vrow = &vs[(kb * 32 + 8 * (e >> 2) + 4 * half + (e & 3)) * VS + c];
+#pragma unroll
+                for (int d = 0; d < DV / 32; ++d)
+                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * d], sacc[kb][e], oacc[d], 0, 0, 0);
+            }
+    }
+
+    if (q_ok) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        float* orow = p.out + (int64_t)b * p.o_batch + (int64_t)query * p.ldo + h * DV + 4 * half;
+#pragma unroll
+        for (int d = 0; d < DV / 32; ++d)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 o = { oacc[d][4 * g] * inv, oacc[d][4 * g + 1] * inv, oacc[d][4 * g + 2] * inv, oacc[d][4 * g + 3] * inv };
+                *reinterpret_cast<f32x4*>(orow + 32 * d + 8 * g) = o;
+            }
+    }
+}
+
+template <int DK, int DV>
+static void flash_launch(const FlashParams& p, int batch)
+{
+    const dim3 grid((unsigned)((p.t + 127) / 128), (unsigned)(batch * p.heads));
+    hipLaunchKernelGGL((flash_prefill_kernel<DK, DV>), grid, dim3(256), 0, stream(), p);
+}
+
+static bool flash_enabled()
+{
+    static const bool on = [] {
+        const char* e = std::getenv("FDX_FLASH");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+// true when the fused kernel took the call
+static bool flash_prefill(const FlashParams& p, int batch, int dk, int dv)
+{
+    if (!flash_enabled())
+        return false;
+    auto aligned = [](const void* ptr, int64_t ld, int64_t bs) {
+        return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0 && (ld & 3) == 0 && (bs & 3) == 0;
+    };
+    if (!aligned(p.q, p.ldq, p.q_batch) || !aligned(p.k, p.ldk, p.k_batch) || !aligned(p.v, p.ldv, p.v_batch)
+        || !aligned(p.out, p.ldo, p.o_batch))
+        return false;
+    profile_begin();
+    if (dk == 64 && dv == 64)
+        flash_launch<64, 64>(p, batch);
+    else if (dk == 32 && dv == 32)
+        flash_launch<32, 32>(p, batch);
+    else if (dk == 128 && dv == 128)
+        flash_launch<128, 128>(p, batch);
+    else
+        return false;
+    const double pairs = p.causal ? (double)p.t * (p.s - p.t) + 0.5 * (double)p.t * (p.t + 1) : (double)p.t * p.s;
+    profile_end("mha_flash_f32", 2.0 * batch * p.heads * pairs * (dk + dv),
+        4.0 * batch * p.heads * ((double)p.t * (dk + dv) + (double)p.s * (dk + dv)));
+    return true;
+}
+
 } // namespace fdx
 
 using namespace fdx;
@@ -114,11 +341,18 @@ fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, con
     FDX_REQUIRE(batch > 0 && t > 0 && s > 0 && heads > 0 && dk > 0 && dv > 0, "mha_prefill: bad shape");
     FDX_REQUIRE(!causal || s >= t, "mha_prefill: causal attention needs at least as many keys as queries");
     FDX_REQUIRE((int64_t)batch * heads <= 65535, "mha_prefill: batch * heads too large");
+    // 1 / sqrt(key_dim) applied to the scores after the product (multi_head_attention_layer.hpp:91-93)
+    const float scale = (float)(1.0 / std::sqrt((double)dk));
+    {
+        FlashParams fp { q, ldq, q_batch, k, ldk, k_batch, v, ldv, v_batch, out, ldo, o_batch, t, s, heads, causal, scale };
+        if (flash_prefill(fp, batch, dk, dv)) {
+            FDX_LAUNCH_CHECK();
+            return FDX_OK;
+        }
+    }
     float* scores = static_cast<float*>(scratch_dev);
     float* vt = scores + (((size_t)batch * heads * t * s + 3) & ~(size_t)3);
     const int64_t v_row = (int64_t)heads * dv;
-    // 1 / sqrt(key_dim) applied to the scores after the product (multi_head_attention_layer.hpp:91-93)
-    const float scale = (float)(1.0 / std::sqrt((double)dk));
     fdx_gemm_batch bt {};
     bt.batch = batch * heads;
     bt.inner = heads;

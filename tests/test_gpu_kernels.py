@@ -242,7 +242,13 @@ def numpy_attention(q, k, v, heads, dk, dv, causal):
 
 @pytest.mark.parametrize("b,t,s,heads,dk,dv,causal", [(2, 5, 7, 3, 4, 5, False), (2, 16, 16, 2, 64, 64, True),
                                                       (1, 33, 33, 4, 16, 16, True), (2, 64, 64, 8, 64, 64, False),
-                                                      (1, 3, 9, 2, 8, 8, True)])
+                                                      (1, 3, 9, 2, 8, 8, True),
+                                                      # depths the fused (flash-style) kernel takes: ragged tiles, key
+                                                      # prefix longer than the queries, several query tiles, one query
+                                                      (2, 256, 256, 4, 64, 64, False), (2, 130, 200, 3, 64, 64, True),
+                                                      (1, 300, 300, 2, 64, 64, True), (2, 100, 300, 3, 32, 32, False),
+                                                      (1, 129, 129, 2, 128, 128, True), (3, 1, 70, 2, 64, 64, False),
+                                                      (2, 64, 65, 2, 32, 32, True)])
 def test_mha_prefill(fdx, oracle, b, t, s, heads, dk, dv, causal):
     say("mha prefill", b, t, s, heads, dk, dv, causal)
     r = rng_for("mha", b, t, s, heads, dk, dv, causal)
