@@ -26,7 +26,10 @@
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(GemmParams p)
+// (the second bound asks for two waves per SIMD where the split variant of the largest four-wave tile would otherwise
+// settle for one: its reduction holds the accumulators in ordinary registers next to the prefetched operands)
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (SPLIT && WAVES_M * WAVES_N == 4 && BM * BN >= 128 * 128) ? 2 : 1)
+void igemm_fast_kernel(GemmParams p)
 {
     constexpr int NT = 64 * WAVES_M * WAVES_N;
     static_assert(NT == 256 || NT == 512, "four or eight waves");
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
 
         if (SPLIT && su_done >= 0) {
             constexpr int TILE_F = BM * BN;
-            const int out_tile = su_done / S, my_split = su_done - out_tile * S; // out_tile counts from the first split tile
+            const int out_tile = su_done / S; // counts from the first split tile
             float* mine = p.split_ws + (int64_t)su_done * TILE_F + t;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -268,27 +271,28 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_fast_kernel(Gemm
                     break;
                 continue;
             }
-            f32x16 own[TM][TN];
+            // every unit, this one included, has left its partial in the workspace: they are summed from there in
+            // split order (re-reading the own one costs a tile of loads and saves a second copy of the accumulators,
+            // which would halve the number of resident workgroups)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    own[i][j] = acc[i][j];
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
                     for (int e = 0; e < 16; ++e)
                         acc[i][j][e] = 0.f;
-                }
             for (int sp = 0; sp < S; ++sp) {
                 const float* part = p.split_ws + ((int64_t)out_tile * S + sp) * TILE_F + t;
-                const bool self = sp == my_split;
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j)
+                    for (int j = 0; j < TN; ++j) {
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            acc[i][j][e] += self ? own[i][j][e]
-                                                 : __hip_atomic_load(part + ((i * TN + j) * 16 + e) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            acc[i][j][e] += __hip_atomic_load(part + ((i * TN + j) * 16 + e) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        // one 32x32 block's loads at a time: hoisting all of them would need a register per load
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
             }
         }
 
