@@ -358,10 +358,25 @@ static bool split_fits(int cfg, int splits, int64_t split_tiles, const GemmParam
 // One launch of the split variant.  hybrid: the tiles that fill whole rounds of resident workgroups are computed
 // whole and only the last, partial round is cut into K ranges, so that every workgroup ends at about the same time;
 // otherwise every tile is cut.  Returns false when the cut does not fit the scratch.
+// mode 2 (stream-K, splits == 0): one workgroup per resident slot, each with an equal stretch of the slabs of all tiles;
+// needs two workspace slots per workgroup and a ticket per tile.
 template <typename K>
-static bool launch_split(K kernel, int tiles, int splits, bool hybrid, int cfg, GemmParams& q, hipStream_t s)
+static bool launch_split(K kernel, int tiles, int splits, int mode, int cfg, GemmParams& q, hipStream_t s)
 {
     const int resident = g_persist_scale > 0 ? g_persist_scale : resident_workgroups(kernel, 256);
+    if (mode == 2) {
+        int bm, bn, bk;
+        tile_of(cfg, bm, bn, bk);
+        const int64_t slabs = (int64_t)tiles * (q.K / bk);
+        const int grid = (int)std::min<int64_t>(resident, slabs);
+        if (tiles > kSplitTickets || (size_t)grid * 2 * bm * bn * sizeof(float) > kSplitWsBytes || slabs >= (1LL << 40))
+            return false;
+        q.splits = 0;
+        q.split_dp_tiles = 0;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, q);
+        return true;
+    }
+    const bool hybrid = mode == 1;
     const int dp = hybrid ? (tiles / resident) * resident : 0;
     if (tiles - dp > 0 && !split_fits(cfg, splits, tiles - dp, q))
         return false;
@@ -370,7 +385,7 @@ static bool launch_split(K kernel, int tiles, int splits, bool hybrid, int cfg, 
     return true;
 }
 
-static bool launch_fast(int cfg, int splits, bool hybrid, const GemmParams& q0, bool conv, int batch, hipStream_t s)
+static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, bool conv, int batch, hipStream_t s)
 {
     GemmParams q = q0;
     q.splits = splits;
@@ -381,11 +396,11 @@ static bool launch_fast(int cfg, int splits, bool hybrid, const GemmParams& q0, 
 #define FDX_FAST(BM_, BN_, BK_)                                                                                  \
     {                                                                                                            \
         const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
-        if (splits > 1) {                                                                                        \
+        if (splits > 1 || mode == 2) {                                                                           \
             if (conv)                                                                                            \
-                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles, splits, hybrid, cfg, q, s); \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles, splits, mode, cfg, q, s); \
             else                                                                                                 \
-                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles, splits, hybrid, cfg, q, s); \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles, splits, mode, cfg, q, s); \
         } else if (conv)                                                                                         \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s);                        \
         else                                                                                                     \
@@ -420,7 +435,8 @@ static bool launch_fast(int cfg, int splits, bool hybrid, const GemmParams& q0, 
 // First sight of a problem shape on the fast path: time every tile configuration once on the
 // real operands (the launches are idempotent) and remember the winner.  Tile count versus
 // resident workgroups, K depth and output width interact too irregularly for a closed rule.
-// A choice is (configuration, K splits, hybrid) packed as cfg + 100 * splits + 10000 * hybrid.  Cutting every tile
+// A choice is (configuration, K splits, mode) packed as cfg + 100 * splits + 10000 * mode, mode 0 = every tile cut into
+// `splits` K ranges, 1 = hybrid (only the last partial round is cut), 2 = stream-K (splits unused).  Cutting every tile
 // is tried only where a configuration has few tiles for the chip; the hybrid cut of the last partial round wherever
 // there is one.
 struct TuneKey {
@@ -462,21 +478,21 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
         const int64_t tiles = (int64_t)((q.M + bm - 1) / bm) * ((q.N + bn - 1) / bn) * batch;
         if (bn > 64 && q.N <= bn / 2)
             continue; // a tile at least twice as wide as the output only idles half of every MFMA
-        static const int kChoices[][2] = { { 1, 0 }, { 2, 0 }, { 3, 0 }, { 4, 0 }, { 2, 1 }, { 3, 1 }, { 4, 1 }, { 6, 1 }, { 8, 1 } };
+        static const int kChoices[][2] = { { 1, 0 }, { 2, 0 }, { 3, 0 }, { 4, 0 }, { 2, 1 }, { 3, 1 }, { 4, 1 }, { 6, 1 }, { 8, 1 }, { 0, 2 } };
         for (const auto& ch : kChoices) {
-            const int splits = ch[0];
-            const bool hybrid = ch[1] != 0;
-            if (splits > 1 && !(can_split && cfg <= 15))
+            const int splits = ch[0], mode = ch[1];
+            const bool hybrid = mode == 1;
+            if (splits != 1 && !(can_split && cfg <= 15))
                 continue;
-            if (splits > 1 && !hybrid && !(tiles <= 1024 && split_fits(cfg, splits, tiles, q)))
+            if (splits > 1 && mode == 0 && !(tiles <= 1024 && split_fits(cfg, splits, tiles, q)))
                 continue;
             if (hybrid && tiles > 16384)
                 continue;
-            if (!launch_fast(cfg, splits, hybrid, q, conv, batch, s)) // warm-up; false = the cut does not fit
+            if (!launch_fast(cfg, splits, mode, q, conv, batch, s)) // warm-up; false = the cut does not fit
                 continue;
             (void)hipEventRecord(a, s);
             for (int r = 0; r < 3; ++r)
-                launch_fast(cfg, splits, hybrid, q, conv, batch, s);
+                launch_fast(cfg, splits, mode, q, conv, batch, s);
             (void)hipEventRecord(b, s);
             float ms = 1e30f;
             if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
@@ -488,7 +504,7 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
                 }
             } else if (ms < best_split_ms) {
                 best_split_ms = ms;
-                best_split = cfg + 100 * splits + (hybrid ? 10000 : 0);
+                best_split = cfg + 100 * splits + 10000 * mode;
             }
         }
     }
@@ -539,21 +555,24 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
     const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31);
     const int unit = conv ? p.Cin : p.K;
 
-    int cfg = g_forced_tile, splits = 1;
-    bool hybrid = false;
-    auto unpack = [&]() { // configuration + 100 * splits + 10000 * hybrid
-        hybrid = cfg >= 10000;
-        splits = std::max(1, (cfg % 10000) / 100);
+    int cfg = g_forced_tile, splits = 1, mode = 0;
+    auto unpack = [&]() { // configuration + 100 * splits + 10000 * mode
+        mode = cfg / 10000;
+        splits = mode == 2 ? 0 : std::max(1, (cfg % 10000) / 100);
         cfg %= 100;
     };
     if (cfg >= 100)
         unpack();
     if (cfg >= 10 && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
         cfg = -1;
-    if (cfg < 10)
+    if (cfg < 10 || mode > 2) {
         splits = 1;
-    if (cfg >= 10 && splits > 1 && (cfg > 15 || !split_prepare()))
+        mode = 0;
+    }
+    if (cfg >= 10 && splits != 1 && (cfg > 15 || !split_prepare())) {
         splits = 1;
+        mode = 0;
+    }
     if (cfg < 0) {
         if (fast_ok && p.N >= 64 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
             GemmParams q = p;
@@ -597,8 +616,8 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         q.a_records = (uint32_t)a_bytes;
         q.b_records = (uint32_t)b_bytes;
         q.batch = batch;
-        if (!launch_fast(cfg, splits, hybrid, q, conv, batch, s))
-            launch_fast(cfg, 1, false, q, conv, batch, s); // the requested cut does not fit the scratch
+        if (!launch_fast(cfg, splits, mode, q, conv, batch, s))
+            launch_fast(cfg, 1, 0, q, conv, batch, s); // the requested cut does not fit the scratch
     } else {
         switch (cfg) {
         case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;

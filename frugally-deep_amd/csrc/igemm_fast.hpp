@@ -23,6 +23,12 @@
 //    in split order (so the sum does not depend on arrival order) and runs the epilogue.
 //    Nothing waits on another workgroup.  Partials are written and read with agent-scope
 //    accesses, which pass the per-XCD L2s, instead of a fence that writes a whole L2 back.
+//  * SPLIT with splits == 0 ("stream-K"): the slabs of all tiles form one line that is cut into
+//    as many equal pieces as there are workgroups, so every workgroup does the same amount of
+//    MFMA work whatever the tile count.  A workgroup's piece covers the end of one tile, some
+//    whole tiles and the beginning of another; the (at most two) partial tiles go through the
+//    same workspace / ticket / ordered-sum path, with the number of contributors of a tile
+//    and their workspace slots computed from the cut points.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false>
@@ -66,6 +72,17 @@ void igemm_fast_kernel(GemmParams p)
     const int alo = xcd * (n_dp >> 3) + (xcd < (n_dp & 7) ? xcd : (n_dp & 7)), na = (n_dp >> 3) + (xcd < (n_dp & 7) ? 1 : 0);
     const int blo = xcd * (n_su >> 3) + (xcd < (n_su & 7) ? xcd : (n_su & 7)), nb = (n_su >> 3) + (xcd < (n_su & 7) ? 1 : 0);
     const int hi = na + nb; // local unit indices [0, hi)
+    const int KT = p.K / BKT;
+
+    // stream-K: workgroup g (numbered XCD by XCD, so an XCD owns a contiguous stretch of tiles) takes the slabs
+    // [g * W / G, (g + 1) * W / G) of the W = tiles * KT slabs; its units are the tiles that stretch touches
+    const bool sk = SPLIT && p.splits == 0;
+    const int G = (int)gridDim.x;
+    const int g_lin = xcd * (G >> 3) + (xcd < (G & 7) ? xcd : (G & 7)) + wg_in_xcd;
+    const int64_t W = (int64_t)all_tiles * KT;
+    const int64_t sk_lo = sk ? g_lin * W / G : 0, sk_hi = sk ? (g_lin + 1) * W / G : 0;
+    const int sk_first = sk ? (int)(sk_lo / KT) : 0;
+    const int sk_units = (sk && sk_hi > sk_lo) ? (int)((sk_hi - 1) / KT) - sk_first + 1 : 0;
 
     // ---- per-tile loader state
     uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
@@ -73,18 +90,32 @@ void igemm_fast_kernel(GemmParams p)
     __amdgpu_buffer_rsrc_t srd_a, srd_b;
     int tap, fx, fy, c0, soff_a, soff_b;
     f32x4 ra[A_LOADS], rb[B_LOADS];
-    const int KT = p.K / BKT;
     int kt_n = KT; // slabs of the current unit
 
-    int cur_su = -1; // split unit of the current work item, -1 for a whole tile
+    int cur_su = -1;  // workspace slot of the current work item's partial tile, -1 for a whole tile
+    int cur_tile = 0; // its output tile
     auto setup = [&](int local, int& m0, int& n0, int64_t& c_off) {
-        int tile = alo + local, split = 0;
+        int tile = alo + local, kt_lo = 0;
         cur_su = -1;
-        if (SPLIT && local >= na) {
+        kt_n = KT;
+        if (sk) {
+            tile = sk_first + local;
+            const int64_t t0 = (int64_t)tile * KT;
+            kt_lo = sk_lo > t0 ? (int)(sk_lo - t0) : 0;
+            const int kt_hi = sk_hi - t0 < KT ? (int)(sk_hi - t0) : KT;
+            kt_n = kt_hi - kt_lo;
+            // a workgroup leaves at most two partial tiles: one that began before its stretch (slot 2g) and one that
+            // ends after it (slot 2g + 1)
+            if (kt_n < KT)
+                cur_su = 2 * g_lin + (sk_lo > t0 ? 0 : 1);
+        } else if (SPLIT && local >= na) {
             cur_su = blo + (local - na);
             tile = n_dp + cur_su / S;
-            split = cur_su - (cur_su / S) * S;
+            const int split = cur_su - (cur_su / S) * S;
+            kt_lo = (int)((int64_t)split * KT / S);
+            kt_n = (int)((int64_t)(split + 1) * KT / S) - kt_lo;
         }
+        cur_tile = tile;
         const int z = tile / per_problem, id = tile - z * per_problem;
         m0 = (id / tiles_n) * BM;
         n0 = (id % tiles_n) * BN;
@@ -128,10 +159,7 @@ void igemm_fast_kernel(GemmParams p)
         }
         tap = fx = fy = c0 = 0;
         soff_a = soff_b = 0;
-        kt_n = KT;
-        if (SPLIT && cur_su >= 0) {
-            const int kt_lo = (int)((int64_t)split * KT / S);
-            kt_n = (int)((int64_t)(split + 1) * KT / S) - kt_lo;
+        if (SPLIT && kt_lo > 0) {
             const int k_start = kt_lo * BKT;
             soff_b = k_start * 4;
             if (CONV) {
@@ -181,8 +209,9 @@ void igemm_fast_kernel(GemmParams p)
             *reinterpret_cast<f32x4*>(&bs[(r0 + i * RPP) * STRIDE + kq * 4]) = rb[i];
     };
 
-    int tile = wg_in_xcd; // local unit index
-    if (tile >= hi)
+    int tile = sk ? 0 : wg_in_xcd; // local unit index
+    const int unit_step = sk ? 1 : wgs_in_xcd, unit_end = sk ? sk_units : hi;
+    if (tile >= unit_end)
         return; // uniform per workgroup
     int m0, n0;
     int64_t c_off;
@@ -234,9 +263,9 @@ void igemm_fast_kernel(GemmParams p)
         const int em0 = m0, en0 = n0;
         float* __restrict__ C = p.C + c_off;
         const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
-        const int su_done = cur_su;
-        tile += wgs_in_xcd;
-        const bool more = tile < hi;
+        const int su_done = cur_su, tile_done = cur_tile;
+        tile += unit_step;
+        const bool more = tile < unit_end;
         if (more) {
             setup(tile, m0, n0, c_off);
             load_tiles(); // in flight while this tile is written out
@@ -244,7 +273,19 @@ void igemm_fast_kernel(GemmParams p)
 
         if (SPLIT && su_done >= 0) {
             constexpr int TILE_F = BM * BN;
-            const int out_tile = su_done / S; // counts from the first split tile
+            // contributors of this output tile, its ticket, and where contributor number sp left its partial
+            int parts = S, out_tile = sk ? tile_done : su_done / S, g_a = 0;
+            const int64_t t0 = (int64_t)tile_done * KT;
+            if (sk) {
+                g_a = (int)(((t0 + 1) * G + W - 1) / W) - 1; // the workgroup whose stretch holds the tile's first slab
+                parts = (int)(((t0 + KT) * G + W - 1) / W) - g_a; // ... up to the one that holds its last slab
+            }
+            auto slot_of = [&](int sp) -> int64_t {
+                if (!sk)
+                    return (int64_t)out_tile * S + sp;
+                const int gg = g_a + sp;
+                return 2 * (int64_t)gg + (gg * W / G > t0 ? 0 : 1);
+            };
             float* mine = p.split_ws + (int64_t)su_done * TILE_F + t;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -258,7 +299,7 @@ void igemm_fast_kernel(GemmParams p)
             __syncthreads();
             if (t == 0) {
                 const int ticket = __hip_atomic_fetch_add(p.split_tickets + out_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const int last = ticket == S - 1;
+                const int last = ticket == parts - 1;
                 if (last)
                     __hip_atomic_store(p.split_tickets + out_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // next launch
                 last_flag = last;
@@ -281,8 +322,8 @@ void igemm_fast_kernel(GemmParams p)
 #pragma unroll
                     for (int e = 0; e < 16; ++e)
                         acc[i][j][e] = 0.f;
-            for (int sp = 0; sp < S; ++sp) {
-                const float* part = p.split_ws + ((int64_t)out_tile * S + sp) * TILE_F + t;
+            for (int sp = 0; sp < parts; ++sp) {
+                const float* part = p.split_ws + slot_of(sp) * TILE_F + t;
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll

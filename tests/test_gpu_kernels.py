@@ -420,6 +420,54 @@ def test_conv2d_hybrid_whole_tiles_plus_split_remainder(fdx, oracle, tile, cap):
     assert np.array_equal(first, second)
 
 
+@pytest.mark.parametrize("tile,cap", [(20010, 0), (20011, 0), (20012, 0), (20013, 0), (20014, 0), (20015, 0),
+                                      (20015, 9), (20012, 40), (20010, 8), (20011, 24), (20014, 133)])
+def test_conv2d_stream_k(fdx, oracle, tile, cap):
+    """Stream-K scheduling (20000 + configuration): the slabs of all tiles are dealt out in equal stretches, one per
+    workgroup, so tiles are shared by two or more workgroups at arbitrary cut points; grid sizes from 8 workgroups (a
+    stretch spans several tiles) to the resident count (several workgroups per tile). Result equals the oracle and
+    repeats bit for bit."""
+    say("conv2d stream-K", tile, cap)
+    n, h, w, cin, cout = 3, 20, 19, 64, 96
+    r = rng_for("conv-streamk", tile, cap)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wj = (r.standard_normal((cout, 3, 3, cin)) / np.sqrt(9 * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    wo = oracle.conv2d_prepare(wj, cout, 3, 3, cin)
+    conv = np.stack([oracle.conv2d(x[i], wo, b, cout, 3, 3, (1, 1), (1, 1), "same") for i in range(n)])
+    res = r.standard_normal(conv.shape).astype(np.float32)
+    want = oracle.relu(oracle.add(res, conv))
+    fdx.lib.fdx_debug_force_tile(tile)
+    fdx.lib.fdx_debug_persist_cap(cap)
+    try:
+        first = fdx.conv2d(x, wj, b, (1, 1), (1, 1), "same", residual=res, act=fdx.relu_act())
+        second = fdx.conv2d(x, wj, b, (1, 1), (1, 1), "same", residual=res, act=fdx.relu_act())
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+        fdx.lib.fdx_debug_persist_cap(0)
+    assert rel(first, want) <= TOL
+    assert np.array_equal(first, second)
+
+
+@pytest.mark.parametrize("m,n,k,tile", [(1000, 256, 512, 20010), (4096, 128, 1024, 20011), (300, 64, 2048, 20015),
+                                        (129, 132, 64, 20012)])
+def test_gemm_stream_k(fdx, m, n, k, tile):
+    say("gemm stream-K", m, n, k, tile)
+    r = rng_for("gemm-streamk", m, n, k)
+    a = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    want = a.astype(np.float64) @ w.astype(np.float64).T + bias
+    fdx.lib.fdx_debug_force_tile(tile)
+    try:
+        got = fdx.gemm(a, w, bias)
+        again = fdx.gemm(a, w, bias)
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(got, want) <= TOL
+    assert np.array_equal(got, again)
+
+
 @pytest.mark.parametrize("case", [
     # n, h, w, cin, cout, k, padding, explicit zero frame (top/left = bottom/right)
     (2, 30, 30, 3, 64, 7, "valid", 3),   # ResNet stem: ZeroPadding2D(3) then 7x7 / 2 valid
