@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
 
 #include "common.hpp"
 #include "igemm_params.hpp"
@@ -522,8 +523,13 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     return best;
 }
 
+// the tuner's table and its timing runs, and the order in which launches that share the split workspace reach the
+// stream, are per process: host threads take turns here
+static std::mutex g_igemm_mutex;
+
 static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* family, double algorithmic_flops = 0.0)
 {
+    std::lock_guard<std::mutex> lock(g_igemm_mutex);
     int a_mode;
     if (conv)
         a_mode = (p.Cin % 4 == 0 && aligned16(p.A)) ? A_CONV_VEC : A_CONV_SCALAR;

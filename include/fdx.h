@@ -12,6 +12,10 @@
  *   - tensors are fp32, channels-last, batch outermost: [n][h][w][c] / [n][rows][depth].
  *   - "dev" pointers are device memory of the current GPU; the per-kernel launchers
  *     take device pointers only and enqueue on the library stream (fdx_sync waits).
+ *   - host threads: every call enqueues on the one library stream, so work from several
+ *     threads runs in the order the calls were made; a model (and a session) serialises
+ *     its own calls, the convolution / GEMM launcher serialises its tuner and scratch.
+ *     The profile and stopwatch calls (fdx_profile_*, fdx_timer_*) are meant for one thread.
  */
 #ifndef FDX_H
 #define FDX_H
@@ -348,6 +352,17 @@ fdx_status fdx_session_decode_step(fdx_session* s, const float* ids_dev, float* 
 fdx_status fdx_session_decode_greedy(fdx_session* s, const float* first_ids_dev, int steps, float* tokens_dev,
     float* last_logits_dev);
 fdx_status fdx_session_length(const fdx_session* s, int* len);
+
+/*
+ * Test hooks (no counterpart in the reference; process-wide, meant for one thread): the parity tests use them to drive
+ * every tile configuration and scheduling form of the convolution / GEMM kernels on small problems, where the tuner
+ * would never pick them.
+ *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; + 100 * splits
+ *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
+ *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
+ */
+fdx_status fdx_debug_force_tile(int cfg);
+fdx_status fdx_debug_persist_cap(int workgroups);
 
 #ifdef __cplusplus
 }
