@@ -1172,6 +1172,16 @@ namespace {
                 if (fdx_conv2d_s2d_prepare(o.hw[0].data(), o.cout, o.n_in, o.kh, o.hw[2].data()) != FDX_OK)
                     return FDX_ERR_INVALID;
             }
+            // self-attention (query, value and key are one tensor): the three projections become one GEMM over the
+            // stacked kernels, whose column blocks the attention core then reads in place
+            if (o.kind == OpKind::MHA && o.hw.size() >= 6 && o.in.size() >= 2 && o.in[0] == o.in[1]
+                && (o.in.size() == 2 || o.in[2] == o.in[0]) && (o.heads * o.dk) % 4 == 0 && (o.heads * o.dv) % 4 == 0) {
+                o.hw.resize(std::max<size_t>(o.hw.size(), 12));
+                for (int part = 0; part < 3; ++part) {
+                    o.hw[10].insert(o.hw[10].end(), o.hw[(size_t)2 * part].begin(), o.hw[(size_t)2 * part].end());
+                    o.hw[11].insert(o.hw[11].end(), o.hw[(size_t)2 * part + 1].begin(), o.hw[(size_t)2 * part + 1].end());
+                }
+            }
             o.dw.assign(o.hw.size(), nullptr);
             for (size_t i = 0; i < o.hw.size(); ++i) {
                 if (o.hw[i].empty())
@@ -1506,7 +1516,9 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
         if (o.kind == OpKind::MHA) { // per-op scratch: placed while inputs and output are live, free again afterwards
             const int64_t T = p->shapes[o.in[0]][0], S = p->shapes[o.in[1]][0];
             const size_t nk = (size_t)o.heads * o.dk, nv = (size_t)o.heads * o.dv, fb = sizeof(float) * (size_t)batch;
-            const size_t sizes[6] = { fb * T * nk, fb * S * nk, fb * S * nv, fb * T * nv,
+            const bool stacked = o.dw.size() > 11 && o.dw[10]; // one buffer holds [q | k | v] per row
+            const size_t sizes[6] = { stacked ? fb * T * (2 * nk + nv) : fb * T * nk, stacked ? (size_t)256 : fb * S * nk,
+                stacked ? (size_t)256 : fb * S * nv, fb * T * nv,
                 fdx_mha_scratch_bytes(batch, o.heads, (int)T, (int)S, o.dv), o.gate ? fb * T * nv : (size_t)256 };
             std::vector<int> held;
             for (size_t sz : sizes) {
@@ -1837,14 +1849,23 @@ namespace {
             const int64_t nk = (int64_t)H * o.dk, nv = (int64_t)H * o.dv;
             const std::vector<float*>& tmp = p.temps[idx];
             float *q = tmp[0], *k = tmp[1], *v = tmp[2], *merged = tmp[3], *scratch = tmp[4];
-            if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[0], D, B * T, (int)nk, D, 1.f, o.dw[1], 0, nullptr, nullptr, q, nk, nullptr)) != FDX_OK)
-                return st;
-            if ((st = fdx_gemm_bias_act_f32(xk, D, o.dw[2], D, B * S, (int)nk, D, 1.f, o.dw[3], 0, nullptr, nullptr, k, nk, nullptr)) != FDX_OK)
-                return st;
-            if ((st = fdx_gemm_bias_act_f32(xv, D, o.dw[4], D, B * S, (int)nv, D, 1.f, o.dw[5], 0, nullptr, nullptr, v, nv, nullptr)) != FDX_OK)
-                return st;
-            if ((st = fdx_mha_prefill_f32(q, k, v, B, T, S, H, o.dk, o.dv, 0, merged, scratch)) != FDX_OK)
-                return st;
+            if (o.dw.size() > 11 && o.dw[10]) {
+                const int64_t nt = 2 * nk + nv;
+                if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[10], D, B * T, (int)nt, D, 1.f, o.dw[11], 0, nullptr, nullptr, q, nt, nullptr)) != FDX_OK)
+                    return st;
+                if ((st = mha_prefill_strided(q, nt, T * nt, q + nk, nt, T * nt, q + 2 * nk, nt, T * nt, B, T, S, H, o.dk, o.dv, 0, merged,
+                         nv, T * nv, scratch)) != FDX_OK)
+                    return st;
+            } else {
+                if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[0], D, B * T, (int)nk, D, 1.f, o.dw[1], 0, nullptr, nullptr, q, nk, nullptr)) != FDX_OK)
+                    return st;
+                if ((st = fdx_gemm_bias_act_f32(xk, D, o.dw[2], D, B * S, (int)nk, D, 1.f, o.dw[3], 0, nullptr, nullptr, k, nk, nullptr)) != FDX_OK)
+                    return st;
+                if ((st = fdx_gemm_bias_act_f32(xv, D, o.dw[4], D, B * S, (int)nv, D, 1.f, o.dw[5], 0, nullptr, nullptr, v, nv, nullptr)) != FDX_OK)
+                    return st;
+                if ((st = fdx_mha_prefill_f32(q, k, v, B, T, S, H, o.dk, o.dv, 0, merged, scratch)) != FDX_OK)
+                    return st;
+            }
             if (o.gate) { // attention output times sigmoid(gate projection of the query) (group_query_attention_layer.hpp:157-164)
                 float* gbuf = tmp[5];
                 const fdx_act sg = { FDX_ACT_SIGMOID, 0.f, 0.f, 0.f };
