@@ -251,7 +251,7 @@ def bench_gpt2(fdx, modelgen, args):
         "prefill_ms": round(prefill_ms, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4), "bytes_per_step_mean": round(total_bytes / new),
-                     "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 49 of the step's 64 launches)",
+                     "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 48 of the step's 64 launches plus the LM head's striding variant)",
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
         "load_seconds": round(load_s, 2),
     }

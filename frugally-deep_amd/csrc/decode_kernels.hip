@@ -224,6 +224,168 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
     }
 }
 
+// Wide outputs (a vocabulary projection: thousands of 16-column groups, K <= 1024): one workgroup per column
+// group would run the chip in rounds, each paying the full load -> multiply -> reduce -> store latency chain with
+// little in flight.  Here a fixed set of resident workgroups strides through the column groups: the activation
+// rows (and the LayerNorm statistics) are taken once, and while one group's products are reduced and stored the next
+// group's weights -- and its bias / residual / row-sum operands -- are already on their way in a second register set.
+// (second bound: four waves per SIMD, i.e. two of these workgroups per CU)
+template <int CHUNK>
+__global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int tiles)
+{
+    __shared__ float red[SK_WAVES * 256];
+    __shared__ float stat[SK_WAVES * 16];
+    __shared__ float row_mean[16], row_rstd[16];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int i = lane & 15, kq = lane >> 4;
+    const int K = p.K;
+    const int per_wave = ((K + SK_WAVES * 16 - 1) / (SK_WAVES * 16)) * 16;
+    const int k_begin = wave * per_wave;
+    const int k_end = k_begin + per_wave < K ? k_begin + per_wave : K;
+    const int slabs = k_end > k_begin ? (k_end - k_begin + 15) / 16 : 0;
+    const int spw = per_wave / 16;
+    const bool m_ok = i < p.M;
+
+    f32x4 a0[CHUNK];
+    {
+        const float* xrow = p.X + (int64_t)(m_ok ? i : 0) * p.ldx;
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s) {
+            const int k = k_begin + s * 16 + kq * 4;
+            a0[s] = (m_ok && s < slabs && k < k_end) ? *reinterpret_cast<const f32x4*>(xrow + k) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+        }
+    }
+    auto load_w = [&](f32x4 (&wreg)[CHUNK], int tile) {
+        const int n = tile * 16 + i;
+        const bool n_ok = n < p.N;
+        const float* wrow = p.W + (int64_t)(n_ok ? n : 0) * p.ldw;
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s) {
+            const int k = k_begin + s * 16 + kq * 4;
+            f32x4 wv = { 0.f, 0.f, 0.f, 0.f };
+            if (p.packed) {
+                if (s < spw)
+                    wv = reinterpret_cast<const f32x4*>(p.W)[(((int64_t)tile * SK_WAVES + wave) * spw + s) * 64 + lane];
+            } else if (n_ok && s < slabs && k < k_end)
+                wv = *reinterpret_cast<const f32x4*>(wrow + k);
+            wreg[s] = wv;
+        }
+    };
+    // epilogue operands of output element (row em, column tile * 16 + ec), fetched with the tile's weights
+    const int em = t >> 4, ec = t & 15;
+    struct Epi {
+        float bias, res, wsum;
+    };
+    auto load_epi = [&](int tile) {
+        Epi e { 0.f, 0.f, 0.f };
+        const int col = tile * 16 + ec;
+        if (t < 256 && em < p.M && col < p.N) {
+            if (p.bias)
+                e.bias = p.bias[col];
+            if (p.residual)
+                e.res = p.residual[(int64_t)em * p.ldr + col];
+            if (p.ln)
+                e.wsum = p.w_rowsum[col];
+        }
+        return e;
+    };
+
+    int tile = blockIdx.x;
+    f32x4 w0[CHUNK], w1[CHUNK];
+    load_w(w0, tile);
+    Epi e0 = load_epi(tile);
+
+    if (p.ln) { // statistics of the (at most 16) rows, from the registers that hold them; two-pass variance
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < CHUNK; ++c)
+            s += (a0[c][0] + a0[c][1]) + (a0[c][2] + a0[c][3]);
+        s += __shfl_xor(s, 16, 64);
+        s += __shfl_xor(s, 32, 64);
+        if (kq == 0)
+            stat[wave * 16 + i] = s;
+        __syncthreads();
+        if (t < 16) {
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+                tot += stat[w * 16 + t];
+            row_mean[t] = tot / (float)K;
+        }
+        __syncthreads();
+        const float mean = row_mean[i];
+        float q = 0.f;
+#pragma unroll
+        for (int c = 0; c < CHUNK; ++c) {
+            const int k = k_begin + c * 16 + kq * 4;
+            if (c < slabs && k < k_end) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float d = a0[c][e] - mean;
+                    q += d * d;
+                }
+            }
+        }
+        q += __shfl_xor(q, 16, 64);
+        q += __shfl_xor(q, 32, 64);
+        __syncthreads();
+        if (kq == 0)
+            stat[wave * 16 + i] = q;
+        __syncthreads();
+        if (t < 16) {
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+                tot += stat[w * 16 + t];
+            row_rstd[t] = 1.0f / sqrtf(tot / (float)K + p.ln_eps);
+        }
+        __syncthreads();
+    }
+
+    const int64_t len_shift = p.seg[0].len_stride ? (int64_t)(*p.len_dev) : 0; // only read when a segment asks for it
+    for (; tile < tiles; tile += gridDim.x) {
+        const int next = tile + gridDim.x;
+        Epi e1 { 0.f, 0.f, 0.f };
+        if (next < tiles) {
+            load_w(w1, next);
+            e1 = load_epi(next);
+        }
+        f32x4 acc = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s][e], w0[s][e], acc, 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            red[wave * 256 + (4 * kq + e) * 16 + i] = acc[e];
+        __syncthreads();
+        const int col = tile * 16 + ec;
+        if (t < 256 && em < p.M && col < p.N) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w)
+                v += red[w * 256 + t];
+            if (p.ln)
+                v = row_rstd[em] * (v - row_mean[em] * e0.wsum);
+            v = apply_act(v + e0.bias + e0.res, p.act);
+            int sgi = 0;
+            if (p.n_seg > 1 && col >= p.seg[1].col_begin)
+                sgi = 1;
+            if (p.n_seg > 2 && col >= p.seg[2].col_begin)
+                sgi = 2;
+            const SkinnySegment& sg = p.seg[sgi];
+            const int64_t shift = sg.len_stride ? (sgi == 0 ? len_shift : (int64_t)(*p.len_dev)) * sg.len_stride : 0;
+            sg.ptr[shift + (int64_t)em * sg.ld + (col - sg.col_begin)] = v;
+        }
+        __syncthreads(); // the reduction buffer is rewritten by the next column group
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s)
+            w0[s] = w1[s];
+        e0 = e1;
+    }
+}
+
 // [N][K] -> [column tile][wave][slab][lane] 16-byte pieces in exactly the order the GEMM's lanes consume
 // them (lane l of wave w, slab s holds W[tile*16 + l%16][w*per_wave + s*16 + (l/16)*4 ..+3], zero beyond N or K),
 // so every wave-wide load is one contiguous kilobyte
@@ -492,9 +654,25 @@ static bool ensure_splitk_workspace()
     return true;
 }
 
+// workgroups of the wide-output kernel that are resident at once (queried once, outside any stream capture)
+static int wide_resident()
+{
+    static const int resident = [] {
+        int per_cu = 1, dev = 0, cus = 256;
+        hipDeviceProp_t prop;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, skinny_wide_kernel<SK_CHUNK>, 512, 0) != hipSuccess || per_cu < 1)
+            per_cu = 1;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        return per_cu * cus;
+    }();
+    return resident;
+}
+
 // allocates the split-K scratch ahead of time (it must not happen inside a stream capture)
 fdx_status skinny_prepare()
 {
+    (void)wide_resident();
     if (!ensure_splitk_workspace()) {
         set_error("dense_rows: out of device memory for the split-K workspace");
         return FDX_ERR_HIP;
@@ -531,6 +709,14 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
     const int per_wg = ((p.K + ksplit * 16 - 1) / (ksplit * 16)) * 16; // as the kernel derives it
     const dim3 grid((unsigned)tiles, (unsigned)ksplit);
     profile_begin();
+    // many column groups and a short K: resident workgroups stride through the groups instead of one group each
+    const int wide_grid = wide_resident();
+    if (ksplit == 1 && per_wg <= SK_WAVES * SK_CHUNK * 16 && tiles >= 4 * wide_grid) {
+        hipLaunchKernelGGL((skinny_wide_kernel<SK_CHUNK>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
+        profile_end("dense_rows_f32", 2.0 * p.M * (double)p.N * p.K, 4.0 * ((double)p.N * p.K + (double)p.M * (p.K + p.N)));
+        FDX_LAUNCH_CHECK();
+        return FDX_OK;
+    }
     // every load of a workgroup in flight at once when its K range fits 8 (or 24) slabs per wave
     if (per_wg <= SK_WAVES * SK_CHUNK * 16)
         hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK, true>), grid, dim3(512), 0, stream(), q);
