@@ -41,8 +41,7 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
 {
     __shared__ float red[SK_WAVES * 256];
     __shared__ int is_last;
-    __shared__ float stat[SK_WAVES * 16];
-    __shared__ float row_mean[16], row_rstd[16];
+    __shared__ float stat[SK_WAVES * 16], stat2[SK_WAVES * 16]; // per-wave row sums / sums of squared deviations
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int i = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.x * 16;
@@ -129,15 +128,13 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
         if (kq == 0)
             stat[wave * 16 + i] = s;
         __syncthreads();
-        if (t < 16) {
-            float tot = 0.f;
+        // every thread adds the eight partial sums of its row itself (same order everywhere, so the same value): the
+        // mean costs this one barrier, and the squared deviations ride on the barrier of the product reduction
+        float tot = 0.f;
 #pragma unroll
-            for (int w = 0; w < SK_WAVES; ++w)
-                tot += stat[w * 16 + t];
-            row_mean[t] = tot / (float)K;
-        }
-        __syncthreads();
-        const float mean = row_mean[i];
+        for (int w = 0; w < SK_WAVES; ++w)
+            tot += stat[w * 16 + i];
+        const float mean = tot / (float)K;
         float q = 0.f;
 #pragma unroll
         for (int c = 0; c < CHUNK; ++c) {
@@ -152,17 +149,8 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
         }
         q += __shfl_xor(q, 16, 64);
         q += __shfl_xor(q, 32, 64);
-        __syncthreads();
         if (kq == 0)
-            stat[wave * 16 + i] = q;
-        __syncthreads();
-        if (t < 16) {
-            float tot = 0.f;
-#pragma unroll
-            for (int w = 0; w < SK_WAVES; ++w)
-                tot += stat[w * 16 + t];
-            row_rstd[t] = 1.0f / sqrtf(tot / (float)K + p.ln_eps);
-        }
+            stat2[wave * 16 + i] = q;
         compute_chunk(w0, a0);
     } else if (SINGLE) {
         compute_chunk(w0, a0);
@@ -216,8 +204,15 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
         }
     }
     if (e_ok) {
-        if (p.ln)
-            v = row_rstd[em] * (v - row_mean[em] * e_wsum);
+        if (p.ln) {
+            float tot = 0.f, dev = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w) {
+                tot += stat[w * 16 + em];
+                dev += stat2[w * 16 + em];
+            }
+            v = (1.0f / sqrtf(dev / (float)K + p.ln_eps)) * (v - (tot / (float)K) * e_wsum);
+        }
         v = apply_act(v + e_bias + e_res, p.act);
         const SkinnySegment& sg = p.seg[e_seg];
         sg.ptr[e_shift + (int64_t)em * sg.ld + (ecol - sg.col_begin)] = v;
@@ -718,7 +713,9 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
         return FDX_OK;
     }
     // every load of a workgroup in flight at once when its K range fits 8 (or 24) slabs per wave
-    if (per_wg <= SK_WAVES * SK_CHUNK * 16)
+    if (per_wg <= SK_WAVES * 6 * 16) // K = 768 and the halves / quarters of longer rows: no empty register slots
+        hipLaunchKernelGGL((skinny_gemm_kernel<6, true>), grid, dim3(512), 0, stream(), q);
+    else if (per_wg <= SK_WAVES * SK_CHUNK * 16)
         hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK, true>), grid, dim3(512), 0, stream(), q);
     else if (per_wg <= SK_WAVES * SK_CHUNK_LONG * 16)
         hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK_LONG, true>), grid, dim3(512), 0, stream(), q);
