@@ -286,9 +286,17 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
     };
 
     int tile = blockIdx.x;
-    f32x4 w0[CHUNK], w1[CHUNK];
+    // short rows leave room for three register sets: the weights of the next TWO column groups are in flight while one
+    // is multiplied; longer rows keep one group ahead
+    constexpr bool AHEAD2 = CHUNK <= 6;
+    f32x4 w0[CHUNK], w1[CHUNK], w2[AHEAD2 ? CHUNK : 1];
     load_w(w0, tile);
     Epi e0 = load_epi(tile);
+    Epi e1 { 0.f, 0.f, 0.f };
+    if (AHEAD2 && tile + (int)gridDim.x < tiles) {
+        load_w(w1, tile + gridDim.x);
+        e1 = load_epi(tile + gridDim.x);
+    }
 
     if (p.ln) { // statistics of the (at most 16) rows, from the registers that hold them; two-pass variance
         float s = 0.f;
@@ -339,11 +347,14 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
 
     const int64_t len_shift = p.seg[0].len_stride ? (int64_t)(*p.len_dev) : 0; // only read when a segment asks for it
     for (; tile < tiles; tile += gridDim.x) {
-        const int next = tile + gridDim.x;
-        Epi e1 { 0.f, 0.f, 0.f };
+        const int next = tile + (AHEAD2 ? 2 : 1) * gridDim.x;
+        Epi e2 { 0.f, 0.f, 0.f };
         if (next < tiles) {
-            load_w(w1, next);
-            e1 = load_epi(next);
+            if constexpr (AHEAD2)
+                load_w(w2, next);
+            else
+                load_w(w1, next);
+            e2 = load_epi(next);
         }
         f32x4 acc = { 0.f, 0.f, 0.f, 0.f };
 #pragma unroll
@@ -375,9 +386,13 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
         }
         __syncthreads(); // the reduction buffer is rewritten by the next column group
 #pragma unroll
-        for (int s = 0; s < CHUNK; ++s)
+        for (int s = 0; s < CHUNK; ++s) {
             w0[s] = w1[s];
-        e0 = e1;
+            if constexpr (AHEAD2)
+                w1[s] = w2[s];
+        }
+        e0 = AHEAD2 ? e1 : e2;
+        e1 = e2;
     }
 }
 
@@ -707,7 +722,10 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
     // many column groups and a short K: resident workgroups stride through the groups instead of one group each
     const int wide_grid = wide_resident();
     if (ksplit == 1 && per_wg <= SK_WAVES * SK_CHUNK * 16 && tiles >= 4 * wide_grid) {
-        hipLaunchKernelGGL((skinny_wide_kernel<SK_CHUNK>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
+        if (per_wg <= SK_WAVES * 6 * 16)
+            hipLaunchKernelGGL((skinny_wide_kernel<6>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
+        else
+            hipLaunchKernelGGL((skinny_wide_kernel<SK_CHUNK>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
         profile_end("dense_rows_f32", 2.0 * p.M * (double)p.N * p.K, 4.0 * ((double)p.N * p.K + (double)p.M * (p.K + p.N)));
         FDX_LAUNCH_CHECK();
         return FDX_OK;
