@@ -5,9 +5,9 @@
 // (16 bytes each, sixteen lanes per cached row so a wave touches four whole rows per load)
 // before anything is used; the values do not depend on the softmax, so they travel while the
 // scores are reduced.  Scores stay in registers; max / sum / output reductions use wave
-// shuffles and one small LDS exchange between the four waves.  Softmax is the reference's
-// exp(x - m - log(sum)) form (include/fdeep/tensor.hpp:1165-1192); the scale multiplies the
-// scores after the dot product (layers/multi_head_attention_layer.hpp:91-93).
+// shuffles and ONE small LDS exchange between the four waves.  Softmax weights equal the
+// reference's exp(x - m - log(sum)) (include/fdeep/tensor.hpp:1165-1192) up to rounding; the
+// scale multiplies the scores after the dot product (layers/multi_head_attention_layer.hpp:91-93).
 #include <cfloat>
 #include <cmath>
 
@@ -22,7 +22,7 @@ __global__ __launch_bounds__(256) void mha_decode_fast_kernel(const float* __res
     const float* __restrict__ kc, const float* __restrict__ vc, float* __restrict__ out, int heads,
     const int* __restrict__ len_dev, int max_len, float scale)
 {
-    __shared__ float red[4];
+    __shared__ float red[4], red_sum[4];
     __shared__ float osum[4][64];
     const int tid = threadIdx.x, part = tid & 15, slot = tid >> 4, wave = tid >> 6;
     const int b = blockIdx.x / heads, h = blockIdx.x % heads;
@@ -55,36 +55,24 @@ __global__ __launch_bounds__(256) void mha_decode_fast_kernel(const float* __res
         sc[u] = slot + 16 * u < len ? s * scale : -FLT_MAX;
         m = fmaxf(m, sc[u]);
     }
-    // maximum over all keys: the other slots of this wave sit 16 and 32 lanes away, then the other waves
+    // Each wave finishes its own quarter of the keys against its OWN maximum (the other slots of the wave sit 16 and
+    // 32 lanes away): probabilities, their sum and the weighted values.  The four quarters then meet once in LDS and
+    // are rescaled to the common maximum, exp(m_w - m) each -- one barrier instead of one per reduction.  The result
+    // is the reference's exp(x - m - log(sum)) weighting up to rounding.
     m = fmaxf(m, __shfl_xor(m, 16, 64));
     m = fmaxf(m, __shfl_xor(m, 32, 64));
-    if ((tid & 63) == 0)
-        red[wave] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     float sum = 0.f;
-#pragma unroll
-    for (int u = 0; u < 16; ++u)
-        sum += slot + 16 * u < len ? expf(sc[u] - m) : 0.f;
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-    __syncthreads();
-    if ((tid & 63) == 0)
-        red[wave] = sum;
-    __syncthreads();
-    const float ls = logf((red[0] + red[1]) + (red[2] + red[3]));
     f32x4 acc = { 0.f, 0.f, 0.f, 0.f };
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-        float pr = 0.f;
-        if (slot + 16 * u < len) {
-            pr = expf(sc[u] - m - ls);
-            pr = isinf(pr) ? 0.f : pr;
-        }
+        const float pr = slot + 16 * u < len ? expf(sc[u] - m) : 0.f;
+        sum += pr;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             acc[e] += pr * vv[u][e];
     }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         acc[e] += __shfl_xor(acc[e], 16, 64);
@@ -95,9 +83,22 @@ __global__ __launch_bounds__(256) void mha_decode_fast_kernel(const float* __res
         for (int e = 0; e < 4; ++e)
             osum[wave][part * 4 + e] = acc[e];
     }
+    if ((tid & 63) == 0) {
+        red[wave] = m;
+        red_sum[wave] = sum;
+    }
     __syncthreads();
-    if (tid < 64)
-        out[(int64_t)b * row + h * 64 + tid] = (osum[0][tid] + osum[1][tid]) + (osum[2][tid] + osum[3][tid]);
+    if (tid < 64) {
+        const float mm = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        float f[4], denom = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            f[w] = expf(red[w] - mm); // a wave without a visible key has m_w = -FLT_MAX: weight 0
+            denom += f[w] * red_sum[w];
+            o += f[w] * osum[w][tid];
+        }
+        out[(int64_t)b * row + h * 64 + tid] = o / denom;
+    }
 }
 
 // true if the fast kernel covers this shape; launches it
