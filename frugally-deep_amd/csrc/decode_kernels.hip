@@ -219,6 +219,8 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
     }
 }
 
+__device__ __forceinline__ unsigned long long pack_max(float v, int col);
+
 // Wide outputs (a vocabulary projection: thousands of 16-column groups, K <= 1024): one workgroup per column
 // group would run the chip in rounds, each paying the full load -> multiply -> reduce -> store latency chain with
 // little in flight.  Here a fixed set of resident workgroups strides through the column groups: the activation
@@ -346,6 +348,7 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
     }
 
     const int64_t len_shift = p.seg[0].len_stride ? (int64_t)(*p.len_dev) : 0; // only read when a segment asks for it
+    unsigned long long best = 0ull; // packed maximum of this thread's output elements (one row, one column per group)
     for (; tile < tiles; tile += gridDim.x) {
         const int next = tile + (AHEAD2 ? 2 : 1) * gridDim.x;
         Epi e2 { 0.f, 0.f, 0.f };
@@ -375,6 +378,10 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
             if (p.ln)
                 v = row_rstd[em] * (v - row_mean[em] * e0.wsum);
             v = apply_act(v + e0.bias + e0.res, p.act);
+            if (p.amax_parts) {
+                const unsigned long long pk = pack_max(v, col);
+                best = pk > best ? pk : best;
+            }
             int sgi = 0;
             if (p.n_seg > 1 && col >= p.seg[1].col_begin)
                 sgi = 1;
@@ -393,6 +400,15 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
         }
         e0 = AHEAD2 ? e1 : e2;
         e1 = e2;
+    }
+    if (p.amax_parts && t < 256) { // the 16 lanes that share a row sit next to each other
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) {
+            const unsigned long long other = __shfl_xor(best, o, 64);
+            best = other > best ? other : best;
+        }
+        if (ec == 0)
+            p.amax_parts[(int64_t)blockIdx.x * 16 + em] = best; // rows beyond M keep 0 = "no value"
     }
 }
 
@@ -627,6 +643,32 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
     }
 }
 
+// per-workgroup partial maxima [parts][16] -> float ids, then as argmax_finish_kernel
+__global__ __launch_bounds__(1024) void argmax_parts_kernel(const unsigned long long* __restrict__ parts, int n_parts, int rows,
+    float* __restrict__ out_idx_f, int* __restrict__ len_dev, float* __restrict__ history)
+{
+    __shared__ unsigned long long sm[64][16];
+    const int r = threadIdx.x & 15, lane_part = threadIdx.x >> 4; // 64 threads per row
+    unsigned long long best = 0ull;
+    for (int q = lane_part; q < n_parts; q += 64) {
+        const unsigned long long pk = parts[(int64_t)q * 16 + r];
+        best = pk > best ? pk : best;
+    }
+    sm[lane_part][r] = best;
+    __syncthreads();
+    if (threadIdx.x < 16 && r < rows) {
+        for (int q = 0; q < 64; ++q)
+            best = sm[q][r] > best ? sm[q][r] : best;
+        const float id = best == 0ull ? 0.f : (float)(0xFFFFFFFFu - (unsigned int)(best & 0xFFFFFFFFull));
+        out_idx_f[r] = id;
+        if (history && len_dev)
+            history[(int64_t)(*len_dev) * rows + r] = id;
+    }
+    __syncthreads();
+    if (len_dev && threadIdx.x == 0)
+        *len_dev += 1;
+}
+
 // packed winners -> float ids; optionally advances the session length (every other kernel of the step
 // has finished by stream order)
 __global__ void argmax_finish_kernel(const unsigned long long* __restrict__ amax, int rows, float* __restrict__ out_idx_f,
@@ -690,6 +732,27 @@ fdx_status skinny_prepare()
     return FDX_OK;
 }
 
+// (rows this short are never split along K, so the choice depends on K and the number of column groups alone)
+int skinny_wide_grid(const SkinnyParams& p)
+{
+    const int tiles = (p.N + 15) / 16;
+    if (p.M <= 0 || p.M > 16 || p.K <= 0)
+        return 0;
+    const int per_wg = ((p.K + 15) / 16) * 16;
+    const int grid = wide_resident();
+    return (per_wg <= SK_WAVES * SK_CHUNK * 16 && tiles >= 4 * grid) ? grid : 0;
+}
+
+fdx_status argmax_parts_launch(const unsigned long long* amax_parts, int parts, int rows, float* out_idx_f, int* len_dev, float* history)
+{
+    FDX_REQUIRE(amax_parts && out_idx_f && parts > 0 && rows > 0 && rows <= 16, "argmax: bad arguments");
+    profile_begin();
+    hipLaunchKernelGGL(argmax_parts_kernel, dim3(1), dim3(1024), 0, stream(), amax_parts, parts, rows, out_idx_f, len_dev, history);
+    profile_end("argmax_f32", 0.0, 8.0 * parts * 16);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
 fdx_status skinny_gemm_launch(const SkinnyParams& p)
 {
     FDX_REQUIRE(p.X && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0, "dense_rows: bad arguments");
@@ -720,8 +783,9 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
     const dim3 grid((unsigned)tiles, (unsigned)ksplit);
     profile_begin();
     // many column groups and a short K: resident workgroups stride through the groups instead of one group each
-    const int wide_grid = wide_resident();
-    if (ksplit == 1 && per_wg <= SK_WAVES * SK_CHUNK * 16 && tiles >= 4 * wide_grid) {
+    const int wide_grid = skinny_wide_grid(p);
+    FDX_REQUIRE(!p.amax_parts || (wide_grid > 0 && ksplit == 1), "dense_rows: partial arg-max cells need the wide-output kernel");
+    if (ksplit == 1 && wide_grid > 0) {
         if (per_wg <= SK_WAVES * 6 * 16)
             hipLaunchKernelGGL((skinny_wide_kernel<6>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
         else

@@ -48,6 +48,8 @@ struct fdx_session {
     float* ids_buf = nullptr;           // ids consumed by the next step (argmax writes them)
     const float* logits_buf = nullptr;
     unsigned long long* amax = nullptr; // per sequence: packed running arg-max of the step's logits
+    unsigned long long* amax_parts = nullptr; // [workgroups of the logits launch][16] when that launch leaves partial maxima
+    int amax_part_count = 0;
     float* history = nullptr;           // [max_len][batch] greedy ids by the position that produced them
     hipGraphExec_t step_graph = nullptr; // one decode step (ids_buf -> ids_buf) captured for replay
     float* splitk_ws = nullptr;         // partial tiles of split-K decode GEMMs
@@ -578,6 +580,18 @@ bool build_fast_plan(fdx_session* s)
     // the embedding launch opens every step and clears the packed arg-max cells the last launch fills
     if (s->steps.empty() || s->steps.front().kind != fdx_session::Step::EmbedAdd)
         return false;
+    // a vocabulary-sized logits launch leaves per-workgroup maxima next to the logits, which saves the pass over them
+    if (s->steps.back().kind == fdx_session::Step::Gemm && s->steps.back().g.n_seg == 1 && s->steps.back().g.seg[0].ptr == s->logits_buf && s->batch <= 16) {
+        SkinnyParams& g = s->steps.back().g;
+        const int parts = skinny_wide_grid(g);
+        if (parts > 0) {
+            s->amax_parts = reinterpret_cast<unsigned long long*>(alloc((size_t)parts * 16 * 2));
+            if (!s->amax_parts)
+                return false;
+            g.amax_parts = s->amax_parts;
+            s->amax_part_count = parts;
+        }
+    }
     return set_int_launch(s->len_dev, 0) == FDX_OK;
 }
 
@@ -620,6 +634,8 @@ fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
     }
     // greedy ids (first maximum wins); the same launch records them by position and advances the cached
     // length on the device
+    if (s->amax_part_count > 0)
+        return argmax_parts_launch(s->amax_parts, s->amax_part_count, B, next_dev, s->len_dev, s->history);
     return argmax_bump_launch(s->logits_buf, B, s->vocab, next_dev, s->len_dev, s->amax, s->history);
 }
 

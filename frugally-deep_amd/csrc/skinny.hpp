@@ -33,9 +33,16 @@ struct SkinnyParams {
     int64_t workspace_floats;
     int* tickets;
     int ticket_count;
+    // optional, wide-output launches only (skinny_wide_grid(p) > 0): every workgroup leaves the packed (value, column)
+    // maximum of each row over the columns it produced in amax_parts[workgroup][16]; argmax_parts_launch picks the winner
+    unsigned long long* amax_parts;
 };
 
 fdx_status skinny_gemm_launch(const SkinnyParams& p);
+// number of workgroups the launch would use if it takes the wide-output kernel (one that strides over column groups), else 0
+int skinny_wide_grid(const SkinnyParams& p);
+// greedy ids from per-workgroup partial maxima [parts][16] (first maximum wins), then as argmax_bump_launch
+fdx_status argmax_parts_launch(const unsigned long long* amax_parts, int parts, int rows, float* out_idx_f, int* len_dev, float* history);
 fdx_status skinny_prepare();
 int64_t packed_weight_floats(int n, int k);
 fdx_status pack_weights_launch(const float* w, int n, int k, int64_t ldw, float* out);

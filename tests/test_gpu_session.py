@@ -113,3 +113,28 @@ def test_session_rejects_non_decoder_models_and_overflow(fdx, modelgen):
     sess.decode_step(np.zeros(2))
     with pytest.raises(fdx.FdxError, match="exceeds max_len"):
         sess.decode_step(np.zeros(2))
+
+
+def test_vocabulary_sized_head_leaves_its_own_argmax(fdx, modelgen):
+    """With tens of thousands of logits per row the logits launch strides over the column groups and leaves
+    per-workgroup maxima, from which the greedy ids are picked without another pass over the logits: the ids must be
+    the first maximum of the logits the same step returns, for batch sizes that fill and do not fill the 16 rows,
+    and the captured loop must produce the same tokens as single steps."""
+    say("session with a vocabulary-sized head")
+    cfg = dict(layers=1, d_model=64, heads=1, vocab=40009, max_pos=32)
+    js = modelgen.dumps(modelgen.gpt2(seed=36, bias_std=0.1, random_affine=True, std=0.2, **cfg))
+    model = fdx.Model(js)
+    for B in (16, 5):
+        prompts = np.random.default_rng(37 + B).integers(0, cfg["vocab"], (B, 6))
+        sess = fdx.Session(model, B, 32)
+        logits, first = sess.prefill(prompts)
+        assert np.array_equal(first, np.argmax(logits, -1).astype(first.dtype))
+        tokens, last_logits = sess.decode_greedy(first, 7)
+        sess2 = fdx.Session(model, B, 32)
+        _, cur = sess2.prefill(prompts)
+        for i in range(7):
+            logits, nxt = sess2.decode_step(cur)
+            assert np.array_equal(nxt, np.argmax(logits, -1).astype(nxt.dtype)), (B, i)
+            assert np.array_equal(nxt, tokens[i]), (B, i)
+            cur = nxt
+        assert rel(logits, last_logits) <= 1e-6
