@@ -485,6 +485,9 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
             const bool hybrid = mode == 1;
             if (splits != 1 && !(can_split && cfg <= 15))
                 continue;
+            static const bool streamk_on = [] { const char* e = std::getenv("FDX_STREAMK"); return !(e && e[0] == '0'); }();
+            if (mode == 2 && !streamk_on)
+                continue;
             if (splits > 1 && mode == 0 && !(tiles <= 1024 && split_fits(cfg, splits, tiles, q)))
                 continue;
             if (hybrid && tiles > 16384)
