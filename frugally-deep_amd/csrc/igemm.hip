@@ -558,7 +558,7 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         a_bytes = ((int64_t)(p.M / (p.OH * p.OW)) * p.H * p.W * p.pix_stride + a_shift) * 4 + 64;
         a_ok = a_mode == A_CONV_VEC && p.Cin % 16 == 0 && p.kh * p.kw <= 64;
     } else {
-        a_bytes = ((int64_t)(p.M - 1) * p.lda + p.K) * 4;
+        a_bytes = ((int64_t)(p.M - 1) * p.lda + (p.a_valid_k > 0 ? p.a_valid_k : p.K)) * 4;
         a_ok = a_mode == A_ROWS_VEC && p.K % 16 == 0;
     }
     const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31);
@@ -614,6 +614,10 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             cfg = 3;
     }
 
+    if (cfg < 10 && p.a_valid_k > 0) { // only the buffer loads of the fast path stop at the real extent
+        set_error("igemm: rows shorter than K need the fast path");
+        return FDX_ERR_UNSUPPORTED;
+    }
     if (cfg < 10 && conv && p.pix_stride != p.Cin) {
         set_error("igemm: a strided-pixel view needs the fast path");
         return FDX_ERR_INVALID;
@@ -785,6 +789,32 @@ extern "C" fdx_status fdx_conv2d_nhwc_f32(const float* in, int n, int h, int w, 
     }
     return run_igemm(p, true, 1, "conv_igemm_f32");
 }
+
+namespace fdx {
+// Pointwise (1x1, stride 1) convolution whose channel count is a multiple of 4 but not of the 16-float slab of the fast
+// path: the filter rows were padded with zero taps to k_padded at load, and the pixels are read as rows of k_padded
+// floats that are only cin apart -- the surplus floats belong to the next pixel and meet zero taps (the very last
+// pixel's surplus lies beyond the buffer extent, which the loads answer with zeros).  Returns FDX_ERR_UNSUPPORTED,
+// with nothing launched, where the fast path does not apply; the caller then uses the unpadded filter.
+fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const float* w_padded, int k_padded, const float* bias,
+    int cout, const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(in && w_padded && out && rows > 0 && rows < (1LL << 31) && cin > 0 && cin % 4 == 0 && k_padded > cin
+            && k_padded % 16 == 0 && cout > 0,
+        "conv1x1_padded: bad arguments");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    if (cout % 4 != 0 || cout < 64 || !aligned16(in) || !aligned16(w_padded) || !aligned16(out) || (residual && !aligned16(residual))
+        || (bias && !aligned16(bias)) || ((rows - 1) * cin + k_padded) * 4 >= (1LL << 31))
+        return FDX_ERR_UNSUPPORTED;
+    GemmParams p {};
+    p.A = in; p.B = w_padded; p.C = out; p.bias = bias; p.residual = residual;
+    p.M = (int)rows; p.N = cout; p.K = k_padded; p.lda = cin; p.ldb = k_padded; p.ldc = cout;
+    p.alpha = 1.f; p.bias_per_row = 0; p.act = make_act(act);
+    p.inner = 1;
+    p.a_valid_k = cin;
+    return run_igemm(p, false, 1, "conv1x1_gemm_f32", 2.0 * (double)rows * cout * cin);
+}
+} // namespace fdx
 
 extern "C" fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const float* b_nk, int64_t ldb,
     int m, int n, int k, float alpha, const float* bias, int bias_per_row,

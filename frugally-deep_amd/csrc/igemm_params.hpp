@@ -28,6 +28,9 @@ struct GemmParams {
     // fast path only: byte extents of one problem's A (counted from the shifted base) and B operands
     uint32_t a_records, b_records;
     int batch; // number of independent problems folded into the persistent tile walk
+    // rows of A that are shorter than K (a pointwise convolution whose channel count was rounded up to the slab with
+    // zero filter taps): floats of a row that really exist, 0 = K.  The loads of the last row stop at the real extent.
+    int a_valid_k;
     // split-K variant of the fast path: K ranges per tile, partial-tile workspace, one ticket per tile (zero between launches)
     int splits;
     int split_dp_tiles; // leading tiles that are computed whole (one unit each); the rest are cut into `splits` K ranges

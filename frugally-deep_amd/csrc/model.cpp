@@ -1172,6 +1172,16 @@ namespace {
                 if (fdx_conv2d_s2d_prepare(o.hw[0].data(), o.cout, o.n_in, o.kh, o.hw[2].data()) != FDX_OK)
                     return FDX_ERR_INVALID;
             }
+            // pointwise convolutions whose channel count is a multiple of 4 but not of 16 (24, 40, 72 ...): a fourth weight
+            // array holds the filter rows padded with zero taps to the next multiple of 16, see conv1x1_padded_launch
+            if (o.kind == OpKind::Conv2D && o.hw.size() == 2 && o.kh == 1 && o.kw == 1 && o.sy == 1 && o.sx == 1 && o.n_in % 4 == 0
+                && o.n_in % 16 != 0 && o.cout % 4 == 0 && o.cout >= 64) {
+                const int kp = (o.n_in + 15) / 16 * 16;
+                o.hw.resize(4);
+                o.hw[3].assign((size_t)o.cout * kp, 0.f);
+                for (int n = 0; n < o.cout; ++n)
+                    std::copy_n(&o.hw[0][(size_t)n * o.n_in], o.n_in, &o.hw[3][(size_t)n * kp]);
+            }
             // self-attention (query, value and key are one tensor): the three projections become one GEMM over the
             // stacked kernels, whose column blocks the attention core then reads in place
             if (o.kind == OpKind::MHA && o.hw.size() >= 6 && o.in.size() >= 2 && o.in[0] == o.in[1]
@@ -1589,6 +1599,11 @@ namespace {
             const int h = one_d ? 1 : (int)(*is)[0], w = (int)(*is)[one_d ? 0 : 1], c = (int)is->back();
             if ((st = window(h, w, o, true, g)) != FDX_OK)
                 return st;
+            if (o.kind == OpKind::Conv2D && o.dw.size() > 3 && o.dw[3] && g[0] + o.zp[0] == 0 && g[2] + o.zp[2] == 0 && g[4] == h && g[5] == w) {
+                st = conv1x1_padded_launch(in0, (int64_t)B * h * w, c, o.dw[3], (c + 15) / 16 * 16, o.dw[1], o.cout, res, actp, out);
+                if (st != FDX_ERR_UNSUPPORTED)
+                    break;
+            }
             if (o.kind == OpKind::Conv2D && !p.temps[idx].empty())
                 st = fdx_conv2d_s2d_nhwc_f32(in0, B, h, w, c, o.dw[2], o.dw[1], o.cout, o.kh, g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5],
                     res, actp, p.temps[idx][0], out);

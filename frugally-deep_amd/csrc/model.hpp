@@ -121,6 +121,8 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
 float* plan_alloc(Plan& p, size_t bytes, int* block_index);
 std::vector<int> topo_order(const fdx_model& m); // producers before consumers, dead ops skipped by callers
 fdx_status positions_launch(float* out, int batch, int t, int start);
+fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const float* w_padded, int k_padded, const float* bias,
+    int cout, const float* residual, const fdx_act* act, float* out);
 fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, const float* k, int64_t ldk, int64_t k_batch,
     const float* v, int64_t ldv, int64_t v_batch, int batch, int t, int s, int heads, int dk, int dv, int causal,
     float* out, int64_t ldo, int64_t o_batch, void* scratch_dev);

@@ -167,3 +167,22 @@ def test_variable_input_size_cycles_through_more_shapes_than_cached_plans(fdx, o
         assert rel(got, want) <= TOL, s
     with pytest.raises(fdx.FdxError, match="Invalid inputs shape"):
         model.predict([np.zeros((1, 8, 8, 4), np.float32)])
+
+
+@pytest.mark.parametrize("cin,cout", [(24, 144), (40, 96), (72, 64), (8, 64)])
+def test_pointwise_convolution_on_channel_counts_between_slabs(fdx, oracle, modelgen, cin, cout):
+    """1x1 convolutions whose channel count is a multiple of 4 but not of 16 read each pixel as a 16-float-aligned row
+    that laps into the next pixel, against filter rows padded with zero taps; the last pixel of the last image has
+    nothing behind it. With BatchNormalization folded in, ReLU6 and a residual Add behind the convolution."""
+    say("pointwise conv", cin, cout)
+    b = modelgen.Builder("pw_%d_%d" % (cin, cout), 50 + cin)
+    x = b.input((9, 7, cin), "img")
+    skip = b.conv2d(x, cout, 3, "skip", padding="same", bias_std=0.1)
+    y = b.conv2d(x, cout, 1, "pw", use_bias=False)
+    y = b.batchnorm(y, "pw_bn", random_stats=True)
+    y = b.relu(y, "pw_relu", max_value=6.0)
+    z = b.conv2d(y, cout, 1, "pw2", bias_std=0.2) if cout % 16 else b.conv2d(x, cout, 1, "pw2", bias_std=0.2)
+    out = b.add([z, skip], "sum")
+    spec = b.finish([out, y])
+    xs = np.random.default_rng(51).standard_normal((5, 9, 7, cin)).astype(np.float32)
+    run_both(fdx, oracle, modelgen, spec, [xs])
