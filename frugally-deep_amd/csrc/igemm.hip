@@ -448,7 +448,10 @@ static std::map<TuneKey, int> g_tuned;
 static int g_autotune = -1;
 static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range per tile
 
-static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s)
+// general_cfg >= 0: the general kernel's configuration for this shape competes too (narrow outputs, where half of a
+// 64-wide fast tile is idle); general_launch runs it once on the caller's unshifted parameters
+template <typename F>
+static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s, int general_cfg, F general_launch)
 {
     if (g_autotune < 0) {
         const char* e = std::getenv("FDX_AUTOTUNE");
@@ -510,6 +513,18 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
                 best_split_ms = ms;
                 best_split = cfg + 100 * splits + 10000 * mode;
             }
+        }
+    }
+    if (general_cfg >= 0) {
+        general_launch();
+        (void)hipEventRecord(a, s);
+        for (int r = 0; r < 3; ++r)
+            general_launch();
+        (void)hipEventRecord(b, s);
+        float ms = 1e30f;
+        if (hipEventSynchronize(b) == hipSuccess && hipEventElapsedTime(&ms, a, b) == hipSuccess && ms < best_ms) {
+            best_ms = ms;
+            best = general_cfg;
         }
     }
     (void)hipEventDestroy(a);
@@ -582,18 +597,30 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         splits = 1;
         mode = 0;
     }
+    auto launch_general = [&](int c) {
+        switch (c) {
+        case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        case 1: launch_cfg<128, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        case 2: launch_cfg<128, 32, 4, 1>(p, a_mode, b_vec, batch, s); break;
+        default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
+        }
+    };
     if (cfg < 0) {
-        if (fast_ok && p.N >= 64 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
+        if (fast_ok && p.N >= 16 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
             GemmParams q = p;
             q.A = p.A - a_shift;
             q.a_records = (uint32_t)a_bytes;
             q.b_records = (uint32_t)b_bytes;
             q.batch = batch;
-            cfg = autotune(q, conv, batch, unit, s);
+            // below 64 output columns the general kernel's narrow tile is a candidate of its own, unless only the
+            // fast path can read this operand
+            const bool general_ok = p.N < 64 && p.a_valid_k == 0 && !(conv && p.pix_stride != p.Cin);
+            const int general_cfg = !general_ok ? -1 : p.N <= 32 ? 2 : (blocks(128, 64) >= 512 ? 1 : 3);
+            cfg = autotune(q, conv, batch, unit, s, general_cfg, [&] { launch_general(general_cfg); });
             if (cfg >= 100)
                 unpack();
         }
-        if (cfg >= 10) {
+        if (cfg >= 0) {
         } else if (fast_ok && p.N >= 64) {
             // the largest tile that still gives every CU a few workgroups
             if (blocks(128, 128) >= 1024 && p.N % 128 == 0)
@@ -632,12 +659,7 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         if (!launch_fast(cfg, splits, mode, q, conv, batch, s))
             launch_fast(cfg, 1, 0, q, conv, batch, s); // the requested cut does not fit the scratch
     } else {
-        switch (cfg) {
-        case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
-        case 1: launch_cfg<128, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
-        case 2: launch_cfg<128, 32, 4, 1>(p, a_mode, b_vec, batch, s); break;
-        default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
-        }
+        launch_general(cfg);
     }
     const double flops = algorithmic_flops > 0.0 ? algorithmic_flops : 2.0 * p.M * (double)p.N * p.K * batch;
     profile_end(family, flops, 0.0);
