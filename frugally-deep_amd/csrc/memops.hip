@@ -384,6 +384,53 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const float* __rest
     }
 }
 
+// Same, 16 bytes per lane and access (depth a multiple of 4, at most 256 * NV): a row is NV wave-wide loads.
+template <int NV>
+__global__ __launch_bounds__(256) void layernorm_wave4_kernel(const float* __restrict__ x, float* __restrict__ out,
+    int64_t rows, int depth, const float* __restrict__ gamma, const float* __restrict__ beta, float eps)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blockIdx.x * 4LL + (threadIdx.x >> 6);
+    if (row >= rows)
+        return;
+    const float* xr = x + row * depth;
+    f32x4 v[NV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int z = (lane + i * 64) * 4;
+        v[i] = z < depth ? *reinterpret_cast<const f32x4*>(xr + z) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+        s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+    }
+    const float mean = wave_sum(s) / (float)depth;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+        if ((lane + i * 64) * 4 < depth)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float d = v[i][e] - mean;
+                q += d * d;
+            }
+    const float rs = 1.0f / sqrtf(wave_sum(q) / (float)depth + eps);
+    float* orow = out + row * depth;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int z = (lane + i * 64) * 4;
+        if (z < depth) {
+            const f32x4 g = gamma ? *reinterpret_cast<const f32x4*>(gamma + z) : f32x4 { 1.f, 1.f, 1.f, 1.f };
+            const f32x4 b = beta ? *reinterpret_cast<const f32x4*>(beta + z) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float inv = rs * g[e];
+                o[e] = v[i][e] * inv + (b[e] - mean * inv);
+            }
+            *reinterpret_cast<f32x4*>(orow + z) = o;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void layernorm_block_kernel(const float* __restrict__ x, float* __restrict__ out,
     int depth, const float* __restrict__ gamma, const float* __restrict__ beta, float eps)
 {
@@ -697,7 +744,17 @@ extern "C" fdx_status fdx_layernorm_f32(const float* x, int64_t rows, int depth,
     FDX_REQUIRE(x && out && rows > 0 && depth > 0, "layernorm: bad arguments");
     profile_begin();
     const dim3 g4((unsigned)((rows + 3) / 4));
-    if (depth <= 256)
+    auto a16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    if (depth % 4 == 0 && depth <= 1024 && a16(x) && a16(out) && a16(gamma) && a16(beta)) {
+        if (depth <= 256)
+            hipLaunchKernelGGL(layernorm_wave4_kernel<1>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
+        else if (depth <= 512)
+            hipLaunchKernelGGL(layernorm_wave4_kernel<2>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
+        else if (depth <= 768)
+            hipLaunchKernelGGL(layernorm_wave4_kernel<3>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
+        else
+            hipLaunchKernelGGL(layernorm_wave4_kernel<4>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
+    } else if (depth <= 256)
         hipLaunchKernelGGL(layernorm_wave_kernel<4>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
     else if (depth <= 1024)
         hipLaunchKernelGGL(layernorm_wave_kernel<16>, g4, dim3(256), 0, stream(), x, out, rows, depth, gamma, beta, eps);
