@@ -242,7 +242,7 @@ __global__ __launch_bounds__(256) void flash_prefill_kernel(FlashParams p)
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float pv = expf(sacc[kb][e] - m_use);
+                const float pv = __expf(sacc[kb][e] - m_use);
                 sacc[kb][e] = pv;
                 rs += pv;
             }
