@@ -397,7 +397,12 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
 #define FDX_FAST(BM_, BN_, BK_)                                                                                  \
     {                                                                                                            \
         const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
-        if (splits > 1 || mode == 2) {                                                                           \
+        if (mode == 2) {                                                                                         \
+            if (conv)                                                                                            \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true, true>, tiles, splits, mode, cfg, q, s); \
+            else                                                                                                 \
+                ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true, true>, tiles, splits, mode, cfg, q, s); \
+        } else if (splits > 1) {                                                                                 \
             if (conv)                                                                                            \
                 ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true, true>, tiles, splits, mode, cfg, q, s); \
             else                                                                                                 \

@@ -31,7 +31,7 @@
 //    and their workspace slots computed from the cut points.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false, bool STREAMK = false>
 // (the second bound asks for two waves per SIMD where the split variant of the largest four-wave tile would otherwise
 // settle for one: its reduction holds the accumulators in ordinary registers next to the prefetched operands)
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (SPLIT && WAVES_M * WAVES_N == 4 && BM * BN >= 128 * 128) ? 2 : 1)
@@ -76,7 +76,10 @@ void igemm_fast_kernel(GemmParams p)
 
     // stream-K: workgroup g (numbered XCD by XCD, so an XCD owns a contiguous stretch of tiles) takes the slabs
     // [g * W / G, (g + 1) * W / G) of the W = tiles * KT slabs; its units are the tiles that stretch touches
-    const bool sk = SPLIT && p.splits == 0;
+    // (a template argument: carried as a run-time flag, the extra index arithmetic cost the plain split variant a
+    // tenth of its speed)
+    static_assert(!STREAMK || SPLIT, "stream-K is a form of the split variant");
+    constexpr bool sk = STREAMK;
     const int G = (int)gridDim.x;
     const int g_lin = xcd * (G >> 3) + (xcd < (G & 7) ? xcd : (G & 7)) + wg_in_xcd;
     const int64_t W = (int64_t)all_tiles * KT;
@@ -312,9 +315,20 @@ void igemm_fast_kernel(GemmParams p)
                     break;
                 continue;
             }
-            // every unit, this one included, has left its partial in the workspace: they are summed from there in
-            // split order (re-reading the own one costs a tile of loads and saves a second copy of the accumulators,
-            // which would halve the number of resident workgroups)
+            // Partials are summed in split order.  The own one comes from the workspace like the others where a second
+            // copy of the accumulators would halve the number of resident workgroups (128 x 128 tiles: re-reading it
+            // costs a tile of loads); smaller tiles keep it in registers.
+            constexpr bool REREAD_OWN = TM * TN >= 4;
+            f32x16 own[REREAD_OWN ? 1 : TM][REREAD_OWN ? 1 : TN];
+            int my_part = -1;
+            if (!REREAD_OWN) {
+                my_part = sk ? g_lin - g_a : su_done - out_tile * S;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        own[REREAD_OWN ? 0 : i][REREAD_OWN ? 0 : j] = acc[i][j];
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -324,13 +338,15 @@ void igemm_fast_kernel(GemmParams p)
                         acc[i][j][e] = 0.f;
             for (int sp = 0; sp < parts; ++sp) {
                 const float* part = p.split_ws + slot_of(sp) * TILE_F + t;
+                const bool self = sp == my_part;
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            acc[i][j][e] += __hip_atomic_load(part + ((i * TN + j) * 16 + e) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            acc[i][j][e] += self ? own[REREAD_OWN ? 0 : i][REREAD_OWN ? 0 : j][e]
+                                                 : __hip_atomic_load(part + ((i * TN + j) * 16 + e) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         // one 32x32 block's loads at a time: hoisting all of them would need a register per load
                         __builtin_amdgcn_sched_barrier(0);
                     }
