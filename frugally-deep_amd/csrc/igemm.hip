@@ -479,6 +479,21 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     int best = -1, best_split = -1;
     float best_ms = 1e30f, best_split_ms = 1e30f;
     const bool can_split = g_split_enabled && split_prepare();
+    // three launches back to back, the faster of two such rounds: candidates within a percent of each other are
+    // common, and a single round of a 30 us kernel is too short a window to tell them apart
+    auto timed = [&](auto&& launch) -> float {
+        float best_round = 1e30f;
+        for (int round = 0; round < 2; ++round) {
+            (void)hipEventRecord(a, s);
+            for (int r = 0; r < 3; ++r)
+                launch();
+            (void)hipEventRecord(b, s);
+            float ms = 1e30f;
+            if (hipEventSynchronize(b) == hipSuccess && hipEventElapsedTime(&ms, a, b) == hipSuccess && ms < best_round)
+                best_round = ms;
+        }
+        return best_round;
+    };
     for (int cfg = 10; cfg <= 18; ++cfg) {
         if (cfg >= 13 && unit % 32 != 0)
             continue;
@@ -502,13 +517,7 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
                 continue;
             if (!launch_fast(cfg, splits, mode, q, conv, batch, s)) // warm-up; false = the cut does not fit
                 continue;
-            (void)hipEventRecord(a, s);
-            for (int r = 0; r < 3; ++r)
-                launch_fast(cfg, splits, mode, q, conv, batch, s);
-            (void)hipEventRecord(b, s);
-            float ms = 1e30f;
-            if (hipEventSynchronize(b) != hipSuccess || hipEventElapsedTime(&ms, a, b) != hipSuccess)
-                continue;
+            const float ms = timed([&] { launch_fast(cfg, splits, mode, q, conv, batch, s); });
             if (splits == 1) {
                 if (ms < best_ms) {
                     best_ms = ms;
@@ -522,12 +531,8 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     }
     if (general_cfg >= 0) {
         general_launch();
-        (void)hipEventRecord(a, s);
-        for (int r = 0; r < 3; ++r)
-            general_launch();
-        (void)hipEventRecord(b, s);
-        float ms = 1e30f;
-        if (hipEventSynchronize(b) == hipSuccess && hipEventElapsedTime(&ms, a, b) == hipSuccess && ms < best_ms) {
+        const float ms = timed(general_launch);
+        if (ms < best_ms) {
             best_ms = ms;
             best = general_cfg;
         }
