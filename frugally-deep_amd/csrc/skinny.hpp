@@ -39,6 +39,34 @@ struct SkinnyParams {
 };
 
 fdx_status skinny_gemm_launch(const SkinnyParams& p);
+
+// One phase of the persistent decode-step kernel: a Dense launch (as skinny_gemm_launch would run it) or the decode
+// attention of every (sequence, head).
+struct MegaPhase {
+    int kind;    // 0 = Dense, 1 = attention
+    int tiles;   // Dense: 16-column groups; attention: (sequence, head) items
+    int ksplit;  // Dense: K ranges per column group
+    int chunk;   // Dense: 6 or 8 slabs per wave (the kernel instantiation)
+    SkinnyParams g;
+    const float* q;
+    int64_t ldq;
+    const float* kc;
+    const float* vc;
+    float* out;
+    int heads, max_len;
+    float scale;
+};
+// Fills `phase` from a Dense launch's parameters; false when the persistent kernel does not cover the shape.
+bool mega_dense_phase(const SkinnyParams& p, float* workspace, int* tickets, MegaPhase& phase);
+bool mega_attention_phase(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch, int heads, int dk,
+    int dv, const int* len_dev, int max_len, MegaPhase& phase);
+// Device-side state of the persistent kernel's grid barrier (allocated once per session): arrival cells, release cells,
+// epoch, abort flag.
+size_t mega_state_bytes();
+// Runs the phases back to back inside one launch, a grid-wide barrier between consecutive phases.
+fdx_status mega_launch(const MegaPhase* phases_dev, int n_phases, void* state_dev);
+// non-zero after a launch whose barrier gave up waiting (reads the flag back; synchronises the stream)
+fdx_status mega_check(void* state_dev);
 // number of workgroups the launch would use if it takes the wide-output kernel (one that strides over column groups), else 0
 int skinny_wide_grid(const SkinnyParams& p);
 // greedy ids from per-workgroup partial maxima [parts][16] (first maximum wins), then as argmax_bump_launch

@@ -138,3 +138,38 @@ def test_vocabulary_sized_head_leaves_its_own_argmax(fdx, modelgen):
             assert np.array_equal(nxt, tokens[i]), (B, i)
             cur = nxt
         assert rel(logits, last_logits) <= 1e-6
+
+
+def test_persistent_step_kernel_matches_separate_launches(fdx, modelgen, monkeypatch):
+    """FDX_DECODE_MEGA=1 (read at session creation) runs the Dense / attention launches of a step as phases of one
+    persistent kernel with grid-wide barriers in between: same tokens and logits as the separate launches, step by
+    step and in the captured loop, over more steps than one barrier epoch."""
+    say("persistent decode-step kernel")
+    cfg = dict(layers=3, d_model=128, heads=2, vocab=211, max_pos=64)
+    js = modelgen.dumps(modelgen.gpt2(seed=38, bias_std=0.1, random_affine=True, std=0.2, **cfg))
+    model = fdx.Model(js)
+    B, P, N = 5, 7, 20
+    prompts = np.random.default_rng(39).integers(0, cfg["vocab"], (B, P))
+    ref = fdx.Session(model, B, 64)
+    _, first = ref.prefill(prompts)
+    want_tokens, want_logits = ref.decode_greedy(first, N)
+    monkeypatch.setenv("FDX_DECODE_MEGA", "1")
+    sess = fdx.Session(model, B, 64)
+    monkeypatch.delenv("FDX_DECODE_MEGA")
+    _, first2 = sess.prefill(prompts)
+    assert np.array_equal(first2, first)
+    tokens, logits = sess.decode_greedy(first2, N)
+    assert np.array_equal(tokens, want_tokens)
+    assert rel(logits, want_logits) <= 1e-6
+    sess3 = fdx.Session(model, B, 64)  # created without the switch: separate launches again
+    _, cur = sess3.prefill(prompts)
+    monkeypatch.setenv("FDX_DECODE_MEGA", "1")
+    sess4 = fdx.Session(model, B, 64)
+    monkeypatch.delenv("FDX_DECODE_MEGA")
+    _, cur4 = sess4.prefill(prompts)
+    for i in range(6):
+        la, na = sess3.decode_step(cur)
+        lb, nb = sess4.decode_step(cur4)
+        assert np.array_equal(na, nb) and np.array_equal(na, want_tokens[i])
+        assert rel(lb, la) <= 1e-6
+        cur, cur4 = na, nb
