@@ -12,6 +12,7 @@
 #include <cmath>
 
 #include "common.hpp"
+#include "global_ptr.hpp"
 #include "skinny.hpp"
 
 namespace fdx {

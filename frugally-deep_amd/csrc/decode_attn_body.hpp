@@ -1,5 +1,5 @@
 // Body of the decode attention for the common head shape, shared by its own kernel (decode_attn.hip) and the persistent
-// decode-step kernel (decode_kernels.hip).  Included inside namespace fdx after f32x4 is defined.
+// decode-step kernel (decode_kernels.hip).  Included inside namespace fdx after f32x4 and gptr are defined.
 #pragma once
 
 struct MhaDecodeShared {
@@ -20,10 +20,10 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
     float (*osum)[64] = sh.osum;
     const int part = tid & 15, slot = tid >> 4, wave = (tid >> 6) & 3;
     const int b = item / heads, h = item % heads;
-    const int len = active ? *len_dev + 1 : 0;
+    const int len = active ? *as_global(len_dev) + 1 : 0;
     const int64_t row = (int64_t)heads * 64;
-    const float* kbase = kc + (int64_t)b * max_len * row + h * 64 + part * 4;
-    const float* vbase = vc + (int64_t)b * max_len * row + h * 64 + part * 4;
+    const gptr<const float> kbase = as_global(kc) + (int64_t)b * max_len * row + h * 64 + part * 4;
+    const gptr<const float> vbase = as_global(vc) + (int64_t)b * max_len * row + h * 64 + part * 4;
     f32x4 kv[16], vv[16];
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
@@ -31,11 +31,11 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
         kv[u] = f32x4 { 0.f, 0.f, 0.f, 0.f };
         vv[u] = f32x4 { 0.f, 0.f, 0.f, 0.f };
         if (j < len) {
-            kv[u] = *reinterpret_cast<const f32x4*>(kbase + (int64_t)j * row);
-            vv[u] = *reinterpret_cast<const f32x4*>(vbase + (int64_t)j * row);
+            kv[u] = *reinterpret_cast<gptr<const f32x4>>(kbase + (int64_t)j * row);
+            vv[u] = *reinterpret_cast<gptr<const f32x4>>(vbase + (int64_t)j * row);
         }
     }
-    const f32x4 qv = active ? *reinterpret_cast<const f32x4*>(q + (int64_t)b * ldq + h * 64 + part * 4) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+    const f32x4 qv = active ? *reinterpret_cast<gptr<const f32x4>>(as_global(q) + (int64_t)b * ldq + h * 64 + part * 4) : f32x4 { 0.f, 0.f, 0.f, 0.f };
 
     float sc[16];
     float m = -FLT_MAX;
@@ -91,7 +91,7 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
             denom += f[w] * red_sum[w];
             o += f[w] * osum[w][tid];
         }
-        float* dst = out + (int64_t)b * row + h * 64 + tid;
+        const gptr<float> dst = as_global(out) + (int64_t)b * row + h * 64 + tid;
         if (MEGA)
             __hip_atomic_store(dst, o / denom, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else

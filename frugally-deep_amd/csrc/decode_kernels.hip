@@ -22,6 +22,7 @@
 #include <cstring>
 
 #include "common.hpp"
+#include "global_ptr.hpp"
 #include "skinny.hpp"
 
 namespace fdx {
@@ -75,9 +76,10 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
 
     const int n = n0 + i;
     const bool n_ok = n < p.N, m_ok = i < p.M;
-    const float* wrow = p.W + (int64_t)(n_ok ? n : 0) * p.ldw;
+    const gptr<const float> Wg = as_global(p.W);
+    const gptr<const float> wrow = Wg + (int64_t)(n_ok ? n : 0) * p.ldw;
     const int spw = per_wave / 16; // slabs per wave in the packed layout
-    const float* xrow = p.X + (int64_t)(m_ok ? i : 0) * p.ldx;
+    const gptr<const float> xrow = as_global(p.X) + (int64_t)(m_ok ? i : 0) * p.ldx;
     // two named register sets (indexing one array with a run-time buffer number would push it to scratch)
     f32x4 w0[CHUNK], a0[CHUNK];
     auto load_chunk = [&](f32x4 (&wreg)[CHUNK], f32x4 (&areg)[CHUNK], int s0) {
@@ -89,11 +91,11 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
             if (p.packed) {
                 // pre-packed operand: this wave's slab is one contiguous 1 KB run, zeros baked in
                 if (s0 + s < spw)
-                    wv = reinterpret_cast<const f32x4*>(p.W)[(((int64_t)bx * SK_WAVES + wave) * spw + (s0 + s)) * 64 + lane];
+                    wv = reinterpret_cast<gptr<const f32x4>>(Wg)[(((int64_t)bx * SK_WAVES + wave) * spw + (s0 + s)) * 64 + lane];
             } else if (n_ok && k_ok)
-                wv = *reinterpret_cast<const f32x4*>(wrow + k);
+                wv = *reinterpret_cast<gptr<const f32x4>>(wrow + k);
             if (m_ok && k_ok)
-                av = *reinterpret_cast<const f32x4*>(xrow + k);
+                av = *reinterpret_cast<gptr<const f32x4>>(xrow + k);
             wreg[s] = wv;
             areg[s] = av;
         }
@@ -109,17 +111,17 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
     int e_seg = 0;
     if (e_ok) {
         if (p.bias)
-            e_bias = p.bias[ecol];
+            e_bias = as_global(p.bias)[ecol];
         if (p.residual)
-            e_res = p.residual[(int64_t)em * p.ldr + ecol];
+            e_res = as_global(p.residual)[(int64_t)em * p.ldr + ecol];
         if (p.ln)
-            e_wsum = p.w_rowsum[ecol];
+            e_wsum = as_global(p.w_rowsum)[ecol];
         if (p.n_seg > 1 && ecol >= p.seg[1].col_begin)
             e_seg = 1;
         if (p.n_seg > 2 && ecol >= p.seg[2].col_begin)
             e_seg = 2;
         if (p.seg[e_seg].len_stride)
-            e_shift = (int64_t)(*p.len_dev) * p.seg[e_seg].len_stride;
+            e_shift = (int64_t)(*as_global(p.len_dev)) * p.seg[e_seg].len_stride;
     }
 
     // 16x16x4 MFMA: A operand lane (m = i, k slot = kq), B operand lane (n = i, k slot = kq);
@@ -196,7 +198,9 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         // Publish this split's partial tile with device-scope stores (they go past the XCD's L2), wait for
         // them, then take a ticket; only the last arrival continues and adds the partials in split order,
         // which makes the sum independent of arrival order.  No fence that writes back the whole L2.
-        float* part = p.workspace + ((int64_t)by * gx + bx) * 256;
+        const gptr<float> ws = as_global(p.workspace);
+        const gptr<int> tickets = as_global(p.tickets);
+        const gptr<float> part = ws + ((int64_t)by * gx + bx) * 256;
         if (t < 256)
             __hip_atomic_store(part + t, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // every lane's partials have left the CU before the ticket is taken
@@ -204,10 +208,10 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (t == 0) {
-            const int ticket = __hip_atomic_fetch_add(p.tickets + bx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int ticket = __hip_atomic_fetch_add(tickets + bx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             is_last = ticket == ksplit - 1;
             if (is_last)
-                __hip_atomic_store(p.tickets + bx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // next launch
+                __hip_atomic_store(tickets + bx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // next launch
         }
         __syncthreads();
         if (!is_last)
@@ -215,7 +219,7 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         if (t < 256) {
             v = 0.f;
             for (int ks = 0; ks < ksplit; ++ks)
-                v += __hip_atomic_load(p.workspace + ((int64_t)ks * gx + bx) * 256 + t, __ATOMIC_RELAXED,
+                v += __hip_atomic_load(ws + ((int64_t)ks * gx + bx) * 256 + t, __ATOMIC_RELAXED,
                     __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -231,7 +235,7 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         }
         v = apply_act(v + e_bias + e_res, p.act);
         const SkinnySegment& sg = p.seg[e_seg];
-        float* dst = sg.ptr + e_shift + (int64_t)em * sg.ld + (ecol - sg.col_begin);
+        const gptr<float> dst = as_global(sg.ptr) + e_shift + (int64_t)em * sg.ld + (ecol - sg.col_begin);
         if (MEGA)
             __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
