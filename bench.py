@@ -113,7 +113,7 @@ def bench_resnet(fdx, modelgen, args):
     total_ms = sum(v["ms"] for v in fams.values())
 
     result = {
-        "metric": "ResNet50-shape img/s (fp32,b64)",
+        "metric": "ResNet50-shape img/s (fp32,b%d)" % args.batch,
         "value": round(img_s, 2),
         "unit": "img/s",
         "n_gpus": 1,
