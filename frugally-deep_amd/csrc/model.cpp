@@ -177,7 +177,10 @@ namespace {
     const std::set<std::string> kIdentity = { "Identity", "Dropout", "Masking", "ActivityRegularization", "AlphaDropout",
         "FixedDropout", "SpatialDropout1D", "SpatialDropout2D", "SpatialDropout3D", "GaussianDropout", "GaussianNoise",
         "RandomBrightness", "RandomContrast", "RandomCrop", "RandomFlip", "RandomHeight", "RandomRotation",
-        "RandomTranslation", "RandomWidth", "RandomZoom" };
+        "RandomTranslation", "RandomWidth", "RandomZoom", "RandomColorDegeneration", "RandomColorJitter", "RandomElasticTransform", "RandomErasing", "RandomGaussianBlur",
+        "RandomGrayscale", "RandomHue", "RandomInvert", "RandomPerspective", "RandomPosterization", "RandomSaturation",
+        "RandomSharpness", "RandomShear", "AugMix", "CutMix", "Equalization", "MaxNumBoundingBoxes", "MixUp", "Pipeline",
+        "RandAugment", "Solarization" };
 
     // Sets an activation by name; returns false for "softmax" (caller schedules the softmax kernel).
     // import_model.hpp:1649-1700; relu parameters only when max_value is present and non-null (:1289-1302).
@@ -591,6 +594,42 @@ namespace {
                     op.hw[1][i] = (beta.empty() ? 0.f : beta[i]) - mean[i] * inv;
                 }
                 op.cout = (int)mean.size();
+                result = add_op(std::move(op));
+            } else if (cls == "Rescaling") {
+                // y = scale * x + offset with one pair for the whole tensor (layers/rescaling_layer.hpp:30-40)
+                op.kind = OpKind::Affine;
+                op.hw.resize(2);
+                op.hw[0] = { (float)cfg.at("scale").number() };
+                op.hw[1] = { (float)cfg.at("offset").number() };
+                op.cout = 1;
+                op.affine_scalar = true;
+                result = add_op(std::move(op));
+            } else if (cls == "Normalization") {
+                // (x - mean) / max(sqrt(variance), 1e-7), or its inverse; one pair for the whole tensor or one per slice of
+                // the given axis (layers/normalization_layer.hpp:36-75, import_model.hpp:1392-1404)
+                op.kind = OpKind::Affine;
+                const std::vector<float> mean = decode_floats(param(sc, c.layer, "mean"));
+                const std::vector<float> var = decode_floats(param(sc, c.layer, "variance"));
+                const Value& ax = cfg.at("axis");
+                const size_t n_axes = ax.is_array() ? ax.size() : (ax.is_null() ? 0 : 1);
+                if (n_axes > 1)
+                    throw FormatError("Unsupported number of axes for Normalization layer");
+                if (mean.size() != var.size() || var.empty() || (n_axes == 0 && var.size() != 1))
+                    throw FormatError("Invalid number of variance values in Normalization layer.");
+                const Value* inv = cfg.find("invert");
+                const bool invert = inv && inv->boolean();
+                op.hw.resize(2);
+                op.hw[0].resize(var.size());
+                op.hw[1].resize(var.size());
+                for (size_t i = 0; i < var.size(); ++i) {
+                    const float sd = std::fmax(std::sqrt(var[i]), 1e-7f);
+                    op.hw[0][i] = invert ? sd : 1.0f / sd;
+                    op.hw[1][i] = invert ? mean[i] : -mean[i] / sd;
+                }
+                op.cout = (int)var.size();
+                op.affine_scalar = n_axes == 0;
+                if (n_axes == 1)
+                    op.ln_axes = (int)(ax.is_array() ? ax.at((size_t)0).integer() : ax.integer());
                 result = add_op(std::move(op));
             } else if (cls == "SeparableConv2D" || cls == "SeparableConv1D") {
                 // depthwise part without bias or activation, then a 1x1 valid convolution that carries the bias and the
@@ -1076,7 +1115,7 @@ namespace {
         // 1. BatchNormalization on the channel axis into the producing convolution / dense weights
         for (size_t i = 0; i < m.ops.size(); ++i) {
             Op& bn = m.ops[i];
-            if (bn.dead || bn.kind != OpKind::Affine)
+            if (bn.dead || bn.kind != OpKind::Affine || bn.affine_scalar)
                 continue;
             Op& p = m.ops[bn.in[0]];
             const bool producer_ok = (is_gemm_like(p) || p.kind == OpKind::DWConv2D) && p.act.kind == FDX_ACT_NONE
@@ -1623,10 +1662,14 @@ namespace {
             break;
         }
         case OpKind::Affine: {
+            if (o.affine_scalar) { // one (scale, shift) pair for every element
+                st = fdx_channel_affine_f32(in0, (size_t)B * (size_t)volume(*is), 1, o.dw[0], o.dw[1], actp, out);
+                break;
+            }
             const int rank = (int)is->size();
             const int axis = o.ln_axes < 0 ? o.ln_axes + rank + 1 : o.ln_axes;
             if (axis != rank || is->back() != o.cout) {
-                set_error("%s: BatchNormalization is supported on the last axis only", o.name.c_str());
+                set_error("%s: %s is supported on the last axis only", o.name.c_str(), o.cls.c_str());
                 return FDX_ERR_UNSUPPORTED;
             }
             st = fdx_channel_affine_f32(in0, (size_t)B * (size_t)volume(*is) / (size_t)o.cout, o.cout, o.dw[0], o.dw[1], actp, out);

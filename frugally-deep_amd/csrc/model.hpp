@@ -59,6 +59,7 @@ struct Op {
     bool log_after = false;          // Softmax op that is a log_softmax
     bool rms = false;                // LayerNorm op that is an RMSNormalization
     bool bilinear = false;           // Resize: interpolation (kh / kw hold the factors; Crop keeps its margins in zp)
+    bool affine_scalar = false;      // Affine with one (scale, shift) pair for the whole tensor (Rescaling, axis-less Normalization)
     bool trailing = false;           // Dilate: zero insertion in front of a "same" transposed convolution (kh / kw hold the rates)
     bool gate = false;               // attention with a sigmoid gate on its output (GroupQueryAttention use_gate)
     std::vector<int64_t> shared_axes; // PReLU

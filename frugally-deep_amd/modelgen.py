@@ -166,6 +166,16 @@ class Builder:
         cfg = {"axis": len(x.shape), "epsilon": eps, "center": True, "scale": True}
         return self._add("BatchNormalization", name, cfg, [x], x.shape)
 
+    def rescaling(self, x, name, scale, offset=0.0):
+        return self._add("Rescaling", name, {"scale": float(scale), "offset": float(offset)}, [x], x.shape)
+
+    def normalization(self, x, name, axis=-1, invert=False):
+        """Keras Normalization with random statistics; axis None = one mean / variance for the whole tensor."""
+        n = 1 if axis is None else x.shape[axis if axis < 0 else axis - 1]
+        self.params[name] = {"mean": self.normal((n,), 0.5), "variance": (0.25 + self.rng.random(n)).astype(np.float32)}
+        cfg = {"axis": [] if axis is None else [axis], "invert": bool(invert)}
+        return self._add("Normalization", name, cfg, [x], x.shape)
+
     def layernorm(self, x, name, eps=1e-3, random_affine=False):
         d = x.shape[-1]
         if random_affine:

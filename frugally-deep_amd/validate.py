@@ -13,6 +13,10 @@ IDENTITY = {
     "Identity", "Dropout", "Masking", "ActivityRegularization", "AlphaDropout", "FixedDropout", "SpatialDropout1D",
     "SpatialDropout2D", "SpatialDropout3D", "GaussianDropout", "GaussianNoise", "RandomBrightness", "RandomContrast",
     "RandomCrop", "RandomFlip", "RandomHeight", "RandomRotation", "RandomTranslation", "RandomWidth", "RandomZoom",
+    "RandomColorDegeneration", "RandomColorJitter", "RandomElasticTransform", "RandomErasing", "RandomGaussianBlur",
+    "RandomGrayscale", "RandomHue", "RandomInvert", "RandomPerspective", "RandomPosterization", "RandomSaturation",
+    "RandomSharpness", "RandomShear", "AugMix", "CutMix", "Equalization", "MaxNumBoundingBoxes", "MixUp", "Pipeline",
+    "RandAugment", "Solarization",
 }
 
 ACTIVATION_LAYERS = {
@@ -42,6 +46,8 @@ REQUIRED_CONFIG = {
     "BatchNormalization": ("epsilon", "center", "scale", "axis"),
     "LayerNormalization": ("epsilon", "center", "scale", "axis"),
     "RMSNormalization": ("epsilon", "axis"),
+    "Rescaling": ("scale", "offset"),
+    "Normalization": ("axis",),
     "MaxPooling1D": _POOL_KEYS, "MaxPooling2D": _POOL_KEYS, "AveragePooling1D": _POOL_KEYS, "AveragePooling2D": _POOL_KEYS,
     "ZeroPadding1D": ("padding",), "ZeroPadding2D": ("padding",),
     "Cropping1D": ("cropping",), "Cropping2D": ("cropping",),
@@ -224,6 +230,16 @@ class _Walk:
                 g = self.count(where, owner, key, need=bool(cfg[flag]))
                 if g is not None and m is not None and cfg[flag] and g != m:
                     self.add(where, "%s has %d values, moving_mean %d" % (key, g, m))
+        elif cls == "Normalization":
+            m, v = self.count(where, owner, "mean"), self.count(where, owner, "variance")
+            if m is not None and v is not None and m != v:
+                self.add(where, "mean and variance differ in length")
+            ax = cfg["axis"]
+            n_axes = len(ax) if isinstance(ax, (list, tuple)) else (0 if ax is None else 1)
+            if n_axes > 1:
+                self.add(where, "more than one Normalization axis")
+            if n_axes == 0 and v is not None and v != 1:
+                self.add(where, "axis-less Normalization needs exactly one mean / variance")
         elif cls == "LayerNormalization":
             for key, flag in (("gamma", "scale"), ("beta", "center")):
                 self.count(where, owner, key, need=bool(cfg[flag]))

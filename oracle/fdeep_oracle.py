@@ -40,6 +40,10 @@ IDENTITY_LAYERS = {
     "SpatialDropout1D", "SpatialDropout2D", "SpatialDropout3D", "GaussianDropout", "GaussianNoise",
     "RandomBrightness", "RandomContrast", "RandomCrop", "RandomFlip", "RandomHeight",
     "RandomRotation", "RandomTranslation", "RandomWidth", "RandomZoom",
+    "RandomColorDegeneration", "RandomColorJitter", "RandomElasticTransform", "RandomErasing", "RandomGaussianBlur",
+    "RandomGrayscale", "RandomHue", "RandomInvert", "RandomPerspective", "RandomPosterization", "RandomSaturation",
+    "RandomSharpness", "RandomShear", "AugMix", "CutMix", "Equalization", "MaxNumBoundingBoxes", "MixUp", "Pipeline",
+    "RandAugment", "Solarization",
 }
 
 
@@ -497,6 +501,9 @@ class _Layer:
             self.p["var"] = decode_floats(get_param(name, "moving_variance"))
             self.p["gamma"] = decode_floats(get_param(name, "gamma")) if c["scale"] else None
             self.p["beta"] = decode_floats(get_param(name, "beta")) if c["center"] else None
+        elif cls == "Normalization":
+            self.p["mean"] = decode_floats(get_param(name, "mean"))
+            self.p["var"] = decode_floats(get_param(name, "variance"))
         elif cls == "LayerNormalization":
             self.p["gamma"] = decode_floats(get_param(name, "gamma")) if c["scale"] else None
             self.p["beta"] = decode_floats(get_param(name, "beta")) if c["center"] else None
@@ -547,6 +554,29 @@ class _Layer:
                                    c["dilation_rate"], c["padding"])
         elif cls == "Dense":
             out = dense(ins[0], p["w"], p["b"], int(c["units"]))
+        elif cls == "Rescaling":
+            # layers/rescaling_layer.hpp:30-40
+            out = (np.float32(c["scale"]) * ins[0] + np.float32(c["offset"])).astype(np.float32)
+        elif cls == "Normalization":
+            # layers/normalization_layer.hpp:36-75: per slice of the axis, (x - mean) / max(sqrt(var), 1e-7) or,
+            # inverted, mean + x * max(sqrt(var), 1e-7); no axis: one pair for the whole tensor
+            x = ins[0]
+            axes = c["axis"] if isinstance(c["axis"], (list, tuple)) else ([] if c["axis"] is None else [c["axis"]])
+            if len(axes) > 1:
+                raise ValueError("Unsupported number of axes for Normalization layer")
+            sd = np.maximum(np.sqrt(p["var"]), np.float32(1e-7)).astype(np.float32)
+            mean = p["mean"]
+            if not axes:
+                if sd.size != 1:
+                    raise ValueError("Invalid number of variance values in Normalization layer.")
+            else:
+                axis = axes[0] if axes[0] >= 0 else axes[0] + x.ndim + 1  # Keras axes count the batch dimension
+                if x.shape[axis - 1] != sd.size:
+                    raise ValueError("Invalid number of variance values in Normalization layer.")
+                shape = [1] * x.ndim
+                shape[axis - 1] = sd.size
+                sd, mean = sd.reshape(shape), mean.reshape(shape)
+            out = ((mean + x * sd) if c.get("invert", False) else ((x - mean) / sd)).astype(np.float32)
         elif cls == "BatchNormalization":
             axis = c["axis"][0] if isinstance(c["axis"], list) else c["axis"]
             x = ins[0]

@@ -469,3 +469,41 @@ def test_decoder_model_with_transposed_convolutions(fdx, oracle, modelgen):
     errs = [rel(g, w) for g, w in zip(got, want)]
     say("  rel errors:", ["%.2e" % e for e in errs])
     assert max(errs) <= TOL
+
+
+def test_model_with_rescaling_normalization_and_passthrough_layers(fdx, oracle, modelgen):
+    """Preprocessing layers in front of a small CNN: Rescaling (one pair), Normalization on the channel axis (plain
+    and inverted), axis-less Normalization, augmentation layers that pass their input through; the Normalization behind
+    a convolution folds into it, the one behind an activation runs as its own launch."""
+    say("Rescaling / Normalization / passthrough model")
+    b = modelgen.Builder("prep_cnn", 92)
+    img = b.input((12, 10, 3), "img")
+    x = b.rescaling(img, "scale", 1 / 127.5, -1.0)
+    x = b._add("RandomFlip", "flip", {}, [x], x.shape)
+    x = b._add("RandAugment", "ra", {}, [x], x.shape)
+    x = b.normalization(x, "norm", axis=-1)
+    c = b.conv2d(x, 8, 3, "c1", padding="same", bias_std=0.1)
+    c = b.normalization(c, "norm_folded", axis=-1)
+    c = b.relu(c, "r1")
+    c = b.normalization(c, "norm_alone", axis=3, invert=True)
+    c = b.normalization(c, "norm_all", axis=None)
+    seq = b.input((7, 6), "seq")
+    s = b.normalization(seq, "norm_seq", axis=-1)
+    s = b.rescaling(s, "scale_seq", -0.5, 3.0)
+    js = modelgen.dumps(b.finish([c, s]))
+    r = np.random.default_rng(23)
+    xi = r.uniform(0, 255, (5, 12, 10, 3)).astype(np.float32)
+    xs = r.standard_normal((5, 7, 6)).astype(np.float32)
+    ref = oracle.OracleModel(js)
+    want = [ref.predict([xi[i], xs[i]]) for i in range(5)]
+    want = [np.stack([w[k] for w in want]) for k in range(2)]
+    got = fdx.Model(js).predict([xi, xs])
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        assert rel(g, w) <= TOL
+    # on another axis than the last the launch is refused, not approximated
+    b2 = modelgen.Builder("prep_bad", 93)
+    x2 = b2.input((4, 5, 6), "x")
+    y2 = b2.normalization(x2, "n", axis=2)
+    with pytest.raises(Exception, match="last axis"):
+        fdx.Model(modelgen.dumps(b2.finish([y2]))).predict([np.zeros((1, 4, 5, 6), np.float32)])

@@ -246,3 +246,41 @@ def test_upsampling_vs_torch_interpolate(oracle):
         assert np.array_equal(oracle.upsample2d(x, fy, fx), near.astype(np.float32))
         bil = torch.nn.functional.interpolate(xt, scale_factor=(fy, fx), mode="bilinear", align_corners=False)[0]
         assert rel(oracle.upsample2d(x, fy, fx, bilinear=True), bil.permute(1, 2, 0).numpy()) <= 2e-6
+
+
+def test_rescaling_normalization_and_passthrough_layers(oracle, modelgen):
+    """Rescaling and Normalization pinned by what the arithmetic fixes: statistics taken from the data itself give
+    zero mean / unit variance per slice; the inverted layer undoes the plain one; an axis-less layer uses one pair;
+    a variance of zero divides by the 1e-7 floor (layers/normalization_layer.hpp:38-45); augmentation layers pass
+    their input through (import_model.hpp:1796-1838)."""
+    r = np.random.default_rng(31)
+    x = (r.standard_normal((6, 5, 4)) * 3 + 2).astype(np.float32)
+    b = modelgen.Builder("prep", 31)
+    xin = b.input(x.shape, "x")
+    y0 = b.rescaling(xin, "scale", 1 / 127.5, -1.0)
+    y1 = b.normalization(xin, "norm_c", axis=-1)
+    y2 = b.normalization(y1, "denorm_c", axis=-1, invert=True)
+    y3 = b.normalization(xin, "norm_w", axis=2)
+    y4 = b.normalization(xin, "norm_all", axis=None)
+    y5 = b._add("RandomHue", "aug", {}, [xin], x.shape)
+    y5 = b._add("Pipeline", "aug2", {}, [y5], x.shape)
+    b.params["norm_c"] = {"mean": x.mean((0, 1)), "variance": x.var((0, 1))}
+    b.params["denorm_c"] = dict(b.params["norm_c"])
+    b.params["norm_w"] = {"mean": x.mean((0, 2)), "variance": np.zeros(5, np.float32)}
+    b.params["norm_all"] = {"mean": np.array([2.5], np.float32), "variance": np.array([4.0], np.float32)}
+    out = oracle.OracleModel(modelgen.dumps(b.finish([y0, y1, y2, y3, y4, y5]))).predict([x])
+    assert np.allclose(out[0], x.astype(np.float64) / 127.5 - 1.0, atol=1e-6)
+    assert np.abs(out[1].mean((0, 1))).max() < 1e-5 and np.abs(out[1].var((0, 1)) - 1).max() < 1e-4
+    assert rel(out[2], x) < 1e-6
+    want3 = (x.astype(np.float64) - x.mean((0, 2)).astype(np.float64)[None, :, None]) / 1e-7
+    assert rel(out[3], want3) < 1e-5
+    assert rel(out[4], (x.astype(np.float64) - 2.5) / 2.0) < 1e-6
+    assert np.array_equal(out[5], x)
+    # two axes are refused, as in the reference (layers/normalization_layer.hpp:32)
+    bad = modelgen.Builder("bad", 1)
+    xb = bad.input((3, 4), "x")
+    yb = bad.normalization(xb, "n", axis=-1)
+    spec = bad.finish([yb])
+    [l for l in spec["architecture"]["config"]["layers"] if l["name"] == "n"][0]["config"]["axis"] = [1, 2]
+    with pytest.raises(Exception):
+        oracle.OracleModel(modelgen.dumps(spec)).predict([np.zeros((3, 4), np.float32)])
