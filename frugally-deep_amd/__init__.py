@@ -173,6 +173,23 @@ def dwconv2d(x, w_chw, bias, strides=(1, 1), dilation=(1, 1), padding="valid", a
     return out.to_host((n, g["out_h"], g["out_w"], c))
 
 
+def dwconv_pointwise(x, dw_w_chw, dw_bias, stride, padding, dw_act, pw_w_nc, pw_bias, residual=None, act=None):
+    """Depthwise 3x3 then 1x1 convolution in one launch.  x [n,h,w,c]; dw_w_chw [c,3,3]; pw_w_nc [n_out,c]."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, wd, c = x.shape
+    g = window_geometry(h, wd, 3, 3, stride, stride, padding)
+    n_out = pw_w_nc.shape[0]
+    dx, dw = DevBuf.from_host(x), DevBuf.from_host(np.transpose(dw_w_chw, (1, 2, 0)))
+    db = None if dw_bias is None else DevBuf.from_host(dw_bias)
+    pw, pb = DevBuf.from_host(pw_w_nc), (None if pw_bias is None else DevBuf.from_host(pw_bias))
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * n_out)
+    check(lib.fdx_dwconv_pointwise_nhwc_f32(_dp(dx), n, h, wd, c, _dp(dw), _dp(db), stride, g["pad_top"], g["pad_left"],
+                                            g["out_h"], g["out_w"], _act_ref(dw_act), _dp(pw), _dp(pb), n_out, _dp(dr),
+                                            _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], n_out))
+
+
 def gemm(a, b_nk, bias=None, alpha=1.0, bias_per_row=False, residual=None, act=None):
     a, b_nk = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b_nk, np.float32)
     m, k = a.shape

@@ -1194,6 +1194,24 @@ namespace {
                 }
             }
         }
+        // last: depthwise 3x3 convolutions whose only consumer is a 1x1 convolution (the second half of an
+        // inverted-residual block, a SeparableConv2D) are marked; whether the pair runs as one launch is decided per plan
+        // by timing both forms
+        static const bool dwpw_on = [] { const char* e = std::getenv("FDX_DWPW"); return !(e && e[0] == '0'); }();
+        for (size_t i = 0; dwpw_on && i < m.ops.size(); ++i) {
+            Op& c = m.ops[i];
+            if (c.dead || c.kind != OpKind::Conv2D || c.kh != 1 || c.kw != 1 || c.sy != 1 || c.sx != 1 || c.softmax
+                || c.zp[0] || c.zp[1] || c.zp[2] || c.zp[3] || c.in.empty())
+                continue;
+            Op& d = m.ops[c.in[0]];
+            if (d.dead || d.kind != OpKind::DWConv2D || d.kh != 3 || d.kw != 3 || d.dy != 1 || d.dx != 1 || d.sy != d.sx
+                || d.consumers != 1 || d.softmax || d.residual >= 0 || d.fused_into >= 0 || c.residual == c.in[0])
+                continue;
+            if (!fdx_dwconv_pointwise_supported(d.cout, c.cout, d.sy))
+                continue;
+            c.fuse_dw = c.in[0];
+            d.fused_into = (int)i;
+        }
     }
 
     fdx_status upload(fdx_model& m)
@@ -1529,6 +1547,7 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->block_of.assign(n, -1);
     p->last_use.assign(n, -1);
     p->temps.assign(n, {});
+    p->dw_fused.assign(n, 0);
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -1542,6 +1561,9 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
             p->last_use[root[i]] = (int)pos;
         if (o.residual >= 0)
             p->last_use[root[o.residual]] = (int)pos;
+        if (o.fuse_dw >= 0) // run as one launch, the pair reads the depthwise convolution's input here
+            for (int i : m->ops[o.fuse_dw].in)
+                p->last_use[root[i]] = (int)pos;
     }
     for (int o : m->outputs)
         p->last_use[root[o]] = 1 << 30;
@@ -1994,12 +2016,89 @@ namespace {
         }
     }
 
+    // The depthwise 3x3 convolution in front of 1x1 convolution `idx` and that convolution as one launch.
+    fdx_status run_dw_fused(fdx_model& m, Plan& p, int idx)
+    {
+        const Op& c = m.ops[idx];
+        const Op& d = m.ops[c.fuse_dw];
+        const Shape& is = p.shapes[d.in[0]];
+        if (is.size() != 3)
+            return FDX_ERR_UNSUPPORTED;
+        const int h = (int)is[0], w = (int)is[1], ch = (int)is[2];
+        int g[6];
+        fdx_status st = window(h, w, d, true, g);
+        if (st != FDX_OK)
+            return st;
+        const fdx_act a1 = to_c(d.act), a2 = to_c(c.act);
+        return fdx_dwconv_pointwise_nhwc_f32(p.out[d.in[0]], p.batch, h, w, ch, d.dw[0], d.dw[1], d.sy, g[0] + d.zp[0], g[2] + d.zp[2],
+            g[4], g[5], d.act.kind == FDX_ACT_NONE ? nullptr : &a1, c.dw[0], c.dw[1], c.cout,
+            c.residual >= 0 ? p.out[c.residual] : nullptr, c.act.kind == FDX_ACT_NONE ? nullptr : &a2, p.out[idx]);
+    }
+
+    // First execution of a plan: both forms of the pair are timed on the real operands (either leaves the same result
+    // in the convolution's output buffer) and the plan remembers the faster one.
+    fdx_status choose_dw_fusion(fdx_model& m, Plan& p, int idx)
+    {
+        const int dw_idx = m.ops[idx].fuse_dw;
+        fdx_status st = run_op(m, p, dw_idx);
+        if (st == FDX_OK)
+            st = run_op(m, p, idx);
+        if (st != FDX_OK)
+            return st;
+        p.dw_fused[idx] = 2;
+        if (run_dw_fused(m, p, idx) != FDX_OK) // a shape the launcher does not take: two launches it is
+            return FDX_OK;
+        hipEvent_t e0, e1;
+        if (hipEventCreate(&e0) != hipSuccess)
+            return FDX_OK;
+        if (hipEventCreate(&e1) != hipSuccess) {
+            (void)hipEventDestroy(e0);
+            return FDX_OK;
+        }
+        float ms[2] = { 1e30f, 1e30f };
+        for (int form = 0; form < 2 && st == FDX_OK; ++form) {
+            for (int round = 0; round < 2 && st == FDX_OK; ++round) {
+                (void)hipEventRecord(e0, stream());
+                for (int r = 0; r < 3 && st == FDX_OK; ++r) {
+                    if (form == 0) {
+                        st = run_op(m, p, dw_idx);
+                        if (st == FDX_OK)
+                            st = run_op(m, p, idx);
+                    } else
+                        st = run_dw_fused(m, p, idx);
+                }
+                (void)hipEventRecord(e1, stream());
+                float t = 1e30f;
+                if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess && t < ms[form])
+                    ms[form] = t;
+            }
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        if (st == FDX_OK && ms[1] < ms[0])
+            p.dw_fused[idx] = 1;
+        static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
+        if (log_picks)
+            std::fprintf(stderr, "[fdx tune] %s + %s: two launches %.1f us, one launch %.1f us\n", m.ops[dw_idx].name.c_str(),
+                m.ops[idx].name.c_str(), ms[0] * 1e3f / 3, ms[1] * 1e3f / 3);
+        return st;
+    }
+
     fdx_status execute(fdx_model& m, Plan& p)
     {
         for (int idx : p.order) {
-            if (m.ops[idx].dead)
+            const Op& o = m.ops[idx];
+            if (o.dead)
                 continue;
-            fdx_status st = run_op(m, p, idx);
+            fdx_status st = FDX_OK;
+            if (o.fused_into >= 0 && p.dw_fused[o.fused_into] != 2)
+                continue; // absorbed by (or timed together with) the 1x1 convolution behind it
+            if (o.fuse_dw >= 0 && p.dw_fused[idx] == 0)
+                st = choose_dw_fusion(m, p, idx);
+            else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 1)
+                st = run_dw_fused(m, p, idx);
+            else
+                st = run_op(m, p, idx);
             if (st != FDX_OK)
                 return st;
         }

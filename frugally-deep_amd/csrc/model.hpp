@@ -31,6 +31,8 @@ struct Op {
     std::string name, cls;
     std::vector<int> in; // producer op indices
     int residual = -1;   // op whose output is added in the producer's epilogue
+    int fuse_dw = -1;    // 1x1 Conv2D: the depthwise 3x3 op in front of it that one launch can absorb (fdx_dwconv_pointwise_nhwc_f32)
+    int fused_into = -1; // that depthwise op: the convolution which may absorb it
     bool dead = false;
     int consumers = 0;
 
@@ -86,6 +88,7 @@ struct Plan {
     std::vector<int> last_use;   // position in order of the last consumer
     std::vector<Block> blocks;
     std::vector<std::vector<float*>> temps; // per op: scratch placed at plan time
+    std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = one launch, 2 = two
     double flops = 0;
     ~Plan();
 };

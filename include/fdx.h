@@ -122,6 +122,23 @@ fdx_status fdx_dwconv2d_nhwc_f32(const float* in, int n, int h, int w, int c,
     const fdx_act* act, float* out);
 
 /*
+ * Depthwise 3x3 convolution (stride 1 or 2 in both directions, no dilation) followed by a 1x1 convolution, as one
+ * launch whose intermediate tensor stays on the chip:
+ *   mid[y][x][c]  = dw_act(dw_bias[c] + sum_taps dw_weights_hwc[fy][fx][c] * in[y*s - pad_top + fy][x*s - pad_left + fx][c])
+ *   out[y][x][o]  = act(pw_bias[o] + sum_c pw_weights_nc[o][c] * mid[y][x][c] + residual[y][x][o])
+ * replaces depthwise_convolve (include/fdeep/depthwise_convolution.hpp:21-99) followed by convolve with a 1x1 filter
+ * (include/fdeep/convolution.hpp:398-429), the pair a SeparableConv2D is made of
+ * (include/fdeep/layers/separable_conv_2d_layer.hpp:26-55) and the second half of an inverted-residual block
+ * (DepthwiseConv2D, folded BatchNormalization, ReLU6, Conv2D 1x1).  Same results as the two launches up to the
+ * summation order of the 1x1 product.  Needs c % 4 == 0, n_out <= 96, both activations NONE / RELU / GELU;
+ * fdx_dwconv_pointwise_supported answers that without launching (FDX_ERR_UNSUPPORTED otherwise).
+ */
+int fdx_dwconv_pointwise_supported(int c, int n_out, int stride);
+fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int h, int w, int c, const float* dw_weights_hwc,
+    const float* dw_bias, int stride, int pad_top, int pad_left, int out_h, int out_w, const fdx_act* dw_act,
+    const float* pw_weights_nc, const float* pw_bias, int n_out, const float* residual, const fdx_act* act, float* out);
+
+/*
  * Row-major GEMM with fused epilogue, fp32 MFMA:
  *   c[m][n] = act(alpha * sum_k a[m][k] * b_nk[n][k] + bias + residual[m][n])
  * replaces dense_layer::apply_impl (include/fdeep/layers/dense_layer.hpp:76-86; weights arrive

@@ -128,6 +128,52 @@ def test_dwconv_vs_oracle(fdx, oracle, case):
     assert rel(got6, want6) <= TOL
 
 
+@pytest.mark.parametrize("case", [
+    # n, h, w, c, n_out, stride, padding: the three tile forms (<= 32, <= 96, more channels), widths that are not a
+    # multiple of a run of 8, one-column images, channel counts that end inside a slab, 1..3 column tiles
+    (2, 9, 8, 32, 16, 1, "same"), (2, 12, 11, 96, 24, 2, "same"), (1, 14, 14, 144, 24, 1, "same"),
+    (2, 7, 7, 192, 32, 1, "same"), (1, 15, 13, 64, 96, 2, "valid"), (1, 5, 1, 8, 4, 1, "same"), (3, 3, 3, 4, 5, 2, "valid"),
+    (1, 10, 17, 40, 33, 1, "valid"), (2, 6, 9, 20, 70, 1, "same"), (1, 28, 28, 160, 64, 1, "same"), (2, 17, 16, 36, 96, 2, "same"),
+    (4, 56, 56, 144, 32, 2, "same")])
+def test_dwconv_pointwise_vs_oracle(fdx, oracle, case):
+    """Depthwise 3x3 + ReLU6 + 1x1 convolution (+ residual) in one launch against the oracle's two layers."""
+    n, h, w, c, n_out, stride, padding = case
+    say("dwconv_pointwise", case)
+    r = rng_for("dwpw", case)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    wd = r.standard_normal((c, 3, 3)).astype(np.float32) * 0.5
+    bd = r.standard_normal(c).astype(np.float32)
+    wp = (r.standard_normal((n_out, c)) / np.sqrt(c)).astype(np.float32)
+    bp = r.standard_normal(n_out).astype(np.float32)
+    mid = [oracle.relu(oracle.depthwise_conv2d(x[i], wd, bd, 3, 3, (stride, stride), (1, 1), padding), 6.0, 0.0, 0.0) for i in range(n)]
+    # 1x1 filter in converted-JSON order [cout][1][1][cin] is the [n_out][c] matrix itself
+    want = np.stack([oracle.conv2d(m, oracle.conv2d_prepare(wp.reshape(-1), n_out, 1, 1, c), bp, n_out, 1, 1) for m in mid])
+    got = fdx.dwconv_pointwise(x, wd, bd, stride, padding, fdx.relu_act(6.0), wp, bp)
+    assert got.shape == want.shape
+    assert rel(got, want) <= TOL
+    res = r.standard_normal(want.shape).astype(np.float32)
+    got_r = fdx.dwconv_pointwise(x, wd, None, stride, padding, None, wp, None, residual=res, act=fdx.relu_act())
+    mid0 = [oracle.depthwise_conv2d(x[i], wd, None, 3, 3, (stride, stride), (1, 1), padding) for i in range(n)]
+    want_r = np.stack([oracle.relu(oracle.conv2d(m, oracle.conv2d_prepare(wp.reshape(-1), n_out, 1, 1, c), None, n_out, 1, 1) + res[i])
+                       for i, m in enumerate(mid0)])
+    assert rel(got_r, want_r) <= TOL
+
+
+def test_dwconv_pointwise_rejects_what_it_does_not_cover(fdx):
+    x = np.zeros((1, 4, 4, 6), np.float32)
+    with pytest.raises(RuntimeError):
+        fdx.dwconv_pointwise(x, np.zeros((6, 3, 3), np.float32), None, 1, "same", None, np.zeros((8, 6), np.float32), None)
+    x = np.zeros((1, 4, 4, 8), np.float32)
+    with pytest.raises(RuntimeError):
+        fdx.dwconv_pointwise(x, np.zeros((8, 3, 3), np.float32), None, 1, "same", None, np.zeros((100, 8), np.float32), None)
+    assert fdx.lib.fdx_dwconv_pointwise_supported(32, 16, 1) == 1 and fdx.lib.fdx_dwconv_pointwise_supported(32, 16, 3) == 0
+    # the 1x1 filter has to fit the LDS
+    assert fdx.lib.fdx_dwconv_pointwise_supported(192, 32, 1) == 1 and fdx.lib.fdx_dwconv_pointwise_supported(576, 96, 1) == 0
+    x = np.zeros((1, 4, 4, 576), np.float32)
+    with pytest.raises(RuntimeError):
+        fdx.dwconv_pointwise(x, np.zeros((576, 3, 3), np.float32), None, 1, "same", None, np.zeros((96, 576), np.float32), None)
+
+
 @pytest.mark.parametrize("case", [(2, 8, 8, 5, 2, 2, "valid"), (2, 9, 7, 4, 3, 2, "same"), (1, 9, 7, 3, 3, 2, "valid"),
                                   (2, 5, 5, 64, 2, 1, "same"), (1, 7, 10, 6, 3, 3, "same")])
 @pytest.mark.parametrize("mode", ["max", "avg"])
