@@ -51,6 +51,26 @@ __device__ __forceinline__ float apply_act(float x, const Act& a)
     return x;
 }
 
+// The same for a block of values, with the switch on the kind outside the element loop and a branch-free ReLU that
+// keeps the order of the tests above (x >= max first, then x >= threshold).  Per element, apply_act's tests become
+// exec-mask branches, which in a short kernel can cost more instructions than the arithmetic around them.
+template <int COUNT>
+__device__ __forceinline__ void apply_act_block(float (&v)[COUNT], const Act& a)
+{
+    if (a.kind == FDX_ACT_RELU) {
+#pragma unroll
+        for (int z = 0; z < COUNT; ++z) {
+            const float x = v[z];
+            const float low = x >= a.threshold ? x : a.negative_slope * (x - a.threshold);
+            v[z] = x >= a.max_value ? a.max_value : low;
+        }
+    } else if (a.kind == FDX_ACT_GELU) {
+#pragma unroll
+        for (int z = 0; z < COUNT; ++z)
+            v[z] = 0.5f * v[z] * (1.0f + erff(v[z] * 0.70710678118654752440f));
+    }
+}
+
 // every activation kind (stand-alone activation kernel only; the epilogues keep the two-way switch above
 // so that the GEMM kernels do not carry transcendental code they never run)
 __device__ __forceinline__ float apply_act_full(float x, const Act& a)

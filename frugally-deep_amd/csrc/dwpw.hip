@@ -36,26 +36,6 @@ constexpr int DWPW_TX = 4;    // output pixels per run
 constexpr int DWPW_KC = 32;   // channels per slab
 constexpr int DWPW_AS = DWPW_KC + 4; // padded LDS row: conflict-free 128-bit fragment reads
 
-// Activation of a block of values with the switch on its kind outside the element loop (apply_act's per-element
-// branches cost more instructions here than the stencil itself); the ReLU form is branch-free and keeps the reference's
-// order of tests: x >= max first, then x >= threshold (include/fdeep/layers/relu_layer.hpp:40-46).
-template <int COUNT>
-__device__ __forceinline__ void act_block(float (&v)[COUNT], const Act& a)
-{
-    if (a.kind == FDX_ACT_RELU) {
-#pragma unroll
-        for (int z = 0; z < COUNT; ++z) {
-            const float x = v[z];
-            const float low = x >= a.threshold ? x : a.negative_slope * (x - a.threshold);
-            v[z] = x >= a.max_value ? a.max_value : low;
-        }
-    } else if (a.kind == FDX_ACT_GELU) {
-#pragma unroll
-        for (int z = 0; z < COUNT; ++z)
-            v[z] = 0.5f * v[z] * (1.0f + erff(v[z] * 0.70710678118654752440f));
-    }
-}
-
 // Every wave works on its own: a tile of 8 runs of 4 consecutive output pixels (32 GEMM rows), one stencil item
 // (run, 4 channels) per lane and 32-channel slab, its own A slab in LDS, its own accumulators.  Only the 1x1 filter is
 // shared: the whole [N][c] matrix sits in LDS for the lifetime of the workgroup (zero-padded to whole slabs and column
@@ -150,7 +130,7 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
                         for (int v = 0; v < 4; ++v)
                             o[j * 4 + v] += col[j * STRIDE + fx][v] * wv[fy * 3 + fx][v];
             }
-            act_block(o, p.act1);
+            apply_act_block(o, p.act1);
             // rows of pixels beyond the row end, of runs beyond the last and of channels beyond the last are zero (an
             // activation may map 0 to something else)
 #pragma unroll
@@ -207,7 +187,7 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
                     if (p.residual && rx0 + e < p.ow)
                         v[e] += p.residual[base + (int64_t)e * p.N];
                 }
-                act_block(v, p.act2);
+                apply_act_block(v, p.act2);
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (rx0 + e < p.ow)

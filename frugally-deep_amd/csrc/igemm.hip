@@ -236,18 +236,24 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParam
         const float bcol = (p.bias && !p.bias_per_row) ? p.bias[n] : 0.f;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
+            float r[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + wm * WTM + i * 32 + 8 * (e >> 2) + 4 * fh + (e & 3);
+                r[e] = acc[i][j][e] * p.alpha + bcol;
                 if (m < p.M) {
-                    float v = acc[i][j][e] * p.alpha + bcol;
                     if (p.bias && p.bias_per_row)
-                        v += p.bias[m];
-                    const int64_t off = (int64_t)m * p.ldc + n;
+                        r[e] += p.bias[m];
                     if (R)
-                        v += R[off];
-                    C[off] = apply_act(v, p.act);
+                        r[e] += R[(int64_t)m * p.ldc + n];
                 }
+            }
+            apply_act_block(r, p.act);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (e >> 2) + 4 * fh + (e & 3);
+                if (m < p.M)
+                    C[(int64_t)m * p.ldc + n] = r[e];
             }
         }
     }

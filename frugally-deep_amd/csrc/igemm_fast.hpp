@@ -391,10 +391,12 @@ void igemm_fast_kernel(GemmParams p)
                 if (m < p.M && n_ok) {
                     f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
                     const int64_t off = (int64_t)m * p.ldc + n;
+                    float r[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        v[e] = apply_act(v[e] * p.alpha + bias4[e] + rr[ps][e], p.act);
-                    *reinterpret_cast<f32x4*>(C + off) = v;
+                        r[e] = v[e] * p.alpha + bias4[e] + rr[ps][e];
+                    apply_act_block(r, p.act);
+                    *reinterpret_cast<f32x4*>(C + off) = f32x4 { r[0], r[1], r[2], r[3] };
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -89,11 +89,9 @@ __global__ void dwconv_kernel(const float* __restrict__ in, const float* __restr
         }
         float* op = out + (((int64_t)img * oh + oy) * ow + ox) * c + c0;
         if (VEC == 4) {
-            f32x4 r;
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                r[v] = apply_act(acc[v], act);
-            *reinterpret_cast<f32x4*>(op) = r;
+            float r[4] = { acc[0], acc[1], acc[2], acc[3] };
+            apply_act_block(r, act);
+            *reinterpret_cast<f32x4*>(op) = f32x4 { r[0], r[1], r[2], r[3] };
         } else {
             op[0] = apply_act(acc[0], act);
         }
@@ -153,15 +151,17 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const float* __restrict_
                         acc[j][v] += col[j * STRIDE + fx][v] * wv[fy * 3 + fx][v];
         }
         float* op = out + (((int64_t)img * oh + oy) * ow + ox0) * c + c0;
+        float r[TX * 4];
 #pragma unroll
         for (int j = 0; j < TX; ++j)
-            if (ox0 + j < ow) {
-                f32x4 r;
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    r[v] = apply_act(acc[j][v], act);
-                *reinterpret_cast<f32x4*>(op + (int64_t)j * c) = r;
-            }
+            for (int v = 0; v < 4; ++v)
+                r[j * 4 + v] = acc[j][v];
+        apply_act_block(r, act);
+#pragma unroll
+        for (int j = 0; j < TX; ++j)
+            if (ox0 + j < ow)
+                *reinterpret_cast<f32x4*>(op + (int64_t)j * c) = f32x4 { r[j * 4], r[j * 4 + 1], r[j * 4 + 2], r[j * 4 + 3] };
     }
 }
 
@@ -261,11 +261,9 @@ __global__ void add_kernel(const float* __restrict__ a, const float* __restrict_
         if (VEC == 4) {
             const f32x4 x = reinterpret_cast<const f32x4*>(a)[i];
             const f32x4 y = reinterpret_cast<const f32x4*>(b)[b_count == count ? i : i % (b_count / 4)];
-            f32x4 r;
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                r[v] = apply_act(x[v] + y[v], act);
-            reinterpret_cast<f32x4*>(out)[i] = r;
+            float r[4] = { x[0] + y[0], x[1] + y[1], x[2] + y[2], x[3] + y[3] };
+            apply_act_block(r, act);
+            reinterpret_cast<f32x4*>(out)[i] = f32x4 { r[0], r[1], r[2], r[3] };
         } else {
             out[i] = apply_act(a[i] + b[b_count == count ? i : i % b_count], act);
         }
