@@ -384,20 +384,25 @@ void igemm_fast_kernel(GemmParams p)
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // all rows of the band are finished in registers before the first of them is stored: the wait for the
+            // residual loads would otherwise also wait, pass after pass, for the store of the pass before
+            f32x4 done[32 / RPS];
 #pragma unroll
             for (int ps = 0; ps < 32 / RPS; ++ps) {
                 const int row = ps * RPS + srow;
-                const int m = em0 + wm * WTM + i * 32 + row;
-                if (m < p.M && n_ok) {
-                    f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
-                    const int64_t off = (int64_t)m * p.ldc + n;
-                    float r[4];
+                const f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
+                float r[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        r[e] = v[e] * p.alpha + bias4[e] + rr[ps][e];
-                    apply_act_block(r, p.act);
-                    *reinterpret_cast<f32x4*>(C + off) = f32x4 { r[0], r[1], r[2], r[3] };
-                }
+                for (int e = 0; e < 4; ++e)
+                    r[e] = v[e] * p.alpha + bias4[e] + rr[ps][e];
+                apply_act_block(r, p.act);
+                done[ps] = f32x4 { r[0], r[1], r[2], r[3] };
+            }
+#pragma unroll
+            for (int ps = 0; ps < 32 / RPS; ++ps) {
+                const int m = em0 + wm * WTM + i * 32 + ps * RPS + srow;
+                if (m < p.M && n_ok)
+                    *reinterpret_cast<f32x4*>(C + (int64_t)m * p.ldc + n) = done[ps];
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
