@@ -41,7 +41,9 @@ constexpr int DWPW_AS = DWPW_KC + 4; // padded LDS row: conflict-free 128-bit fr
 // shared: the whole [N][c] matrix sits in LDS for the lifetime of the workgroup (zero-padded to whole slabs and column
 // tiles), loaded once.  Without workgroup barriers in the loop the waves of a CU drift apart and cover each other's
 // load latency, as in the stand-alone depthwise kernel.
-template <int STRIDE, int CT>
+// B_LDS = false: the filter is too large for the LDS; every wave then takes its B fragments of a slab straight from
+// memory (the filter is a few hundred KB, read by every tile: it stays in L2), requested ahead of the slab's taps.
+template <int STRIDE, int CT, bool B_LDS>
 __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
 {
     constexpr int TX = DWPW_TX, COLS = (TX - 1) * STRIDE + 3, KC = DWPW_KC, AS = DWPW_AS;
@@ -49,17 +51,20 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int fr = lane & 31, fh = lane >> 5;
     const int c = p.c, BS = p.c_pad + 4;
-    float* Bs = lds;                                  // [CT * 32][c_pad + 4]
-    float* As = lds + CT * 32 * BS + wave * (32 * AS); // this wave's [32][KC + 4]
+    float* Bs = lds;                                  // [CT * 32][c_pad + 4] (B_LDS only)
+    float* As = lds + (B_LDS ? CT * 32 * BS : 0) + wave * (32 * AS); // this wave's [32][KC + 4]
 
-    for (int idx = t; idx < CT * 32 * (p.c_pad / 4); idx += 256) {
-        const int nrow = idx / (p.c_pad / 4), ch = (idx % (p.c_pad / 4)) * 4;
-        f32x4 w4 = { 0.f, 0.f, 0.f, 0.f };
-        if (nrow < p.N && ch < c)
-            w4 = *reinterpret_cast<const f32x4*>(p.pw_w + (int64_t)nrow * c + ch);
-        *reinterpret_cast<f32x4*>(&Bs[nrow * BS + ch]) = w4;
+    if (B_LDS) {
+        for (int idx = t; idx < CT * 32 * (p.c_pad / 4); idx += 256) {
+            const int nrow = idx / (p.c_pad / 4), ch = (idx % (p.c_pad / 4)) * 4;
+            f32x4 w4 = { 0.f, 0.f, 0.f, 0.f };
+            if (nrow < p.N && ch < c)
+                w4 = *reinterpret_cast<const f32x4*>(p.pw_w + (int64_t)nrow * c + ch);
+            *reinterpret_cast<f32x4*>(&Bs[nrow * BS + ch]) = w4;
+        }
+        __syncthreads();
     }
-    __syncthreads();
+    const __amdgpu_buffer_rsrc_t srd_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.pw_w), 0, p.N * c * 4, 0x00020000);
 
     constexpr uint32_t OOB = 0x80000000u; // beyond any extent the host accepts
     const __amdgpu_buffer_rsrc_t srd_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.in), 0, (int)p.in_bytes, 0x00020000);
@@ -100,6 +105,18 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
                 acc[i][e] = 0.f;
 
         for (int c_base = 0; c_base < c; c_base += KC) {
+            // (filter fragments of this slab first: loads return in order, and the product needs them last)
+            f32x4 bw[B_LDS ? 1 : CT * (KC / 8)];
+            if (!B_LDS) {
+#pragma unroll
+                for (int i = 0; i < CT; ++i)
+#pragma unroll
+                    for (int k8 = 0; k8 < KC / 8; ++k8) {
+                        const int nrow = i * 32 + fr, ch = c_base + k8 * 8 + fh * 4;
+                        const uint32_t vo = (nrow < p.N && ch < c) ? (uint32_t)(nrow * c + ch) * 4u : OOB;
+                        bw[i * (KC / 8) + k8] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_w, (int)vo, 0, 0));
+                    }
+            }
             const int c0 = c_base + 4 * q;
             const bool c_ok = c0 < c;
             const int cw = c_ok ? c0 : 0; // filter taps and bias of a quad beyond the last channel: any valid address, unused
@@ -146,7 +163,8 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
                 const f32x4 af = *reinterpret_cast<const f32x4*>(&As[fr * AS + k8 * 8 + fh * 4]);
 #pragma unroll
                 for (int i = 0; i < CT; ++i) {
-                    const f32x4 bf = *reinterpret_cast<const f32x4*>(&Bs[(i * 32 + fr) * BS + c_base + k8 * 8 + fh * 4]);
+                    const f32x4 bf = B_LDS ? *reinterpret_cast<const f32x4*>(&Bs[(i * 32 + fr) * BS + c_base + k8 * 8 + fh * 4])
+                                           : bw[B_LDS ? 0 : i * (KC / 8) + k8];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[e], bf[e], acc[i], 0, 0, 0);
@@ -210,10 +228,13 @@ static int64_t dwpw_resident(K kernel, size_t lds)
     return (int64_t)per_cu * cus;
 }
 
-static size_t dwpw_lds_bytes(int c, int n_out)
+// LDS of a workgroup: the waves' A slabs, plus the whole 1x1 filter where that still leaves room for a second workgroup
+static size_t dwpw_lds_bytes(int c, int n_out, bool* filter_in_lds)
 {
     const int c_pad = (c + DWPW_KC - 1) / DWPW_KC * DWPW_KC, ct = (n_out + 31) / 32;
-    return sizeof(float) * ((size_t)ct * 32 * (c_pad + 4) + 4 * 32 * DWPW_AS);
+    const size_t slabs = sizeof(float) * 4 * 32 * DWPW_AS, filter = sizeof(float) * (size_t)ct * 32 * (c_pad + 4);
+    *filter_in_lds = slabs + filter <= 64 * 1024;
+    return slabs + (*filter_in_lds ? filter : 0);
 }
 
 static bool al16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -224,9 +245,8 @@ using namespace fdx;
 
 extern "C" int fdx_dwconv_pointwise_supported(int c, int n_out, int stride)
 {
-    // the whole 1x1 filter has to fit the LDS next to the waves' slabs, with room for a second workgroup on the CU
     return c > 0 && c % 4 == 0 && n_out > 0 && n_out <= DWPW_NP && (stride == 1 || stride == 2)
-        && dwpw_lds_bytes(c, n_out) <= 64 * 1024;
+        && (int64_t)n_out * c * 4 < (1LL << 31);
 }
 
 extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int h, int w, int c, const float* dw_weights_hwc,
@@ -236,8 +256,7 @@ extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int 
     FDX_REQUIRE(in && dw_weights_hwc && pw_weights_nc && out, "dwconv_pointwise: null pointer");
     FDX_REQUIRE(n > 0 && h > 0 && w > 0 && out_h > 0 && out_w > 0, "dwconv_pointwise: bad shape");
     if (!fdx_dwconv_pointwise_supported(c, n_out, stride)) {
-        set_error("dwconv_pointwise: needs channels %% 4 == 0, at most %d output channels, stride 1 or 2 and a 1x1 filter that fits the LDS",
-            DWPW_NP);
+        set_error("dwconv_pointwise: needs channels %% 4 == 0, at most %d output channels and stride 1 or 2", DWPW_NP);
         return FDX_ERR_UNSUPPORTED;
     }
     FDX_REQUIRE_EPILOGUE_ACT(dw_act);
@@ -259,16 +278,24 @@ extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int 
     p.act1 = make_act(dw_act);
     p.act2 = make_act(act);
     const int ct = (n_out + 31) / 32;
-    const size_t lds = dwpw_lds_bytes(c, n_out);
+    bool in_lds = false;
+    const size_t lds = dwpw_lds_bytes(c, n_out, &in_lds);
     const int64_t tiles = ((int64_t)p.runs + 7) / 8;
     // persistent waves: exactly the workgroups that are resident at once (a second round would run on a part of the chip)
     const int64_t want = (tiles + 3) / 4;
     profile_begin();
+#define FDX_DWPW_L(S_, CT_, L_)                                                                              \
+    {                                                                                                        \
+        const int64_t resident = dwpw_resident(dwpw_kernel<S_, CT_, L_>, lds);                               \
+        const unsigned grid = (unsigned)(want < resident ? want : resident);                                 \
+        hipLaunchKernelGGL((dwpw_kernel<S_, CT_, L_>), dim3(grid), dim3(256), lds, stream(), p);             \
+    }
 #define FDX_DWPW(S_, CT_)                                                                                    \
     {                                                                                                        \
-        const int64_t resident = dwpw_resident(dwpw_kernel<S_, CT_>, lds);                                   \
-        const unsigned grid = (unsigned)(want < resident ? want : resident);                                 \
-        hipLaunchKernelGGL((dwpw_kernel<S_, CT_>), dim3(grid), dim3(256), lds, stream(), p);                 \
+        if (in_lds)                                                                                          \
+            FDX_DWPW_L(S_, CT_, true)                                                                        \
+        else                                                                                                 \
+            FDX_DWPW_L(S_, CT_, false)                                                                       \
     }
     if (stride == 1) {
         if (ct == 1) FDX_DWPW(1, 1) else if (ct == 2) FDX_DWPW(1, 2) else FDX_DWPW(1, 3)
@@ -276,6 +303,7 @@ extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int 
         if (ct == 1) FDX_DWPW(2, 1) else if (ct == 2) FDX_DWPW(2, 2) else FDX_DWPW(2, 3)
     }
 #undef FDX_DWPW
+#undef FDX_DWPW_L
     const double pix_in = (double)n * h * w, pix_out = (double)n * out_h * out_w;
     profile_end("dwconv_pointwise_f32", 2.0 * pix_out * c * n_out,
         4.0 * (pix_in * c + pix_out * n_out * (residual ? 2.0 : 1.0) + 9.0 * c + (double)n_out * c));
