@@ -1521,6 +1521,16 @@ namespace {
 
 } // namespace
 
+// test hook: -1 = a plan times both forms of a depthwise + 1x1 pair, 0 = always two launches, 1 = always one
+static int g_force_dw_fusion = -1;
+
+extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
+{
+    FDX_REQUIRE(mode >= -1 && mode <= 1, "fdx_debug_force_dw_fusion: mode must be -1, 0 or 1");
+    g_force_dw_fusion = mode;
+    return FDX_OK;
+}
+
 fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out)
 {
     for (size_t i = 0; i < m->plans.size(); ++i)
@@ -1547,7 +1557,7 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->block_of.assign(n, -1);
     p->last_use.assign(n, -1);
     p->temps.assign(n, {});
-    p->dw_fused.assign(n, 0);
+    p->dw_fused.assign(n, g_force_dw_fusion < 0 ? 0 : (g_force_dw_fusion ? 1 : 2));
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -2095,9 +2105,15 @@ namespace {
                 continue; // absorbed by (or timed together with) the 1x1 convolution behind it
             if (o.fuse_dw >= 0 && p.dw_fused[idx] == 0)
                 st = choose_dw_fusion(m, p, idx);
-            else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 1)
+            else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 1) {
                 st = run_dw_fused(m, p, idx);
-            else
+                if (st == FDX_ERR_UNSUPPORTED) { // forced by a test on a pair the launcher does not take
+                    p.dw_fused[idx] = 2;
+                    st = run_op(m, p, m.ops[idx].fuse_dw);
+                    if (st == FDX_OK)
+                        st = run_op(m, p, idx);
+                }
+            } else
                 st = run_op(m, p, idx);
             if (st != FDX_OK)
                 return st;

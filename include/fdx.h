@@ -377,9 +377,12 @@ fdx_status fdx_session_length(const fdx_session* s, int* len);
  *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; + 100 * splits
  *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
  *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
+ *   fdx_debug_force_dw_fusion: how plans built from now on run a depthwise 3x3 convolution and the 1x1 convolution behind
+ *     it: -1 = timed once per plan (the default), 0 = always two launches, 1 = one launch wherever the pair qualifies.
  */
 fdx_status fdx_debug_force_tile(int cfg);
 fdx_status fdx_debug_persist_cap(int workgroups);
+fdx_status fdx_debug_force_dw_fusion(int mode);
 
 #ifdef __cplusplus
 }

@@ -104,6 +104,28 @@ def test_mobilenet_v2_truncated(fdx, oracle, modelgen):
     run_both(fdx, oracle, modelgen, spec, [x])
 
 
+@pytest.mark.parametrize("mode", [1, 0])
+def test_depthwise_pointwise_pairs_forced_either_way(fdx, oracle, modelgen, mode):
+    """The depthwise 3x3 + 1x1 pairs of inverted-residual blocks (stride 1 and 2 with the folded ZeroPadding2D, folded
+    BatchNormalization, ReLU6 in between, residual Add behind) and of SeparableConv2D, forced to run as one launch each
+    and as two: both must match the oracle.  (Left to itself a plan times both forms and keeps the faster.)"""
+    say("depthwise + pointwise pairs, forced fusion mode", mode)
+    spec = modelgen.mobilenet_v2(seed=25, input_size=64, classes=20, random_bn=True, truncate=11)
+    x = np.random.default_rng(18).uniform(0, 1, (5, 64, 64, 3)).astype(np.float32)
+    b = modelgen.Builder("sep", 26)
+    img = b.input((13, 11, 8), "img")
+    s1 = b.separable_conv2d(img, 24, 3, "sep1", padding="same", activation="relu")
+    s2 = b.separable_conv2d(s1, 10, 3, "sep2", strides=2, padding="valid", use_bias=False)
+    sep = b.finish([s2])
+    xs = np.random.default_rng(19).standard_normal((3, 13, 11, 8)).astype(np.float32)
+    fdx.check(fdx.lib.fdx_debug_force_dw_fusion(mode))
+    try:
+        run_both(fdx, oracle, modelgen, spec, [x])
+        run_both(fdx, oracle, modelgen, sep, [xs])
+    finally:
+        fdx.check(fdx.lib.fdx_debug_force_dw_fusion(-1))
+
+
 def test_encoder_small(fdx, oracle, modelgen):
     say("encoder")
     spec = modelgen.encoder(seed=23, layers=2, seq=24, d_model=64, heads=4, ffn=128, bias_std=0.1, random_affine=True)
