@@ -59,7 +59,7 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
     f32x4 acc = { 0.f, 0.f, 0.f, 0.f };
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
-        const float pr = slot + 16 * u < len ? expf(sc[u] - m) : 0.f;
+        const float pr = slot + 16 * u < len ? __expf(sc[u] - m) : 0.f; // as the prefill kernel: the hardware exponential, relative error ~1e-7
         sum += pr;
 #pragma unroll
         for (int e = 0; e < 4; ++e)

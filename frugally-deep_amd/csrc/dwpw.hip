@@ -10,6 +10,9 @@
 // The reference computes the two layers one after the other: depthwise_convolve
 // (include/fdeep/depthwise_convolution.hpp:21-99), the activation layer, convolve (include/fdeep/convolution.hpp:398-429);
 // SeparableConv2D is the same pair without anything in between (include/fdeep/layers/separable_conv_2d_layer.hpp:26-55).
+#include <map>
+#include <mutex>
+
 #include "common.hpp"
 #include "igemm_params.hpp"
 
@@ -215,17 +218,23 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
     }
 }
 
+// workgroups of `kernel` with `lds` bytes of dynamic LDS that are resident at once (remembered per LDS size: one static
+// table per kernel instantiation; launches are serialised by the caller's stream order, the table by this mutex)
 template <typename K>
 static int64_t dwpw_resident(K kernel, size_t lds)
 {
+    static std::mutex mu;
+    static std::map<size_t, int64_t> known;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = known.find(lds);
+    if (it != known.end())
+        return it->second;
     int per_cu = 1, dev = 0;
     hipDeviceProp_t prop;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds) != hipSuccess || per_cu < 1)
         per_cu = 1;
-    static int cus = 0;
-    if (cus == 0)
-        cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
-    return (int64_t)per_cu * cus;
+    const int cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+    return known[lds] = (int64_t)per_cu * cus;
 }
 
 // LDS of a workgroup: the waves' A slabs, plus the whole 1x1 filter where that still leaves room for a second workgroup
