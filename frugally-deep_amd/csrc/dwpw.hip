@@ -1,7 +1,7 @@
 // Depthwise 3x3 convolution fused into the pointwise (1x1) convolution that consumes it, gfx950.
 //
 // An inverted-residual block writes its widest tensor twice and reads it twice: the expanded activations go
-// expand -> HBM -> depthwise -> HBM -> projection.  Here the depthwise result never reaches memory: a workgroup
+// expand -> HBM -> depthwise -> HBM -> projection.  Here the depthwise result never reaches memory: a wave
 // computes the depthwise outputs of a tile of pixels for a slab of channels straight into LDS (the A operand),
 // multiplies them by the matching slab of the 1x1 filter on fp32 MFMA, and walks the channel slabs with the
 // projection's accumulators in registers.  Traffic: input once (plus the cache-served 3x3 neighbourhood), output
