@@ -31,6 +31,7 @@ struct DwPwParams {
     int runs;           // n * oh * xt (the host keeps it below 2^31: 32-bit index arithmetic in the kernel)
     int c_pad;          // c rounded up to the channel slab
     uint32_t in_bytes;  // extent of the input tensor (below 2^31)
+    uint32_t out_bytes; // extent of the output tensor and of the residual (below 2^31)
     Act act1, act2;
 };
 
@@ -70,6 +71,9 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
     const __amdgpu_buffer_rsrc_t srd_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.pw_w), 0, p.N * c * 4, 0x00020000);
 
     constexpr uint32_t OOB = 0x80000000u; // beyond any extent the host accepts
+    const __amdgpu_buffer_rsrc_t srd_out = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)p.out_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srd_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual ? p.residual : p.out), 0,
+        (int)p.out_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t srd_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.in), 0, (int)p.in_bytes, 0x00020000);
     const int run_local = lane >> 3, q = lane & 7; // stencil item of this lane: run of the tile, channel quad of the slab
     const int tiles = (p.runs + 7) / 8;
@@ -178,42 +182,50 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
 
         // ---- epilogue.  32x32 accumulator layout: element e of lane l is row 8*(e/4) + 4*(l/32) + e%4, column l%32;
         // a row is pixel e%4 of run 2*(e/4) + l/32 of the tile.
+        // Output and residual through buffer resources too: an element outside the tensor (column beyond N, pixel beyond
+        // the row end, run beyond the last) gets an out-of-range offset, which the hardware drops (store) or answers with
+        // zero (load) -- no branch per element.
+        // this lane's four runs are two apart: one division for the first, carries for the rest
+        int line0 = (int)((unsigned)(tile * 8 + fh) / (unsigned)p.xt); // img * oh + oy
+        int xr0 = tile * 8 + fh - line0 * p.xt;
+        uint32_t pix_off[4]; // byte offset of (run g, pixel 0, column 0), OOB for a run beyond the last
+        int px_left[4];      // pixels of run g inside the row
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if (g > 0) {
+                xr0 += 2;
+                while (xr0 >= p.xt) {
+                    xr0 -= p.xt;
+                    ++line0;
+                }
+            }
+            const bool r_ok = tile * 8 + 2 * g + fh < p.runs;
+            pix_off[g] = (uint32_t)((line0 * p.ow + xr0 * TX) * p.N) * 4u;
+            px_left[g] = r_ok ? p.ow - xr0 * TX : 0;
+        }
 #pragma unroll
         for (int i = 0; i < CT; ++i) {
             const int ncol = i * 32 + fr;
-            if (ncol >= p.N)
-                continue;
-            const float bcol = p.pw_b ? p.pw_b[ncol] : 0.f;
-            // this lane's four runs are two apart: one division for the first, carries for the rest
-            int line = (int)((unsigned)(tile * 8 + fh) / (unsigned)p.xt); // img * oh + oy
-            int xr = tile * 8 + fh - line * p.xt;
+            const bool n_ok = ncol < p.N;
+            const float bcol = (p.pw_b && n_ok) ? p.pw_b[ncol] : 0.f;
+            float v[16];
+            uint32_t off[16];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int r = tile * 8 + 2 * g + fh;
-                if (g > 0) {
-                    xr += 2;
-                    while (xr >= p.xt) {
-                        xr -= p.xt;
-                        ++line;
-                    }
-                }
-                if (r >= p.runs)
-                    continue;
-                const int rx0 = xr * TX;
-                const int64_t base = ((int64_t)line * p.ow + rx0) * p.N + ncol;
-                float v[4];
+            for (int g = 0; g < 4; ++g)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    v[e] = acc[i][g * 4 + e] + bcol;
-                    if (p.residual && rx0 + e < p.ow)
-                        v[e] += p.residual[base + (int64_t)e * p.N];
+                    off[g * 4 + e] = (n_ok && e < px_left[g]) ? pix_off[g] + (uint32_t)(e * p.N + ncol) * 4u : OOB;
+                    v[g * 4 + e] = acc[i][g * 4 + e] + bcol;
                 }
-                apply_act_block(v, p.act2);
+            if (p.residual) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (rx0 + e < p.ow)
-                        p.out[base + (int64_t)e * p.N] = v[e];
+                for (int z = 0; z < 16; ++z)
+                    v[z] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srd_res, (int)off[z], 0, 0));
             }
+            apply_act_block(v, p.act2);
+#pragma unroll
+            for (int z = 0; z < 16; ++z)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[z]), srd_out, (int)off[z], 0, 0);
         }
     }
 }
@@ -284,6 +296,8 @@ extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int 
     p.c_pad = (c + DWPW_KC - 1) / DWPW_KC * DWPW_KC;
     FDX_REQUIRE((int64_t)n * h * w * c * 4 < (1LL << 31), "dwconv_pointwise: input tensor beyond 2 GiB");
     p.in_bytes = (uint32_t)((int64_t)n * h * w * c * 4);
+    FDX_REQUIRE((int64_t)n * out_h * out_w * n_out * 4 < (1LL << 31), "dwconv_pointwise: output tensor beyond 2 GiB");
+    p.out_bytes = (uint32_t)((int64_t)n * out_h * out_w * n_out * 4);
     p.act1 = make_act(dw_act);
     p.act2 = make_act(act);
     const int ct = (n_out + 31) / 32;
