@@ -89,7 +89,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParam
     }
     // conv k-state of this thread's quarter: input channel, filter column, filter row
     int kc = 0, kfx = 0, kfy = 0;
-    if (A_MODE == A_CONV_VEC) {
+    if (A_MODE == A_CONV_VEC || A_MODE == A_CONV_SCALAR) {
         const int kk = kq * 4, tap = kk / p.Cin;
         kc = kk - tap * p.Cin;
         kfy = tap / p.kw;
@@ -127,23 +127,31 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParam
                 if (a_ok[i] && kfy < p.kh && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W)
                     v = *reinterpret_cast<const f32x4*>(a_ptr[i] + ((int64_t)(iy * p.W + ix) * p.Cin + kc));
             } else {
+                // the quarter's four k values one by one, (channel, filter column, filter row) carried along instead of
+                // divided out of k for every element (two integer divisions per loaded float made the 3-channel stem
+                // convolutions instruction-bound); k < K is the same as filter row < kh
                 if (a_ok[i]) {
+                    int c = kc, fx = kfx, fy = kfy;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const int kk = k + j;
-                        if (kk < p.K) {
-                            const int tap = kk / p.Cin, c = kk - tap * p.Cin;
-                            const int fy = tap / p.kw, fx = tap - fy * p.kw;
+                        if (fy < p.kh) {
                             const int iy = a_iy0[i] + fy * p.dy, ix = a_ix0[i] + fx * p.dx;
                             if (iy >= 0 && iy < p.H && ix >= 0 && ix < p.W)
                                 v[j] = a_ptr[i][(int64_t)(iy * p.W + ix) * p.Cin + c];
+                        }
+                        if (++c == p.Cin) {
+                            c = 0;
+                            if (++fx == p.kw) {
+                                fx = 0;
+                                ++fy;
+                            }
                         }
                     }
                 }
             }
             ra[i] = v;
         }
-        if (A_MODE == A_CONV_VEC) { // advance the quarter's (fy, fx, c) by one slab
+        if (A_MODE == A_CONV_VEC || A_MODE == A_CONV_SCALAR) { // advance the quarter's (fy, fx, c) by one slab
             kc += BK;
             while (kc >= p.Cin) {
                 kc -= p.Cin;
