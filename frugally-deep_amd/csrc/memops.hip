@@ -108,16 +108,17 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const float* __restrict_
     int oh, int ow, Act act)
 {
     constexpr int COLS = (TX - 1) * STRIDE + 3;
-    const int cv = c / 4, xt = (ow + TX - 1) / TX;
-    const int64_t total = (int64_t)n * oh * xt * cv;
-    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
-         idx += (int64_t)gridDim.x * blockDim.x) {
-        const int cq = (int)(idx % cv);
-        int64_t rest = idx / cv;
-        const int ox0 = (int)(rest % xt) * TX;
-        rest /= xt;
-        const int oy = (int)(rest % oh);
-        const int img = (int)(rest / oh);
+    const unsigned cv = (unsigned)c / 4, xt = (unsigned)(ow + TX - 1) / TX;
+    // item index in 32 bits (the host launches this kernel only below 2^31 items): a 64-bit division costs several
+    // times the arithmetic of an item
+    const unsigned total = (unsigned)n * (unsigned)oh * xt * cv;
+    for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        unsigned rest = idx / cv;
+        const int cq = (int)(idx - rest * cv);
+        unsigned rest2 = rest / xt;
+        const int ox0 = (int)(rest - rest2 * xt) * TX;
+        const int img = (int)(rest2 / (unsigned)oh);
+        const int oy = (int)(rest2 - (unsigned)img * (unsigned)oh);
         const int c0 = cq * 4;
         f32x4 wv[9];
 #pragma unroll
@@ -585,7 +586,8 @@ extern "C" fdx_status fdx_dwconv2d_nhwc_f32(const float* in, int n, int h, int w
     const bool vec = c % 4 == 0 && al16(in) && al16(weights_hwc) && al16(out);
     const size_t items = (size_t)n * out_h * out_w * (vec ? c / 4 : c);
     profile_begin();
-    const bool k3 = vec && kh == 3 && kw == 3 && dy == 1 && dx == 1 && sy == sx && (sy == 1 || sy == 2) && (!bias || al16(bias));
+    const bool k3 = vec && kh == 3 && kw == 3 && dy == 1 && dx == 1 && sy == sx && (sy == 1 || sy == 2) && (!bias || al16(bias))
+        && (uint64_t)n * out_h * ((out_w + 3) / 4) * (c / 4) < (1ull << 31); // 32-bit item index in the 3x3 kernel
     if (k3 && sy == 1)
         hipLaunchKernelGGL((dwconv3x3_kernel<1, 8>), dim3(grid_for((size_t)n * out_h * ((out_w + 7) / 8) * (c / 4), 256)), dim3(256), 0,
             stream(), in, weights_hwc, bias, out, n, h, w, c, pad_top, pad_left, out_h, out_w, a);
