@@ -323,6 +323,8 @@ static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStrea
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), 0, s, q);
 }
 
+#include "pw_stream.hpp"
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // library-owned scratch of the split-K variant: partial tiles and one ticket per output tile
@@ -469,8 +471,11 @@ static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range p
 
 // general_cfg >= 0: the general kernel's configuration for this shape competes too (narrow outputs, where half of a
 // 64-wide fast tile is idle); general_launch runs it once on the caller's unshifted parameters
-template <typename F>
-static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s, int general_cfg, F general_launch)
+// stream_ok: the row-streaming short-K kernel (configuration 30, pw_stream.hpp) competes as well
+constexpr int kStreamCfg = 30;
+template <typename F, typename G>
+static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s, int general_cfg, F general_launch,
+    bool stream_ok, G stream_launch)
 {
     if (g_autotune < 0) {
         const char* e = std::getenv("FDX_AUTOTUNE");
@@ -551,6 +556,14 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
             best = general_cfg;
         }
     }
+    if (stream_ok) {
+        stream_launch();
+        const float ms = timed(stream_launch);
+        if (ms < best_ms) {
+            best_ms = ms;
+            best = kStreamCfg;
+        }
+    }
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
     static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
@@ -611,9 +624,16 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
     };
     if (cfg >= 100)
         unpack();
-    if (cfg >= 10 && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
+    const bool stream_ok = pw_stream_ok(p, conv, batch, a_bytes, b_bytes) && b_vec;
+    if (cfg == kStreamCfg && !stream_ok)
+        cfg = -1;
+    if (cfg >= 10 && cfg != kStreamCfg && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
         cfg = -1;
     if (cfg < 10 || mode > 2) {
+        splits = 1;
+        mode = 0;
+    }
+    if (cfg == kStreamCfg) {
         splits = 1;
         mode = 0;
     }
@@ -640,7 +660,8 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             // fast path can read this operand
             const bool general_ok = p.N < 64 && p.a_valid_k == 0 && !(conv && p.pix_stride != p.Cin);
             const int general_cfg = !general_ok ? -1 : p.N <= 32 ? 2 : (blocks(128, 64) >= 512 ? 1 : 3);
-            cfg = autotune(q, conv, batch, unit, s, general_cfg, [&] { launch_general(general_cfg); });
+            cfg = autotune(q, conv, batch, unit, s, general_cfg, [&] { launch_general(general_cfg); }, stream_ok,
+                [&] { pw_stream_launch(p, a_bytes, b_bytes, s); });
             if (cfg >= 100)
                 unpack();
         }
@@ -674,7 +695,9 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         return FDX_ERR_INVALID;
     }
     profile_begin();
-    if (cfg >= 10) {
+    if (cfg == kStreamCfg) {
+        pw_stream_launch(p, a_bytes, b_bytes, s);
+    } else if (cfg >= 10) {
         GemmParams q = p;
         q.A = p.A - a_shift;
         q.a_records = (uint32_t)a_bytes;

@@ -374,7 +374,8 @@ fdx_status fdx_session_length(const fdx_session* s, int* len);
  * Test hooks (no counterpart in the reference; process-wide, meant for one thread): the parity tests use them to drive
  * every tile configuration and scheduling form of the convolution / GEMM kernels on small problems, where the tuner
  * would never pick them.
- *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; + 100 * splits
+ *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; 30 = the row-streaming
+ *     kernel for K <= 128 (where it does not apply the tuner decides); + 100 * splits
  *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
  *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
  *   fdx_debug_force_dw_fusion: how plans built from now on run a depthwise 3x3 convolution and the 1x1 convolution behind

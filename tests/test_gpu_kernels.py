@@ -80,11 +80,35 @@ def test_conv2d_epilogue_residual_relu(fdx, oracle):
     assert rel(got, want) <= TOL
 
 
+@pytest.mark.parametrize("m,n,k", [(1000, 96, 16), (33, 144, 24), (4096, 192, 32), (257, 960, 96), (64, 4, 8), (31, 33, 128),
+                                   (500, 256, 64), (129, 576, 96), (70, 100, 40)])
+def test_row_streaming_gemm_short_k(fdx, oracle, m, n, k):
+    """The row-streaming kernel for K <= 128 (tile configuration 30), forced: rows and columns that end inside a
+    32-wide group, every epilogue operand, k counts that fill the register blocks only partly."""
+    say("row-streaming gemm", m, n, k)
+    r = rng_for("pws", m, n, k)
+    a = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    b = r.standard_normal(n).astype(np.float32)
+    res = r.standard_normal((m, n)).astype(np.float32)
+    ref = a.astype(np.float64) @ w.astype(np.float64).T
+    fdx.lib.fdx_debug_force_tile(30)
+    try:
+        got = fdx.gemm(a, w, None)
+        got_full = fdx.gemm(a, w, b, alpha=0.75, residual=res, act=fdx.relu_act(6.0))
+        got_gelu = fdx.gemm(a, w, b, act=fdx.gelu_act())
+    finally:
+        fdx.lib.fdx_debug_force_tile(-1)
+    assert rel(got, ref) <= TOL
+    assert rel(got_full, np.clip(0.75 * ref + b + res, 0.0, 6.0)) <= TOL
+    assert rel(got_gelu, oracle.gelu((ref + b).astype(np.float32))) <= TOL
+
+
 GEMM_CASES = [(1, 10, 32), (16, 768, 768), (37, 50, 29), (256, 2048, 512), (130, 1000, 2048), (5, 3, 7), (64, 64, 16),
               (300, 96, 100)]
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 17, 18])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 10, 11, 12, 13, 14, 15, 16, 17, 18, 30])
 @pytest.mark.parametrize("m,n,k", GEMM_CASES)
 def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
     say("gemm", m, n, k, "tile", tile)
