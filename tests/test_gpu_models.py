@@ -126,6 +126,30 @@ def test_depthwise_pointwise_pairs_forced_either_way(fdx, oracle, modelgen, mode
         fdx.check(fdx.lib.fdx_debug_force_dw_fusion(-1))
 
 
+def test_mobilenet_v2_full_size_fusion_invariance(fdx, oracle, modelgen):
+    """At the real layer shapes (224x224, all 17 blocks, batch 8): one launch per depthwise + 1x1 pair, two launches per
+    pair and the timed choice give the same features, and one image agrees with the oracle."""
+    say("mobilenet_v2 full size, fused vs two launches")
+    spec = modelgen.mobilenet_v2(seed=27, random_bn=True)
+    spec = with_taps(spec, ["global_average_pooling2d"])
+    x = np.random.default_rng(20).uniform(0, 1, (8, 224, 224, 3)).astype(np.float32)
+    spec = fix_tap_shapes(spec, oracle, modelgen, [x[0]])
+    js = modelgen.dumps(spec)
+    outs = []
+    try:
+        for mode in (1, 0, -1):
+            fdx.check(fdx.lib.fdx_debug_force_dw_fusion(mode))
+            outs.append(fdx.Model(js, verify=False).predict([x]))
+    finally:
+        fdx.check(fdx.lib.fdx_debug_force_dw_fusion(-1))
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert rel(a, b) <= 1e-5
+    want = oracle.OracleModel(js).predict([x[0]])
+    for g, w in zip(outs[0], want):
+        assert rel(g[0], w) <= TOL
+
+
 def test_encoder_small(fdx, oracle, modelgen):
     say("encoder")
     spec = modelgen.encoder(seed=23, layers=2, seq=24, d_model=64, heads=4, ffn=128, bias_std=0.1, random_affine=True)
