@@ -1,5 +1,6 @@
 // Row-streaming GEMM for short K (K <= 128): C[M][N] = act(alpha * A[M][K] * B[N][K]^T + bias + residual).
-// Included by igemm.hip inside namespace fdx.
+// Included by igemm.hip inside namespace fdx.  One more form of the product behind convolve with a 1x1 filter
+// (include/fdeep/convolution.hpp:398-429) and dense_layer::apply_impl (include/fdeep/layers/dense_layer.hpp:76-86).
 //
 // The pointwise convolutions that widen a tensor (K = 16..128 input channels, N = 96..960 outputs) are one or two K
 // slabs of arithmetic around a large output: the tiled kernel spends its time in tile set-up, LDS staging and barriers
