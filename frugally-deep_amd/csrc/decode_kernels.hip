@@ -50,8 +50,10 @@ struct SkinnyShared {
 
 // The work of workgroup (bx, by) of a (gx, gy) grid.  MEGA: called from the persistent decode-step kernel, where the
 // results must be visible to workgroups on other XCDs after a grid-wide barrier inside the same launch: they are
-// written with agent-scope stores (which pass this XCD's L2); the operands are read with ordinary loads, which is
-// safe there because every buffer of a step is written by one phase and not read before that phase in the same launch.
+// written with agent-scope stores (which pass this XCD's L2); the operands are read with ordinary loads: every buffer
+// of a step is written by one phase and not read before that phase in the same launch, so no cache holds an older
+// copy.  What this takes for granted is that an acknowledged agent-scope store (s_waitcnt vmcnt(0)) is in memory; the
+// persistent kernel has once produced different tokens than the separate launches, so it is not used by default.
 template <int CHUNK, bool SINGLE, bool MEGA>
 __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, int by, int gx, int gy, SkinnyShared& sh)
 {

@@ -1183,8 +1183,9 @@ namespace {
                 continue;
             for (int side = 1; side >= 0; --side) {
                 Op& p = m.ops[add.in[side]];
-                if (is_gemm_like(p) && p.consumers == 1 && p.residual < 0 && !p.softmax && p.act.kind == FDX_ACT_NONE
-                    && !p.dead) {
+                // (an attention op ends in its output projection, a GEMM with the same epilogue)
+                if ((is_gemm_like(p) || p.kind == OpKind::MHA) && p.consumers == 1 && p.residual < 0 && !p.softmax
+                    && p.act.kind == FDX_ACT_NONE && !p.dead) {
                     p.residual = add.in[1 - side];
                     p.act = add.act;
                     add.dead = true;
@@ -1966,7 +1967,7 @@ namespace {
                     || (st = fdx_broadcast_combine_f32(FDX_COMBINE_MUL, merged, flat, gbuf, flat, 0, 1, 1.0f, nullptr, merged, nullptr)) != FDX_OK)
                     return st;
             }
-            st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, B * T, o.dout, (int)nv, 1.f, o.dw[7], 0, nullptr, nullptr, out,
+            st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, B * T, o.dout, (int)nv, 1.f, o.dw[7], 0, res, actp, out,
                 o.dout, nullptr);
             break;
         }

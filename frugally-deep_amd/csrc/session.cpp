@@ -266,7 +266,7 @@ fdx_status run(fdx_session* s, const float* ids_dev, int T, float* logits_dev, f
                 }
             }
             if (st == FDX_OK)
-                st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, (int)R, o.dout, (int)nv, 1.f, o.dw[7], 0, nullptr, nullptr, out, o.dout,
+                st = fdx_gemm_bias_act_f32(merged, nv, o.dw[6], nv, (int)R, o.dout, (int)nv, 1.f, o.dw[7], 0, res, actp, out, o.dout,
                     nullptr);
             break;
         }
@@ -508,10 +508,17 @@ bool build_fast_plan(fdx_session* s)
             std::memset(&og, 0, sizeof og);
             og.X = merged; og.ldx = nv; og.W = o.dw[6]; og.ldw = nv; og.M = B; og.N = o.dout; og.K = nv; og.bias = o.dw[7];
             og.act = Act { FDX_ACT_NONE, 3.402823466e+38f, 0.f, 0.f };
+            if (o.residual >= 0) { // the Add behind the attention was folded into it at load
+                if (lazy_ln[o.residual] >= 0 || !buf[o.residual])
+                    return false;
+                og.residual = buf[o.residual];
+                og.ldr = o.dout;
+                og.act = o.act;
+            }
             bool is_output = false;
             for (int out : m.outputs)
                 is_output = is_output || out == idx;
-            if (!is_output && users[idx].size() == 1) {
+            if (!is_output && users[idx].size() == 1 && o.residual < 0) {
                 const int ai = users[idx][0];
                 const Op& add = m.ops[ai];
                 if (add.kind == OpKind::Add && add.in.size() == 2 && add.in[0] != add.in[1]) {
@@ -599,8 +606,8 @@ bool build_fast_plan(fdx_session* s)
     }
     // With FDX_DECODE_MEGA=1 (read when the session is created) the run of Dense / attention launches between the
     // embedding and the logits launch becomes one persistent kernel, if every one of them has a phase form.  Off by
-    // default: a phase costs 7.9 us against 7.3 us per separate launch on the GPT-2-small shape as long as the next
-    // phase's weights are not requested before the barrier.
+    // default: a phase costs 7.6 us against 7.3 us per separate launch on the GPT-2-small shape, and the exchange between
+    // phases is not verified to the bar of the separate launches (see skinny_gemm_body): for measurement only.
     const char* mega_env = std::getenv("FDX_DECODE_MEGA");
     const bool mega_on = mega_env && mega_env[0] == '1';
     if (mega_on && s->steps.size() >= 4) {
