@@ -15,6 +15,9 @@ namespace fdx {
 void set_error(const char* fmt, ...);
 hipStream_t stream();
 bool profiling();
+// Clears library-owned scratch at set-up time, on the library stream (which does not synchronise with the null
+// stream) and waits for it, so that the first kernel that reads the cells sees zeros.  Not for use inside a stream capture.
+hipError_t zero_device(void* p, size_t bytes);
 // records one launch for the per-kernel profile (flops / bytes are algorithmic figures)
 void profile_begin();
 void profile_end(const char* family, double flops, double bytes);

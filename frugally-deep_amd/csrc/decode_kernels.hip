@@ -944,7 +944,7 @@ static bool ensure_splitk_workspace()
     if (hipMalloc(&g_splitk_ws, sizeof(float) * kSplitWsFloats) != hipSuccess)
         return false;
     if (hipMalloc(&g_splitk_tickets, sizeof(int) * kSplitTickets) != hipSuccess
-        || hipMemset(g_splitk_tickets, 0, sizeof(int) * kSplitTickets) != hipSuccess)
+        || zero_device(g_splitk_tickets, sizeof(int) * kSplitTickets) != hipSuccess)
         return false;
     return true;
 }

@@ -341,7 +341,7 @@ static bool split_prepare()
     if (hipMalloc(&g_split_ws, kSplitWsBytes) != hipSuccess)
         return false;
     if (hipMalloc(&g_split_tickets, sizeof(int) * kSplitTickets) != hipSuccess
-        || hipMemset(g_split_tickets, 0, sizeof(int) * kSplitTickets) != hipSuccess)
+        || zero_device(g_split_tickets, sizeof(int) * kSplitTickets) != hipSuccess)
         return false;
     return true;
 }

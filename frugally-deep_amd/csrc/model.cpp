@@ -1110,6 +1110,28 @@ namespace {
         }
         std::vector<Shape> shapes;
         const bool have_shapes = infer_shapes(m, dummy, shapes, topo_order(m)) == FDX_OK;
+        // Two tensors that agree under one dummy extent need not agree at run time (a variable dimension against a fixed
+        // one of that extent, or two different variable dimensions): an Add only counts as an equal-shape sum if its
+        // operands also agree with every variable dimension at a second extent and, where the graph accepts it, with
+        // every variable dimension at an extent of its own.
+        std::vector<Shape> shapes_b, shapes_c;
+        bool have_b = false, have_c = false;
+        {
+            std::vector<Shape> dummy_b = m.in_decl, dummy_c = m.in_decl;
+            int64_t next = 11;
+            for (size_t i = 0; i < dummy_b.size(); ++i)
+                for (size_t d = 0; d < dummy_b[i].size(); ++d)
+                    if (dummy_b[i][d] < 0) {
+                        dummy_b[i][d] = 7;
+                        dummy_c[i][d] = next;
+                        next += 2;
+                    }
+            have_b = infer_shapes(m, dummy_b, shapes_b, topo_order(m)) == FDX_OK;
+            have_c = infer_shapes(m, dummy_c, shapes_c, topo_order(m)) == FDX_OK;
+        }
+        auto same_shape_always = [&](int x, int y) {
+            return shapes[x] == shapes[y] && have_b && shapes_b[x] == shapes_b[y] && (!have_c || shapes_c[x] == shapes_c[y]);
+        };
 
         count_consumers(m);
         // 1. BatchNormalization on the channel axis into the producing convolution / dense weights
@@ -1179,7 +1201,7 @@ namespace {
             if (add.dead || add.kind != OpKind::Add || add.in.size() != 2 || add.in[0] == add.in[1] || add.combine != FDX_COMBINE_ADD
                 || add.scale != 1.0f)
                 continue;
-            if (shapes[add.in[0]] != shapes[add.in[1]])
+            if (!same_shape_always(add.in[0], add.in[1]))
                 continue;
             for (int side = 1; side >= 0; --side) {
                 Op& p = m.ops[add.in[side]];
@@ -1264,7 +1286,7 @@ namespace {
             o.hw.shrink_to_fit();
         }
         FDX_HIP(hipMalloc(&m.err_flag, sizeof(int)));
-        FDX_HIP(hipMemset(m.err_flag, 0, sizeof(int)));
+        FDX_HIP(zero_device(m.err_flag, sizeof(int)));
         return FDX_OK;
     }
 

@@ -50,6 +50,15 @@ hipStream_t stream()
 }
 bool profiling() { return g_profile; }
 
+hipError_t zero_device(void* p, size_t bytes)
+{
+    hipStream_t s = stream();
+    hipError_t e = hipMemsetAsync(p, 0, bytes, s);
+    if (e != hipSuccess)
+        return e;
+    return hipStreamSynchronize(s);
+}
+
 static hipEvent_t get_event()
 {
     if (!g_event_pool.empty()) {

@@ -340,14 +340,14 @@ bool build_fast_plan(fdx_session* s)
     s->amax = reinterpret_cast<unsigned long long*>(alloc((size_t)2 * B + 4));
     if (!s->ids_buf || !s->amax)
         return false;
-    if (hipMemset(s->amax, 0, sizeof(unsigned long long) * B) != hipSuccess)
+    if (zero_device(s->amax, sizeof(unsigned long long) * B) != hipSuccess)
         return false;
     s->history = alloc((size_t)s->max_len * B);
     if (!s->history || skinny_prepare() != FDX_OK)
         return false;
     s->splitk_ws = alloc((size_t)fdx_session::kWsFloats);
     s->splitk_tickets = reinterpret_cast<int*>(alloc((size_t)fdx_session::kTickets));
-    if (!s->splitk_ws || !s->splitk_tickets || hipMemset(s->splitk_tickets, 0, sizeof(int) * fdx_session::kTickets) != hipSuccess)
+    if (!s->splitk_ws || !s->splitk_tickets || zero_device(s->splitk_tickets, sizeof(int) * fdx_session::kTickets) != hipSuccess)
         return false;
     std::vector<char> skip(m.ops.size(), 0);
     const int ids_op = m.inputs[0], pos_op = m.inputs[1];
@@ -633,7 +633,7 @@ bool build_fast_plan(fdx_session* s)
             s->mega_state = alloc((mega_state_bytes() + 3) / 4);
             if (!s->mega_phases || !s->mega_state
                 || hipMemcpy(s->mega_phases, phases.data(), sizeof(MegaPhase) * phases.size(), hipMemcpyHostToDevice) != hipSuccess
-                || hipMemset(s->mega_state, 0, mega_state_bytes()) != hipSuccess)
+                || zero_device(s->mega_state, mega_state_bytes()) != hipSuccess)
                 return false;
             s->mega_count = (int)phases.size();
             s->mega_first = first;
@@ -785,8 +785,26 @@ extern "C" fdx_status fdx_session_create(fdx_model* m, int batch, int max_len, f
             return FDX_ERR_UNSUPPORTED;
         }
         switch (o.kind) {
-        case OpKind::Input: case OpKind::Embedding: case OpKind::Add: case OpKind::LayerNorm: case OpKind::Act:
-        case OpKind::Softmax: case OpKind::Dense: case OpKind::View:
+        case OpKind::LayerNorm: {
+            // a position is one (1, depth) row of the (T, depth) sample: only statistics over the depth axis keep
+            // positions apart (layers/layer_normalization_layer.hpp:37-63 takes any axis set)
+            const bool last_only = o.target_shape.size() == 1 && (o.target_shape[0] == -1 || o.target_shape[0] == 2);
+            if (!last_only) {
+                set_error("session_create: %s normalises over an axis other than the last; its statistics would mix positions",
+                    o.name.c_str());
+                return FDX_ERR_UNSUPPORTED;
+            }
+            break;
+        }
+        case OpKind::View:
+            // Flatten / Reshape regroup the (T, depth) sample across positions; identity layers carry neither attribute
+            if (o.flatten || !o.target_shape.empty()) {
+                set_error("session_create: %s (%s) reshapes across positions", o.name.c_str(), o.cls.c_str());
+                return FDX_ERR_UNSUPPORTED;
+            }
+            break;
+        case OpKind::Input: case OpKind::Embedding: case OpKind::Add: case OpKind::Act:
+        case OpKind::Softmax: case OpKind::Dense: // softmax runs along depth only (tensor.hpp:1165-1192)
             break;
         case OpKind::MHA: {
             const bool self = o.in[0] == o.in[1] && (o.in.size() == 2 || o.in[2] == o.in[0]);
