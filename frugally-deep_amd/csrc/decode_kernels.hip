@@ -996,6 +996,20 @@ fdx_status argmax_parts_launch(const unsigned long long* amax_parts, int parts, 
     return FDX_OK;
 }
 
+// K ranges per column group of a launch without LayerNorm prologue and pre-packed operand
+static int skinny_ksplit(int K, int tiles)
+{
+    // spread a narrow projection over the chip: a CU pulls only a few tens of GB/s on its own
+    // long K only: below that the ticket exchange costs more than the idle CUs
+    int ksplit = 1;
+    while (ksplit < 8 && K / ksplit > SK_WAVES * SK_CHUNK * 16 && K / (ksplit * 2) >= 128)
+        ksplit *= 2;
+    if (ksplit > 1)
+        while (ksplit < 8 && tiles * ksplit < 192 && K / (ksplit * 2) >= 256)
+            ksplit *= 2;
+    return ksplit;
+}
+
 fdx_status skinny_gemm_launch(const SkinnyParams& p)
 {
     FDX_REQUIRE(p.X && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0, "dense_rows: bad arguments");
@@ -1009,18 +1023,18 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
     // more than one chunk; LayerNorm launches keep whole rows in one workgroup
     int ksplit = 1;
     SkinnyParams q = p;
-    if (!p.ln && !p.packed && ensure_splitk_workspace()) {
-        // spread a narrow projection over the chip: a CU pulls only a few tens of GB/s on its own
-        // long K only: below that the ticket exchange costs more than the idle CUs
-        while (ksplit < 8 && p.K / ksplit > SK_WAVES * SK_CHUNK * 16 && p.K / (ksplit * 2) >= 128)
-            ksplit *= 2;
-        if (ksplit > 1)
-            while (ksplit < 8 && tiles * ksplit < 192 && p.K / (ksplit * 2) >= 256)
-                ksplit *= 2;
-        if ((int64_t)tiles * ksplit * 256 > kSplitWsFloats || tiles > kSplitTickets)
+    // the caller's workspace (the entry point that allocates nothing brings its own) or the library's, allocated on first use
+    const bool own_ws = p.workspace && p.tickets;
+    if (!p.ln && !p.packed && (own_ws || ensure_splitk_workspace())) {
+        const int64_t ws_floats = own_ws ? p.workspace_floats : kSplitWsFloats;
+        const int ticket_count = own_ws ? p.ticket_count : kSplitTickets;
+        ksplit = skinny_ksplit(p.K, tiles);
+        if ((int64_t)tiles * ksplit * 256 > ws_floats || tiles > ticket_count)
             ksplit = 1;
-        q.workspace = g_splitk_ws;
-        q.tickets = g_splitk_tickets;
+        if (!own_ws) {
+            q.workspace = g_splitk_ws;
+            q.tickets = g_splitk_tickets;
+        }
     }
     const int per_wg = ((p.K + ksplit * 16 - 1) / (ksplit * 16)) * 16; // as the kernel derives it
     const dim3 grid((unsigned)tiles, (unsigned)ksplit);
@@ -1143,6 +1157,70 @@ extern "C" fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const flo
     p.act = fdx::make_act(act);
     p.n_seg = 1;
     p.seg[0] = { out, n, 0, 0 };
+    return fdx::skinny_gemm_launch(p);
+}
+
+// ---- the Dense entry point that allocates nothing -----------------------------------------------------------------
+// Split-K partial tiles and tickets of fdx_dense_rows_noalloc_f32 live in this file-scope device array instead of
+// memory from hipMalloc: [kNoAllocWsFloats] partial-tile floats, then [kNoAllocTickets] ticket ints.  The GPU holds
+// it (4 MiB + 16 KiB) until the process ends.  Host code never passes the array's name to a kernel: its device
+// address is looked up once, at library set-up, and kept in g_noalloc_ptr.
+namespace fdx {
+constexpr int64_t kNoAllocWsFloats = 1 << 20;
+constexpr int kNoAllocTickets = 4096;
+static __device__ __align__(256) float scratch[kNoAllocWsFloats + kNoAllocTickets];
+static float* g_noalloc_ptr = nullptr; // device address of `scratch` on the library's device
+
+__global__ void clear_ints_kernel(int* p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        p[i] = 0;
+}
+
+// called from the library's set-up (runtime.cpp:ensure_init) with the library's device current
+hipError_t noalloc_setup()
+{
+    (void)wide_resident(); // occupancy query of the wide-output kernel, cached: not to be made inside a capture
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess)
+        return e;
+    g_noalloc_ptr = static_cast<float*>(ptr);
+    return hipSuccess;
+}
+} // namespace fdx
+
+extern "C" fdx_status fdx_dense_rows_noalloc_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
+    const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(x && w_nk && out, "dense_rows_noalloc: null pointer");
+    FDX_REQUIRE(fdx::g_noalloc_ptr, "dense_rows_noalloc: call fdx_init first (the library's set-up looks up the scratch array's address)");
+    FDX_REQUIRE(m > 0 && m <= 16, "dense_rows_noalloc: 1 to 16 rows, got %d", m);
+    FDX_REQUIRE(n > 0 && n <= 16 * fdx::kNoAllocTickets, "dense_rows_noalloc: at most %d output columns, got %d", 16 * fdx::kNoAllocTickets, n);
+    FDX_REQUIRE(k > 0 && k <= 32768, "dense_rows_noalloc: at most 32768 input columns, got %d", k);
+    const int tiles = (n + 15) / 16;
+    const int ksplit = fdx::skinny_ksplit(k, tiles);
+    FDX_REQUIRE((int64_t)tiles * ksplit * 256 <= fdx::kNoAllocWsFloats,
+        "dense_rows_noalloc: %d column groups x %d K ranges exceed the fixed scratch of %lld floats", tiles, ksplit,
+        (long long)fdx::kNoAllocWsFloats);
+    fdx::SkinnyParams p;
+    std::memset(&p, 0, sizeof p);
+    p.X = x; p.ldx = k; p.W = w_nk; p.ldw = k; p.M = m; p.N = n; p.K = k; p.bias = bias; p.residual = residual; p.ldr = n;
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    p.act = fdx::make_act(act);
+    p.n_seg = 1;
+    p.seg[0] = { out, n, 0, 0 };
+    p.workspace = fdx::g_noalloc_ptr;
+    p.workspace_floats = fdx::kNoAllocWsFloats;
+    p.tickets = reinterpret_cast<int*>(fdx::g_noalloc_ptr + fdx::kNoAllocWsFloats);
+    p.ticket_count = fdx::kNoAllocTickets;
+    if (ksplit > 1) {
+        // every call on this GPU shares the array, which keeps the last call's contents: the tickets this launch counts
+        // on start at zero (a fill kernel, not a memset, so that a caller may capture the call)
+        hipLaunchKernelGGL(fdx::clear_ints_kernel, dim3((unsigned)((tiles + 255) / 256)), dim3(256), 0, fdx::stream(), p.tickets, tiles);
+        FDX_LAUNCH_CHECK();
+    }
     return fdx::skinny_gemm_launch(p);
 }
 

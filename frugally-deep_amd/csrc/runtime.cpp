@@ -42,6 +42,7 @@ void set_error(const char* fmt, ...)
 }
 
 fdx_status ensure_init();
+hipError_t noalloc_setup(); // decode_kernels.hip: device address of the scratch array of fdx_dense_rows_noalloc_f32
 hipStream_t stream()
 {
     if (!g_inited)
@@ -127,6 +128,7 @@ fdx_status ensure_init()
     FDX_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     FDX_HIP(hipEventCreate(&g_t0));
     FDX_HIP(hipEventCreate(&g_t1));
+    FDX_HIP(noalloc_setup());
     g_inited = true;
     return FDX_OK;
 }

@@ -162,6 +162,19 @@ fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const float* b_nk,
 fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
     const float* residual, const fdx_act* act, float* out);
 /*
+ * fdx_dense_rows_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arithmetic, same kernels and the
+ * same results as fdx_dense_rows_f32; the split-K partial tiles and tickets it needs for k > 1024 live in a fixed
+ * array of device memory inside the library (4 MiB + 16 KiB per GPU, held until the process ends) instead of a
+ * workspace allocated on first use.  The call makes no hipMalloc / hipFree and uses no allocating library routine.
+ * Needs fdx_init (or any earlier library call) to have run; limits: m <= 16, n <= 65536, k <= 32768 and
+ * ceil(n / 16) * splits * 256 <= 1048576 floats (splits <= 8, chosen from k and n), otherwise FDX_ERR_INVALID with the
+ * reason in fdx_last_error.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (other than
+ * in order on the library's stream) race.
+ */
+fdx_status fdx_dense_rows_noalloc_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
+    const float* residual, const fdx_act* act, float* out);
+/*
  * LayerNormalization followed by Dense in one launch (layers/layer_normalization_layer.hpp:37-63 then
  * layers/dense_layer.hpp:76-86).  fdx_fold_layernorm_f32 prepares, once per layer pair,
  *   w_folded[n][k] = w[n][k] * gamma[k],  w_rowsum[n] = sum_k w_folded[n][k],  bias_folded[n] = bias[n] + sum_k w[n][k] * beta[k]
