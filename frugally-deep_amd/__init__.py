@@ -90,6 +90,23 @@ def _act_ref(act):
     return None if act is None else ctypes.byref(act)
 
 
+def tuner_export():
+    """The per-shape tuning table of this process as text (fdx_tuner_export)."""
+    need = ctypes.c_size_t()
+    check(lib.fdx_tuner_export(None, ctypes.c_size_t(0), ctypes.byref(need)))
+    buf = ctypes.create_string_buffer(need.value)
+    check(lib.fdx_tuner_export(buf, ctypes.c_size_t(need.value), ctypes.byref(need)))
+    return buf.value.decode()
+
+
+def tuner_import(text):
+    check(lib.fdx_tuner_import(text.encode()))
+
+
+def tuner_freeze(on=True):
+    check(lib.fdx_tuner_freeze(1 if on else 0))
+
+
 class DevBuf:
     """Device buffer owned by the library's allocator; holds fp32 (or raw bytes)."""
 

@@ -461,11 +461,30 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
 // `splits` K ranges, 1 = hybrid (only the last partial round is cut), 2 = stream-K (splits unused).  Cutting every tile
 // is tried only where a configuration has few tiles for the chip; the hybrid cut of the last partial round wherever
 // there is one.
-struct TuneKey {
-    int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
-    bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }
-};
+// (TuneKey: igemm_params.hpp; conv = 2 rows hold the one-launch / two-launch choice of a depthwise + 1x1 pair)
 static std::map<TuneKey, int> g_tuned;
+static std::mutex g_tune_mutex; // the table only; never held across a launch
+static bool g_tune_frozen = false;
+
+bool tune_lookup(const TuneKey& key, int* choice)
+{
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    auto it = g_tuned.find(key);
+    if (it == g_tuned.end())
+        return false;
+    *choice = it->second;
+    return true;
+}
+void tune_store(const TuneKey& key, int choice)
+{
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    g_tuned[key] = choice;
+}
+bool tune_frozen()
+{
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    return g_tune_frozen;
+}
 static int g_autotune = -1;
 static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range per tile
 
@@ -489,9 +508,11 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     std::memset(&key, 0, sizeof key);
     key.conv = conv; key.M = q.M; key.N = q.N; key.K = q.K; key.Cin = conv ? q.Cin : 0; key.kh = conv ? q.kh : 0;
     key.kw = conv ? q.kw : 0; key.sy = conv ? q.sy : 0; key.sx = conv ? q.sx : 0; key.batch = batch; key.res = q.residual != nullptr;
-    auto it = g_tuned.find(key);
-    if (it != g_tuned.end())
-        return it->second;
+    int known = -1;
+    if (tune_lookup(key, &known))
+        return known;
+    if (tune_frozen())
+        return -1; // an unseen shape under a frozen table takes the closed rule of run_igemm: no timing, same choice every run
     hipEvent_t a, b;
     if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess)
         return -1;
@@ -574,7 +595,7 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
         best = best_split;
     if (log_picks)
         std::fprintf(stderr, "[fdx tune]   -> %d\n", best);
-    g_tuned[key] = best;
+    tune_store(key, best);
     return best;
 }
 
@@ -907,4 +928,60 @@ extern "C" fdx_status fdx_gemm_bias_act_f32(const float* a, int64_t lda, const f
         p.c_outer = batch->c_outer; p.c_inner = batch->c_inner;
     }
     return run_igemm(p, false, nb, "gemm_f32");
+}
+
+// ---- the tuner's table as text: one line per shape, "conv M N K Cin kh kw sy sx batch res choice"
+extern "C" fdx_status fdx_tuner_export(char* text, size_t capacity, size_t* needed)
+{
+    std::string out;
+    {
+        std::lock_guard<std::mutex> lock(fdx::g_tune_mutex);
+        char line[256];
+        for (const auto& kv : fdx::g_tuned) {
+            const fdx::TuneKey& k = kv.first;
+            std::snprintf(line, sizeof line, "%d %d %d %d %d %d %d %d %d %d %d %d\n", k.conv, k.M, k.N, k.K, k.Cin, k.kh, k.kw, k.sy, k.sx,
+                k.batch, k.res, kv.second);
+            out += line;
+        }
+    }
+    if (needed)
+        *needed = out.size() + 1;
+    if (text && capacity > 0) {
+        FDX_REQUIRE(capacity >= out.size() + 1, "tuner_export: buffer of %zu bytes, %zu needed", capacity, out.size() + 1);
+        std::memcpy(text, out.c_str(), out.size() + 1);
+    }
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_tuner_import(const char* text)
+{
+    FDX_REQUIRE(text, "tuner_import: null text");
+    std::vector<std::pair<fdx::TuneKey, int>> rows;
+    const char* p = text;
+    while (*p) {
+        fdx::TuneKey k;
+        std::memset(&k, 0, sizeof k);
+        int choice = 0, used = 0;
+        const int got = std::sscanf(p, "%d %d %d %d %d %d %d %d %d %d %d %d%n", &k.conv, &k.M, &k.N, &k.K, &k.Cin, &k.kh, &k.kw, &k.sy,
+            &k.sx, &k.batch, &k.res, &choice, &used);
+        if (got <= 0)
+            break; // trailing white space
+        FDX_REQUIRE(got == 12, "tuner_import: malformed line near offset %d", (int)(p - text));
+        FDX_REQUIRE(k.conv >= 0 && k.conv <= 2 && choice >= -1, "tuner_import: value out of range near offset %d", (int)(p - text));
+        rows.emplace_back(k, choice);
+        p += used;
+        while (*p == '\n' || *p == '\r' || *p == ' ')
+            ++p;
+    }
+    std::lock_guard<std::mutex> lock(fdx::g_tune_mutex);
+    for (const auto& r : rows)
+        fdx::g_tuned[r.first] = r.second;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_tuner_freeze(int on)
+{
+    std::lock_guard<std::mutex> lock(fdx::g_tune_mutex);
+    fdx::g_tune_frozen = on != 0;
+    return FDX_OK;
 }

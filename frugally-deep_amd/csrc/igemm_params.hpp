@@ -1,5 +1,6 @@
 // Launch parameters shared by the implicit-GEMM kernels.
 #pragma once
+#include <cstring>
 #include "common.hpp"
 
 namespace fdx {
@@ -38,5 +39,15 @@ struct GemmParams {
     int* split_tickets;
 };
 
+// Key of the per-process tuning table (igemm.hip).  conv = 0 / 1: a GEMM / convolution shape and its tile choice
+// (configuration + 100 * splits + 10000 * mode); conv = 2: a depthwise 3x3 + 1x1 pair (M = height, Cin = width,
+// K = channels, N = filters, sy = stride, res = residual) and whether it runs as one launch (1) or two (2).
+struct TuneKey {
+    int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
+    bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }
+};
+bool tune_lookup(const TuneKey& key, int* choice);
+void tune_store(const TuneKey& key, int choice);
+bool tune_frozen(); // fdx_tuner_freeze(1): shapes not in the table take the closed rules, nothing is timed
 
 } // namespace fdx

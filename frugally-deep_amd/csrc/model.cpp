@@ -17,6 +17,7 @@
 #include <tuple>
 
 #include "einsum.hpp"
+#include "igemm_params.hpp"
 #include "json.hpp"
 
 using namespace fdx;
@@ -2073,6 +2074,34 @@ namespace {
     fdx_status choose_dw_fusion(fdx_model& m, Plan& p, int idx)
     {
         const int dw_idx = m.ops[idx].fuse_dw;
+        // the choice is kept per shape in the tuner's table, so that an exported table pins it too
+        TuneKey key;
+        std::memset(&key, 0, sizeof key);
+        {
+            const Op& c = m.ops[idx];
+            const Op& d = m.ops[dw_idx];
+            const Shape& is = p.shapes[d.in[0]];
+            key.conv = 2;
+            key.M = is.size() == 3 ? (int)is[0] : 0;
+            key.Cin = is.size() == 3 ? (int)is[1] : 0;
+            key.K = is.size() == 3 ? (int)is[2] : 0;
+            key.N = c.cout;
+            key.sy = d.sy;
+            key.batch = p.batch;
+            key.res = c.residual >= 0;
+            int known = 0;
+            if (tune_lookup(key, &known) || tune_frozen()) {
+                p.dw_fused[idx] = known == 1 ? 1 : 2; // frozen and unseen: two launches
+                if (p.dw_fused[idx] == 1) {
+                    const fdx_status fs = run_dw_fused(m, p, idx);
+                    if (fs != FDX_ERR_UNSUPPORTED)
+                        return fs;
+                    p.dw_fused[idx] = 2;
+                }
+                fdx_status st2 = run_op(m, p, dw_idx);
+                return st2 == FDX_OK ? run_op(m, p, idx) : st2;
+            }
+        }
         fdx_status st = run_op(m, p, dw_idx);
         if (st == FDX_OK)
             st = run_op(m, p, idx);
@@ -2110,6 +2139,8 @@ namespace {
         (void)hipEventDestroy(e1);
         if (st == FDX_OK && ms[1] < ms[0])
             p.dw_fused[idx] = 1;
+        if (st == FDX_OK)
+            tune_store(key, p.dw_fused[idx]);
         static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
         if (log_picks)
             std::fprintf(stderr, "[fdx tune] %s + %s: two launches %.1f us, one launch %.1f us\n", m.ops[dw_idx].name.c_str(),

@@ -384,6 +384,19 @@ fdx_status fdx_session_decode_greedy(fdx_session* s, const float* first_ids_dev,
 fdx_status fdx_session_length(const fdx_session* s, int* len);
 
 /*
+ * The per-shape tuning table.  The first launch of a convolution / GEMM shape (and of a depthwise 3x3 + 1x1 pair) times
+ * the candidate kernels once per process and keeps the winner; candidates sum in different orders, so two processes may
+ * return results that differ in the last bits (all within the reference tolerance; the reference itself leaves the
+ * summation order to Eigen, convolution.hpp:134-148).  For bit-identical results run to run, export the table of a
+ * warmed-up process, import it at start-up and freeze it: under a frozen table a shape that is not listed takes a fixed
+ * rule and nothing is timed.  Text format: one line per shape, "conv M N K Cin kh kw sy sx batch res choice".
+ * fdx_tuner_export: `needed` receives the size including the terminator; text may be NULL to query it.
+ */
+fdx_status fdx_tuner_export(char* text, size_t capacity, size_t* needed);
+fdx_status fdx_tuner_import(const char* text);
+fdx_status fdx_tuner_freeze(int on);
+
+/*
  * Test hooks (no counterpart in the reference; process-wide, meant for one thread): the parity tests use them to drive
  * every tile configuration and scheduling form of the convolution / GEMM kernels on small problems, where the tuner
  * would never pick them.

@@ -115,6 +115,35 @@ def test_session_rejects_non_decoder_models_and_overflow(fdx, modelgen):
         sess.decode_step(np.zeros(2))
 
 
+def test_session_rejects_layers_that_mix_positions(fdx, modelgen):
+    """A cached decode step works on one position at a time: LayerNormalization over anything but the depth axis and
+    Flatten / Reshape layers (which regroup the (T, depth) sample) are refused when the session is created, instead of
+    being computed over one position's depth."""
+    say("session: position-mixing layers")
+    import copy
+    base = modelgen.gpt2(seed=40, layers=1, d_model=16, heads=2, vocab=19, max_pos=16)
+    for axis in ([1], [1, 2], [-2]):
+        spec = copy.deepcopy(base)
+        for layer in spec["architecture"]["config"]["layers"]:
+            if layer["name"] == "h0_ln2":
+                layer["config"]["axis"] = axis
+        with pytest.raises(fdx.FdxError, match="axis other than the last"):
+            fdx.Session(fdx.Model(modelgen.dumps(spec), verify=False), 2, 8)
+    for cls, cfg in (("Reshape", {"target_shape": [-1, 16]}), ("Flatten", {})):
+        b = modelgen.Builder("mix", 41)
+        ids, pos = b.input((None,), "ids"), b.input((None,), "positions")
+        x = b.add([b.embedding(ids, 19, 16, "wte"), b.embedding(pos, 16, 16, "wpe")], "embed_add")
+        h = b.layernorm(x, "ln1", 1e-5)
+        h = b.mha(h, h, "attn", 2, 8)
+        x = b.add([x, h], "add1")
+        x = b._add(cls, "regroup", cfg, [x], x.shape)
+        x = b.dense(x, 19, "lm_head")
+        model = fdx.Model(modelgen.dumps(b.finish([x])), verify=False)
+        with pytest.raises(fdx.FdxError, match="reshapes across positions"):
+            fdx.Session(model, 2, 8)
+    fdx.Session(fdx.Model(modelgen.dumps(base), verify=False), 2, 8)  # the unmodified decoder is accepted
+
+
 def test_vocabulary_sized_head_leaves_its_own_argmax(fdx, modelgen):
     """With tens of thousands of logits per row the logits launch strides over the column groups and leaves
     per-workgroup maxima, from which the greedy ids are picked without another pass over the logits: the ids must be
