@@ -52,18 +52,64 @@ def profile_families(fdx):
     return fams
 
 
-def cpu_baseline_resnet(js, x, cores, passes=2):
-    """The oracle (a port of the reference CPU path) timed with one prediction per core in parallel."""
+def host_cores():
+    """Host threads the CPU baseline uses: the cores this process may run on, at most the 16 a one-GPU box grants."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n = os.cpu_count() or 1
+    return max(1, min(n, 16))
+
+
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline_resnet(js, x, cores, warmup=3, passes=5):
+    """The oracle (a port of the reference CPU path) timed with one prediction per core in parallel threads, 3 warm-up
+    and 5 timed passes as the reference's own harness does (test/applications_performance.cpp:59-77)."""
     import fdeep_oracle
     ref = fdeep_oracle.OracleModel(js)
     samples = [x[i % x.shape[0]] for i in range(cores)]
     with concurrent.futures.ThreadPoolExecutor(cores) as pool:
-        list(pool.map(lambda s: ref.predict([s]), samples))  # warm-up pass
+        for _ in range(warmup):
+            list(pool.map(lambda s: ref.predict([s]), samples))
         t0 = time.perf_counter()
         for _ in range(passes):
             list(pool.map(lambda s: ref.predict([s]), samples))
         dt = time.perf_counter() - t0
     return cores * passes / dt
+
+
+def cpu_baseline_decode(js, cores, prompt=4, warmup=3, timed=5):
+    """KV-cached greedy decoding on the CPU oracle, one sequence per core in parallel threads: a short prompt and 3
+    warm-up steps per sequence, then 5 timed steps each (a step streams every weight of the model once per sequence,
+    whatever the context length, so the short context hardly changes its cost)."""
+    import fdeep_oracle
+    ref = fdeep_oracle.OracleModel(js)
+    rng = np.random.default_rng(7)
+    decoders = [fdeep_oracle.CachedDecoder(ref) for _ in range(cores)]
+    state = [int(t) for t in rng.integers(0, 50257, cores)]
+
+    def run(i, steps):
+        tok = state[i]
+        for _ in range(steps):
+            tok = fdeep_oracle.argmax(decoders[i].step(tok))
+        state[i] = tok
+
+    with concurrent.futures.ThreadPoolExecutor(cores) as pool:
+        list(pool.map(lambda i: run(i, prompt + warmup), range(cores)))
+        t0 = time.perf_counter()
+        list(pool.map(lambda i: run(i, timed), range(cores)))
+        dt = time.perf_counter() - t0
+    return cores * timed / dt
 
 
 def bench_resnet(fdx, modelgen, args):
@@ -144,12 +190,23 @@ def bench_resnet(fdx, modelgen, args):
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
         "load_seconds": round(load_s, 2),
     }
+    # what a model.predict caller with host tensors sees: the same batch through fdx_model_predict, host-to-device copy
+    # of the 38.5 MB input and device-to-host copy of the outputs included (pageable host memory)
+    model.predict([x])
+    reps = max(3, args.steps // 4)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        model.predict([x])
+    e2e_s = (time.perf_counter() - t0) / reps
+    result["end_to_end"] = {"value": round(batch / e2e_s, 1), "unit": "img/s", "ms_per_step": round(e2e_s * 1e3, 3),
+                            "what": "fdx_model_predict on host pointers, batch %d: input H2D + forward + output D2H, wall clock" % batch}
     if not args.no_cpu_baseline:
-        cores = min(os.cpu_count() or 1, 16)
+        cores = host_cores()
         cpu = cpu_baseline_resnet(js, x, cores)
         result["cpu_baseline"] = {"value": round(cpu, 3), "unit": "img/s", "cores": cores, "kind": "port",
+                                  "cpu": cpu_model_name(),
                                   "sample": "%d ResNet50 predictions per pass (one per core, in parallel threads), "
-                                            "1 warm-up + 2 timed passes of the CPU oracle" % cores}
+                                            "3 warm-up + 5 timed passes of the CPU oracle" % cores}
     model.close()
     return result
 
@@ -220,6 +277,13 @@ def bench_gpt2(fdx, modelgen, args):
     t0 = time.perf_counter()
     model = fdx.Model(js, verify=False)
     load_s = time.perf_counter() - t0
+    cpu = None
+    if not args.no_cpu_baseline:
+        cores = host_cores()
+        cpu = {"value": round(cpu_baseline_decode(js, cores), 2), "unit": "tok/s", "cores": cores, "kind": "port",
+               "cpu": cpu_model_name(),
+               "sample": "%d sequences (one per core, in parallel threads) on the CPU oracle's KV-cached decoder: 4 prompt + 3 "
+                         "warm-up steps, then 5 timed greedy steps each" % cores}
     del js
     ids = np.random.default_rng(99).integers(0, 50257, (batch, prompt)).astype(np.float32)
     sess = fdx.Session(model, batch, prompt + new)
@@ -255,6 +319,8 @@ def bench_gpt2(fdx, modelgen, args):
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
         "load_seconds": round(load_s, 2),
     }
+    if cpu:
+        out["cpu_baseline"] = cpu
     sess.close()
     model.close()
     return out

@@ -248,11 +248,24 @@ using tensors_vec = std::vector<tensors>;
 
 inline std::string show_tensor(const tensor& t)
 {
-    std::ostringstream os;
-    os.setf(std::ios::fixed);
-    os.precision(4);
+    // every value with four decimals, padded on the left with spaces to the longest of them
+    // (include/fdeep/tensor.hpp:1203-1218), nested by dim5 / dim4 / height / width / depth
     const auto& v = *t.as_vector();
     const auto& s = t.shape();
+    std::vector<std::string> strs;
+    strs.reserve(v.size());
+    std::size_t longest = 0;
+    for (float_type f : v) {
+        std::ostringstream one;
+        one.setf(std::ios::fixed);
+        one.precision(4);
+        one << f;
+        strs.push_back(one.str());
+        longest = std::max(longest, strs.back().size());
+    }
+    for (auto& str : strs)
+        str.insert(0, longest - str.size(), ' ');
+    std::ostringstream os;
     std::size_t i = 0;
     os << "[";
     for (std::size_t d5 = 0; d5 < s.size_dim_5_; ++d5) {
@@ -264,7 +277,7 @@ inline std::string show_tensor(const tensor& t)
                 for (std::size_t x = 0; x < s.width_; ++x) {
                     os << (x ? ", [" : "[");
                     for (std::size_t z = 0; z < s.depth_; ++z)
-                        os << (z ? ", " : "") << v[i++];
+                        os << (z ? ", " : "") << strs[i++];
                     os << "]";
                 }
                 os << "]";

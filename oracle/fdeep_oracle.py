@@ -742,7 +742,8 @@ class _Graph:
                 layer = self.layers[lname]
                 ins = [get(cn) for cn in layer.nodes[node]]
                 if causal and layer.cls == "MultiHeadAttention":
-                    memo[key] = [OracleModel._causal_mha(layer, ins)]
+                    hook = causal if callable(causal) else OracleModel._causal_mha
+                    memo[key] = [hook(layer, ins)]
                 else:
                     memo[key] = [layer.apply(ins)]
             return memo[key][0]
@@ -808,6 +809,7 @@ class OracleModel:
         out = self.predict(inputs)
         return argmax(out[0])
 
+
     def run_embedded_tests(self, eps=1e-4):
         """Replays the file's own test cases, absolute tolerance, NaN == NaN passes.
         include/fdeep/model.hpp:254-267, import_model.hpp:1990-2021"""
@@ -820,3 +822,57 @@ class OracleModel:
                 if bad.any():
                     raise RuntimeError("test failed")
         return True
+
+
+class CachedDecoder:
+    """One sequence decoded token by token with the projected keys / values of every self-attention layer
+    kept between steps: the CPU counterpart of a KV-cache decode session, used as the timed CPU baseline of
+    the decode benchmark and as a second statement of the causal definition.
+
+    Step t feeds (id, position t) through the layer graph as a one-row sample.  Every layer other than
+    attention works on rows independently; a self-attention layer projects the new row with the layer's
+    per-head Dense kernels (multi_head_attention_layer.hpp:47-59: q_w (D, H, dk) read as a Dense kernel
+    [D][H*dk], o_w (H, dv, D) as [H*dv][D]), appends k and v to its cache and evaluates
+    softmax(q K^T * 1/sqrt(dk)) V per head over the cached rows (same file :74-95, scale applied to the
+    scores, softmax in the reference's exp(x - m - log sum) form), which is what the reference computes
+    for MultiHeadAttention(query = x[t:t+1], value = x[0:t+1])."""
+
+    def __init__(self, model):
+        self.model = model
+        self.cache = {}
+        self.t = 0
+
+    def _attend(self, layer, ins):
+        c, w = layer.cfg, layer.p["w"]
+        heads, dk = int(c["num_heads"]), int(c["key_dim"])
+        dv = int(c.get("value_dim") or dk)
+        if c["use_bias"]:
+            qw, qb, kw, kb, vw, vb, ow, ob = w
+        else:
+            (qw, kw, vw, ow), qb, kb, vb, ob = w, None, None, None, None
+        x = ins[0]
+        assert x.shape[0] == 1 and all(i is ins[0] or np.array_equal(i, x) for i in ins[1:]), "self-attention on one new row"
+        zk, zv = np.zeros(heads * dk, np.float32), np.zeros(heads * dv, np.float32)
+        q = dense(x, qw, qb if qb is not None else zk, heads * dk)[0]
+        k = dense(x, kw, kb if kb is not None else zk, heads * dk)[0]
+        v = dense(x, vw, vb if vb is not None else zv, heads * dv)[0]
+        ks, vs = self.cache.setdefault(layer.name, ([], []))
+        ks.append(k)
+        vs.append(v)
+        K = np.stack(ks).reshape(len(ks), heads, dk)
+        V = np.stack(vs).reshape(len(vs), heads, dv)
+        scale = np.float32(1.0 / np.sqrt(float(dk)))
+        merged = np.empty(heads * dv, np.float32)
+        for h in range(heads):
+            scores = (K[:, h, :] @ q[h * dk:(h + 1) * dk]).astype(np.float32) * scale
+            merged[h * dv:(h + 1) * dv] = softmax(scores[None, :])[0] @ V[:, h, :]
+        dout = ow.size // (heads * dv)
+        return dense(merged[None, :], ow, ob if ob is not None else np.zeros(dout, np.float32), dout)
+
+    def step(self, token):
+        """Feeds one token id; returns the logits row for the next position."""
+        ids = np.array([token], np.float32)
+        pos = np.array([self.t], np.float32)
+        out = self.model.graph.run([ids, pos], self._attend)[0]
+        self.t += 1
+        return out[-1]

@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <fdeep/fdeep.hpp>
+#include <thread>
 
 #define EXPECT(cond)                                                     \
     do {                                                                 \
@@ -75,6 +76,28 @@ int main(int argc, char** argv)
     const fdeep::model copy = model;
     EXPECT(copy.predict({ x })[0].to_vector() == out[0].to_vector());
 
+    // predict is const and thread-safe (FAQ.md:103-114): four host threads on one model and on a copy of it, each
+    // mixing predict and predict_multi, get what the serial calls above returned
+    {
+        int bad[4] = { 0, 0, 0, 0 };
+        std::vector<std::thread> workers;
+        for (int t = 0; t < 4; ++t)
+            workers.emplace_back([&, t] {
+                const fdeep::model& mine = (t % 2) ? copy : model;
+                for (int it = 0; it < 20; ++it) {
+                    if (mine.predict({ x })[0].to_vector() != out[0].to_vector())
+                        ++bad[t];
+                    const auto multi = mine.predict_multi(std::vector<fdeep::tensors>(3 + t, dummy), it % 2 == 0);
+                    for (const auto& r : multi)
+                        if (r[0].to_vector() != serial[0][0].to_vector())
+                            ++bad[t];
+                }
+            });
+        for (auto& w : workers)
+            w.join();
+        EXPECT(bad[0] + bad[1] + bad[2] + bad[3] == 0);
+    }
+
     // error behaviour (include/fdeep/model.hpp:137-139, 293; tensor_shape.hpp:246-250)
     EXPECT(throws_with([&] { model.predict({ fdeep::tensor(fdeep::tensor_shape(32, 32, 4), 0.0f) }); }, "Invalid inputs shape"));
     EXPECT(throws_with([&] { model.predict({ fdeep::tensor(fdeep::tensor_shape(3072), 0.0f) }); }, "Invalid inputs shape"));
@@ -91,6 +114,9 @@ int main(int argc, char** argv)
     for (int i = 0; i < 6; ++i)
         EXPECT(back[static_cast<std::size_t>(i)] == px[i]);
     EXPECT(fdeep::show_tensor_shape(t.shape()) == "3(1, 2, 3)");
+    // show_tensor pads every value to the longest one (include/fdeep/tensor.hpp:1203-1218)
+    EXPECT(fdeep::show_tensor(fdeep::tensor(fdeep::tensor_shape(2, 2), std::vector<float> { 1.5f, -12.25f, 0.0f, 3.0f }))
+        == "[[[[[  1.5000, -12.2500], [  0.0000,   3.0000]]]]]");
     // dimensions() covers the rank only (include/fdeep/tensor_shape.hpp:153-164)
     EXPECT((fdeep::tensor_shape(7, 5).dimensions() == std::vector<std::size_t> { 7, 5 }));
     EXPECT((fdeep::tensor_pos(1, 2, 3).dimensions() == std::vector<std::size_t> { 1, 2, 3 }));

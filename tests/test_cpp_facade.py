@@ -17,7 +17,7 @@ def compile_facade():
             os.path.join(ROOT, "include", "fdeep", "fdeep.hpp")), os.path.getmtime(os.path.join(PKG, "libfdx.so"))):
         return
     subprocess.check_call(["g++", "-std=c++14", "-O1", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), src,
-                           "-L", PKG, "-lfdx", "-Wl,-rpath," + PKG, "-Wl,-rpath,/opt/rocm/lib", "-o", EXE])
+                           "-L", PKG, "-lfdx", "-Wl,-rpath," + PKG, "-Wl,-rpath,/opt/rocm/lib", "-pthread", "-o", EXE])
 
 
 def test_facade_compiles_and_links(fdx):

@@ -73,6 +73,21 @@ def test_causal_prefix_identity_equals_sdpa_is_causal(oracle, modelgen):
     assert rel(oracle.OracleModel(modelgen.dumps(spec)).predict([x])[0], np.einsum("htk,hkd->td", o, ow) + ob) <= 2e-6
 
 
+def test_cached_decoder_equals_causal_prediction_rows(oracle, modelgen):
+    """The oracle's KV-cached decoder (the timed CPU baseline of the decode benchmark) fed token by token returns, at
+    step t, row t of the causal prediction of the whole sequence, which is defined through the reference's own
+    MultiHeadAttention(query = x[t:t+1], value = x[0:t+1]); with and without attention biases."""
+    for bias_std in (0.1, 0.0):
+        spec = modelgen.gpt2(seed=61, layers=2, d_model=32, heads=4, vocab=53, max_pos=16, bias_std=bias_std,
+                             random_affine=True, std=0.2)
+        ref = oracle.OracleModel(modelgen.dumps(spec))
+        ids = np.random.default_rng(62).integers(0, 53, 11).astype(np.float32)
+        want = ref.predict([ids, np.arange(11, dtype=np.float32)], causal=True)[0]
+        dec = oracle.CachedDecoder(ref)
+        for t in range(11):
+            assert rel(dec.step(ids[t]), want[t]) <= 2e-6, t
+
+
 def test_batchnorm_equals_folded_convolution(oracle, modelgen):
     """conv -> BN equals a convolution with W' = W * inv[n], b' = b * inv + beta - mean * inv (the load-time fold
     the GPU path applies), to 1e-6."""
