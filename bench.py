@@ -338,7 +338,7 @@ def bench_gpt2_kernels(fdx, args):
     out = []
     ms = ctypes.c_float()
     for name, k, n, ln, res in shapes:
-        copies = max(2, int(600e6 // (4 * k * n)))
+        copies = max(1, int(args.ring_mb * 1e6 // (4 * k * n)))
         w = fdx.DevBuf(4 * k * n * copies)
         host = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
         for c in range(copies):
@@ -386,6 +386,9 @@ def main():
     ap.add_argument("--decode-reps", type=int, default=2)
     ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels", "mobilenet_v2", "encoder"], default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ring-mb", type=float, default=600.0,
+                    help="gpt2_kernels: total size of the ring of weight copies a kernel cycles through (larger than the "
+                         "caches by default, so every launch streams from HBM)")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also launch one plain device copy (act_kernel, no activation) of this many MiB, whose known "
                          "traffic scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")

@@ -1,19 +1,21 @@
-// Body of the decode attention for the common head shape, shared by its own kernel (decode_attn.hip) and the persistent
-// decode-step kernel (decode_kernels.hip).  Included inside namespace fdx after f32x4 and gptr are defined.
+// Body of the decode attention for the common head shape, shared by the attention kernel and the kernel that also
+// applies the output projection (both in decode_attn.hip).  Included inside namespace fdx after f32x4 and gptr are defined.
 #pragma once
 
 struct MhaDecodeShared {
     float red[4], red_sum[4];
     float osum[4][64];
+    float oval[64]; // KEEP: the head's output row for the code that follows in the same workgroup
 };
 
-// The work of one (sequence, head) item by 256 threads.  MEGA: called from the persistent decode-step kernel by a
-// 512-thread workgroup whose upper half idles (active = false: no loads, no stores, same barriers); the output is
-// written with agent-scope stores so that workgroups on other XCDs see it after the grid-wide barrier of that kernel.
-template <bool MEGA>
+// The work of one (sequence, head) item by 256 threads.  KEEP: the 64 output values stay in sh.oval (valid after the
+// caller's next barrier) instead of going to `out`.
+// after_loads() runs once every key / value / query load has been issued and before the first of them is used: the place
+// where a caller requests operands of its own that do not depend on the attention result.
+template <bool KEEP, typename AfterLoads>
 __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q, int64_t ldq, const float* __restrict__ kc,
     const float* __restrict__ vc, float* __restrict__ out, int heads, const int* __restrict__ len_dev, int max_len, float scale,
-    int item, int tid, bool active, MhaDecodeShared& sh)
+    int item, int tid, bool active, MhaDecodeShared& sh, AfterLoads after_loads)
 {
     float* red = sh.red;
     float* red_sum = sh.red_sum;
@@ -36,6 +38,7 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
         }
     }
     const f32x4 qv = active ? *reinterpret_cast<gptr<const f32x4>>(as_global(q) + (int64_t)b * ldq + h * 64 + part * 4) : f32x4 { 0.f, 0.f, 0.f, 0.f };
+    after_loads();
 
     float sc[16];
     float m = -FLT_MAX;
@@ -91,11 +94,10 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
             denom += f[w] * red_sum[w];
             o += f[w] * osum[w][tid];
         }
-        const gptr<float> dst = as_global(out) + (int64_t)b * row + h * 64 + tid;
-        if (MEGA)
-            __hip_atomic_store(dst, o / denom, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (KEEP)
+            sh.oval[tid] = o / denom;
         else
-            *dst = o / denom;
+            as_global(out)[(int64_t)b * row + h * 64 + tid] = o / denom;
     }
 }
 

@@ -19,6 +19,7 @@
 // Up to three output segments let one launch write q and the new key / value cache rows.
 #include <cfloat>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.hpp"
@@ -33,10 +34,6 @@ constexpr int SK_WAVES = 8;
 constexpr int SK_CHUNK = 8;       // slabs of 16 k-values whose loads are issued together (8 waves x 8 x 16 = 1024 k)
 constexpr int SK_CHUNK_LONG = 24; // long-K launches (up to 3072) still issue everything at once, one workgroup per CU
 
-// split-K scratch a session hands to the persistent decode-step kernel (floats / tickets); see session.cpp
-static int64_t fdx_mega_ws_floats() { return 1 << 20; }
-static int fdx_mega_tickets() { return 4096; }
-
 // SINGLE: the workgroup's K range fits one chunk per wave (only one register set is live, which
 // triples the number of resident workgroups).  gridDim.y > 1 splits K across workgroups: partial
 // tiles go to a workspace and the last workgroup to arrive at a column group (atomic ticket) adds
@@ -48,13 +45,8 @@ struct SkinnyShared {
     float stat[SK_WAVES * 16], stat2[SK_WAVES * 16]; // per-wave row sums / sums of squared deviations
 };
 
-// The work of workgroup (bx, by) of a (gx, gy) grid.  MEGA: called from the persistent decode-step kernel, where the
-// results must be visible to workgroups on other XCDs after a grid-wide barrier inside the same launch: they are
-// written with agent-scope stores (which pass this XCD's L2); the operands are read with ordinary loads: every buffer
-// of a step is written by one phase and not read before that phase in the same launch, so no cache holds an older
-// copy.  What this takes for granted is that an acknowledged agent-scope store (s_waitcnt vmcnt(0)) is in memory; the
-// persistent kernel has once produced different tokens than the separate launches, so it is not used by default.
-template <int CHUNK, bool SINGLE, bool MEGA>
+// The work of workgroup (bx, by) of a (gx, gy) grid.
+template <int CHUNK, bool SINGLE>
 __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, int by, int gx, int gy, SkinnyShared& sh)
 {
     float* red = sh.red;
@@ -238,10 +230,7 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         v = apply_act(v + e_bias + e_res, p.act);
         const SkinnySegment& sg = p.seg[e_seg];
         const gptr<float> dst = as_global(sg.ptr) + e_shift + (int64_t)em * sg.ld + (ecol - sg.col_begin);
-        if (MEGA)
-            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else
-            *dst = v;
+        *dst = v;
     }
 }
 
@@ -249,7 +238,7 @@ template <int CHUNK, bool SINGLE>
 __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
 {
     __shared__ SkinnyShared sh;
-    skinny_gemm_body<CHUNK, SINGLE, false>(p, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, sh);
+    skinny_gemm_body<CHUNK, SINGLE>(p, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, sh);
 }
 
 
@@ -444,215 +433,6 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
         if (ec == 0)
             p.amax_parts[(int64_t)blockIdx.x * 16 + em] = best; // rows beyond M keep 0 = "no value"
     }
-}
-
-// ---- the decode step as ONE launch -------------------------------------------------------------------------------
-//
-// A step of the cached decoder is a chain of some sixty small launches, each a few microseconds of load -> multiply ->
-// store latency plus the launch itself.  Here one workgroup per CU stays resident and walks the same chain as phases,
-// with a grid-wide barrier between phases instead of a launch boundary.
-//
-// Barrier: every workgroup writes the phase number into its own arrival cell (256 bytes apart); workgroup 0 gathers
-// them, one thread per cell, and writes eight release cells (one per XCD residue of the workgroup index); the others
-// poll their release cell.  No read-modify-write and nobody polls a cell that many others write: 1.5 us for 256
-// workgroups, against 11 us for a shared atomic counter.  Every wait is bounded; a workgroup that gives up raises the
-// abort flag and all workgroups leave at their next barrier.
-//
-// Visibility between phases without a cache flush (an agent-scope release / acquire fence pair costs 30 us here):
-// results are written with agent-scope stores, which pass the writer's L2, and waited for before the arrival cell is
-// written; operands are read with ordinary loads, which miss the reader's L2 because every buffer of a step is
-// written by exactly one phase and read by nobody before that phase within the launch (launch boundaries take care
-// of the previous step's lines).
-#include "decode_attn_body.hpp"
-
-struct MegaState {
-    unsigned arrive[1024 * 64]; // cell w at arrive[w * 64]
-    unsigned go[8 * 64];
-    unsigned epoch;             // phase number reached by the previous launches
-    int abort;
-};
-constexpr int kMegaSpinLimit = 200000;
-
-__device__ __forceinline__ bool mega_barrier(MegaState* st, unsigned phase_no, int* bad)
-{
-    // this workgroup's results have left the CU
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const int nwg = (int)gridDim.x;
-    if (threadIdx.x == 0)
-        __hip_atomic_store(&st->arrive[blockIdx.x * 64], phase_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (blockIdx.x == 0) {
-        for (int w = threadIdx.x; w < nwg; w += blockDim.x) {
-            int spins = 0;
-            while (__hip_atomic_load(&st->arrive[w * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < phase_no) {
-                if (++spins > kMegaSpinLimit
-                    || __hip_atomic_load(&st->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-                    *bad = 1;
-                    break;
-                }
-            }
-        }
-        __syncthreads();
-        if (*bad && threadIdx.x == 0)
-            __hip_atomic_store(&st->abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (threadIdx.x < 8)
-            __hip_atomic_store(&st->go[threadIdx.x * 64], phase_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (threadIdx.x == 0) {
-        int spins = 0;
-        while (__hip_atomic_load(&st->go[(blockIdx.x & 7) * 64], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < phase_no) {
-            if (++spins > kMegaSpinLimit) {
-                *bad = 1;
-                __hip_atomic_store(&st->abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
-        }
-        if (__hip_atomic_load(&st->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-            *bad = 1;
-    }
-    __syncthreads();
-    return *bad == 0;
-}
-
-__global__ __launch_bounds__(512) void decode_mega_kernel(const MegaPhase* __restrict__ phases, int n_phases, MegaState* st)
-{
-    __shared__ SkinnyShared sh;
-    __shared__ MhaDecodeShared ash;
-    __shared__ int bad;
-    // all phase descriptors, staged once: fetching each one when its phase starts would put a dependent global load
-    // behind every barrier
-    extern __shared__ __attribute__((aligned(16))) int phase_words[];
-    const MegaPhase* sph = reinterpret_cast<const MegaPhase*>(phase_words);
-    if (threadIdx.x == 0)
-        bad = 0;
-    {
-        const int* src = reinterpret_cast<const int*>(phases);
-        const int words = n_phases * (int)(sizeof(MegaPhase) / sizeof(int));
-        for (int z = threadIdx.x; z < words; z += blockDim.x)
-            phase_words[z] = src[z];
-    }
-    const unsigned base = st->epoch;
-    const int G = (int)gridDim.x;
-    __syncthreads();
-    for (int pi = 0; pi < n_phases; ++pi) {
-        const MegaPhase& ph = sph[pi];
-        if (ph.kind == 0) {
-            const int units = ph.tiles * ph.ksplit;
-            for (int u = blockIdx.x; u < units; u += G) {
-                const int bx = u % ph.tiles, by = u / ph.tiles;
-                if (ph.chunk == 6)
-                    skinny_gemm_body<6, true, true>(ph.g, bx, by, ph.tiles, ph.ksplit, sh);
-                else
-                    skinny_gemm_body<SK_CHUNK, true, true>(ph.g, bx, by, ph.tiles, ph.ksplit, sh);
-                __syncthreads(); // the reduction scratch is reused by the next unit
-            }
-        } else {
-            for (int item = blockIdx.x; item < ph.tiles; item += G)
-                mha_decode_fast_body<true>(ph.q, ph.ldq, ph.kc, ph.vc, ph.out, ph.heads, ph.g.len_dev, ph.max_len, ph.scale, item,
-                    threadIdx.x & 255, threadIdx.x < 256, ash);
-        }
-        if (pi + 1 < n_phases && !mega_barrier(st, base + (unsigned)pi + 1u, &bad))
-            return; // uniform: every thread of the workgroup reads the same flag after the barrier's last __syncthreads
-    }
-    // the epoch moves on for the next launch (this launch's last barrier lies behind every workgroup that reaches here
-    // only if n_phases > 1; the epoch cell is read at launch start and launches do not overlap)
-    if (blockIdx.x == 0 && threadIdx.x == 0)
-        st->epoch = base + (unsigned)n_phases;
-}
-
-bool mega_dense_phase(const SkinnyParams& p, float* workspace, int* tickets, MegaPhase& phase)
-{
-    if (!(p.X && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0 && p.K % 4 == 0 && p.ldx % 4 == 0 && p.ldw % 4 == 0 && p.n_seg >= 1
-            && p.n_seg <= 3))
-        return false;
-    if (p.ln && !(p.K <= SK_WAVES * SK_CHUNK * 16 && p.w_rowsum))
-        return false;
-    if (p.amax_parts)
-        return false;
-    const int tiles = (p.N + 15) / 16;
-    int ksplit = 1;
-    if (!p.ln && !p.packed) { // as skinny_gemm_launch splits
-        while (ksplit < 8 && p.K / ksplit > SK_WAVES * SK_CHUNK * 16 && p.K / (ksplit * 2) >= 128)
-            ksplit *= 2;
-        if (ksplit > 1)
-            while (ksplit < 8 && tiles * ksplit < 192 && p.K / (ksplit * 2) >= 256)
-                ksplit *= 2;
-    }
-    const int per_wg = ((p.K + ksplit * 16 - 1) / (ksplit * 16)) * 16;
-    if (per_wg > SK_WAVES * SK_CHUNK * 16)
-        return false;
-    if (ksplit > 1 && (!workspace || !tickets || (int64_t)tiles * ksplit * 256 > fdx_mega_ws_floats() || tiles > fdx_mega_tickets()))
-        return false;
-    std::memset(&phase, 0, sizeof phase);
-    phase.kind = 0;
-    phase.tiles = tiles;
-    phase.ksplit = ksplit;
-    phase.chunk = per_wg <= SK_WAVES * 6 * 16 ? 6 : SK_CHUNK;
-    phase.g = p;
-    phase.g.workspace = workspace;
-    phase.g.tickets = tickets;
-    return true;
-}
-
-bool mega_attention_phase(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch, int heads, int dk,
-    int dv, const int* len_dev, int max_len, MegaPhase& phase)
-{
-    if (!(q && kc && vc && out && len_dev) || dk != 64 || dv != 64 || max_len > 256 || ldq % 4 != 0 || batch <= 0 || heads <= 0)
-        return false;
-    std::memset(&phase, 0, sizeof phase);
-    phase.kind = 1;
-    phase.tiles = batch * heads;
-    phase.q = q; phase.ldq = ldq; phase.kc = kc; phase.vc = vc; phase.out = out;
-    phase.heads = heads; phase.max_len = max_len;
-    phase.scale = (float)(1.0 / std::sqrt((double)dk));
-    phase.g.len_dev = len_dev;
-    return true;
-}
-
-// one workgroup per CU: all of them are resident at once, which the barrier relies on (queried outside any stream capture)
-static int mega_grid()
-{
-    static const int grid = [] {
-        int dev = 0, cus = 256;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        return cus < 1024 ? cus : 1024;
-    }();
-    return grid;
-}
-
-size_t mega_state_bytes()
-{
-    (void)mega_grid();
-    return sizeof(MegaState);
-}
-
-fdx_status mega_launch(const MegaPhase* phases_dev, int n_phases, void* state_dev)
-{
-    FDX_REQUIRE(phases_dev && state_dev && n_phases > 0, "decode step kernel: bad arguments");
-    const size_t lds = sizeof(MegaPhase) * (size_t)n_phases;
-    FDX_REQUIRE(lds <= 48 * 1024, "decode step kernel: %d phases do not fit its descriptor table", n_phases);
-    const int grid = mega_grid();
-    profile_begin();
-    hipLaunchKernelGGL(decode_mega_kernel, dim3((unsigned)grid), dim3(512), lds, stream(), phases_dev, n_phases,
-        static_cast<MegaState*>(state_dev));
-    profile_end("decode_step_f32", 0.0, 0.0);
-    FDX_LAUNCH_CHECK();
-    return FDX_OK;
-}
-
-fdx_status mega_check(void* state_dev)
-{
-    FDX_REQUIRE(state_dev, "decode step kernel: no state");
-    int flag = 0;
-    FDX_HIP(hipMemcpyAsync(&flag, &static_cast<MegaState*>(state_dev)->abort, sizeof(int), hipMemcpyDeviceToHost, stream()));
-    FDX_HIP(hipStreamSynchronize(stream()));
-    if (flag != 0) {
-        set_error("decode step kernel: a grid-wide barrier gave up waiting");
-        return FDX_ERR_HIP;
-    }
-    return FDX_OK;
 }
 
 // [N][K] -> [column tile][wave][slab][lane] 16-byte pieces in exactly the order the GEMM's lanes consume

@@ -34,12 +34,18 @@ struct fdx_session {
     // ---- decode fast path (one new token per sequence, batch <= 16): a fixed list of fused launches
     // over buffers allocated once; built at creation when the graph has the expected decoder structure
     struct Step {
-        enum Kind { EmbedAdd, Gemm, Attn, LayerNorm, Add, Act, Softmax } kind;
+        enum Kind { EmbedAdd, Gemm, Attn, AttnProj, LayerNorm, Add, Act, Softmax } kind;
         SkinnyParams g;                 // Gemm
         const float *a = nullptr, *b = nullptr; // operands of the other kinds
         float* out = nullptr;
         int op = -1;                    // model op this step realises
         int depth = 0;
+        // AttnProj: the output projection that rides in the attention launch
+        const float* proj_w = nullptr;  // [heads][64][depth]
+        const float* proj_bias = nullptr;
+        const float* proj_residual = nullptr;
+        fdx::Act proj_act { FDX_ACT_NONE, 3.402823466e+38f, 0.f, 0.f };
+        int mha_op = -1;
     };
     bool fast = false;
     std::vector<Step> steps;
@@ -48,23 +54,19 @@ struct fdx_session {
     float* ids_buf = nullptr;           // ids consumed by the next step (argmax writes them)
     const float* logits_buf = nullptr;
     unsigned long long* amax = nullptr; // per sequence: packed running arg-max of the step's logits
-    // the Dense / attention launches of a step as phases of one persistent kernel (steps[mega_first .. mega_last])
-    MegaPhase* mega_phases = nullptr;
-    void* mega_state = nullptr;
-    int mega_count = 0, mega_first = -1, mega_last = -1;
-    bool mega_used = false; // a launch has run since the abort flag was last read back
     unsigned long long* amax_parts = nullptr; // [workgroups of the logits launch][16] when that launch leaves partial maxima
     int amax_part_count = 0;
     float* history = nullptr;           // [max_len][batch] greedy ids by the position that produced them
     hipGraphExec_t step_graph = nullptr; // one decode step (ids_buf -> ids_buf) captured for replay
-    float* splitk_ws = nullptr;         // partial tiles of split-K decode GEMMs
-    int* splitk_tickets = nullptr;
+    float* splitk_ws = nullptr;         // per-head partial rows of the attention + projection launches
+    int* splitk_tickets = nullptr;      // their tickets, one per sequence, zero between launches
     static constexpr int64_t kWsFloats = 1 << 20;
     static constexpr int kTickets = 4096;
     float* positions = nullptr;
     ~fdx_session()
     {
         (void)hipStreamSynchronize(stream());
+
         for (auto& c : chunks)
             (void)hipFree(c.p);
         for (auto& kv : kc)
@@ -322,20 +324,30 @@ bool build_fast_plan(fdx_session* s)
         if (o.residual >= 0)
             users[o.residual].push_back(idx);
     }
+    // Every buffer of the decode step comes out of a few large allocations: hundreds of separate small ones would each sit
+    // on pages of their own, and a launch that touches a dozen operands would miss the address translation caches for
+    // most of them.
+    char* chunk = nullptr;
+    size_t chunk_left = 0;
     auto alloc = [&](size_t floats) -> float* {
-        void* p = nullptr;
-        if (hipMalloc(&p, floats * sizeof(float)) != hipSuccess)
-            return nullptr;
-        s->owned.push_back(p);
-        return static_cast<float*>(p);
+        const size_t bytes = (floats * sizeof(float) + 255) & ~(size_t)255;
+        if (bytes > chunk_left) {
+            const size_t want = std::max(bytes, (size_t)256 << 20);
+            void* p = nullptr;
+            if (hipMalloc(&p, want) != hipSuccess)
+                return nullptr;
+            s->owned.push_back(p);
+            chunk = static_cast<char*>(p);
+            chunk_left = want;
+        }
+        float* r = reinterpret_cast<float*>(chunk);
+        chunk += bytes;
+        chunk_left -= bytes;
+        return r;
     };
-    {
-        void* p = nullptr;
-        if (hipMalloc(&p, sizeof(int)) != hipSuccess)
-            return false;
-        s->owned.push_back(p);
-        s->len_dev = static_cast<int*>(p);
-    }
+    s->len_dev = reinterpret_cast<int*>(alloc(1));
+    if (!s->len_dev)
+        return false;
     s->ids_buf = alloc((size_t)B);
     s->amax = reinterpret_cast<unsigned long long*>(alloc((size_t)2 * B + 4));
     if (!s->ids_buf || !s->amax)
@@ -474,12 +486,15 @@ bool build_fast_plan(fdx_session* s)
             if (!wqkv || !bqkv || !q || !merged)
                 return false;
             const size_t f = sizeof(float);
-            if (hipMemcpy(wqkv, o.dw[0], f * nk * D, hipMemcpyDeviceToDevice) != hipSuccess
-                || hipMemcpy(wqkv + (size_t)nk * D, o.dw[2], f * nk * D, hipMemcpyDeviceToDevice) != hipSuccess
-                || hipMemcpy(wqkv + (size_t)2 * nk * D, o.dw[4], f * nv * D, hipMemcpyDeviceToDevice) != hipSuccess
-                || hipMemcpy(bqkv, o.dw[1], f * nk, hipMemcpyDeviceToDevice) != hipSuccess
-                || hipMemcpy(bqkv + nk, o.dw[3], f * nk, hipMemcpyDeviceToDevice) != hipSuccess
-                || hipMemcpy(bqkv + 2 * nk, o.dw[5], f * nv, hipMemcpyDeviceToDevice) != hipSuccess)
+            // on the library stream, like the launches that read the copies (a plain device-to-device hipMemcpy runs on the
+            // null stream, which this stream does not wait for, and may return before the copy has happened)
+            hipStream_t cs = stream();
+            if (hipMemcpyAsync(wqkv, o.dw[0], f * nk * D, hipMemcpyDeviceToDevice, cs) != hipSuccess
+                || hipMemcpyAsync(wqkv + (size_t)nk * D, o.dw[2], f * nk * D, hipMemcpyDeviceToDevice, cs) != hipSuccess
+                || hipMemcpyAsync(wqkv + (size_t)2 * nk * D, o.dw[4], f * nv * D, hipMemcpyDeviceToDevice, cs) != hipSuccess
+                || hipMemcpyAsync(bqkv, o.dw[1], f * nk, hipMemcpyDeviceToDevice, cs) != hipSuccess
+                || hipMemcpyAsync(bqkv + nk, o.dw[3], f * nk, hipMemcpyDeviceToDevice, cs) != hipSuccess
+                || hipMemcpyAsync(bqkv + 2 * nk, o.dw[5], f * nv, hipMemcpyDeviceToDevice, cs) != hipSuccess)
                 return false;
             fdx_session::Step pr;
             pr.kind = fdx_session::Step::Gemm;
@@ -496,12 +511,6 @@ bool build_fast_plan(fdx_session* s)
             g.seg[2] = { s->vc[idx], (int64_t)s->max_len * nv, 2 * nk, nv };
             g.len_dev = s->len_dev;
             s->steps.push_back(pr);
-            fdx_session::Step at;
-            at.kind = fdx_session::Step::Attn;
-            at.op = idx;
-            at.a = q;
-            at.out = merged;
-            s->steps.push_back(at);
             // output projection; a following two-input Add becomes its residual operand
             st.kind = fdx_session::Step::Gemm;
             SkinnyParams& og = st.g;
@@ -531,6 +540,34 @@ bool build_fast_plan(fdx_session* s)
                         skip[ai] = 1;
                     }
                 }
+            }
+            // Attention and this projection as one launch where the kernel covers the shape: one dependent launch less
+            // per block, against an exchange of per-head partial rows between workgroups that costs about half a launch
+            // itself.  Measured on the GPT-2-small shape (batch 16): 0.498 ms per step against 0.484 ms for the two
+            // launches, so it is off unless FDX_DECODE_FUSE_PROJ=1 is set when the session is created.
+            const char* fuse_env = std::getenv("FDX_DECODE_FUSE_PROJ");
+            const bool fuse_proj = fuse_env && fuse_env[0] == '1';
+            const bool act_ok = og.act.kind == FDX_ACT_NONE || og.act.kind == FDX_ACT_RELU || og.act.kind == FDX_ACT_GELU;
+            if (fuse_proj && act_ok
+                && mha_decode_proj_supported(B, H, o.dk, o.dv, s->max_len, nk, o.dout, fdx_session::kWsFloats, fdx_session::kTickets)) {
+                float* wt = alloc((size_t)H * o.dout * 64);
+                if (!wt || pack_proj_heads_launch(o.dw[6], H, o.dout, wt) != FDX_OK)
+                    return false;
+                st.kind = fdx_session::Step::AttnProj;
+                st.a = q;
+                st.proj_w = wt;
+                st.proj_bias = o.dw[7];
+                st.proj_residual = og.residual;
+                st.proj_act = og.act;
+                st.mha_op = idx;
+                std::memset(&og, 0, sizeof og);
+            } else {
+                fdx_session::Step at;
+                at.kind = fdx_session::Step::Attn;
+                at.op = idx;
+                at.a = q;
+                at.out = merged;
+                s->steps.push_back(at);
             }
             break;
         }
@@ -604,42 +641,6 @@ bool build_fast_plan(fdx_session* s)
             s->amax_part_count = parts;
         }
     }
-    // With FDX_DECODE_MEGA=1 (read when the session is created) the run of Dense / attention launches between the
-    // embedding and the logits launch becomes one persistent kernel, if every one of them has a phase form.  Off by
-    // default: a phase costs 7.6 us against 7.3 us per separate launch on the GPT-2-small shape, and the exchange between
-    // phases is not verified to the bar of the separate launches (see skinny_gemm_body): for measurement only.
-    const char* mega_env = std::getenv("FDX_DECODE_MEGA");
-    const bool mega_on = mega_env && mega_env[0] == '1';
-    if (mega_on && s->steps.size() >= 4) {
-        std::vector<MegaPhase> phases;
-        const int first = 1, last = (int)s->steps.size() - 2;
-        bool ok = true;
-        for (int i = first; i <= last && ok; ++i) {
-            const fdx_session::Step& step = s->steps[(size_t)i];
-            const Op& o = m.ops[step.op];
-            MegaPhase ph;
-            if (step.kind == fdx_session::Step::Gemm)
-                ok = mega_dense_phase(step.g, s->splitk_ws, s->splitk_tickets, ph);
-            else if (step.kind == fdx_session::Step::Attn)
-                ok = mega_attention_phase(step.a, (int64_t)o.heads * o.dk, s->kc[step.op], s->vc[step.op], step.out, B, o.heads, o.dk,
-                    o.dv, s->len_dev, s->max_len, ph);
-            else
-                ok = false;
-            if (ok)
-                phases.push_back(ph);
-        }
-        if (ok && phases.size() >= 2) {
-            s->mega_phases = reinterpret_cast<MegaPhase*>(alloc((sizeof(MegaPhase) * phases.size() + 3) / 4));
-            s->mega_state = alloc((mega_state_bytes() + 3) / 4);
-            if (!s->mega_phases || !s->mega_state
-                || hipMemcpy(s->mega_phases, phases.data(), sizeof(MegaPhase) * phases.size(), hipMemcpyHostToDevice) != hipSuccess
-                || zero_device(s->mega_state, mega_state_bytes()) != hipSuccess)
-                return false;
-            s->mega_count = (int)phases.size();
-            s->mega_first = first;
-            s->mega_last = last;
-        }
-    }
     return set_int_launch(s->len_dev, 0) == FDX_OK;
 }
 
@@ -650,13 +651,6 @@ fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
     const int B = s->batch;
     fdx_status st = FDX_OK;
     for (size_t si = 0; si < s->steps.size(); ++si) {
-        if ((int)si == s->mega_first && s->mega_count > 0) {
-            if ((st = mega_launch(s->mega_phases, s->mega_count, s->mega_state)) != FDX_OK)
-                return st;
-            s->mega_used = true;
-            si = (size_t)s->mega_last;
-            continue;
-        }
         const auto& step = s->steps[si];
         const Op& o = m.ops[step.op];
         const fdx_act act = to_c(o.act);
@@ -672,6 +666,13 @@ fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
             st = mha_decode_dyn_launch(step.a, (int64_t)o.heads * o.dk, s->kc[step.op], s->vc[step.op], step.out, B, o.heads, o.dk, o.dv,
                 s->len_dev, s->max_len, s->len + 1);
             break;
+        case fdx_session::Step::AttnProj: {
+            const Op& mo = m.ops[step.mha_op];
+            st = mha_decode_proj_launch(step.a, (int64_t)mo.heads * mo.dk, s->kc[step.mha_op], s->vc[step.mha_op], B, mo.heads, s->len_dev,
+                s->max_len, step.proj_w, step.proj_bias, step.proj_residual, step.depth, step.proj_act, step.depth, s->splitk_ws,
+                fdx_session::kWsFloats, s->splitk_tickets, fdx_session::kTickets, step.out, s->len + 1);
+            break;
+        }
         case fdx_session::Step::LayerNorm:
             st = fdx_layernorm_f32(step.a, B, step.depth, o.dw[0], o.dw[1], o.eps, step.out);
             break;
@@ -702,12 +703,6 @@ fdx_status run_fast(fdx_session* s, const float* ids_dev, float* logits_dev, flo
     FDX_REQUIRE(ids_dev, "session: null ids");
     FDX_REQUIRE(s->len + 1 <= s->max_len, "session: sequence length %d exceeds max_len %d", s->len + 1, s->max_len);
     std::lock_guard<std::mutex> lock(m.mu);
-    if (s->mega_used) { // did a barrier of the previous persistent launches give up?
-        s->mega_used = false;
-        const fdx_status ms = mega_check(s->mega_state);
-        if (ms != FDX_OK)
-            return ms;
-    }
     fdx_status st = launch_steps(s, ids_dev, next_ids_dev ? next_ids_dev : s->ids_buf);
     if (st != FDX_OK)
         return st;
@@ -725,12 +720,6 @@ fdx_status run_fast_greedy(fdx_session* s, const float* first_ids_dev, int steps
     fdx_model& m = *s->m;
     FDX_REQUIRE(s->len + steps <= s->max_len, "session: sequence length %d exceeds max_len %d", s->len + steps, s->max_len);
     std::lock_guard<std::mutex> lock(m.mu);
-    if (s->mega_used) {
-        s->mega_used = false;
-        const fdx_status ms = mega_check(s->mega_state);
-        if (ms != FDX_OK)
-            return ms;
-    }
     const int B = s->batch;
     hipStream_t st = stream();
     FDX_HIP(hipMemcpyAsync(s->ids_buf, first_ids_dev, sizeof(float) * B, hipMemcpyDeviceToDevice, st));

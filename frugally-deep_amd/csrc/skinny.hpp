@@ -40,33 +40,6 @@ struct SkinnyParams {
 
 fdx_status skinny_gemm_launch(const SkinnyParams& p);
 
-// One phase of the persistent decode-step kernel: a Dense launch (as skinny_gemm_launch would run it) or the decode
-// attention of every (sequence, head).
-struct MegaPhase {
-    int kind;    // 0 = Dense, 1 = attention
-    int tiles;   // Dense: 16-column groups; attention: (sequence, head) items
-    int ksplit;  // Dense: K ranges per column group
-    int chunk;   // Dense: 6 or 8 slabs per wave (the kernel instantiation)
-    SkinnyParams g;
-    const float* q;
-    int64_t ldq;
-    const float* kc;
-    const float* vc;
-    float* out;
-    int heads, max_len;
-    float scale;
-};
-// Fills `phase` from a Dense launch's parameters; false when the persistent kernel does not cover the shape.
-bool mega_dense_phase(const SkinnyParams& p, float* workspace, int* tickets, MegaPhase& phase);
-bool mega_attention_phase(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch, int heads, int dk,
-    int dv, const int* len_dev, int max_len, MegaPhase& phase);
-// Device-side state of the persistent kernel's grid barrier (allocated once per session): arrival cells, release cells,
-// epoch, abort flag.
-size_t mega_state_bytes();
-// Runs the phases back to back inside one launch, a grid-wide barrier between consecutive phases.
-fdx_status mega_launch(const MegaPhase* phases_dev, int n_phases, void* state_dev);
-// non-zero after a launch whose barrier gave up waiting (reads the flag back; synchronises the stream)
-fdx_status mega_check(void* state_dev);
 // number of workgroups the launch would use if it takes the wide-output kernel (one that strides over column groups), else 0
 int skinny_wide_grid(const SkinnyParams& p);
 // greedy ids from per-workgroup partial maxima [parts][16] (first maximum wins), then as argmax_bump_launch
@@ -78,6 +51,15 @@ fdx_status fold_layernorm_launch(const float* gamma, const float* beta, const fl
     float* w_out, float* wsum, float* bias_out);
 fdx_status embed_add_launch(const float* ids, int batch, const float* ta, int dim_a, const float* tb, int dim_b,
     const int* len_dev, int depth, float* out, int* err, unsigned long long* amax);
+// Decode attention (64-wide heads, at most 256 cached positions) and the layer's output projection with bias, residual and
+// activation as one launch (decode_attn.hip); wt is the projection kernel re-laid by pack_proj_heads_launch, workspace
+// holds batch * heads * n_out partial sums, tickets one zero-initialised cell per sequence.
+bool mha_decode_proj_supported(int batch, int heads, int dk, int dv, int max_len, int64_t ldq, int n_out, int64_t workspace_floats,
+    int ticket_count);
+fdx_status pack_proj_heads_launch(const float* w_nk, int heads, int n_out, float* out);
+fdx_status mha_decode_proj_launch(const float* q, int64_t ldq, const float* kc, const float* vc, int batch, int heads,
+    const int* len_dev, int max_len, const float* wt, const float* bias, const float* residual, int64_t ldr, const Act& act, int n_out,
+    float* workspace, int64_t workspace_floats, int* tickets, int ticket_count, float* out, int len_hint);
 fdx_status mha_decode_dyn_launch(const float* q, int64_t ldq, const float* kc, const float* vc, float* out, int batch,
     int heads, int dk, int dv, const int* len_dev, int max_len, int len_hint);
 fdx_status argmax_bump_launch(const float* x, int rows, int depth, float* out_idx_f, int* len_dev, unsigned long long* amax,
