@@ -108,6 +108,24 @@ __device__ __forceinline__ float apply_act_full(float x, const Act& a)
     }
 }
 
+// Sum over the sixteen lanes of a row (lanes 16r .. 16r+15), left in every lane of the row, on the VALU's data-parallel
+// primitives: swaps inside quads, then the mirror inside each half row and inside the row (after the quad steps all lanes
+// of a quad agree, so the mirrored partner holds the other quads' sum).  __shfl_xor compiles to ds_bpermute_b32, a trip
+// through the LDS crossbar with an address register and a wait of its own per step.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += dpp_move<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+    v += dpp_move<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+    v += dpp_move<0x141>(v); // row_half_mirror
+    v += dpp_move<0x140>(v); // row_mirror
+    return v;
+}
+
 // activations an epilogue can carry
 inline bool epilogue_act_ok(const fdx_act* a) { return !a || a->kind == FDX_ACT_NONE || a->kind == FDX_ACT_RELU || a->kind == FDX_ACT_GELU; }
 

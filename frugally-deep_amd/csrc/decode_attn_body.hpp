@@ -45,10 +45,7 @@ __device__ __forceinline__ void mha_decode_fast_body(const float* __restrict__ q
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
         float s = qv[0] * kv[u][0] + qv[1] * kv[u][1] + qv[2] * kv[u][2] + qv[3] * kv[u][3];
-        s += __shfl_xor(s, 8, 64);
-        s += __shfl_xor(s, 4, 64);
-        s += __shfl_xor(s, 2, 64);
-        s += __shfl_xor(s, 1, 64);
+        s = row16_sum(s);
         sc[u] = slot + 16 * u < len ? s * scale : -FLT_MAX;
         m = fmaxf(m, sc[u]);
     }

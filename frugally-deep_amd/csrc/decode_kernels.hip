@@ -211,10 +211,17 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         if (!is_last)
             return;
         if (t < 256) {
+            // all partials are requested before the first is used (a loop of load-and-add would pay one round trip to
+            // memory per K range), then added in split order
+            float pv[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+                pv[ks] = ks < ksplit ? __hip_atomic_load(ws + ((int64_t)ks * gx + bx) * 256 + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
             v = 0.f;
-            for (int ks = 0; ks < ksplit; ++ks)
-                v += __hip_atomic_load(ws + ((int64_t)ks * gx + bx) * 256 + t, __ATOMIC_RELAXED,
-                    __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+                if (ks < ksplit)
+                    v += pv[ks];
         }
     }
     if (e_ok) {
