@@ -207,6 +207,28 @@ def dwconv_pointwise(x, dw_w_chw, dw_bias, stride, padding, dw_act, pw_w_nc, pw_
     return out.to_host((n, g["out_h"], g["out_w"], n_out))
 
 
+def inverted_residual(x, exp_w_ec, exp_bias, exp_act, dw_w_chw, dw_bias, stride, padding, dw_act, pw_w_nc, pw_bias,
+                      residual=None, act=None, zero_frame=(0, 0, 0, 0)):
+    """1x1 expansion, depthwise 3x3, 1x1 projection in one launch.  x [n,h,w,cin]; exp_w_ec [ce,cin]; dw_w_chw [ce,3,3];
+    pw_w_nc [n_out,ce]; zero_frame = (top, left, bottom, right) of an explicit ZeroPadding2D in front of the depthwise layer."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, wd, cin = x.shape
+    zt, zl, zb, zr = zero_frame
+    g = window_geometry(h + zt + zb, wd + zl + zr, 3, 3, stride, stride, padding)
+    ce, n_out = exp_w_ec.shape[0], pw_w_nc.shape[0]
+    dx, ew = DevBuf.from_host(x), DevBuf.from_host(exp_w_ec)
+    eb = None if exp_bias is None else DevBuf.from_host(exp_bias)
+    dw = DevBuf.from_host(np.transpose(dw_w_chw, (1, 2, 0)))
+    db = None if dw_bias is None else DevBuf.from_host(dw_bias)
+    pw, pb = DevBuf.from_host(pw_w_nc), (None if pw_bias is None else DevBuf.from_host(pw_bias))
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * n_out)
+    check(lib.fdx_inverted_residual_nhwc_f32(_dp(dx), n, h, wd, cin, _dp(ew), _dp(eb), _act_ref(exp_act), ce, _dp(dw), _dp(db),
+                                             stride, g["pad_top"] + zt, g["pad_left"] + zl, g["out_h"], g["out_w"], _act_ref(dw_act),
+                                             _dp(pw), _dp(pb), n_out, _dp(dr), _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], n_out))
+
+
 def gemm(a, b_nk, bias=None, alpha=1.0, bias_per_row=False, residual=None, act=None):
     a, b_nk = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b_nk, np.float32)
     m, k = a.shape

@@ -1235,6 +1235,18 @@ namespace {
                 continue;
             c.fuse_dw = c.in[0];
             d.fused_into = (int)i;
+            // ... and the 1x1 expansion in front of the depthwise convolution, where one launch covers the whole block
+            if (d.in.empty())
+                continue;
+            Op& e = m.ops[d.in[0]];
+            const bool act_ok = e.act.kind == FDX_ACT_NONE || e.act.kind == FDX_ACT_RELU || e.act.kind == FDX_ACT_GELU;
+            if (!e.dead && e.kind == OpKind::Conv2D && e.kh == 1 && e.kw == 1 && e.sy == 1 && e.sx == 1 && !e.softmax && e.residual < 0
+                && e.consumers == 1 && e.fuse_dw < 0 && e.exp_into < 0 && !e.zp[0] && !e.zp[1] && !e.zp[2] && !e.zp[3] && act_ok
+                && !e.hw.empty() && e.cout > 0 && e.hw[0].size() % (size_t)e.cout == 0
+                && fdx_inverted_residual_supported((int)(e.hw[0].size() / (size_t)e.cout), e.cout, c.cout, d.sy)) {
+                c.fuse_exp = d.in[0];
+                e.exp_into = (int)i;
+            }
         }
     }
 
@@ -1550,7 +1562,7 @@ static int g_force_dw_fusion = -1;
 
 extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
 {
-    FDX_REQUIRE(mode >= -1 && mode <= 1, "fdx_debug_force_dw_fusion: mode must be -1, 0 or 1");
+    FDX_REQUIRE(mode >= -1 && mode <= 2, "fdx_debug_force_dw_fusion: mode must be -1, 0, 1 or 2");
     g_force_dw_fusion = mode;
     return FDX_OK;
 }
@@ -1581,7 +1593,7 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->block_of.assign(n, -1);
     p->last_use.assign(n, -1);
     p->temps.assign(n, {});
-    p->dw_fused.assign(n, g_force_dw_fusion < 0 ? 0 : (g_force_dw_fusion ? 1 : 2));
+    p->dw_fused.assign(n, g_force_dw_fusion < 0 ? 0 : (g_force_dw_fusion == 1 ? 1 : (g_force_dw_fusion == 2 ? 3 : 2)));
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -1597,6 +1609,9 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
             p->last_use[root[o.residual]] = (int)pos;
         if (o.fuse_dw >= 0) // run as one launch, the pair reads the depthwise convolution's input here
             for (int i : m->ops[o.fuse_dw].in)
+                p->last_use[root[i]] = (int)pos;
+        if (o.fuse_exp >= 0) // ... and the whole block the expansion's input
+            for (int i : m->ops[o.fuse_exp].in)
                 p->last_use[root[i]] = (int)pos;
     }
     for (int o : m->outputs)
@@ -2069,17 +2084,67 @@ namespace {
             c.residual >= 0 ? p.out[c.residual] : nullptr, c.act.kind == FDX_ACT_NONE ? nullptr : &a2, p.out[idx]);
     }
 
-    // First execution of a plan: both forms of the pair are timed on the real operands (either leaves the same result
-    // in the convolution's output buffer) and the plan remembers the faster one.
+    // Expansion, depthwise 3x3 convolution and 1x1 convolution `idx` as one launch.
+    fdx_status run_block_fused(fdx_model& m, Plan& p, int idx)
+    {
+        const Op& c = m.ops[idx];
+        const Op& d = m.ops[c.fuse_dw];
+        const Op& e = m.ops[c.fuse_exp];
+        const Shape& is = p.shapes[e.in[0]];
+        if (is.size() != 3)
+            return FDX_ERR_UNSUPPORTED;
+        const int h = (int)is[0], w = (int)is[1], cin = (int)is[2];
+        int g[6];
+        fdx_status st = window(h, w, d, true, g);
+        if (st != FDX_OK)
+            return st;
+        const fdx_act a0 = to_c(e.act), a1 = to_c(d.act), a2 = to_c(c.act);
+        return fdx_inverted_residual_nhwc_f32(p.out[e.in[0]], p.batch, h, w, cin, e.dw[0], e.dw[1], e.act.kind == FDX_ACT_NONE ? nullptr : &a0,
+            e.cout, d.dw[0], d.dw[1], d.sy, g[0] + d.zp[0], g[2] + d.zp[2], g[4], g[5], d.act.kind == FDX_ACT_NONE ? nullptr : &a1, c.dw[0],
+            c.dw[1], c.cout, c.residual >= 0 ? p.out[c.residual] : nullptr, c.act.kind == FDX_ACT_NONE ? nullptr : &a2, p.out[idx]);
+    }
+
+    // One of the three forms of a block that ends in 1x1 convolution `idx`: 3 = expansion + depthwise + projection as one
+    // launch, 1 = (expansion,) depthwise + projection as one launch, 2 = a launch per layer.  A form the launchers do not
+    // take falls back to the next; p.dw_fused[idx] is left at the form that ran.
+    fdx_status run_block_form(fdx_model& m, Plan& p, int idx, int form)
+    {
+        const Op& c = m.ops[idx];
+        fdx_status st = FDX_OK;
+        if (form == 3 && c.fuse_exp >= 0) {
+            st = run_block_fused(m, p, idx);
+            if (st != FDX_ERR_UNSUPPORTED) {
+                p.dw_fused[idx] = 3;
+                return st;
+            }
+        }
+        if (form == 3)
+            form = 1;
+        if (c.fuse_exp >= 0 && (st = run_op(m, p, c.fuse_exp)) != FDX_OK) // the expansion was skipped in the op walk
+            return st;
+        if (form == 1) {
+            st = run_dw_fused(m, p, idx);
+            if (st != FDX_ERR_UNSUPPORTED) {
+                p.dw_fused[idx] = 1;
+                return st;
+            }
+        }
+        p.dw_fused[idx] = 2;
+        if ((st = run_op(m, p, c.fuse_dw)) != FDX_OK)
+            return st;
+        return run_op(m, p, idx);
+    }
+
+    // First execution of a plan: the forms of the block are timed on the real operands (each leaves the same result in the
+    // convolution's output buffer) and the plan remembers the fastest; the choice is kept per shape in the tuner's table,
+    // so that an exported table pins it too.
     fdx_status choose_dw_fusion(fdx_model& m, Plan& p, int idx)
     {
-        const int dw_idx = m.ops[idx].fuse_dw;
-        // the choice is kept per shape in the tuner's table, so that an exported table pins it too
+        const Op& c = m.ops[idx];
+        const Op& d = m.ops[c.fuse_dw];
         TuneKey key;
         std::memset(&key, 0, sizeof key);
         {
-            const Op& c = m.ops[idx];
-            const Op& d = m.ops[dw_idx];
             const Shape& is = p.shapes[d.in[0]];
             key.conv = 2;
             key.M = is.size() == 3 ? (int)is[0] : 0;
@@ -2089,62 +2154,52 @@ namespace {
             key.sy = d.sy;
             key.batch = p.batch;
             key.res = c.residual >= 0;
-            int known = 0;
-            if (tune_lookup(key, &known) || tune_frozen()) {
-                p.dw_fused[idx] = known == 1 ? 1 : 2; // frozen and unseen: two launches
-                if (p.dw_fused[idx] == 1) {
-                    const fdx_status fs = run_dw_fused(m, p, idx);
-                    if (fs != FDX_ERR_UNSUPPORTED)
-                        return fs;
-                    p.dw_fused[idx] = 2;
-                }
-                fdx_status st2 = run_op(m, p, dw_idx);
-                return st2 == FDX_OK ? run_op(m, p, idx) : st2;
-            }
+            key.kh = c.fuse_exp >= 0 ? (int)p.shapes[m.ops[c.fuse_exp].in[0]].back() : 0; // input channels of a whole block
         }
-        fdx_status st = run_op(m, p, dw_idx);
-        if (st == FDX_OK)
-            st = run_op(m, p, idx);
-        if (st != FDX_OK)
-            return st;
-        p.dw_fused[idx] = 2;
-        if (run_dw_fused(m, p, idx) != FDX_OK) // a shape the launcher does not take: two launches it is
-            return FDX_OK;
+        int known = 0;
+        if (tune_lookup(key, &known) || tune_frozen()) // frozen and unseen: a launch per layer
+            return run_block_form(m, p, idx, known == 1 || known == 3 ? known : 2);
         hipEvent_t e0, e1;
         if (hipEventCreate(&e0) != hipSuccess)
-            return FDX_OK;
+            return run_block_form(m, p, idx, 2);
         if (hipEventCreate(&e1) != hipSuccess) {
             (void)hipEventDestroy(e0);
-            return FDX_OK;
+            return run_block_form(m, p, idx, 2);
         }
-        float ms[2] = { 1e30f, 1e30f };
-        for (int form = 0; form < 2 && st == FDX_OK; ++form) {
+        const int forms[3] = { 2, 1, 3 };
+        float ms[3] = { 1e30f, 1e30f, 1e30f };
+        fdx_status st = FDX_OK;
+        for (int f = 0; f < 3 && st == FDX_OK; ++f) {
+            if (forms[f] == 3 && c.fuse_exp < 0)
+                continue;
+            st = run_block_form(m, p, idx, forms[f]); // warm-up; tells whether the launcher takes the shape
+            if (st != FDX_OK || p.dw_fused[idx] != forms[f])
+                continue;
             for (int round = 0; round < 2 && st == FDX_OK; ++round) {
                 (void)hipEventRecord(e0, stream());
-                for (int r = 0; r < 3 && st == FDX_OK; ++r) {
-                    if (form == 0) {
-                        st = run_op(m, p, dw_idx);
-                        if (st == FDX_OK)
-                            st = run_op(m, p, idx);
-                    } else
-                        st = run_dw_fused(m, p, idx);
-                }
+                for (int r = 0; r < 3 && st == FDX_OK; ++r)
+                    st = run_block_form(m, p, idx, forms[f]);
                 (void)hipEventRecord(e1, stream());
                 float t = 1e30f;
-                if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess && t < ms[form])
-                    ms[form] = t;
+                if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess && t < ms[f])
+                    ms[f] = t;
             }
         }
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
-        if (st == FDX_OK && ms[1] < ms[0])
-            p.dw_fused[idx] = 1;
-        if (st == FDX_OK)
-            tune_store(key, p.dw_fused[idx]);
+        if (st != FDX_OK)
+            return st;
+        int best = 0;
+        for (int f = 1; f < 3; ++f)
+            if (ms[f] < ms[best])
+                best = f;
         static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
         if (log_picks)
-            std::fprintf(stderr, "[fdx tune] %s + %s: two launches %.1f us, one launch %.1f us\n", m.ops[dw_idx].name.c_str(),
-                m.ops[idx].name.c_str(), ms[0] * 1e3f / 3, ms[1] * 1e3f / 3);
+            std::fprintf(stderr, "[fdx tune] %s + %s: a launch per layer %.1f us, depthwise + projection %.1f us, whole block %.1f us\n",
+                d.name.c_str(), c.name.c_str(), ms[0] * 1e3f / 3, ms[1] * 1e3f / 3, ms[2] * 1e3f / 3);
+        st = run_block_form(m, p, idx, forms[best]); // leaves the chosen form's state (and its result) behind
+        if (st == FDX_OK)
+            tune_store(key, p.dw_fused[idx]);
         return st;
     }
 
@@ -2157,9 +2212,20 @@ namespace {
             fdx_status st = FDX_OK;
             if (o.fused_into >= 0 && p.dw_fused[o.fused_into] != 2)
                 continue; // absorbed by (or timed together with) the 1x1 convolution behind it
+            if (o.exp_into >= 0 && (p.dw_fused[o.exp_into] == 0 || p.dw_fused[o.exp_into] == 3))
+                continue; // the expansion of a block that runs as one launch, or whose forms are about to be timed
             if (o.fuse_dw >= 0 && p.dw_fused[idx] == 0)
                 st = choose_dw_fusion(m, p, idx);
-            else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 1) {
+            else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 3) {
+                if (o.fuse_exp >= 0) {
+                    st = run_block_fused(m, p, idx);
+                    if (st == FDX_ERR_UNSUPPORTED)
+                        st = run_block_form(m, p, idx, 1);
+                } else { // forced by a test on a pair without an expansion in front
+                    p.dw_fused[idx] = 1;
+                    st = run_block_form(m, p, idx, 1);
+                }
+            } else if (o.fuse_dw >= 0 && p.dw_fused[idx] == 1) {
                 st = run_dw_fused(m, p, idx);
                 if (st == FDX_ERR_UNSUPPORTED) { // forced by a test on a pair the launcher does not take
                     p.dw_fused[idx] = 2;

@@ -33,6 +33,8 @@ struct Op {
     int residual = -1;   // op whose output is added in the producer's epilogue
     int fuse_dw = -1;    // 1x1 Conv2D: the depthwise 3x3 op in front of it that one launch can absorb (fdx_dwconv_pointwise_nhwc_f32)
     int fused_into = -1; // that depthwise op: the convolution which may absorb it
+    int fuse_exp = -1;   // 1x1 Conv2D with fuse_dw >= 0: the 1x1 expansion in front of the depthwise op, if one launch can run all three (fdx_inverted_residual_nhwc_f32)
+    int exp_into = -1;   // that expansion: the projection which may absorb it
     bool dead = false;
     int consumers = 0;
 
@@ -88,7 +90,7 @@ struct Plan {
     std::vector<int> last_use;   // position in order of the last consumer
     std::vector<Block> blocks;
     std::vector<std::vector<float*>> temps; // per op: scratch placed at plan time
-    std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = one launch, 2 = two
+    std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = depthwise + projection as one launch, 2 = one launch per layer, 3 = expansion + depthwise + projection as one launch
     double flops = 0;
     ~Plan();
 };

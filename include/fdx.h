@@ -139,6 +139,21 @@ fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int h, int w, i
     const float* pw_weights_nc, const float* pw_bias, int n_out, const float* residual, const fdx_act* act, float* out);
 
 /*
+ * A whole inverted-residual block as one launch: 1x1 convolution (expansion, cin -> ce) + activation, depthwise 3x3
+ * (stride 1 or 2) + activation, 1x1 convolution (projection, ce -> n_out) + optional residual + activation; the expanded
+ * tensor stays on chip (convolution.hpp:398-429, depthwise_convolution.hpp:21-99, convolution.hpp:398-429 run back to
+ * back by the reference).  exp_weights_ec is [ce][cin], dw_weights_hwc [3][3][ce], pw_weights_nc [n_out][ce]; biases
+ * may be NULL.  The padding (pad_top, pad_left; bottom / right implied by out_h, out_w) belongs to the depthwise
+ * convolution and pads the expanded, activated tensor with zeros.  fdx_inverted_residual_supported tells whether the
+ * kernel covers a shape: cin 16 / 24 / 32, ce % 4 == 0 within the LDS budget, n_out <= 64.
+ */
+int fdx_inverted_residual_supported(int cin, int ce, int n_out, int stride);
+fdx_status fdx_inverted_residual_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* exp_weights_ec,
+    const float* exp_bias, const fdx_act* exp_act, int ce, const float* dw_weights_hwc, const float* dw_bias, int stride, int pad_top,
+    int pad_left, int out_h, int out_w, const fdx_act* dw_act, const float* pw_weights_nc, const float* pw_bias, int n_out,
+    const float* residual, const fdx_act* act, float* out);
+
+/*
  * Row-major GEMM with fused epilogue, fp32 MFMA:
  *   c[m][n] = act(alpha * sum_k a[m][k] * b_nk[n][k] + bias + residual[m][n])
  * replaces dense_layer::apply_impl (include/fdeep/layers/dense_layer.hpp:76-86; weights arrive

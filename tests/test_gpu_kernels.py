@@ -185,6 +185,59 @@ def test_dwconv_pointwise_vs_oracle(fdx, oracle, case):
     assert rel(got_r, want_r) <= TOL
 
 
+@pytest.mark.parametrize("case", [
+    # n, h, w, cin, ce, n_out, stride, padding, zero_frame: MobileNetV2's first blocks, odd sizes that leave partial tiles,
+    # an expansion that does not fill its last 32-channel slab, two projection tiles
+    (2, 16, 16, 16, 96, 24, 2, "valid", (0, 0, 1, 1)), (2, 12, 20, 24, 144, 24, 1, "same", (0, 0, 0, 0)),
+    (1, 13, 11, 24, 144, 32, 2, "valid", (0, 0, 1, 1)), (3, 9, 7, 32, 192, 32, 1, "same", (0, 0, 0, 0)),
+    (1, 10, 10, 32, 192, 64, 1, "same", (0, 0, 0, 0)), (2, 5, 3, 16, 20, 8, 1, "same", (0, 0, 0, 0)),
+    (1, 56, 56, 24, 144, 24, 1, "same", (0, 0, 0, 0)), (1, 33, 47, 16, 96, 40, 2, "same", (0, 0, 0, 0))])
+def test_inverted_residual_block_vs_oracle(fdx, oracle, case):
+    """1x1 expansion + ReLU6, depthwise 3x3 + ReLU6, 1x1 projection (+ residual) as one launch against the oracle's three
+    layers; the depthwise padding pads the expanded tensor with zeros (not with expand(0))."""
+    n, h, w, cin, ce, n_out, stride, padding, frame = case
+    say("inverted_residual", case)
+    r = rng_for("irb", case)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    we = (r.standard_normal((ce, cin)) / np.sqrt(cin)).astype(np.float32)
+    be = (r.standard_normal(ce) + 1.0).astype(np.float32)  # a bias that survives ReLU6: padding must still read zero
+    wd = r.standard_normal((ce, 3, 3)).astype(np.float32) * 0.5
+    bd = r.standard_normal(ce).astype(np.float32)
+    wp = (r.standard_normal((n_out, ce)) / np.sqrt(ce)).astype(np.float32)
+    bp = r.standard_normal(n_out).astype(np.float32)
+    zt, zl, zb, zr = frame
+
+    def reference(i, res, with_bias, final_act):
+        e = oracle.conv2d(x[i], oracle.conv2d_prepare(we.reshape(-1), ce, 1, 1, cin), be if with_bias else None, ce, 1, 1)
+        e = oracle.relu(e, 6.0, 0.0, 0.0)
+        e = np.pad(e, ((zt, zb), (zl, zr), (0, 0)))
+        d = oracle.relu(oracle.depthwise_conv2d(e, wd, bd if with_bias else None, 3, 3, (stride, stride), (1, 1), padding), 6.0, 0.0, 0.0)
+        o = oracle.conv2d(d, oracle.conv2d_prepare(wp.reshape(-1), n_out, 1, 1, ce), bp if with_bias else None, n_out, 1, 1)
+        if res is not None:
+            o = o + res[i]
+        return oracle.relu(o) if final_act else o
+
+    want = np.stack([reference(i, None, True, False) for i in range(n)])
+    got = fdx.inverted_residual(x, we, be, fdx.relu_act(6.0), wd, bd, stride, padding, fdx.relu_act(6.0), wp, bp, zero_frame=frame)
+    assert got.shape == want.shape
+    assert rel(got, want) <= TOL
+    res = r.standard_normal(want.shape).astype(np.float32)
+    want_r = np.stack([reference(i, res, False, True) for i in range(n)])
+    got_r = fdx.inverted_residual(x, we, None, fdx.relu_act(6.0), wd, None, stride, padding, fdx.relu_act(6.0), wp, None, residual=res,
+                                  act=fdx.relu_act(), zero_frame=frame)
+    assert rel(got_r, want_r) <= TOL
+
+
+def test_inverted_residual_rejects_what_it_does_not_cover(fdx):
+    assert fdx.lib.fdx_inverted_residual_supported(16, 96, 24, 2) == 1 and fdx.lib.fdx_inverted_residual_supported(24, 144, 32, 1) == 1
+    assert fdx.lib.fdx_inverted_residual_supported(20, 96, 24, 1) == 0 and fdx.lib.fdx_inverted_residual_supported(16, 96, 24, 3) == 0
+    assert fdx.lib.fdx_inverted_residual_supported(32, 192, 65, 1) == 0 and fdx.lib.fdx_inverted_residual_supported(32, 4000, 32, 1) == 0
+    x = np.zeros((1, 4, 4, 20), np.float32)
+    with pytest.raises(RuntimeError):
+        fdx.inverted_residual(x, np.zeros((8, 20), np.float32), None, None, np.zeros((8, 3, 3), np.float32), None, 1, "same", None,
+                              np.zeros((8, 8), np.float32), None)
+
+
 def test_dwconv_pointwise_rejects_what_it_does_not_cover(fdx):
     x = np.zeros((1, 4, 4, 6), np.float32)
     with pytest.raises(RuntimeError):

@@ -104,11 +104,12 @@ def test_mobilenet_v2_truncated(fdx, oracle, modelgen):
     run_both(fdx, oracle, modelgen, spec, [x])
 
 
-@pytest.mark.parametrize("mode", [1, 0])
+@pytest.mark.parametrize("mode", [2, 1, 0])
 def test_depthwise_pointwise_pairs_forced_either_way(fdx, oracle, modelgen, mode):
     """The depthwise 3x3 + 1x1 pairs of inverted-residual blocks (stride 1 and 2 with the folded ZeroPadding2D, folded
     BatchNormalization, ReLU6 in between, residual Add behind) and of SeparableConv2D, forced to run as one launch each
-    and as two: both must match the oracle.  (Left to itself a plan times both forms and keeps the faster.)"""
+    (mode 1), as two (mode 0), and with the 1x1 expansion in front taken into the same launch where the block has one
+    (mode 2): all must match the oracle.  (Left to itself a plan times the forms and keeps the fastest.)"""
     say("depthwise + pointwise pairs, forced fusion mode", mode)
     spec = modelgen.mobilenet_v2(seed=25, input_size=64, classes=20, random_bn=True, truncate=11)
     x = np.random.default_rng(18).uniform(0, 1, (5, 64, 64, 3)).astype(np.float32)
@@ -137,7 +138,7 @@ def test_mobilenet_v2_full_size_fusion_invariance(fdx, oracle, modelgen):
     js = modelgen.dumps(spec)
     outs = []
     try:
-        for mode in (1, 0, -1):
+        for mode in (2, 1, 0, -1):
             fdx.check(fdx.lib.fdx_debug_force_dw_fusion(mode))
             outs.append(fdx.Model(js, verify=False).predict([x]))
     finally:
