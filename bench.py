@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file and scaled by a plain copy of known size (a process cannot read these counters for itself; the
 # summaries under profiles/ give the commands and the raw readings).  Valid for the default configurations only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 169.1e6, "skinny_gemm, GPT-2 decode b16": 10.9e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 165.7e6, "skinny_gemm, GPT-2 decode b16": 11.0e6}
 
 
 def load_package():
@@ -315,7 +315,7 @@ def bench_gpt2(fdx, modelgen, args):
         "prefill_ms": round(prefill_ms, 3),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4), "bytes_per_step_mean": round(total_bytes / new),
-                     "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 48 of the step's 64 launches plus the LM head's striding variant)",
+                     "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 48 of the step's 63 launches plus the LM head's striding variant)",
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
         "load_seconds": round(load_s, 2),
     }
