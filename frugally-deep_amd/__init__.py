@@ -229,6 +229,34 @@ def inverted_residual(x, exp_w_ec, exp_bias, exp_act, dw_w_chw, dw_bias, stride,
     return out.to_host((n, g["out_h"], g["out_w"], n_out))
 
 
+def stem_block(x, conv_w_nkkc, conv_bias, conv_act, conv_stride, conv_padding, dw_w_chw, dw_bias, stride, padding, dw_act,
+               pw_w_nc, pw_bias, residual=None, act=None, conv_zero_frame=(0, 0, 0, 0), zero_frame=(0, 0, 0, 0)):
+    """Small convolution on the image, depthwise 3x3, 1x1 projection in one launch.  x [n,ih,iw,ic]; conv_w_nkkc
+    [ce,ek,ek,ic]; dw_w_chw [ce,3,3]; pw_w_nc [n_out,ce]; the zero frames = (top, left, bottom, right) of explicit
+    ZeroPadding2D layers in front of the convolution / the depthwise layer."""
+    x = np.ascontiguousarray(x, np.float32)
+    n, ih, iw, ic = x.shape
+    ce, ek = conv_w_nkkc.shape[0], conv_w_nkkc.shape[1]
+    ct, cl, cb, cr = conv_zero_frame
+    gc = window_geometry(ih + ct + cb, iw + cl + cr, ek, ek, conv_stride, conv_stride, conv_padding)
+    h, w = gc["out_h"], gc["out_w"]
+    zt, zl, zb, zr = zero_frame
+    g = window_geometry(h + zt + zb, w + zl + zr, 3, 3, stride, stride, padding)
+    n_out = pw_w_nc.shape[0]
+    dx, cw = DevBuf.from_host(x), DevBuf.from_host(conv_w_nkkc)
+    cbias = None if conv_bias is None else DevBuf.from_host(conv_bias)
+    dw = DevBuf.from_host(np.transpose(dw_w_chw, (1, 2, 0)))
+    db = None if dw_bias is None else DevBuf.from_host(dw_bias)
+    pw, pb = DevBuf.from_host(pw_w_nc), (None if pw_bias is None else DevBuf.from_host(pw_bias))
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * n_out)
+    check(lib.fdx_stem_block_nhwc_f32(_dp(dx), n, ih, iw, ic, _dp(cw), _dp(cbias), _act_ref(conv_act), ce, ek, conv_stride,
+                                      gc["pad_top"] + ct, gc["pad_left"] + cl, h, w, _dp(dw), _dp(db), stride, g["pad_top"] + zt,
+                                      g["pad_left"] + zl, g["out_h"], g["out_w"], _act_ref(dw_act), _dp(pw), _dp(pb), n_out, _dp(dr),
+                                      _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], n_out))
+
+
 def gemm(a, b_nk, bias=None, alpha=1.0, bias_per_row=False, residual=None, act=None):
     a, b_nk = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b_nk, np.float32)
     m, k = a.shape

@@ -18,6 +18,7 @@
 //
 // The reference computes the three layers one after the other: convolve (include/fdeep/convolution.hpp:398-429), the
 // activation, depthwise_convolve (include/fdeep/depthwise_convolution.hpp:21-99), the activation, convolve, Add.
+#include <cstring>
 #include <map>
 #include <mutex>
 
@@ -41,6 +42,10 @@ struct IrbParams {
     int ce_pad;                  // ce rounded up to the channel slab
     uint32_t in_bytes, out_bytes; // extents of input and output / residual (below 2^31)
     Act act_exp, act_dw, act_out;
+    // stem form: the first layer is an ek x ek convolution (stride es, padding ept / epl) on the image `in`
+    // [n][ih][iw][ic] with ek * ek * ic <= 32; h and w are then the extents of that convolution's output and exp_w is
+    // [ce][ek][ek][ic]
+    int ih, iw, ic, ek, es, ept, epl;
 };
 
 constexpr int IRB_TH = 4, IRB_TW = 8, IRB_TX = 4; // output tile of a wave; pixels per stencil run
@@ -73,8 +78,11 @@ __device__ __forceinline__ void irb_act(float (&v)[COUNT], const Act& a, bool cl
         apply_act_block(v, a);
 }
 
-// KIN = input channels / 8, CT = 32-column tiles of the projection, NW = waves per workgroup
-template <int STRIDE, int CT, int KIN, int NW>
+// KIN = input channels / 8, CT = 32-column tiles of the projection, NW = waves per workgroup.  STEM: the first layer is
+// a small convolution on an image of a few channels instead of a 1x1 convolution (the first block of MobileNet-like
+// networks: 3x3 / 2 on RGB, depthwise 3x3, 1x1 projection); its taps, (filter row, filter column, channel) = k < 32,
+// take the place of the input channels, and the A operand is gathered from the image tap by tap.
+template <int STRIDE, int CT, int KIN, int NW, bool STEM>
 __global__ __launch_bounds__(NW * 64) void irb_kernel(IrbParams p)
 {
     constexpr int TH = IRB_TH, TW = IRB_TW, TX = IRB_TX, KC = IRB_KC, LS = IRB_LS;
@@ -99,12 +107,20 @@ __global__ __launch_bounds__(NW * 64) void irb_kernel(IrbParams p)
             w4 = *reinterpret_cast<const f32x4*>(p.pw_w + (int64_t)nrow * ce + ch);
         *reinterpret_cast<f32x4*>(&Bs[nrow * BS + ch]) = w4;
     }
-    for (int idx = t; idx < p.ce_pad * KIN * 2; idx += NW * 64) {
-        const int row = idx / (KIN * 2), k4 = (idx % (KIN * 2)) * 4;
-        f32x4 w4 = { 0.f, 0.f, 0.f, 0.f };
-        if (row < ce)
-            w4 = *reinterpret_cast<const f32x4*>(p.exp_w + (int64_t)row * CIN + k4);
-        *reinterpret_cast<f32x4*>(&We[row * WS + k4]) = w4;
+    if (STEM) {
+        const int taps = p.ek * p.ek * p.ic;
+        for (int idx = t; idx < p.ce_pad * CIN; idx += NW * 64) {
+            const int row = idx / CIN, k = idx - row * CIN;
+            We[row * WS + k] = (row < ce && k < taps) ? p.exp_w[(int64_t)row * taps + k] : 0.f;
+        }
+    } else {
+        for (int idx = t; idx < p.ce_pad * KIN * 2; idx += NW * 64) {
+            const int row = idx / (KIN * 2), k4 = (idx % (KIN * 2)) * 4;
+            f32x4 w4 = { 0.f, 0.f, 0.f, 0.f };
+            if (row < ce)
+                w4 = *reinterpret_cast<const f32x4*>(p.exp_w + (int64_t)row * CIN + k4);
+            *reinterpret_cast<f32x4*>(&We[row * WS + k4]) = w4;
+        }
     }
     for (int idx = t; idx < 11 * p.ce_pad; idx += NW * 64) { // every per-slab operand comes from LDS: a global load per slab would stall the wave
         const int row = idx / p.ce_pad, ch = idx - row * p.ce_pad;
@@ -129,30 +145,89 @@ __global__ __launch_bounds__(NW * 64) void irb_kernel(IrbParams p)
     const bool clamp_exp = irb_is_clamp(p.act_exp), clamp_dw = irb_is_clamp(p.act_dw), clamp_out = irb_is_clamp(p.act_out);
     const int run_local = lane >> 3, q = lane & 7; // stencil item of this lane: run of the tile, channel quad of the slab
     const int orow = run_local >> 1, xrun = run_local & 1; // the run's row in the tile and which half of the row
+    // stem form: tap k = kk * 8 + fh * 4 + e of this lane in one word: bits 0-23 its byte offset from the window's
+    // first tap, bits 24-26 the filter row, 27-29 the filter column, bit 31 set for a tap beyond the filter (added to
+    // an offset it points outside every extent, and the load returns zero)
+    uint32_t tap[KIN][4];
+    if (STEM) {
+        const int taps = p.ek * p.ek * p.ic, row_taps = p.ek * p.ic;
+#pragma unroll
+        for (int kk = 0; kk < KIN; ++kk)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int k = kk * 8 + fh * 4 + e;
+                const int ky = k / row_taps, rem = k - ky * row_taps;
+                tap[kk][e] = k < taps ? (uint32_t)((ky * p.iw * p.ic + rem) * 4) | (uint32_t)ky << 24 | (uint32_t)(rem / p.ic) << 27 : OOB;
+            }
+    }
     const int wave_count = (int)gridDim.x * NW;
+    // The input pixels of a tile in MFMA operand order: row block rb, row fr is region pixel rb * 32 + fr; this lane
+    // holds channels kk * 8 + fh * 4 .. + 3 of it.  A pixel outside the image (or beyond the region) reads as zeros.
+    // (Requesting the next tile's pixels once the last slab's expansion has freed these registers was measured: slower,
+    // the longer live ranges cost more than the hidden latency gains.)
+    f32x4 a[RB][KIN];
+    auto request_pixels = [&](int tile) {
+        const int rest = tile / p.tiles_x;
+        const int tx = tile - rest * p.tiles_x;
+        const int img = rest / p.tiles_y;
+        const int ty = rest - img * p.tiles_y;
+        const int iy0 = ty * TH * STRIDE - p.pad_top, ix0 = tx * TW * STRIDE - p.pad_left;
+        const uint32_t img_off = STEM ? (uint32_t)img * (uint32_t)(p.ih * p.iw * p.ic) * 4u : (uint32_t)img * (uint32_t)(p.h * p.w * CIN) * 4u;
+        if (STEM) {
+            // every window of the region inside the image (most tiles): no test per tap
+            const int wy0 = iy0 * p.es - p.ept, wx0 = ix0 * p.es - p.epl;
+            const bool windows_inside = iy0 >= 0 && iy0 + RH <= p.h && ix0 >= 0 && ix0 + RW <= p.w && wy0 >= 0 && wx0 >= 0
+                && wy0 + (RH - 1) * p.es + p.ek <= p.ih && wx0 + (RW - 1) * p.es + p.ek <= p.iw;
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int pidx = rb * 32 + fr;
+                const int ry = pidx / RW, rx = pidx - ry * RW;
+                const int iy = iy0 + ry, ix = ix0 + rx;
+                const int by = iy * p.es - p.ept, bx = ix * p.es - p.epl; // first tap of this pixel's window
+                const uint32_t base = img_off + (uint32_t)((by * p.iw + bx) * p.ic * 4); // wraps below zero and back with the tap's offset
+                if (windows_inside) {
+#pragma unroll
+                    for (int kk = 0; kk < KIN; ++kk)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t off = pidx < PIN ? base + (tap[kk][e] & 0x80FFFFFFu) : OOB;
+                            a[rb][kk][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srd_in, (int)off, 0, 0));
+                        }
+                } else {
+                    const bool ok = pidx < PIN && iy >= 0 && iy < p.h && ix >= 0 && ix < p.w;
+#pragma unroll
+                    for (int kk = 0; kk < KIN; ++kk)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int yy = by + (int)((tap[kk][e] >> 24) & 7u), xx = bx + (int)((tap[kk][e] >> 27) & 7u);
+                            const bool tap_ok = ok && yy >= 0 && yy < p.ih && xx >= 0 && xx < p.iw;
+                            const uint32_t off = tap_ok ? base + (tap[kk][e] & 0x80FFFFFFu) : OOB;
+                            a[rb][kk][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srd_in, (int)off, 0, 0));
+                        }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int pidx = rb * 32 + fr;
+                const int ry = pidx / RW, rx = pidx - ry * RW;
+                const int iy = iy0 + ry, ix = ix0 + rx;
+                const bool ok = pidx < PIN && iy >= 0 && iy < p.h && ix >= 0 && ix < p.w;
+                const uint32_t off = ok ? img_off + (uint32_t)((iy * p.w + ix) * CIN + fh * 4) * 4u : OOB;
+#pragma unroll
+                for (int kk = 0; kk < KIN; ++kk)
+                    a[rb][kk] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)(off + (uint32_t)kk * 32u), 0, 0));
+            }
+        }
+    };
     for (int tile = (int)blockIdx.x * NW + wave; tile < p.tiles; tile += wave_count) {
+        request_pixels(tile);
         const int rest = tile / p.tiles_x;
         const int tx = tile - rest * p.tiles_x;
         const int img = rest / p.tiles_y;
         const int ty = rest - img * p.tiles_y;
         const int oy0 = ty * TH, ox0 = tx * TW;
         const int iy0 = oy0 * STRIDE - p.pad_top, ix0 = ox0 * STRIDE - p.pad_left;
-        const uint32_t img_off = (uint32_t)img * (uint32_t)(p.h * p.w * CIN) * 4u;
-
-        // the tile's input pixels in MFMA operand order: row block rb, row fr is region pixel rb * 32 + fr; this lane
-        // holds channels kk * 8 + fh * 4 .. + 3 of it.  A pixel outside the image (or beyond the region) reads as zeros.
-        f32x4 a[RB][KIN];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const int pidx = rb * 32 + fr;
-            const int ry = pidx / RW, rx = pidx - ry * RW;
-            const int iy = iy0 + ry, ix = ix0 + rx;
-            const bool ok = pidx < PIN && iy >= 0 && iy < p.h && ix >= 0 && ix < p.w;
-            const uint32_t off = ok ? img_off + (uint32_t)((iy * p.w + ix) * CIN + fh * 4) * 4u : OOB;
-#pragma unroll
-            for (int kk = 0; kk < KIN; ++kk)
-                a[rb][kk] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)(off + (uint32_t)kk * 32u), 0, 0));
-        }
         // which of the sixteen accumulator rows of a row block are pixels inside the image: element e of this lane is row
         // 8 * (e / 4) + 4 * fh + e % 4
         // (a tile whose whole region lies inside the image -- most of them -- needs no mask)
@@ -341,6 +416,66 @@ static int64_t irb_resident(K kernel, int threads, size_t lds)
     return known[lds] = (int64_t)per_cu * cus;
 }
 
+// Fills the tile counts and extents of `p` (pointers, image / grid sizes, channel counts and activations are set) and
+// launches the instantiation for (depthwise stride, projection width, K / 8 of the first layer).
+static fdx_status irb_launch(IrbParams& p, int cin, int n_out, int stride, bool stem, int64_t in_floats)
+{
+    p.tiles_x = (p.ow + IRB_TW - 1) / IRB_TW;
+    p.tiles_y = (p.oh + IRB_TH - 1) / IRB_TH;
+    FDX_REQUIRE((int64_t)p.n * p.tiles_x * p.tiles_y < (1LL << 30), "inverted_residual: too many output pixels for one launch");
+    p.tiles = p.n * p.tiles_x * p.tiles_y;
+    p.ce_pad = (p.ce + IRB_KC - 1) / IRB_KC * IRB_KC;
+    FDX_REQUIRE(in_floats * 4 < (1LL << 31), "inverted_residual: input tensor beyond 2 GiB");
+    p.in_bytes = (uint32_t)(in_floats * 4);
+    FDX_REQUIRE((int64_t)p.n * p.oh * p.ow * n_out * 4 < (1LL << 31), "inverted_residual: output tensor beyond 2 GiB");
+    p.out_bytes = (uint32_t)((int64_t)p.n * p.oh * p.ow * n_out * 4);
+    const int ct = (n_out + 31) / 32, kin = cin / 8;
+    const int nw = irb_waves(cin, p.ce, n_out, stride);
+    const size_t lds = irb_lds_bytes(cin, p.ce, n_out, stride, nw);
+    const int64_t want = ((int64_t)p.tiles + nw - 1) / nw;
+    bool launched = false;
+#define FDX_IRB_L(S_, CT_, KIN_, NW_, ST_)                                                                                \
+    {                                                                                                                     \
+        const int64_t resident = irb_resident(irb_kernel<S_, CT_, KIN_, NW_, ST_>, NW_ * 64, lds);                        \
+        if (resident > 0) {                                                                                               \
+            const unsigned grid = (unsigned)(want < resident ? want : resident);                                          \
+            hipLaunchKernelGGL((irb_kernel<S_, CT_, KIN_, NW_, ST_>), dim3(grid), dim3(NW_ * 64), lds, stream(), p);      \
+            launched = true;                                                                                              \
+        }                                                                                                                 \
+    }
+#define FDX_IRB_W(S_, CT_, KIN_, ST_)                                                                                     \
+    {                                                                                                                     \
+        if (nw == 8)                                                                                                      \
+            FDX_IRB_L(S_, CT_, KIN_, 8, ST_)                                                                              \
+        else                                                                                                              \
+            FDX_IRB_L(S_, CT_, KIN_, 4, ST_)                                                                              \
+    }
+#define FDX_IRB_K(S_, CT_)                                                                                                \
+    {                                                                                                                     \
+        if (stem)                                                                                                         \
+            FDX_IRB_W(S_, CT_, 4, true)                                                                                   \
+        else if (kin == 2)                                                                                                \
+            FDX_IRB_W(S_, CT_, 2, false)                                                                                  \
+        else if (kin == 3)                                                                                                \
+            FDX_IRB_W(S_, CT_, 3, false)                                                                                  \
+        else                                                                                                              \
+            FDX_IRB_W(S_, CT_, 4, false)                                                                                  \
+    }
+    if (stride == 1) {
+        if (ct == 1) FDX_IRB_K(1, 1) else FDX_IRB_K(1, 2)
+    } else {
+        if (ct == 1) FDX_IRB_K(2, 1) else FDX_IRB_K(2, 2)
+    }
+#undef FDX_IRB_K
+#undef FDX_IRB_W
+#undef FDX_IRB_L
+    if (!launched) {
+        set_error("inverted_residual: the kernel's LDS request was refused");
+        return FDX_ERR_UNSUPPORTED;
+    }
+    return FDX_OK;
+}
+
 static bool al16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
 } // namespace fdx
@@ -373,67 +508,69 @@ extern "C" fdx_status fdx_inverted_residual_nhwc_f32(const float* in, int n, int
     FDX_REQUIRE(pad_top >= 0 && pad_left >= 0 && (int64_t)(out_h - 1) * stride - pad_top < h && (int64_t)(out_w - 1) * stride - pad_left < w,
         "inverted_residual: output size does not fit the input");
     IrbParams p;
+    std::memset(&p, 0, sizeof p);
     p.in = in; p.exp_w = exp_weights_ec; p.exp_b = exp_bias; p.dw_w = dw_weights_hwc; p.dw_b = dw_bias; p.pw_w = pw_weights_nc;
     p.pw_b = pw_bias; p.residual = residual; p.out = out;
     p.n = n; p.h = h; p.w = w; p.ce = ce; p.pad_top = pad_top; p.pad_left = pad_left; p.oh = out_h; p.ow = out_w; p.N = n_out;
-    p.tiles_x = (out_w + IRB_TW - 1) / IRB_TW;
-    p.tiles_y = (out_h + IRB_TH - 1) / IRB_TH;
-    FDX_REQUIRE((int64_t)n * p.tiles_x * p.tiles_y < (1LL << 30), "inverted_residual: too many output pixels for one launch");
-    p.tiles = n * p.tiles_x * p.tiles_y;
-    p.ce_pad = (ce + IRB_KC - 1) / IRB_KC * IRB_KC;
-    FDX_REQUIRE((int64_t)n * h * w * cin * 4 < (1LL << 31), "inverted_residual: input tensor beyond 2 GiB");
-    p.in_bytes = (uint32_t)((int64_t)n * h * w * cin * 4);
-    FDX_REQUIRE((int64_t)n * out_h * out_w * n_out * 4 < (1LL << 31), "inverted_residual: output tensor beyond 2 GiB");
-    p.out_bytes = (uint32_t)((int64_t)n * out_h * out_w * n_out * 4);
     p.act_exp = make_act(exp_act);
     p.act_dw = make_act(dw_act);
     p.act_out = make_act(act);
-    const int ct = (n_out + 31) / 32, kin = cin / 8;
-    const int nw = irb_waves(cin, ce, n_out, stride);
-    const size_t lds = irb_lds_bytes(cin, ce, n_out, stride, nw);
-    const int64_t want = ((int64_t)p.tiles + nw - 1) / nw;
-    bool launched = false;
     profile_begin();
-#define FDX_IRB_L(S_, CT_, KIN_, NW_)                                                                                     \
-    {                                                                                                                     \
-        const int64_t resident = irb_resident(irb_kernel<S_, CT_, KIN_, NW_>, NW_ * 64, lds);                             \
-        if (resident > 0) {                                                                                               \
-            const unsigned grid = (unsigned)(want < resident ? want : resident);                                          \
-            hipLaunchKernelGGL((irb_kernel<S_, CT_, KIN_, NW_>), dim3(grid), dim3(NW_ * 64), lds, stream(), p);           \
-            launched = true;                                                                                              \
-        }                                                                                                                 \
-    }
-#define FDX_IRB_W(S_, CT_, KIN_)                                                                                          \
-    {                                                                                                                     \
-        if (nw == 8)                                                                                                      \
-            FDX_IRB_L(S_, CT_, KIN_, 8)                                                                                   \
-        else                                                                                                              \
-            FDX_IRB_L(S_, CT_, KIN_, 4)                                                                                   \
-    }
-#define FDX_IRB_K(S_, CT_)                                                                                                \
-    {                                                                                                                     \
-        if (kin == 2)                                                                                                     \
-            FDX_IRB_W(S_, CT_, 2)                                                                                         \
-        else if (kin == 3)                                                                                                \
-            FDX_IRB_W(S_, CT_, 3)                                                                                         \
-        else                                                                                                              \
-            FDX_IRB_W(S_, CT_, 4)                                                                                         \
-    }
-    if (stride == 1) {
-        if (ct == 1) FDX_IRB_K(1, 1) else FDX_IRB_K(1, 2)
-    } else {
-        if (ct == 1) FDX_IRB_K(2, 1) else FDX_IRB_K(2, 2)
-    }
-#undef FDX_IRB_K
-#undef FDX_IRB_W
-#undef FDX_IRB_L
-    if (!launched) {
-        set_error("inverted_residual: the kernel's LDS request was refused");
-        return FDX_ERR_UNSUPPORTED;
-    }
+    const fdx_status st = irb_launch(p, cin, n_out, stride, false, (int64_t)n * h * w * cin);
+    if (st != FDX_OK)
+        return st;
     const double pix_in = (double)n * h * w, pix_out = (double)n * out_h * out_w;
     profile_end("inverted_residual_f32", 2.0 * pix_in * cin * ce + 2.0 * pix_out * ce * n_out,
         4.0 * (pix_in * cin + pix_out * n_out * (residual ? 2.0 : 1.0) + (double)ce * (cin + 9.0 + n_out)));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+extern "C" int fdx_stem_block_supported(int ic, int ek, int ce, int n_out, int stride)
+{
+    return ic > 0 && ek > 0 && ek <= 5 && ek * ek * ic <= 32 && ce > 0 && ce % 4 == 0 && n_out > 0 && n_out <= IRB_NP && (stride == 1 || stride == 2)
+        && irb_waves(32, ce, n_out, stride) > 0;
+}
+
+extern "C" fdx_status fdx_stem_block_nhwc_f32(const float* in, int n, int ih, int iw, int ic, const float* conv_weights_nk,
+    const float* conv_bias, const fdx_act* conv_act, int ce, int ek, int conv_stride, int conv_pad_top, int conv_pad_left, int h, int w,
+    const float* dw_weights_hwc, const float* dw_bias, int stride, int pad_top, int pad_left, int out_h, int out_w, const fdx_act* dw_act,
+    const float* pw_weights_nc, const float* pw_bias, int n_out, const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(in && conv_weights_nk && dw_weights_hwc && pw_weights_nc && out, "stem_block: null pointer");
+    FDX_REQUIRE(n > 0 && ih > 0 && iw > 0 && h > 0 && w > 0 && out_h > 0 && out_w > 0 && conv_stride > 0, "stem_block: bad shape");
+    if (!fdx_stem_block_supported(ic, ek, ce, n_out, stride)) {
+        set_error("stem_block: needs a square filter with at most 32 taps (rows x columns x channels), convolution channels %% 4 == 0 "
+                  "that fit the LDS, at most %d output channels and depthwise stride 1 or 2", IRB_NP);
+        return FDX_ERR_UNSUPPORTED;
+    }
+    FDX_REQUIRE_EPILOGUE_ACT(conv_act);
+    FDX_REQUIRE_EPILOGUE_ACT(dw_act);
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    FDX_REQUIRE(al16(dw_weights_hwc) && al16(pw_weights_nc) && (!dw_bias || al16(dw_bias)), "stem_block: depthwise and projection operands "
+        "must be 16-byte aligned");
+    FDX_REQUIRE(conv_pad_top >= 0 && conv_pad_left >= 0 && conv_pad_top < 256 && conv_pad_left < 256
+            && (int64_t)(h - 1) * conv_stride - conv_pad_top < ih && (int64_t)(w - 1) * conv_stride - conv_pad_left < iw,
+        "stem_block: the convolution's output size does not fit the image");
+    FDX_REQUIRE(pad_top >= 0 && pad_left >= 0 && (int64_t)(out_h - 1) * stride - pad_top < h && (int64_t)(out_w - 1) * stride - pad_left < w,
+        "stem_block: output size does not fit the convolution's output");
+    FDX_REQUIRE((int64_t)iw * ic * ek * 4 < (1LL << 24), "stem_block: image rows too long");
+    IrbParams p;
+    std::memset(&p, 0, sizeof p);
+    p.in = in; p.exp_w = conv_weights_nk; p.exp_b = conv_bias; p.dw_w = dw_weights_hwc; p.dw_b = dw_bias; p.pw_w = pw_weights_nc;
+    p.pw_b = pw_bias; p.residual = residual; p.out = out;
+    p.n = n; p.h = h; p.w = w; p.ce = ce; p.pad_top = pad_top; p.pad_left = pad_left; p.oh = out_h; p.ow = out_w; p.N = n_out;
+    p.ih = ih; p.iw = iw; p.ic = ic; p.ek = ek; p.es = conv_stride; p.ept = conv_pad_top; p.epl = conv_pad_left;
+    p.act_exp = make_act(conv_act);
+    p.act_dw = make_act(dw_act);
+    p.act_out = make_act(act);
+    profile_begin();
+    const fdx_status st = irb_launch(p, 32, n_out, stride, true, (int64_t)n * ih * iw * ic);
+    if (st != FDX_OK)
+        return st;
+    const double pix_mid = (double)n * h * w, pix_out = (double)n * out_h * out_w;
+    profile_end("stem_block_f32", 2.0 * pix_mid * ek * ek * ic * ce + 2.0 * pix_out * ce * n_out,
+        4.0 * ((double)n * ih * iw * ic + pix_out * n_out * (residual ? 2.0 : 1.0) + (double)ce * (ek * ek * ic + 9.0 + n_out)));
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }

@@ -1240,10 +1240,14 @@ namespace {
                 continue;
             Op& e = m.ops[d.in[0]];
             const bool act_ok = e.act.kind == FDX_ACT_NONE || e.act.kind == FDX_ACT_RELU || e.act.kind == FDX_ACT_GELU;
-            if (!e.dead && e.kind == OpKind::Conv2D && e.kh == 1 && e.kw == 1 && e.sy == 1 && e.sx == 1 && !e.softmax && e.residual < 0
-                && e.consumers == 1 && e.fuse_dw < 0 && e.exp_into < 0 && !e.zp[0] && !e.zp[1] && !e.zp[2] && !e.zp[3] && act_ok
-                && !e.hw.empty() && e.cout > 0 && e.hw[0].size() % (size_t)e.cout == 0
-                && fdx_inverted_residual_supported((int)(e.hw[0].size() / (size_t)e.cout), e.cout, c.cout, d.sy)) {
+            if (e.dead || e.kind != OpKind::Conv2D || e.softmax || e.residual >= 0 || e.consumers != 1 || e.fuse_dw >= 0 || e.exp_into >= 0
+                || !act_ok || e.hw.empty() || e.cout <= 0 || e.hw[0].size() % (size_t)e.cout != 0)
+                continue;
+            const bool pointwise = e.kh == 1 && e.kw == 1 && e.sy == 1 && e.sx == 1 && !e.zp[0] && !e.zp[1] && !e.zp[2] && !e.zp[3];
+            // ... or the small convolution on the image a MobileNet-like network starts with (3x3 / 2 on RGB)
+            const bool stem = !pointwise && e.kh == e.kw && e.sy == e.sx && e.dy == 1 && e.dx == 1 && e.n_in > 0
+                && fdx_stem_block_supported(e.n_in, e.kh, e.cout, c.cout, d.sy);
+            if ((pointwise && fdx_inverted_residual_supported((int)(e.hw[0].size() / (size_t)e.cout), e.cout, c.cout, d.sy)) || stem) {
                 c.fuse_exp = d.in[0];
                 e.exp_into = (int)i;
             }
@@ -2093,12 +2097,28 @@ namespace {
         const Shape& is = p.shapes[e.in[0]];
         if (is.size() != 3)
             return FDX_ERR_UNSUPPORTED;
-        const int h = (int)is[0], w = (int)is[1], cin = (int)is[2];
+        int h = (int)is[0], w = (int)is[1];
+        const int cin = (int)is[2];
         int g[6];
-        fdx_status st = window(h, w, d, true, g);
+        fdx_status st;
+        const fdx_act a0 = to_c(e.act), a1 = to_c(d.act), a2 = to_c(c.act);
+        if (e.kh != 1 || e.sy != 1) { // a small convolution on the image in place of the 1x1 expansion
+            int ge[6];
+            if ((st = window(h, w, e, true, ge)) != FDX_OK)
+                return st;
+            const int ih = h, iw = w;
+            h = ge[4];
+            w = ge[5];
+            if ((st = window(h, w, d, true, g)) != FDX_OK)
+                return st;
+            return fdx_stem_block_nhwc_f32(p.out[e.in[0]], p.batch, ih, iw, cin, e.dw[0], e.dw[1], e.act.kind == FDX_ACT_NONE ? nullptr : &a0,
+                e.cout, e.kh, e.sy, ge[0] + e.zp[0], ge[2] + e.zp[2], h, w, d.dw[0], d.dw[1], d.sy, g[0] + d.zp[0], g[2] + d.zp[2], g[4], g[5],
+                d.act.kind == FDX_ACT_NONE ? nullptr : &a1, c.dw[0], c.dw[1], c.cout, c.residual >= 0 ? p.out[c.residual] : nullptr,
+                c.act.kind == FDX_ACT_NONE ? nullptr : &a2, p.out[idx]);
+        }
+        st = window(h, w, d, true, g);
         if (st != FDX_OK)
             return st;
-        const fdx_act a0 = to_c(e.act), a1 = to_c(d.act), a2 = to_c(c.act);
         return fdx_inverted_residual_nhwc_f32(p.out[e.in[0]], p.batch, h, w, cin, e.dw[0], e.dw[1], e.act.kind == FDX_ACT_NONE ? nullptr : &a0,
             e.cout, d.dw[0], d.dw[1], d.sy, g[0] + d.zp[0], g[2] + d.zp[2], g[4], g[5], d.act.kind == FDX_ACT_NONE ? nullptr : &a1, c.dw[0],
             c.dw[1], c.cout, c.residual >= 0 ? p.out[c.residual] : nullptr, c.act.kind == FDX_ACT_NONE ? nullptr : &a2, p.out[idx]);
@@ -2270,9 +2290,30 @@ namespace {
         Plan* p = nullptr;
         if ((st = get_plan(m, batch, shapes, &p)) != FDX_OK)
             return st;
+        // Inputs that already lie in device memory are read where they are (16-byte aligned ones: the kernels' vector
+        // loads need that): the input op and every view of it point at the caller's buffer for this call.  Nothing
+        // writes an input buffer, and the plan is used under the model's lock.
+        struct Restore {
+            Plan* plan;
+            std::vector<std::pair<int, float*>> saved;
+            ~Restore()
+            {
+                for (auto& kv : saved)
+                    plan->out[kv.first] = kv.second;
+            }
+        } restore{ p, {} };
         for (size_t i = 0; i < m->inputs.size(); ++i) {
             FDX_REQUIRE(in[i], "predict: null input %zu", i);
             const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(shapes[i]);
+            if (in_on_device && (reinterpret_cast<uintptr_t>(in[i]) & 15) == 0) {
+                float* own = p->out[m->inputs[i]];
+                for (size_t k = 0; k < p->out.size(); ++k)
+                    if (p->out[k] == own && own) {
+                        restore.saved.emplace_back((int)k, own);
+                        p->out[k] = const_cast<float*>(in[i]);
+                    }
+                continue;
+            }
             FDX_HIP(hipMemcpyAsync(p->out[m->inputs[i]], in[i], bytes, in_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
                 stream()));
         }

@@ -154,6 +154,22 @@ fdx_status fdx_inverted_residual_nhwc_f32(const float* in, int n, int h, int w, 
     const float* residual, const fdx_act* act, float* out);
 
 /*
+ * The first block of a MobileNet-like network as one launch: a small convolution on the image (ek x ek taps on ic
+ * channels with ek * ek * ic <= 32, e.g. 3x3 on RGB; stride conv_stride, zero padding conv_pad_top / conv_pad_left) +
+ * activation, depthwise 3x3 (stride 1 or 2) + activation, 1x1 convolution (ce -> n_out) + optional residual +
+ * activation.  The convolution's output (h x w x ce, the widest tensor of such a network) stays on chip; the reference
+ * runs convolve (convolution.hpp:398-429), depthwise_convolve (depthwise_convolution.hpp:21-99) and convolve one
+ * after the other.  conv_weights_nk is [ce][ek][ek][ic]; the other operands are those of
+ * fdx_inverted_residual_nhwc_f32, (h, w) being the extents of the convolution's output, which the depthwise
+ * convolution pads with zeros.  fdx_stem_block_supported tells whether the kernel covers a shape.
+ */
+int fdx_stem_block_supported(int ic, int ek, int ce, int n_out, int stride);
+fdx_status fdx_stem_block_nhwc_f32(const float* in, int n, int ih, int iw, int ic, const float* conv_weights_nk,
+    const float* conv_bias, const fdx_act* conv_act, int ce, int ek, int conv_stride, int conv_pad_top, int conv_pad_left, int h, int w,
+    const float* dw_weights_hwc, const float* dw_bias, int stride, int pad_top, int pad_left, int out_h, int out_w, const fdx_act* dw_act,
+    const float* pw_weights_nc, const float* pw_bias, int n_out, const float* residual, const fdx_act* act, float* out);
+
+/*
  * Row-major GEMM with fused epilogue, fp32 MFMA:
  *   c[m][n] = act(alpha * sum_k a[m][k] * b_nk[n][k] + bias + residual[m][n])
  * replaces dense_layer::apply_impl (include/fdeep/layers/dense_layer.hpp:76-86; weights arrive
@@ -367,7 +383,9 @@ fdx_status fdx_model_io_shape(const fdx_model* m, int is_output, int index, int*
  * launch sequence.  in[i] points at batch * volume(in_dims[i]) floats (sample-major); in_dims holds
  * 5 right-aligned dims per input and in_ranks its rank (the reference rejects a rank mismatch,
  * tensor_shape.hpp:246-250).  Outputs: out[i] receives batch * volume floats; out_dims/out_ranks are
- * written per output.  Host-pointer and device-pointer variants.
+ * written per output.  Host-pointer and device-pointer variants.  The device-pointer variant returns with its work
+ * queued on the library's stream (fdx_sync waits for it) and reads inputs that are 16-byte aligned where they lie
+ * (others are copied first): such an input must stay unchanged until that work has completed.
  */
 fdx_status fdx_model_predict(fdx_model* m, int batch, const float* const* in, const int64_t* in_dims,
     const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks);

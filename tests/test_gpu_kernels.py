@@ -238,6 +238,66 @@ def test_inverted_residual_rejects_what_it_does_not_cover(fdx):
                               np.zeros((8, 8), np.float32), None)
 
 
+@pytest.mark.parametrize("case", [
+    # n, ih, iw, ic, ek, conv stride, conv padding, conv frame, ce, n_out, depthwise stride, depthwise padding, depthwise frame
+    (2, 32, 32, 3, 3, 2, "same", (0, 0, 0, 0), 32, 16, 1, "same", (0, 0, 0, 0)),     # MobileNetV2's first block
+    (2, 33, 29, 3, 3, 2, "valid", (0, 0, 1, 1), 32, 16, 1, "same", (0, 0, 0, 0)),    # explicit bottom / right padding
+    (1, 20, 24, 1, 5, 1, "same", (0, 0, 0, 0), 16, 24, 2, "same", (0, 0, 0, 0)),     # 25 taps on one channel, stride-2 stencil
+    (2, 17, 19, 4, 2, 2, "valid", (1, 2, 0, 0), 40, 40, 2, "valid", (0, 0, 1, 1)),   # two slabs, two projection tiles
+    (1, 9, 40, 2, 3, 1, "same", (0, 0, 0, 0), 64, 8, 1, "valid", (0, 0, 0, 0)),
+    (3, 70, 45, 3, 3, 2, "same", (0, 0, 0, 0), 32, 16, 1, "same", (0, 0, 0, 0)),     # tiles whose windows lie inside the image
+])
+def test_stem_block_vs_oracle(fdx, oracle, case):
+    """Small convolution + ReLU6, depthwise 3x3 + ReLU6, 1x1 projection (+ residual) as one launch against the oracle's
+    three layers; both paddings (the convolution's on the image, the stencil's on the convolution's output) read zeros."""
+    n, ih, iw, ic, ek, cs, cpad, cframe, ce, n_out, stride, padding, frame = case
+    say("stem_block", case)
+    r = rng_for("stem", case)
+    x = r.standard_normal((n, ih, iw, ic)).astype(np.float32)
+    wc = (r.standard_normal((ce, ek, ek, ic)) / np.sqrt(ek * ek * ic)).astype(np.float32)
+    bc = (r.standard_normal(ce) + 1.0).astype(np.float32)
+    wd = r.standard_normal((ce, 3, 3)).astype(np.float32) * 0.5
+    bd = r.standard_normal(ce).astype(np.float32)
+    wp = (r.standard_normal((n_out, ce)) / np.sqrt(ce)).astype(np.float32)
+    bp = r.standard_normal(n_out).astype(np.float32)
+    ct, cl, cb, cr = cframe
+    zt, zl, zb, zr = frame
+
+    def reference(i, res, with_bias, final_act):
+        img = np.pad(x[i], ((ct, cb), (cl, cr), (0, 0)))
+        e = oracle.conv2d(img, oracle.conv2d_prepare(wc.reshape(-1), ce, ek, ek, ic), bc if with_bias else None, ce, ek, ek, (cs, cs),
+                          (1, 1), cpad)
+        e = oracle.relu(e, 6.0, 0.0, 0.0)
+        e = np.pad(e, ((zt, zb), (zl, zr), (0, 0)))
+        d = oracle.relu(oracle.depthwise_conv2d(e, wd, bd if with_bias else None, 3, 3, (stride, stride), (1, 1), padding), 6.0, 0.0, 0.0)
+        o = oracle.conv2d(d, oracle.conv2d_prepare(wp.reshape(-1), n_out, 1, 1, ce), bp if with_bias else None, n_out, 1, 1)
+        if res is not None:
+            o = o + res[i]
+        return oracle.relu(o) if final_act else o
+
+    want = np.stack([reference(i, None, True, False) for i in range(n)])
+    got = fdx.stem_block(x, wc, bc, fdx.relu_act(6.0), cs, cpad, wd, bd, stride, padding, fdx.relu_act(6.0), wp, bp,
+                         conv_zero_frame=cframe, zero_frame=frame)
+    assert got.shape == want.shape
+    assert rel(got, want) <= TOL
+    res = r.standard_normal(want.shape).astype(np.float32)
+    want_r = np.stack([reference(i, res, False, True) for i in range(n)])
+    got_r = fdx.stem_block(x, wc, None, fdx.relu_act(6.0), cs, cpad, wd, None, stride, padding, fdx.relu_act(6.0), wp, None, residual=res,
+                           act=fdx.relu_act(), conv_zero_frame=cframe, zero_frame=frame)
+    assert rel(got_r, want_r) <= TOL
+
+
+def test_stem_block_rejects_what_it_does_not_cover(fdx):
+    assert fdx.lib.fdx_stem_block_supported(3, 3, 32, 16, 1) == 1 and fdx.lib.fdx_stem_block_supported(1, 5, 16, 24, 2) == 1
+    assert fdx.lib.fdx_stem_block_supported(4, 3, 32, 16, 1) == 0  # 36 taps
+    assert fdx.lib.fdx_stem_block_supported(3, 3, 30, 16, 1) == 0 and fdx.lib.fdx_stem_block_supported(3, 3, 32, 65, 1) == 0
+    assert fdx.lib.fdx_stem_block_supported(3, 3, 32, 16, 3) == 0
+    x = np.zeros((1, 8, 8, 4), np.float32)
+    with pytest.raises(RuntimeError):
+        fdx.stem_block(x, np.zeros((8, 3, 3, 4), np.float32), None, None, 1, "same", np.zeros((8, 3, 3), np.float32), None, 1, "same", None,
+                       np.zeros((8, 8), np.float32), None)
+
+
 def test_dwconv_pointwise_rejects_what_it_does_not_cover(fdx):
     x = np.zeros((1, 4, 4, 6), np.float32)
     with pytest.raises(RuntimeError):

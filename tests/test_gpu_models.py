@@ -168,6 +168,38 @@ def test_gpt2_tiny_predict_is_unmasked(fdx, oracle, modelgen):
     run_both(fdx, oracle, modelgen, spec, [ids, pos])
 
 
+def test_predict_from_device_pointers(fdx, modelgen):
+    """fdx_model_predict_dev reads 16-byte aligned device inputs where they lie and copies misaligned ones first; both
+    return what the host-pointer call returns, also when the same plan is used with another buffer afterwards, with the
+    first buffer overwritten in between, and with host inputs again."""
+    import ctypes
+    say("predict_dev aligned / misaligned inputs")
+    model = fdx.Model(modelgen.dumps(modelgen.small_cnn()))
+    r = np.random.default_rng(77)
+    xs = [r.uniform(-1, 1, (9, 32, 32, 3)).astype(np.float32) for _ in range(3)]
+    want = [model.predict([x])[0] for x in xs]
+    out = fdx.DevBuf(want[0].nbytes)
+    fp = ctypes.POINTER(ctypes.c_float)
+
+    def run(ptr_value):
+        ip = (fp * 1)(ctypes.cast(ctypes.c_void_p(ptr_value), fp))
+        op = (fp * 1)(fdx._dp(out))
+        dims, ranks = model._dims([(32, 32, 3)])
+        fdx.check(fdx.lib.fdx_model_predict_dev(model._h, 9, ip, dims, ranks, op, None, None))
+        fdx.sync()
+        return out.to_host(want[0].shape)
+
+    a = fdx.DevBuf.from_host(xs[0])
+    assert np.array_equal(run(a.ptr.value), want[0])
+    b = fdx.DevBuf(xs[1].nbytes + 16)  # the same data four bytes off a 16-byte boundary
+    fdx.check(fdx.lib.fdx_h2d(ctypes.c_void_p(b.ptr.value + 4), xs[1].ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(xs[1].nbytes)))
+    assert np.array_equal(run(b.ptr.value + 4), want[1])
+    fdx.check(fdx.lib.fdx_h2d(a.ptr, xs[2].ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(xs[2].nbytes)))
+    assert np.array_equal(run(a.ptr.value), want[2])
+    assert np.array_equal(model.predict([xs[0]])[0], want[0])
+    assert np.array_equal(run(b.ptr.value + 4), want[1])
+
+
 def test_input_shape_errors(fdx, modelgen):
     say("shape errors")
     model = fdx.Model(modelgen.dumps(modelgen.small_cnn()))
