@@ -229,6 +229,25 @@ def inverted_residual(x, exp_w_ec, exp_bias, exp_act, dw_w_chw, dw_bias, stride,
     return out.to_host((n, g["out_h"], g["out_w"], n_out))
 
 
+def conv2d_winograd(x, w, bias, padding="same", residual=None, act=None):
+    """3x3 stride-1 convolution in the Winograd F(2x2, 3x3) form.  x [n,h,w,cin]; w in converted-JSON order [cout,3,3,cin]."""
+    x, w = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(w, np.float32)
+    n, h, wd, cin = x.shape
+    cout = w.shape[0]
+    assert w.shape[1:] == (3, 3, cin)
+    g = window_geometry(h, wd, 3, 3, 1, 1, padding)
+    lib.fdx_conv2d_winograd_weight_floats.restype = ctypes.c_size_t
+    u = np.empty(lib.fdx_conv2d_winograd_weight_floats(cout, cin), np.float32)
+    check(lib.fdx_conv2d_winograd_prepare(w.ctypes.data_as(c_float_p), cout, cin, u.ctypes.data_as(c_float_p)))
+    dx, du = DevBuf.from_host(x), DevBuf.from_host(u)
+    db = None if bias is None else DevBuf.from_host(bias)
+    dr = None if residual is None else DevBuf.from_host(residual)
+    out = DevBuf(4 * n * g["out_h"] * g["out_w"] * cout)
+    check(lib.fdx_conv2d_winograd_nhwc_f32(_dp(dx), n, h, wd, cin, _dp(du), _dp(db), cout, g["pad_top"], g["pad_left"], g["out_h"],
+                                           g["out_w"], _dp(dr), _act_ref(act), _dp(out)))
+    return out.to_host((n, g["out_h"], g["out_w"], cout))
+
+
 def stem_block(x, conv_w_nkkc, conv_bias, conv_act, conv_stride, conv_padding, dw_w_chw, dw_bias, stride, padding, dw_act,
                pw_w_nc, pw_bias, residual=None, act=None, conv_zero_frame=(0, 0, 0, 0), zero_frame=(0, 0, 0, 0)):
     """Small convolution on the image, depthwise 3x3, 1x1 projection in one launch.  x [n,ih,iw,ic]; conv_w_nkkc

@@ -1,0 +1,302 @@
+// 3x3 stride-1 convolution in the Winograd F(2x2, 3x3) form on fp32 MFMA, gfx950.
+//
+// A 3x3 convolution spends 9 multiply-adds per output pixel and channel pair.  Computed on 2x2 output tiles from their
+// 4x4 input patches d with the filter g moved into the same 4x4 domain once at load,
+//     Y = At [ sum_c (G g_c Gt) o (Bt d_c B) ] A          (o = element by element),
+// it spends 16 per four pixels, 2.25 times fewer: for each of the 16 positions of the 4x4 domain the sum over the input
+// channels is a GEMM  M_p[tile][cout] = sum_c V_p[tile][c] * U_p[c][cout],  and those run on the matrix cores.
+//
+// A workgroup of four waves owns 32 tiles (of any images, in raster order) and NT * 32 output channels.  Wave xi owns
+// row xi of the 4x4 domain, i.e. the four positions (xi, 0..3):
+//   * per step of 8 input channels a lane takes, for its tile (lane % 32) and its four channels (lane / 32), the two
+//     patch rows that row xi of Bt combines, four pixels each, straight from global memory (a pixel outside the image
+//     is an out-of-range buffer offset and reads as zero: the convolution's padding), forms the four transformed
+//     values with 8 additions per channel, and has the A operands of its four GEMMs in registers -- no LDS, no barrier;
+//   * the B operands come from the transformed filter, laid out at load so that what a wave takes for one position,
+//     one column tile and one step is one contiguous kilobyte: U[cout / 32][cin / 8][position][lane][4], lane =
+//     32 * (channel / 4 % 2) + cout % 32;
+//   * 4 positions x NT column tiles of 32x32x2 MFMA accumulate over the input channels.
+// At the end each wave folds its four positions with At along the row (two values per tile and channel), the four
+// waves meet once in LDS, and wave (i, j) combines the rows with At along the column into output pixel (i, j) of
+// every tile, adds bias and residual, applies the activation and stores 16-byte pieces.
+//
+// Transform matrices (Lavin & Gray, "Fast Algorithms for Convolutional Neural Networks", F(2x2, 3x3)):
+//   Bt = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]   G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]   At = [1 1 1 0; 0 1 -1 -1]
+// Their entries are 0, +-1 and +-1/2: the result differs from the direct sum by a few more roundings (measured against
+// the reference's order of summation in the tests), not by a conditioning problem as the larger tiles have.
+//
+// Replaces convolve for 3x3 filters, stride 1, no dilation (include/fdeep/convolution.hpp:398-429, :107-160).
+#include <cstring>
+#include <vector>
+
+#include "common.hpp"
+#include "igemm_params.hpp"
+
+namespace fdx {
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+struct WinoParams {
+    const float* in;       // [n][h][w][cin]
+    const float* u;        // [cout / 32][cin / 8][16][64][4], see fdx_conv2d_winograd_prepare
+    const float* bias;     // [cout] or null
+    const float* residual; // like out, or null
+    float* out;            // [n][oh][ow][cout]
+    int n, h, w, cin, cout, pad_top, pad_left, oh, ow;
+    int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
+    uint32_t in_bytes, out_bytes, u_bytes;
+    Act act;
+};
+
+constexpr int WINO_TM = 32;  // tiles per workgroup
+constexpr int WINO_PAD = 4;  // padding of an LDS row of the exchange
+
+// NT = 32-column tiles of the output channels per workgroup
+template <int NT, int XI>
+__device__ __forceinline__ void wino_main(const WinoParams& p, const uint32_t (&pix_off)[2][4], const uint32_t (&u_off)[4][NT],
+    f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u)
+{
+    const int steps = p.cin / 8;
+    auto load_a = [&](f32x4 (&d)[2][4], int step) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                d[r][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], step * 32, 0));
+    };
+    auto load_b = [&](f32x4 (&b)[4][NT], int step) {
+#pragma unroll
+        for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                b[nu][nt] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], step * 16384, 0));
+    };
+    f32x4 d[2][4], b[4][NT];
+    load_a(d, 0);
+    load_b(b, 0);
+    for (int step = 0; step < steps; ++step) {
+        // row xi of Bt over the patch rows, then Bt again over the columns
+        f32x4 v[4];
+        {
+            f32x4 t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                t[j] = XI == 1 ? d[0][j] + d[1][j] : (XI == 2 ? d[1][j] - d[0][j] : d[0][j] - d[1][j]);
+            v[0] = t[0] - t[2];
+            v[1] = t[1] + t[2];
+            v[2] = t[2] - t[1];
+            v[3] = t[1] - t[3];
+        }
+        f32x4 bc[4][NT];
+#pragma unroll
+        for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                bc[nu][nt] = b[nu][nt];
+        if (step + 1 < steps) { // the next step's operands travel while this step multiplies
+            load_a(d, step + 1);
+            load_b(b, step + 1);
+        }
+#pragma unroll
+        for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], bc[nu][nt][e], acc[nu][nt], 0, 0, 0);
+    }
+}
+
+template <int NT>
+__global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
+{
+    constexpr int NC = NT * 32, LS = NC + WINO_PAD;
+    extern __shared__ __attribute__((aligned(16))) float lds[]; // [4 rows][2][32 tiles][LS], then 32 tile descriptors
+    const int t = threadIdx.x, lane = t & 63, xi = t >> 6;
+    const int fr = lane & 31, fh = lane >> 5;
+    const int n0 = (int)blockIdx.y * NC;
+    constexpr uint32_t OOB = 0x80000000u;
+    const __amdgpu_buffer_rsrc_t srd_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.in), 0, (int)p.in_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srd_u = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.u), 0, (int)p.u_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srd_out = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)p.out_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srd_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual ? p.residual : p.out), 0,
+        (int)p.out_bytes, 0x00020000);
+
+    // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
+    const int tile = (int)blockIdx.x * WINO_TM + fr;
+    const bool tile_ok = tile < p.tiles;
+    const int rest = tile / p.tiles_x;
+    const int tx = tile - rest * p.tiles_x;
+    const int img = rest / p.tiles_y;
+    const int ty = rest - img * p.tiles_y;
+    uint32_t pix_off[2][4];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const int row = r == 0 ? (xi == 0 ? 0 : 1) : (xi == 0 ? 2 : (xi == 3 ? 3 : 2));
+        const int y = 2 * ty - p.pad_top + row;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int x = 2 * tx - p.pad_left + j;
+            const bool ok = tile_ok && y >= 0 && y < p.h && x >= 0 && x < p.w;
+            pix_off[r][j] = ok ? (uint32_t)(((img * p.h + y) * p.w + x) * p.cin + fh * 4) * 4u : OOB;
+        }
+    }
+    uint32_t u_off[4][NT];
+#pragma unroll
+    for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            u_off[nu][nt] = (uint32_t)(((n0 / 32 + nt) * (p.cin / 8) * 16 + xi * 4 + nu) * 64 + lane) * 16u;
+    // where the tile's outputs go, for the waves that finish them: byte offset of pixel (0, 0) of the tile, channel 0,
+    // or an out-of-range offset; bit 0 / 1 of the second word: the tile's second row / column exists
+    int* tile_desc = reinterpret_cast<int*>(lds + 8 * WINO_TM * LS);
+    if (xi == 0 && fh == 0) {
+        tile_desc[fr * 2] = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
+        tile_desc[fr * 2 + 1] = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
+    }
+
+    f32x16 acc[4][NT];
+#pragma unroll
+    for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                acc[nu][nt][e] = 0.f;
+    switch (xi) { // the row of Bt is a compile-time choice inside the loop
+    case 0: wino_main<NT, 0>(p, pix_off, u_off, acc, srd_in, srd_u); break;
+    case 1: wino_main<NT, 1>(p, pix_off, u_off, acc, srd_in, srd_u); break;
+    case 2: wino_main<NT, 2>(p, pix_off, u_off, acc, srd_in, srd_u); break;
+    default: wino_main<NT, 3>(p, pix_off, u_off, acc, srd_in, srd_u); break;
+    }
+
+    // At along the row: z0 = m0 + m1 + m2, z1 = m1 - m2 - m3.  Element e of a lane is tile 8 * (e / 4) + 4 * fh + e % 4,
+    // channel nt * 32 + fr.
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int row = 8 * (e / 4) + 4 * fh + (e % 4);
+            const float m1 = acc[1][nt][e], m2 = acc[2][nt][e];
+            lds[((xi * 2 + 0) * WINO_TM + row) * LS + nt * 32 + fr] = acc[0][nt][e] + m1 + m2;
+            lds[((xi * 2 + 1) * WINO_TM + row) * LS + nt * 32 + fr] = m1 - m2 - acc[3][nt][e];
+        }
+    __syncthreads();
+
+    // At along the column: wave (i, j) = (xi / 2, xi % 2) finishes pixel (i, j) of every tile
+    const int oi = xi >> 1, oj = xi & 1;
+    constexpr int LANES_PER_TILE = NC / 4, TILES_PER_PASS = 64 / LANES_PER_TILE;
+    const int c4 = (lane % LANES_PER_TILE) * 4;
+    f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
+    if (p.bias)
+        bias4 = *reinterpret_cast<const f32x4*>(p.bias + n0 + c4);
+#pragma unroll 4
+    for (int pass = 0; pass < WINO_TM / TILES_PER_PASS; ++pass) {
+        const int tl = pass * TILES_PER_PASS + lane / LANES_PER_TILE;
+        const int base = tile_desc[tl * 2], flags = tile_desc[tl * 2 + 1];
+        const float* z = lds + (oj * WINO_TM + tl) * LS + c4; // row 0 of the domain, column value oj
+        const f32x4 za = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 0 : 1) * 2 * WINO_TM * LS);
+        const f32x4 zb = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 1 : 2) * 2 * WINO_TM * LS);
+        const f32x4 zc = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 2 : 3) * 2 * WINO_TM * LS);
+        f32x4 y = oi == 0 ? za + zb + zc : za - zb - zc;
+        const bool ok = (oi == 0 || (flags & 1)) && (oj == 0 || (flags & 2));
+        const uint32_t off = ok ? (uint32_t)base + (uint32_t)((oi * p.ow + oj) * p.cout + n0 + c4) * 4u : OOB;
+        y += bias4;
+        if (p.residual)
+            y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_res, (int)off, 0, 0));
+        float v[4] = { y[0], y[1], y[2], y[3] };
+        apply_act_block(v, p.act);
+        const f32x4 r = { v[0], v[1], v[2], v[3] };
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), srd_out, (int)off, 0, 0);
+    }
+}
+
+static size_t wino_lds_bytes(int nt) { return sizeof(float) * (size_t)8 * WINO_TM * (nt * 32 + WINO_PAD) + sizeof(int) * 2 * WINO_TM; }
+
+static bool al16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+} // namespace fdx
+
+using namespace fdx;
+
+extern "C" int fdx_conv2d_winograd_supported(int cin, int cout)
+{
+    return cin > 0 && cin % 8 == 0 && cout > 0 && cout % 64 == 0;
+}
+
+extern "C" size_t fdx_conv2d_winograd_weight_floats(int cout, int cin) { return (size_t)16 * (size_t)cout * (size_t)cin; }
+
+// (G g Gt)[a][b] for the 3x3 filter g of every (cout, cin), in the order the kernel's lanes take it:
+// u[cout / 32][cin / 8][p = 4 a + b][32 * (cin % 8 / 4) + cout % 32][cin % 4]; host memory on both sides
+extern "C" fdx_status fdx_conv2d_winograd_prepare(const float* weights_nkkc, int cout, int cin, float* u_out)
+{
+    FDX_REQUIRE(weights_nkkc && u_out && fdx_conv2d_winograd_supported(cin, cout), "winograd_prepare: bad arguments");
+    static const double G[4][3] = { { 1.0, 0.0, 0.0 }, { 0.5, 0.5, 0.5 }, { 0.5, -0.5, 0.5 }, { 0.0, 0.0, 1.0 } };
+    const size_t steps = (size_t)cin / 8;
+    for (int n = 0; n < cout; ++n)
+        for (int c = 0; c < cin; ++c) {
+            double g[3][3], gg[4][3];
+            for (int y = 0; y < 3; ++y)
+                for (int x = 0; x < 3; ++x)
+                    g[y][x] = weights_nkkc[(((size_t)n * 3 + y) * 3 + x) * cin + c];
+            for (int a = 0; a < 4; ++a)
+                for (int x = 0; x < 3; ++x)
+                    gg[a][x] = G[a][0] * g[0][x] + G[a][1] * g[1][x] + G[a][2] * g[2][x];
+            const size_t lane = (size_t)32 * ((c % 8) / 4) + n % 32;
+            for (int a = 0; a < 4; ++a)
+                for (int b = 0; b < 4; ++b)
+                    u_out[(((((size_t)n / 32) * steps + c / 8) * 16 + (a * 4 + b)) * 64 + lane) * 4 + c % 4]
+                        = (float)(gg[a][0] * G[b][0] + gg[a][1] * G[b][1] + gg[a][2] * G[b][2]);
+        }
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* u_weights, const float* bias,
+    int cout, int pad_top, int pad_left, int out_h, int out_w, const float* residual, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(in && u_weights && out, "conv2d_winograd: null pointer");
+    FDX_REQUIRE(n > 0 && h > 0 && w > 0 && out_h > 0 && out_w > 0, "conv2d_winograd: bad shape");
+    if (!fdx_conv2d_winograd_supported(cin, cout)) {
+        set_error("conv2d_winograd: needs input channels %% 8 == 0 and output channels %% 64 == 0");
+        return FDX_ERR_UNSUPPORTED;
+    }
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    FDX_REQUIRE(al16(in) && al16(u_weights) && al16(out) && (!bias || al16(bias)) && (!residual || al16(residual)),
+        "conv2d_winograd: operands must be 16-byte aligned");
+    FDX_REQUIRE(pad_top >= 0 && pad_left >= 0 && out_h - 1 - pad_top < h && out_w - 1 - pad_left < w,
+        "conv2d_winograd: output size does not fit the input");
+    WinoParams p;
+    std::memset(&p, 0, sizeof p);
+    p.in = in; p.u = u_weights; p.bias = bias; p.residual = residual; p.out = out;
+    p.n = n; p.h = h; p.w = w; p.cin = cin; p.cout = cout; p.pad_top = pad_top; p.pad_left = pad_left; p.oh = out_h; p.ow = out_w;
+    p.tiles_x = (out_w + 1) / 2;
+    p.tiles_y = (out_h + 1) / 2;
+    FDX_REQUIRE((int64_t)n * p.tiles_x * p.tiles_y < (1LL << 30), "conv2d_winograd: too many output pixels for one launch");
+    p.tiles = n * p.tiles_x * p.tiles_y;
+    FDX_REQUIRE((int64_t)n * h * w * cin * 4 < (1LL << 31), "conv2d_winograd: input tensor beyond 2 GiB");
+    p.in_bytes = (uint32_t)((int64_t)n * h * w * cin * 4);
+    FDX_REQUIRE((int64_t)n * out_h * out_w * cout * 4 < (1LL << 31), "conv2d_winograd: output tensor beyond 2 GiB");
+    p.out_bytes = (uint32_t)((int64_t)n * out_h * out_w * cout * 4);
+    FDX_REQUIRE((int64_t)16 * cout * cin * 4 < (1LL << 31), "conv2d_winograd: filter beyond 2 GiB");
+    p.u_bytes = (uint32_t)((int64_t)16 * cout * cin * 4);
+    p.act = make_act(act);
+    const int nt = cout % 128 == 0 && (int64_t)((p.tiles + WINO_TM - 1) / WINO_TM) * (cout / 128) >= 512 ? 4 : 2;
+    const dim3 grid((unsigned)((p.tiles + WINO_TM - 1) / WINO_TM), (unsigned)(cout / (nt * 32)));
+    const size_t lds = wino_lds_bytes(nt);
+    profile_begin();
+    if (nt == 4) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<4>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(4));
+        FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
+        hipLaunchKernelGGL(wino_kernel<4>, grid, dim3(256), lds, stream(), p);
+    } else {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<2>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(2));
+        FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
+        hipLaunchKernelGGL(wino_kernel<2>, grid, dim3(256), lds, stream(), p);
+    }
+    const double pix = (double)n * out_h * out_w;
+    profile_end("conv2d_winograd_f32", 2.0 * pix * 9.0 * cin * cout, 4.0 * ((double)n * h * w * cin + pix * cout * (residual ? 2.0 : 1.0) + 9.0 * cin * cout));
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}

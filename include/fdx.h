@@ -154,6 +154,21 @@ fdx_status fdx_inverted_residual_nhwc_f32(const float* in, int n, int h, int w, 
     const float* residual, const fdx_act* act, float* out);
 
 /*
+ * 3x3 convolution, stride 1, no dilation, in the Winograd F(2x2, 3x3) form: 2.25 times fewer multiply-adds than the
+ * direct sum that convolve runs (include/fdeep/convolution.hpp:398-429, :107-160); same result up to a few more
+ * roundings (the transform matrices hold 0, +-1 and +-1/2 only).  The filter is moved into the transform domain once:
+ * fdx_conv2d_winograd_prepare takes the converted-JSON order [cout][3][3][cin] (host memory) and writes
+ * fdx_conv2d_winograd_weight_floats(cout, cin) floats (host memory), which the caller places on the device as
+ * u_weights.  Needs cin % 8 == 0 and cout % 64 == 0 (fdx_conv2d_winograd_supported); zero padding pad_top / pad_left,
+ * bottom / right implied by out_h / out_w as for fdx_conv2d_nhwc_f32.
+ */
+int fdx_conv2d_winograd_supported(int cin, int cout);
+size_t fdx_conv2d_winograd_weight_floats(int cout, int cin);
+fdx_status fdx_conv2d_winograd_prepare(const float* weights_nkkc, int cout, int cin, float* u_out);
+fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* u_weights, const float* bias,
+    int cout, int pad_top, int pad_left, int out_h, int out_w, const float* residual, const fdx_act* act, float* out);
+
+/*
  * The first block of a MobileNet-like network as one launch: a small convolution on the image (ek x ek taps on ic
  * channels with ek * ek * ic <= 32, e.g. 3x3 on RGB; stride conv_stride, zero padding conv_pad_top / conv_pad_left) +
  * activation, depthwise 3x3 (stride 1 or 2) + activation, 1x1 convolution (ce -> n_out) + optional residual +

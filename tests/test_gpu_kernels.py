@@ -239,6 +239,38 @@ def test_inverted_residual_rejects_what_it_does_not_cover(fdx):
 
 
 @pytest.mark.parametrize("case", [
+    # n, h, w, cin, cout, padding
+    (2, 8, 8, 8, 64, "same"), (1, 7, 7, 16, 64, "same"), (3, 9, 6, 24, 128, "same"), (2, 10, 13, 8, 64, "valid"),
+    (1, 14, 14, 64, 128, "same"), (5, 5, 5, 32, 192, "same"), (2, 4, 3, 8, 64, "valid"), (1, 3, 3, 8, 64, "valid"),
+])
+def test_conv2d_winograd_vs_oracle(fdx, oracle, case):
+    """3x3 stride-1 convolution through the F(2x2, 3x3) transforms against the oracle's direct sum: odd extents (tiles
+    that hang over the output), both paddings, partial tile blocks, bias, residual and activation."""
+    n, h, w, cin, cout, padding = case
+    say("conv2d_winograd", case)
+    r = rng_for("wino", case)
+    x = r.standard_normal((n, h, w, cin)).astype(np.float32)
+    wt = (r.standard_normal((cout, 3, 3, cin)) / np.sqrt(9 * cin)).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    prepared = oracle.conv2d_prepare(wt.reshape(-1), cout, 3, 3, cin)
+    want = np.stack([oracle.conv2d(x[i], prepared, b, cout, 3, 3, (1, 1), (1, 1), padding) for i in range(n)])
+    got = fdx.conv2d_winograd(x, wt, b, padding)
+    assert got.shape == want.shape
+    assert rel(got, want) <= TOL
+    res = r.standard_normal(want.shape).astype(np.float32)
+    want_r = np.stack([oracle.relu(oracle.conv2d(x[i], prepared, None, cout, 3, 3, (1, 1), (1, 1), padding) + res[i]) for i in range(n)])
+    got_r = fdx.conv2d_winograd(x, wt, None, padding, residual=res, act=fdx.relu_act())
+    assert rel(got_r, want_r) <= TOL
+
+
+def test_conv2d_winograd_rejects_what_it_does_not_cover(fdx):
+    assert fdx.lib.fdx_conv2d_winograd_supported(64, 64) == 1 and fdx.lib.fdx_conv2d_winograd_supported(8, 192) == 1
+    assert fdx.lib.fdx_conv2d_winograd_supported(3, 64) == 0 and fdx.lib.fdx_conv2d_winograd_supported(64, 32) == 0
+    with pytest.raises(RuntimeError):
+        fdx.conv2d_winograd(np.zeros((1, 6, 6, 4), np.float32), np.zeros((64, 3, 3, 4), np.float32), None)
+
+
+@pytest.mark.parametrize("case", [
     # n, ih, iw, ic, ek, conv stride, conv padding, conv frame, ce, n_out, depthwise stride, depthwise padding, depthwise frame
     (2, 32, 32, 3, 3, 2, "same", (0, 0, 0, 0), 32, 16, 1, "same", (0, 0, 0, 0)),     # MobileNetV2's first block
     (2, 33, 29, 3, 3, 2, "valid", (0, 0, 1, 1), 32, 16, 1, "same", (0, 0, 0, 0)),    # explicit bottom / right padding
