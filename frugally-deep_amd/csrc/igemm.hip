@@ -967,7 +967,7 @@ extern "C" fdx_status fdx_tuner_import(const char* text)
         if (got <= 0)
             break; // trailing white space
         FDX_REQUIRE(got == 12, "tuner_import: malformed line near offset %d", (int)(p - text));
-        FDX_REQUIRE(k.conv >= 0 && k.conv <= 2 && choice >= -1, "tuner_import: value out of range near offset %d", (int)(p - text));
+        FDX_REQUIRE(k.conv >= 0 && k.conv <= 3 && choice >= -1, "tuner_import: value out of range near offset %d", (int)(p - text));
         rows.emplace_back(k, choice);
         p += used;
         while (*p == '\n' || *p == '\r' || *p == ' ')

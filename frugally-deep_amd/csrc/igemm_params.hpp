@@ -41,7 +41,10 @@ struct GemmParams {
 
 // Key of the per-process tuning table (igemm.hip).  conv = 0 / 1: a GEMM / convolution shape and its tile choice
 // (configuration + 100 * splits + 10000 * mode); conv = 2: a depthwise 3x3 + 1x1 pair (M = height, Cin = width,
-// K = channels, N = filters, sy = stride, res = residual) and whether it runs as one launch (1) or two (2).
+// K = channels, N = filters, sy = stride, res = residual, kh = input channels of a whole block) and the form it runs
+// in (1 = depthwise + projection as one launch, 2 = a launch per layer, 3 = the whole block as one launch);
+// conv = 3: a 3x3 stride-1 convolution (M = output pixels of the batch, kh / kw = input height / width, sy / sx = top /
+// left padding) and its kernel (0 = direct, 1 = Winograd).
 struct TuneKey {
     int conv, M, N, K, Cin, kh, kw, sy, sx, batch, res;
     bool operator<(const TuneKey& o) const { return std::memcmp(this, &o, sizeof(TuneKey)) < 0; }

@@ -1279,6 +1279,16 @@ namespace {
                 for (int n = 0; n < o.cout; ++n)
                     std::copy_n(&o.hw[0][(size_t)n * o.n_in], o.n_in, &o.hw[3][(size_t)n * kp]);
             }
+            // 3x3 stride-1 convolutions get a fifth weight array: the filter in the Winograd F(2x2, 3x3) domain; whether a
+            // plan runs the direct or the Winograd kernel is decided per shape by timing both
+            static const bool wino_on = [] { const char* e = std::getenv("FDX_WINOGRAD"); return !(e && e[0] == '0'); }();
+            if (wino_on && o.kind == OpKind::Conv2D && o.hw.size() == 2 && o.kh == 3 && o.kw == 3 && o.sy == 1 && o.sx == 1 && o.dy == 1
+                && o.dx == 1 && !o.softmax && fdx_conv2d_winograd_supported(o.n_in, o.cout)) {
+                o.hw.resize(5);
+                o.hw[4].resize(fdx_conv2d_winograd_weight_floats(o.cout, o.n_in));
+                if (fdx_conv2d_winograd_prepare(o.hw[0].data(), o.cout, o.n_in, o.hw[4].data()) != FDX_OK)
+                    return FDX_ERR_INVALID;
+            }
             // self-attention (query, value and key are one tensor): the three projections become one GEMM over the
             // stacked kernels, whose column blocks the attention core then reads in place
             if (o.kind == OpKind::MHA && o.hw.size() >= 6 && o.in.size() >= 2 && o.in[0] == o.in[1]
@@ -1571,6 +1581,17 @@ extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
     return FDX_OK;
 }
 
+// test hook: -1 = a plan times the direct and the Winograd kernel of a 3x3 stride-1 convolution, 0 = always direct, 1 = Winograd
+// wherever it applies
+static int g_force_winograd = -1;
+
+extern "C" fdx_status fdx_debug_force_winograd(int mode)
+{
+    FDX_REQUIRE(mode >= -1 && mode <= 1, "fdx_debug_force_winograd: mode must be -1, 0 or 1");
+    g_force_winograd = mode;
+    return FDX_OK;
+}
+
 fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes, Plan** out)
 {
     for (size_t i = 0; i < m->plans.size(); ++i)
@@ -1598,6 +1619,7 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->last_use.assign(n, -1);
     p->temps.assign(n, {});
     p->dw_fused.assign(n, g_force_dw_fusion < 0 ? 0 : (g_force_dw_fusion == 1 ? 1 : (g_force_dw_fusion == 2 ? 3 : 2)));
+    p->conv_form.assign(n, (signed char)g_force_winograd);
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -1690,6 +1712,78 @@ namespace {
 
     fdx_act to_c(const Act& a) { return { a.kind, a.max_value, a.negative_slope, a.threshold }; }
 
+    // First execution of a 3x3 stride-1 convolution that has a Winograd filter: the direct and the Winograd kernel are
+    // timed on the real operands (both leave the same result, up to rounding, in the output buffer), the plan remembers
+    // the faster one and the tuner's table keeps it per shape, so that an exported table pins it too.
+    fdx_status choose_conv_form(fdx_model& m, Plan& p, int idx, const float* in0, int h, int w, int c, const int* g, const float* res,
+        const fdx_act* actp, float* out)
+    {
+        const Op& o = m.ops[idx];
+        const int B = p.batch;
+        auto run = [&](int form) -> fdx_status {
+            if (form == 1)
+                return fdx_conv2d_winograd_nhwc_f32(in0, B, h, w, c, o.dw[4], o.dw[1], o.cout, g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5], res,
+                    actp, out);
+            return fdx_conv2d_nhwc_f32(in0, B, h, w, c, o.dw[0], o.dw[1], o.cout, o.kh, o.kw, o.sy, o.sx, o.dy, o.dx, g[0] + o.zp[0],
+                g[2] + o.zp[2], g[4], g[5], res, actp, out);
+        };
+        TuneKey key;
+        std::memset(&key, 0, sizeof key);
+        key.conv = 3;
+        key.M = B * g[4] * g[5];
+        key.N = o.cout;
+        key.K = 9 * c;
+        key.Cin = c;
+        key.kh = h;
+        key.kw = w;
+        key.sy = g[0] + o.zp[0];
+        key.sx = g[2] + o.zp[2];
+        key.batch = B;
+        key.res = res != nullptr;
+        int known = 0;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if (tune_lookup(key, &known) || tune_frozen() || hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+            if (e0)
+                (void)hipEventDestroy(e0);
+            p.conv_form[idx] = known == 1 ? 1 : 0; // frozen and unseen: the direct kernel
+            fdx_status st = run(p.conv_form[idx]);
+            if (st == FDX_ERR_UNSUPPORTED && p.conv_form[idx] == 1) {
+                p.conv_form[idx] = 0;
+                st = run(0);
+            }
+            return st;
+        }
+        float ms[2] = { 1e30f, 1e30f };
+        fdx_status st = FDX_OK;
+        for (int form = 0; form < 2 && st == FDX_OK; ++form) {
+            st = run(form); // warm-up (the direct kernel picks its tile here); tells whether the launcher takes the shape
+            if (st == FDX_ERR_UNSUPPORTED && form == 1) {
+                st = FDX_OK;
+                continue;
+            }
+            for (int round = 0; round < 3 && st == FDX_OK; ++round) {
+                (void)hipEventRecord(e0, stream());
+                for (int r = 0; r < 3 && st == FDX_OK; ++r)
+                    st = run(form);
+                (void)hipEventRecord(e1, stream());
+                float t = 1e30f;
+                if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess && t < ms[form])
+                    ms[form] = t;
+            }
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        if (st != FDX_OK)
+            return st;
+        const int best = ms[1] < ms[0] ? 1 : 0;
+        static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
+        if (log_picks)
+            std::fprintf(stderr, "[fdx tune] %s: direct %.1f us, Winograd %.1f us\n", o.name.c_str(), ms[0] * 1e3f / 3, ms[1] * 1e3f / 3);
+        p.conv_form[idx] = (signed char)best;
+        tune_store(key, best);
+        return run(best);
+    }
+
     fdx_status run_op(fdx_model& m, Plan& p, int idx)
     {
         const Op& o = m.ops[idx];
@@ -1717,6 +1811,18 @@ namespace {
                 st = conv1x1_padded_launch(in0, (int64_t)B * h * w, c, o.dw[3], (c + 15) / 16 * 16, o.dw[1], o.cout, res, actp, out);
                 if (st != FDX_ERR_UNSUPPORTED)
                     break;
+            }
+            if (o.kind == OpKind::Conv2D && o.dw.size() > 4 && o.dw[4]) {
+                if (p.conv_form[idx] < 0) {
+                    st = choose_conv_form(m, p, idx, in0, h, w, c, g, res, actp, out);
+                    break; // the chosen form ran last and left its result
+                }
+                if (p.conv_form[idx] == 1) {
+                    st = fdx_conv2d_winograd_nhwc_f32(in0, B, h, w, c, o.dw[4], o.dw[1], o.cout, g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5], res,
+                        actp, out);
+                    if (st != FDX_ERR_UNSUPPORTED)
+                        break;
+                }
             }
             if (o.kind == OpKind::Conv2D && !p.temps[idx].empty())
                 st = fdx_conv2d_s2d_nhwc_f32(in0, B, h, w, c, o.dw[2], o.dw[1], o.cout, o.kh, g[0] + o.zp[0], g[2] + o.zp[2], g[4], g[5],

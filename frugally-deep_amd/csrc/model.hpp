@@ -91,6 +91,7 @@ struct Plan {
     std::vector<Block> blocks;
     std::vector<std::vector<float*>> temps; // per op: scratch placed at plan time
     std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = depthwise + projection as one launch, 2 = one launch per layer, 3 = expansion + depthwise + projection as one launch
+    std::vector<signed char> conv_form;     // per 3x3 stride-1 convolution with a Winograd filter: -1 = not timed yet, 0 = direct kernel, 1 = Winograd kernel
     double flops = 0;
     ~Plan();
 };

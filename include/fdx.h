@@ -456,10 +456,14 @@ fdx_status fdx_tuner_freeze(int on);
  *     around it: -1 = the forms are timed once per block shape (the default), 0 = one launch per layer, 1 = depthwise +
  *     projection as one launch wherever the pair qualifies, 2 = expansion + depthwise + projection as one launch
  *     wherever the block qualifies (other blocks as under 1).
+ *   fdx_debug_force_winograd: which kernel plans built from now on run a 3x3 stride-1 convolution with: -1 = the direct and
+ *     the Winograd kernel are timed once per shape (the default), 0 = always the direct kernel, 1 = the Winograd kernel
+ *     wherever it covers the shape.
  */
 fdx_status fdx_debug_force_tile(int cfg);
 fdx_status fdx_debug_persist_cap(int workgroups);
 fdx_status fdx_debug_force_dw_fusion(int mode);
+fdx_status fdx_debug_force_winograd(int mode);
 
 #ifdef __cplusplus
 }

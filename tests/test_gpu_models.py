@@ -168,6 +168,23 @@ def test_gpt2_tiny_predict_is_unmasked(fdx, oracle, modelgen):
     run_both(fdx, oracle, modelgen, spec, [ids, pos])
 
 
+@pytest.mark.parametrize("mode", [1, 0, -1])
+def test_resnet_with_either_3x3_kernel(fdx, oracle, modelgen, mode):
+    """The 3x3 stride-1 convolutions of a (narrow) ResNet50 through the Winograd kernel, through the direct kernel, and
+    with the plan timing both: every form meets the oracle."""
+    say("resnet 3x3 kernels, mode", mode)
+    js = modelgen.dumps(modelgen.resnet50(seed=61, input_size=64, width=64, blocks=(2, 2, 1, 1), classes=10, random_bn=True))
+    x = np.random.default_rng(62).uniform(0, 1, (3, 64, 64, 3)).astype(np.float32)
+    want = [oracle.OracleModel(js).predict([x[i]])[0] for i in range(3)]
+    try:
+        fdx.check(fdx.lib.fdx_debug_force_winograd(mode))
+        got = fdx.Model(js, verify=False).predict([x])[0]
+    finally:
+        fdx.check(fdx.lib.fdx_debug_force_winograd(-1))
+    for i in range(3):
+        assert rel(got[i], want[i]) <= TOL
+
+
 def test_predict_from_device_pointers(fdx, modelgen):
     """fdx_model_predict_dev reads 16-byte aligned device inputs where they lie and copies misaligned ones first; both
     return what the host-pointer call returns, also when the same plan is used with another buffer afterwards, with the
