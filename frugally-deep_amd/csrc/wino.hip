@@ -6,7 +6,8 @@
 // it spends 16 per four pixels, 2.25 times fewer: for each of the 16 positions of the 4x4 domain the sum over the input
 // channels is a GEMM  M_p[tile][cout] = sum_c V_p[tile][c] * U_p[c][cout],  and those run on the matrix cores.
 //
-// A workgroup of four waves owns 32 tiles (of any images, in raster order) and NT * 32 output channels.  Wave xi owns
+// A unit of work is 32 tiles (of any images, in raster order) by NT * 32 output channels; a workgroup of four waves
+// works on one unit at a time (how units are dealt to workgroups: see wino_kernel).  Wave xi owns
 // row xi of the 4x4 domain, i.e. the four positions (xi, 0..3):
 //   * per step of 8 input channels a lane takes, for its tile (lane % 32) and its four channels (lane / 32), the two
 //     patch rows that row xi of Bt combines, four pixels each, straight from global memory (a pixel outside the image
@@ -27,7 +28,7 @@
 //
 // Replaces convolve for 3x3 filters, stride 1, no dilation (include/fdeep/convolution.hpp:398-429, :107-160).
 #include <cstring>
-#include <vector>
+#include <mutex>
 
 #include "common.hpp"
 #include "igemm_params.hpp"
@@ -44,174 +45,284 @@ struct WinoParams {
     float* out;            // [n][oh][ow][cout]
     int n, h, w, cin, cout, pad_top, pad_left, oh, ow;
     int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
-    uint32_t in_bytes, out_bytes, u_bytes;
+    uint32_t in_bytes, out_bytes, u_bytes, ws_bytes;
+    int n_blocks, units; // column blocks of NT * 32 channels; units of work = blocks of 32 tiles x column blocks
+    float* ws;           // shares of units that several workgroups work on: two places per workgroup
+    int* tickets;        // one per unit, zero between launches
     Act act;
 };
 
 constexpr int WINO_TM = 32;  // tiles per workgroup
 constexpr int WINO_PAD = 4;  // padding of an LDS row of the exchange
 
-// NT = 32-column tiles of the output channels per workgroup
+// NT = 32-column tiles of the output channels per workgroup, XI = this wave's row of the transform domain.
+// The operands of a step sit in one of SETS register sets; the loop is unrolled over the sets, so that a set is
+// loaded SETS - 1 steps before it is used and nothing is ever copied from one set to another.
 template <int NT, int XI>
 __device__ __forceinline__ void wino_main(const WinoParams& p, const uint32_t (&pix_off)[2][4], const uint32_t (&u_off)[4][NT],
-    f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u)
+    f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u, int step_begin, int step_end)
 {
-    const int steps = p.cin / 8;
-    auto load_a = [&](f32x4 (&d)[2][4], int step) {
+    constexpr int SETS = NT <= 2 ? 3 : 2;
+    const int steps = step_end - step_begin;
+    f32x4 d[SETS][2][4], b[SETS][4][NT];
+    auto load = [&](f32x4 (&dd)[2][4], f32x4 (&bb)[4][NT], int step) {
 #pragma unroll
         for (int r = 0; r < 2; ++r)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                d[r][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], step * 32, 0));
-    };
-    auto load_b = [&](f32x4 (&b)[4][NT], int step) {
+                dd[r][j] = __builtin_bit_cast(f32x4,
+                    __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], (step_begin + step) * 32, 0));
 #pragma unroll
         for (int nu = 0; nu < 4; ++nu)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
-                b[nu][nt] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], step * 16384, 0));
+                bb[nu][nt] = __builtin_bit_cast(f32x4,
+                    __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], (step_begin + step) * 16384, 0));
     };
-    f32x4 d[2][4], b[4][NT];
-    load_a(d, 0);
-    load_b(b, 0);
-    for (int step = 0; step < steps; ++step) {
-        // row xi of Bt over the patch rows, then Bt again over the columns
-        f32x4 v[4];
-        {
-            f32x4 t[4];
+    auto multiply = [&](const f32x4 (&dd)[2][4], const f32x4 (&bb)[4][NT]) {
+        // row XI of Bt over the patch rows, then Bt again over the columns
+        f32x4 t[4], v[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                t[j] = XI == 1 ? d[0][j] + d[1][j] : (XI == 2 ? d[1][j] - d[0][j] : d[0][j] - d[1][j]);
-            v[0] = t[0] - t[2];
-            v[1] = t[1] + t[2];
-            v[2] = t[2] - t[1];
-            v[3] = t[1] - t[3];
-        }
-        f32x4 bc[4][NT];
-#pragma unroll
-        for (int nu = 0; nu < 4; ++nu)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                bc[nu][nt] = b[nu][nt];
-        if (step + 1 < steps) { // the next step's operands travel while this step multiplies
-            load_a(d, step + 1);
-            load_b(b, step + 1);
-        }
+        for (int j = 0; j < 4; ++j)
+            t[j] = XI == 1 ? dd[0][j] + dd[1][j] : (XI == 2 ? dd[1][j] - dd[0][j] : dd[0][j] - dd[1][j]);
+        v[0] = t[0] - t[2];
+        v[1] = t[1] + t[2];
+        v[2] = t[2] - t[1];
+        v[3] = t[1] - t[3];
 #pragma unroll
         for (int nu = 0; nu < 4; ++nu)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], bc[nu][nt][e], acc[nu][nt], 0, 0, 0);
+                    acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], bb[nu][nt][e], acc[nu][nt], 0, 0, 0);
+    };
+    // Every load below is unconditional (a step index beyond the range is clamped to the last step and its data never
+    // used): with loads behind branches the compiler has to assume the fewest outstanding ones at every wait, which
+    // shortens the distance between a load and its use to nothing.
+    const int last = steps - 1;
+#pragma unroll
+    for (int s0 = 0; s0 < SETS - 1; ++s0)
+        load(d[s0], b[s0], s0 < last ? s0 : last);
+    const int rounds = steps / SETS;
+    for (int r = 0; r < rounds; ++r) {
+#pragma unroll
+        for (int u = 0; u < SETS; ++u) {
+            const int ahead = r * SETS + u + SETS - 1;
+            load(d[(u + SETS - 1) % SETS], b[(u + SETS - 1) % SETS], ahead < last ? ahead : last);
+            __builtin_amdgcn_sched_barrier(0); // the loads stay in front of the step they overlap with (the scheduler
+            multiply(d[u], b[u]);              // would gather them at the end of the loop body, right before their use)
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
+    const int rest = steps - rounds * SETS; // at most SETS - 1 steps, already loaded
+#pragma unroll
+    for (int u = 0; u < SETS - 1; ++u)
+        if (u < rest)
+            multiply(d[u], b[u]);
 }
 
+// Persistent workgroups, balanced over the chip: the units of work (32 tiles x NT * 32 channels, cin / 8 steps each)
+// form one line of steps, cut into as many equal stretches as there are workgroups.  A stretch that covers a unit
+// from its first to its last step finishes it alone.  A unit that two or three stretches share is finished by the
+// last of them to arrive: each leaves its share in the output domain (the transforms are linear, so shares add
+// there) in the workspace with agent-scope stores, waits until they have left the CU, and takes the unit's ticket;
+// the one that draws the last ticket adds all shares in stretch order (the result does not depend on who came last),
+// then bias, residual and activation.  Nobody waits for anybody.  Without this a launch lasts a whole number of
+// units per CU: 392 units on 256 CUs take the time of 512.
 template <int NT>
 __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
 {
     constexpr int NC = NT * 32, LS = NC + WINO_PAD;
+    constexpr int LANES_PER_TILE = NC / 4, TILES_PER_PASS = 64 / LANES_PER_TILE, PASSES = WINO_TM / TILES_PER_PASS;
+    constexpr int kAgentScope = 16; // cache-policy bit of a buffer access: written through to / fetched from memory
     extern __shared__ __attribute__((aligned(16))) float lds[]; // [4 rows][2][32 tiles][LS], then 32 tile descriptors
+    __shared__ int last_flag;
     const int t = threadIdx.x, lane = t & 63, xi = t >> 6;
     const int fr = lane & 31, fh = lane >> 5;
-    const int n0 = (int)blockIdx.y * NC;
     constexpr uint32_t OOB = 0x80000000u;
     const __amdgpu_buffer_rsrc_t srd_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.in), 0, (int)p.in_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t srd_u = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.u), 0, (int)p.u_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t srd_out = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)p.out_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t srd_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual ? p.residual : p.out), 0,
         (int)p.out_bytes, 0x00020000);
-
-    // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
-    const int tile = (int)blockIdx.x * WINO_TM + fr;
-    const bool tile_ok = tile < p.tiles;
-    const int rest = tile / p.tiles_x;
-    const int tx = tile - rest * p.tiles_x;
-    const int img = rest / p.tiles_y;
-    const int ty = rest - img * p.tiles_y;
-    uint32_t pix_off[2][4];
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        const int row = r == 0 ? (xi == 0 ? 0 : 1) : (xi == 0 ? 2 : (xi == 3 ? 3 : 2));
-        const int y = 2 * ty - p.pad_top + row;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int x = 2 * tx - p.pad_left + j;
-            const bool ok = tile_ok && y >= 0 && y < p.h && x >= 0 && x < p.w;
-            pix_off[r][j] = ok ? (uint32_t)(((img * p.h + y) * p.w + x) * p.cin + fh * 4) * 4u : OOB;
-        }
-    }
-    uint32_t u_off[4][NT];
-#pragma unroll
-    for (int nu = 0; nu < 4; ++nu)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            u_off[nu][nt] = (uint32_t)(((n0 / 32 + nt) * (p.cin / 8) * 16 + xi * 4 + nu) * 64 + lane) * 16u;
-    // where the tile's outputs go, for the waves that finish them: byte offset of pixel (0, 0) of the tile, channel 0,
-    // or an out-of-range offset; bit 0 / 1 of the second word: the tile's second row / column exists
+    const __amdgpu_buffer_rsrc_t srd_ws = __builtin_amdgcn_make_buffer_rsrc(p.ws, 0, (int)p.ws_bytes, 0x00020000);
     int* tile_desc = reinterpret_cast<int*>(lds + 8 * WINO_TM * LS);
-    if (xi == 0 && fh == 0) {
-        tile_desc[fr * 2] = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
-        tile_desc[fr * 2 + 1] = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
-    }
+    const int oi = xi >> 1, oj = xi & 1; // the output pixel of every tile this wave finishes
+    const int c4 = (lane % LANES_PER_TILE) * 4;
+    constexpr uint32_t SHARE_BYTES = 4u * PASSES * 64u * 16u; // a unit's share in the workspace: [wave][pass][lane] 16-byte pieces
 
-    f32x16 acc[4][NT];
+    const int G = (int)gridDim.x, g = (int)blockIdx.x;
+    const int spu = p.cin / 8; // steps per unit
+    const int64_t S = (int64_t)p.units * spu;
+    auto stretch_begin = [&](int gg) -> int64_t { return (int64_t)gg * S / G; };
+    auto owner_of = [&](int64_t step) -> int { return (int)(((step + 1) * G - 1) / S); }; // the stretch that holds `step`
+    // a workgroup has two places in the workspace: one for the unit its stretch begins in, one for the unit it ends in
+    auto share_off = [&](int gg, int unit) -> uint32_t {
+        return (uint32_t)(2 * gg + (stretch_begin(gg) / spu == unit ? 0 : 1)) * SHARE_BYTES;
+    };
+    int64_t pos = stretch_begin(g);
+    const int64_t end = stretch_begin(g + 1);
+    while (pos < end) {
+        const int unit = (int)(pos / spu);
+        const int64_t unit_begin = (int64_t)unit * spu;
+        const int s0 = (int)(pos - unit_begin);
+        const int s1 = end - unit_begin < spu ? (int)(end - unit_begin) : spu;
+        const int mb = unit / p.n_blocks, nb = unit - mb * p.n_blocks;
+        const int n0 = nb * NC;
+
+        // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
+        const int tile = mb * WINO_TM + fr;
+        const bool tile_ok = tile < p.tiles;
+        const int rest = tile / p.tiles_x;
+        const int tx = tile - rest * p.tiles_x;
+        const int img = rest / p.tiles_y;
+        const int ty = rest - img * p.tiles_y;
+        uint32_t pix_off[2][4];
 #pragma unroll
-    for (int nu = 0; nu < 4; ++nu)
+        for (int r = 0; r < 2; ++r) {
+            const int row = r == 0 ? (xi == 0 ? 0 : 1) : (xi == 0 ? 2 : (xi == 3 ? 3 : 2));
+            const int y = 2 * ty - p.pad_top + row;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int x = 2 * tx - p.pad_left + j;
+                const bool ok = tile_ok && y >= 0 && y < p.h && x >= 0 && x < p.w;
+                pix_off[r][j] = ok ? (uint32_t)(((img * p.h + y) * p.w + x) * p.cin + fh * 4) * 4u : OOB;
+            }
+        }
+        uint32_t u_off[4][NT];
+#pragma unroll
+        for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                u_off[nu][nt] = (uint32_t)(((n0 / 32 + nt) * spu * 16 + xi * 4 + nu) * 64 + lane) * 16u;
+        // where the tile's outputs go, for the waves that finish them: byte offset of pixel (0, 0) of the tile, channel
+        // 0, or an out-of-range offset; bit 0 / 1 of the second word: the tile's second row / column exists
+        if (xi == 0 && fh == 0) {
+            tile_desc[fr * 2] = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
+            tile_desc[fr * 2 + 1] = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
+        }
+
+        f32x16 acc[4][NT];
+#pragma unroll
+        for (int nu = 0; nu < 4; ++nu)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[nu][nt][e] = 0.f;
+        switch (xi) { // the row of Bt is a compile-time choice inside the loop
+        case 0: wino_main<NT, 0>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
+        case 1: wino_main<NT, 1>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
+        case 2: wino_main<NT, 2>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
+        default: wino_main<NT, 3>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
+        }
+
+        // At along the row: z0 = m0 + m1 + m2, z1 = m1 - m2 - m3.  Element e of a lane is tile 8 * (e / 4) + 4 * fh +
+        // e % 4, channel nt * 32 + fr.
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-                acc[nu][nt][e] = 0.f;
-    switch (xi) { // the row of Bt is a compile-time choice inside the loop
-    case 0: wino_main<NT, 0>(p, pix_off, u_off, acc, srd_in, srd_u); break;
-    case 1: wino_main<NT, 1>(p, pix_off, u_off, acc, srd_in, srd_u); break;
-    case 2: wino_main<NT, 2>(p, pix_off, u_off, acc, srd_in, srd_u); break;
-    default: wino_main<NT, 3>(p, pix_off, u_off, acc, srd_in, srd_u); break;
-    }
+            for (int e = 0; e < 16; ++e) {
+                const int row = 8 * (e / 4) + 4 * fh + (e % 4);
+                const float m1 = acc[1][nt][e], m2 = acc[2][nt][e];
+                lds[((xi * 2 + 0) * WINO_TM + row) * LS + nt * 32 + fr] = acc[0][nt][e] + m1 + m2;
+                lds[((xi * 2 + 1) * WINO_TM + row) * LS + nt * 32 + fr] = m1 - m2 - acc[3][nt][e];
+            }
+        __syncthreads();
 
-    // At along the row: z0 = m0 + m1 + m2, z1 = m1 - m2 - m3.  Element e of a lane is tile 8 * (e / 4) + 4 * fh + e % 4,
-    // channel nt * 32 + fr.
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int row = 8 * (e / 4) + 4 * fh + (e % 4);
-            const float m1 = acc[1][nt][e], m2 = acc[2][nt][e];
-            lds[((xi * 2 + 0) * WINO_TM + row) * LS + nt * 32 + fr] = acc[0][nt][e] + m1 + m2;
-            lds[((xi * 2 + 1) * WINO_TM + row) * LS + nt * 32 + fr] = m1 - m2 - acc[3][nt][e];
-        }
-    __syncthreads();
-
-    // At along the column: wave (i, j) = (xi / 2, xi % 2) finishes pixel (i, j) of every tile
-    const int oi = xi >> 1, oj = xi & 1;
-    constexpr int LANES_PER_TILE = NC / 4, TILES_PER_PASS = 64 / LANES_PER_TILE;
-    const int c4 = (lane % LANES_PER_TILE) * 4;
-    f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
-    if (p.bias)
-        bias4 = *reinterpret_cast<const f32x4*>(p.bias + n0 + c4);
+        // At along the column: wave (oi, oj) combines the rows into its pixel of every tile
+        auto combine = [&](int pass) -> f32x4 {
+            const int tl = pass * TILES_PER_PASS + lane / LANES_PER_TILE;
+            const float* z = lds + (oj * WINO_TM + tl) * LS + c4; // row 0 of the domain, column value oj
+            const f32x4 za = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 0 : 1) * 2 * WINO_TM * LS);
+            const f32x4 zb = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 1 : 2) * 2 * WINO_TM * LS);
+            const f32x4 zc = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 2 : 3) * 2 * WINO_TM * LS);
+            return oi == 0 ? za + zb + zc : za - zb - zc;
+        };
+        f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
+        if (p.bias)
+            bias4 = *reinterpret_cast<const f32x4*>(p.bias + n0 + c4);
+        auto finish = [&](int pass, f32x4 y) {
+            const int tl = pass * TILES_PER_PASS + lane / LANES_PER_TILE;
+            const int base = tile_desc[tl * 2], flags = tile_desc[tl * 2 + 1];
+            const bool ok = (oi == 0 || (flags & 1)) && (oj == 0 || (flags & 2));
+            const uint32_t off = ok ? (uint32_t)base + (uint32_t)((oi * p.ow + oj) * p.cout + n0 + c4) * 4u : OOB;
+            y += bias4;
+            if (p.residual)
+                y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_res, (int)off, 0, 0));
+            float v[4] = { y[0], y[1], y[2], y[3] };
+            apply_act_block(v, p.act);
+            const f32x4 r = { v[0], v[1], v[2], v[3] };
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), srd_out, (int)off, 0, 0);
+        };
+        if (s0 == 0 && s1 == spu) {
 #pragma unroll 4
-    for (int pass = 0; pass < WINO_TM / TILES_PER_PASS; ++pass) {
-        const int tl = pass * TILES_PER_PASS + lane / LANES_PER_TILE;
-        const int base = tile_desc[tl * 2], flags = tile_desc[tl * 2 + 1];
-        const float* z = lds + (oj * WINO_TM + tl) * LS + c4; // row 0 of the domain, column value oj
-        const f32x4 za = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 0 : 1) * 2 * WINO_TM * LS);
-        const f32x4 zb = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 1 : 2) * 2 * WINO_TM * LS);
-        const f32x4 zc = *reinterpret_cast<const f32x4*>(z + (oi == 0 ? 2 : 3) * 2 * WINO_TM * LS);
-        f32x4 y = oi == 0 ? za + zb + zc : za - zb - zc;
-        const bool ok = (oi == 0 || (flags & 1)) && (oj == 0 || (flags & 2));
-        const uint32_t off = ok ? (uint32_t)base + (uint32_t)((oi * p.ow + oj) * p.cout + n0 + c4) * 4u : OOB;
-        y += bias4;
-        if (p.residual)
-            y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_res, (int)off, 0, 0));
-        float v[4] = { y[0], y[1], y[2], y[3] };
-        apply_act_block(v, p.act);
-        const f32x4 r = { v[0], v[1], v[2], v[3] };
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), srd_out, (int)off, 0, 0);
+            for (int pass = 0; pass < PASSES; ++pass)
+                finish(pass, combine(pass));
+        } else {
+            const uint32_t lane_off = (uint32_t)((xi * PASSES) * 64 + lane) * 16u;
+            const uint32_t mine = share_off(g, unit) + lane_off;
+#pragma unroll 4
+            for (int pass = 0; pass < PASSES; ++pass)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, combine(pass)), srd_ws, (int)(mine + (uint32_t)pass * 1024u), 0,
+                    kAgentScope);
+            // every lane's share has left the CU before the ticket is taken
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            const int g_a = owner_of(unit_begin), parts = owner_of(unit_begin + spu - 1) - g_a + 1;
+            if (t == 0) {
+                const int ticket = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int last = ticket == parts - 1;
+                if (last)
+                    __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // for the next launch
+                last_flag = last;
+            }
+            __syncthreads();
+            if (last_flag != 0) {
+                for (int pass = 0; pass < PASSES; ++pass) {
+                    f32x4 y = { 0.f, 0.f, 0.f, 0.f };
+                    for (int sp = 0; sp < parts; ++sp)
+                        y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_ws,
+                            (int)(share_off(g_a + sp, unit) + lane_off + (uint32_t)pass * 1024u), 0, kAgentScope));
+                    finish(pass, y);
+                }
+            }
+        }
+        __syncthreads(); // the next unit overwrites the exchange area, the tile descriptors and last_flag
+        pos = unit_begin + s1;
     }
 }
 
 static size_t wino_lds_bytes(int nt) { return sizeof(float) * (size_t)8 * WINO_TM * (nt * 32 + WINO_PAD) + sizeof(int) * 2 * WINO_TM; }
+
+// library-owned scratch: two shares of 32 KB per workgroup of the persistent grid, one ticket per unit (zero
+// between launches: the workgroup that finishes a unit resets its ticket)
+constexpr int kWinoTickets = 1 << 16;
+constexpr size_t kWinoShareBytes = 32 * 1024;
+static float* g_wino_ws = nullptr;
+static int* g_wino_tickets = nullptr;
+static int g_wino_grid = 0;
+
+static bool wino_prepare()
+{
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    if (g_wino_ws && g_wino_tickets)
+        return true;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount < 1)
+        return false;
+    g_wino_grid = prop.multiProcessorCount;
+    if (!g_wino_ws && hipMalloc(&g_wino_ws, 2 * kWinoShareBytes * (size_t)g_wino_grid) != hipSuccess)
+        return false;
+    if (!g_wino_tickets
+        && (hipMalloc(&g_wino_tickets, sizeof(int) * kWinoTickets) != hipSuccess
+            || zero_device(g_wino_tickets, sizeof(int) * kWinoTickets) != hipSuccess))
+        return false;
+    return true;
+}
 
 static bool al16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
@@ -280,21 +391,30 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     FDX_REQUIRE((int64_t)16 * cout * cin * 4 < (1LL << 31), "conv2d_winograd: filter beyond 2 GiB");
     p.u_bytes = (uint32_t)((int64_t)16 * cout * cin * 4);
     p.act = make_act(act);
-    const int nt = cout % 128 == 0 && (int64_t)((p.tiles + WINO_TM - 1) / WINO_TM) * (cout / 128) >= 512 ? 4 : 2;
-    const dim3 grid((unsigned)((p.tiles + WINO_TM - 1) / WINO_TM), (unsigned)(cout / (nt * 32)));
+    FDX_REQUIRE(wino_prepare(), "conv2d_winograd: no device memory for the workspace");
+    const int m_blocks = (p.tiles + WINO_TM - 1) / WINO_TM;
+    // (128-channel units -- NT = 4 -- were measured: the second register set of operands no longer fits beside 256
+    // accumulators, and with one set the loads are not hidden: slower than 64-channel units on every ResNet50 shape)
+    constexpr int nt = 2;
+    p.n_blocks = cout / (nt * 32);
+    if ((int64_t)m_blocks * p.n_blocks > kWinoTickets) {
+        set_error("conv2d_winograd: more than %d units of work in one launch", kWinoTickets);
+        return FDX_ERR_UNSUPPORTED;
+    }
+    p.units = m_blocks * p.n_blocks;
+    p.ws = g_wino_ws;
+    p.ws_bytes = (uint32_t)(2 * kWinoShareBytes * (size_t)g_wino_grid);
+    p.tickets = g_wino_tickets;
+    // every workgroup gets at least four steps; none gets an empty stretch
+    const int64_t total_steps = (int64_t)p.units * (cin / 8);
+    const int64_t by_steps = total_steps / 4 > 0 ? total_steps / 4 : 1;
+    const dim3 grid((unsigned)(by_steps < g_wino_grid ? by_steps : g_wino_grid));
     const size_t lds = wino_lds_bytes(nt);
     profile_begin();
-    if (nt == 4) {
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<4>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(4));
-        FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
-        hipLaunchKernelGGL(wino_kernel<4>, grid, dim3(256), lds, stream(), p);
-    } else {
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<2>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(2));
-        FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
-        hipLaunchKernelGGL(wino_kernel<2>, grid, dim3(256), lds, stream(), p);
-    }
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<2>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(2));
+    FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
+    hipLaunchKernelGGL(wino_kernel<2>, grid, dim3(256), lds, stream(), p);
     const double pix = (double)n * out_h * out_w;
     profile_end("conv2d_winograd_f32", 2.0 * pix * 9.0 * cin * cout, 4.0 * ((double)n * h * w * cin + pix * cout * (residual ? 2.0 : 1.0) + 9.0 * cin * cout));
     FDX_LAUNCH_CHECK();

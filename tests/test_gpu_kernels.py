@@ -242,10 +242,12 @@ def test_inverted_residual_rejects_what_it_does_not_cover(fdx):
     # n, h, w, cin, cout, padding
     (2, 8, 8, 8, 64, "same"), (1, 7, 7, 16, 64, "same"), (3, 9, 6, 24, 128, "same"), (2, 10, 13, 8, 64, "valid"),
     (1, 14, 14, 64, 128, "same"), (5, 5, 5, 32, 192, "same"), (2, 4, 3, 8, 64, "valid"), (1, 3, 3, 8, 64, "valid"),
+    (4, 28, 28, 40, 64, "same"), (8, 14, 14, 72, 128, "same"), (6, 20, 20, 104, 256, "same"),  # units shared by two or three workgroups
 ])
 def test_conv2d_winograd_vs_oracle(fdx, oracle, case):
     """3x3 stride-1 convolution through the F(2x2, 3x3) transforms against the oracle's direct sum: odd extents (tiles
-    that hang over the output), both paddings, partial tile blocks, bias, residual and activation."""
+    that hang over the output), both paddings, partial tile blocks, bias, residual and activation; twice in a row, since
+    the tickets of shared units must be back at zero after a launch."""
     n, h, w, cin, cout, padding = case
     say("conv2d_winograd", case)
     r = rng_for("wino", case)
@@ -261,6 +263,7 @@ def test_conv2d_winograd_vs_oracle(fdx, oracle, case):
     want_r = np.stack([oracle.relu(oracle.conv2d(x[i], prepared, None, cout, 3, 3, (1, 1), (1, 1), padding) + res[i]) for i in range(n)])
     got_r = fdx.conv2d_winograd(x, wt, None, padding, residual=res, act=fdx.relu_act())
     assert rel(got_r, want_r) <= TOL
+    assert np.array_equal(fdx.conv2d_winograd(x, wt, b, padding), got)  # the same shares, added in the same order
 
 
 def test_conv2d_winograd_rejects_what_it_does_not_cover(fdx):
