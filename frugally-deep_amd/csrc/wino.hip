@@ -47,6 +47,7 @@ struct WinoParams {
     int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
     uint32_t in_bytes, out_bytes, u_bytes, ws_bytes;
     int n_blocks, units; // column blocks of NT * 32 channels; units of work = blocks of 32 tiles x column blocks
+    int per_wg, longer;  // steps per workgroup (total / workgroups) and how many workgroups take one more
     float* ws;           // shares of units that several workgroups work on: two places per workgroup
     int* tickets;        // one per unit, zero between launches
     Act act;
@@ -55,30 +56,49 @@ struct WinoParams {
 constexpr int WINO_TM = 32;  // tiles per workgroup
 constexpr int WINO_PAD = 4;  // padding of an LDS row of the exchange
 
-// NT = 32-column tiles of the output channels per workgroup, XI = this wave's row of the transform domain.
-// The operands of a step sit in one of SETS register sets; the loop is unrolled over the sets, so that a set is
-// loaded SETS - 1 steps before it is used and nothing is ever copied from one set to another.
-template <int NT, int XI>
-__device__ __forceinline__ void wino_main(const WinoParams& p, const uint32_t (&pix_off)[2][4], const uint32_t (&u_off)[4][NT],
-    f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u, int step_begin, int step_end)
+constexpr int WINO_SETS = 3; // register sets of step operands: a set is loaded WINO_SETS - 1 steps before its use
+
+// one step's operands: the eight patch pixels of this lane's tile and the 4 x NT filter pieces of its positions
+template <int NT>
+__device__ __forceinline__ void wino_load(f32x4 (&dd)[2][4], f32x4 (&bb)[4][NT], const uint32_t (&pix_off)[2][4],
+    const uint32_t (&u_off)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u, int step)
 {
-    constexpr int SETS = NT <= 2 ? 3 : 2;
-    const int steps = step_end - step_begin;
-    f32x4 d[SETS][2][4], b[SETS][4][NT];
-    auto load = [&](f32x4 (&dd)[2][4], f32x4 (&bb)[4][NT], int step) {
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < 2; ++r)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                dd[r][j] = __builtin_bit_cast(f32x4,
-                    __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], (step_begin + step) * 32, 0));
+        for (int j = 0; j < 4; ++j)
+            dd[r][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], step * 32, 0));
 #pragma unroll
-        for (int nu = 0; nu < 4; ++nu)
+    for (int nu = 0; nu < 4; ++nu)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                bb[nu][nt] = __builtin_bit_cast(f32x4,
-                    __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], (step_begin + step) * 16384, 0));
-    };
+        for (int nt = 0; nt < NT; ++nt)
+            bb[nu][nt] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], step * 16384, 0));
+}
+
+// The first WINO_SETS - 1 steps of a stretch of steps, requested ahead of wino_steps (for the first unit of a
+// workgroup at its start, for every later one before the previous unit's results are exchanged and stored, so that
+// they travel meanwhile).  Every load here and below is unconditional -- a step beyond the range is clamped to the last
+// one and its data never used: with loads behind branches the compiler has to assume the fewest outstanding ones at
+// every wait, which shortens the distance between a load and its use to nothing.
+template <int NT>
+__device__ __forceinline__ void wino_request(f32x4 (&d)[WINO_SETS][2][4], f32x4 (&b)[WINO_SETS][4][NT], const uint32_t (&pix_off)[2][4],
+    const uint32_t (&u_off)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u, int step_begin, int step_end)
+{
+    const int last = step_end - 1;
+#pragma unroll
+    for (int s0 = 0; s0 < WINO_SETS - 1; ++s0)
+        wino_load<NT>(d[s0], b[s0], pix_off, u_off, srd_in, srd_u, step_begin + s0 < last ? step_begin + s0 : last);
+}
+
+// NT = 32-column tiles of the output channels per workgroup, XI = this wave's row of the transform domain.  The loop
+// is unrolled over the register sets, so that nothing is ever copied from one set to another.
+template <int NT, int XI>
+__device__ __forceinline__ void wino_steps(f32x4 (&d)[WINO_SETS][2][4], f32x4 (&b)[WINO_SETS][4][NT], const uint32_t (&pix_off)[2][4],
+    const uint32_t (&u_off)[4][NT], f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u,
+    int step_begin, int step_end)
+{
+    constexpr int SETS = WINO_SETS;
+    const int steps = step_end - step_begin, last = step_end - 1;
     auto multiply = [&](const f32x4 (&dd)[2][4], const f32x4 (&bb)[4][NT]) {
         // row XI of Bt over the patch rows, then Bt again over the columns
         f32x4 t[4], v[4];
@@ -97,19 +117,12 @@ __device__ __forceinline__ void wino_main(const WinoParams& p, const uint32_t (&
                 for (int e = 0; e < 4; ++e)
                     acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], bb[nu][nt][e], acc[nu][nt], 0, 0, 0);
     };
-    // Every load below is unconditional (a step index beyond the range is clamped to the last step and its data never
-    // used): with loads behind branches the compiler has to assume the fewest outstanding ones at every wait, which
-    // shortens the distance between a load and its use to nothing.
-    const int last = steps - 1;
-#pragma unroll
-    for (int s0 = 0; s0 < SETS - 1; ++s0)
-        load(d[s0], b[s0], s0 < last ? s0 : last);
     const int rounds = steps / SETS;
     for (int r = 0; r < rounds; ++r) {
 #pragma unroll
         for (int u = 0; u < SETS; ++u) {
-            const int ahead = r * SETS + u + SETS - 1;
-            load(d[(u + SETS - 1) % SETS], b[(u + SETS - 1) % SETS], ahead < last ? ahead : last);
+            const int ahead = step_begin + r * SETS + u + SETS - 1;
+            wino_load<NT>(d[(u + SETS - 1) % SETS], b[(u + SETS - 1) % SETS], pix_off, u_off, srd_in, srd_u, ahead < last ? ahead : last);
             __builtin_amdgcn_sched_barrier(0); // the loads stay in front of the step they overlap with (the scheduler
             multiply(d[u], b[u]);              // would gather them at the end of the loop body, right before their use)
             __builtin_amdgcn_sched_barrier(0);
@@ -152,33 +165,37 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     const int c4 = (lane % LANES_PER_TILE) * 4;
     constexpr uint32_t SHARE_BYTES = 4u * PASSES * 64u * 16u; // a unit's share in the workspace: [wave][pass][lane] 16-byte pieces
 
-    const int G = (int)gridDim.x, g = (int)blockIdx.x;
+    const int g = (int)blockIdx.x;
     const int spu = p.cin / 8; // steps per unit
-    const int64_t S = (int64_t)p.units * spu;
-    auto stretch_begin = [&](int gg) -> int64_t { return (int64_t)gg * S / G; };
-    auto owner_of = [&](int64_t step) -> int { return (int)(((step + 1) * G - 1) / S); }; // the stretch that holds `step`
+    // stretches: the first p.longer of them hold p.per_wg + 1 steps, the others p.per_wg (32-bit arithmetic throughout:
+    // a 64-bit division costs more than a hundred instructions, and this runs once per unit)
+    auto stretch_begin = [&](int gg) -> int { return gg * p.per_wg + (gg < p.longer ? gg : p.longer); };
+    auto owner_of = [&](int step) -> int { // the stretch that holds `step`
+        const int knee = p.longer * (p.per_wg + 1);
+        return step < knee ? step / (p.per_wg + 1) : p.longer + (step - knee) / p.per_wg;
+    };
     // a workgroup has two places in the workspace: one for the unit its stretch begins in, one for the unit it ends in
     auto share_off = [&](int gg, int unit) -> uint32_t {
         return (uint32_t)(2 * gg + (stretch_begin(gg) / spu == unit ? 0 : 1)) * SHARE_BYTES;
     };
-    int64_t pos = stretch_begin(g);
-    const int64_t end = stretch_begin(g + 1);
-    while (pos < end) {
-        const int unit = (int)(pos / spu);
-        const int64_t unit_begin = (int64_t)unit * spu;
-        const int s0 = (int)(pos - unit_begin);
-        const int s1 = end - unit_begin < spu ? (int)(end - unit_begin) : spu;
+    // What a lane needs to know of a unit: the offsets of its operands, and -- for the waves that finish the unit's
+    // tiles -- where tile (lane % 32) goes: byte offset of its pixel (0, 0), channel 0, or an out-of-range offset; bit
+    // 0 / 1 of the second word: the tile's second row / column exists.  A unit that is not live (there is none left
+    // in the stretch) gives offsets that are out of range everywhere: loads from them return zeros and move nothing.
+    struct UnitView {
+        uint32_t pix_off[2][4], u_off[4][NT];
+        int desc0, desc1;
+    };
+    const int end = stretch_begin(g + 1);
+    auto view_of = [&](bool live, int unit, UnitView& v) {
         const int mb = unit / p.n_blocks, nb = unit - mb * p.n_blocks;
-        const int n0 = nb * NC;
-
         // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
         const int tile = mb * WINO_TM + fr;
-        const bool tile_ok = tile < p.tiles;
+        const bool tile_ok = live && tile < p.tiles;
         const int rest = tile / p.tiles_x;
         const int tx = tile - rest * p.tiles_x;
         const int img = rest / p.tiles_y;
         const int ty = rest - img * p.tiles_y;
-        uint32_t pix_off[2][4];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const int row = r == 0 ? (xi == 0 ? 0 : 1) : (xi == 0 ? 2 : (xi == 3 ? 3 : 2));
@@ -187,20 +204,33 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
             for (int j = 0; j < 4; ++j) {
                 const int x = 2 * tx - p.pad_left + j;
                 const bool ok = tile_ok && y >= 0 && y < p.h && x >= 0 && x < p.w;
-                pix_off[r][j] = ok ? (uint32_t)(((img * p.h + y) * p.w + x) * p.cin + fh * 4) * 4u : OOB;
+                v.pix_off[r][j] = ok ? (uint32_t)(((img * p.h + y) * p.w + x) * p.cin + fh * 4) * 4u : OOB;
             }
         }
-        uint32_t u_off[4][NT];
 #pragma unroll
         for (int nu = 0; nu < 4; ++nu)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
-                u_off[nu][nt] = (uint32_t)(((n0 / 32 + nt) * spu * 16 + xi * 4 + nu) * 64 + lane) * 16u;
-        // where the tile's outputs go, for the waves that finish them: byte offset of pixel (0, 0) of the tile, channel
-        // 0, or an out-of-range offset; bit 0 / 1 of the second word: the tile's second row / column exists
+                v.u_off[nu][nt] = live ? (uint32_t)(((nb * NT + nt) * spu * 16 + xi * 4 + nu) * 64 + lane) * 16u : OOB;
+        v.desc0 = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
+        v.desc1 = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
+    };
+    f32x4 d[WINO_SETS][2][4], b[WINO_SETS][4][NT];
+    UnitView cur;
+    int pos = stretch_begin(g);
+    int unit = pos / spu; // (the only division by the step count: from here on units are counted up)
+    if (pos < end) {
+        const int unit_begin = unit * spu;
+        view_of(true, unit, cur);
+        wino_request<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, pos - unit_begin, end - unit_begin < spu ? end - unit_begin : spu);
+    }
+    while (pos < end) {
+        const int unit_begin = unit * spu;
+        const int s0 = pos - unit_begin, s1 = end - unit_begin < spu ? end - unit_begin : spu;
+        const int n0 = (unit % p.n_blocks) * NC;
         if (xi == 0 && fh == 0) {
-            tile_desc[fr * 2] = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
-            tile_desc[fr * 2 + 1] = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
+            tile_desc[fr * 2] = cur.desc0;
+            tile_desc[fr * 2 + 1] = cur.desc1;
         }
 
         f32x16 acc[4][NT];
@@ -212,10 +242,17 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
                 for (int e = 0; e < 16; ++e)
                     acc[nu][nt][e] = 0.f;
         switch (xi) { // the row of Bt is a compile-time choice inside the loop
-        case 0: wino_main<NT, 0>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
-        case 1: wino_main<NT, 1>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
-        case 2: wino_main<NT, 2>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
-        default: wino_main<NT, 3>(p, pix_off, u_off, acc, srd_in, srd_u, s0, s1); break;
+        case 0: wino_steps<NT, 0>(d, b, cur.pix_off, cur.u_off, acc, srd_in, srd_u, s0, s1); break;
+        case 1: wino_steps<NT, 1>(d, b, cur.pix_off, cur.u_off, acc, srd_in, srd_u, s0, s1); break;
+        case 2: wino_steps<NT, 2>(d, b, cur.pix_off, cur.u_off, acc, srd_in, srd_u, s0, s1); break;
+        default: wino_steps<NT, 3>(d, b, cur.pix_off, cur.u_off, acc, srd_in, srd_u, s0, s1); break;
+        }
+        // the next unit's first operands set out now and travel while this unit's results are exchanged and stored
+        const int next_pos = unit_begin + s1; // the next unit begins at its first step
+        {
+            const bool live = next_pos < end;
+            view_of(live, unit + 1, cur);
+            wino_request<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, 0, !live || end - next_pos >= spu ? spu : end - next_pos);
         }
 
         // At along the row: z0 = m0 + m1 + m2, z1 = m1 - m2 - m3.  Element e of a lane is tile 8 * (e / 4) + 4 * fh +
@@ -290,7 +327,8 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
             }
         }
         __syncthreads(); // the next unit overwrites the exchange area, the tile descriptors and last_flag
-        pos = unit_begin + s1;
+        pos = next_pos;
+        ++unit;
     }
 }
 
@@ -407,8 +445,11 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     p.tickets = g_wino_tickets;
     // every workgroup gets at least four steps; none gets an empty stretch
     const int64_t total_steps = (int64_t)p.units * (cin / 8);
+    FDX_REQUIRE(total_steps < (1LL << 30), "conv2d_winograd: too many steps for one launch");
     const int64_t by_steps = total_steps / 4 > 0 ? total_steps / 4 : 1;
     const dim3 grid((unsigned)(by_steps < g_wino_grid ? by_steps : g_wino_grid));
+    p.per_wg = (int)(total_steps / grid.x);
+    p.longer = (int)(total_steps % grid.x);
     const size_t lds = wino_lds_bytes(nt);
     profile_begin();
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<2>),
