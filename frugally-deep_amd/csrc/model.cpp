@@ -2301,7 +2301,7 @@ namespace {
             st = run_block_form(m, p, idx, forms[f]); // warm-up; tells whether the launcher takes the shape
             if (st != FDX_OK || p.dw_fused[idx] != forms[f])
                 continue;
-            for (int round = 0; round < 2 && st == FDX_OK; ++round) {
+            for (int round = 0; round < 4 && st == FDX_OK; ++round) { // the shortest of four rounds: a single one is too noisy to rank forms a few percent apart
                 (void)hipEventRecord(e0, stream());
                 for (int r = 0; r < 3 && st == FDX_OK; ++r)
                     st = run_block_form(m, p, idx, forms[f]);
