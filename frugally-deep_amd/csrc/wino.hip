@@ -46,7 +46,7 @@ struct WinoParams {
     int n, h, w, cin, cout, pad_top, pad_left, oh, ow;
     int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
     uint32_t in_bytes, out_bytes, u_bytes, ws_bytes;
-    int n_blocks, units; // column blocks of NT * 32 channels; units of work = blocks of 32 tiles x column blocks
+    int m_blocks, n_blocks, units; // blocks of 32 tiles, column blocks of NT * 32 channels; units of work = their product
     int per_wg, longer;  // steps per workgroup (total / workgroups) and how many workgroups take one more
     float* ws;           // shares of units that several workgroups work on: two places per workgroup
     int* tickets;        // one per unit, zero between launches
@@ -165,7 +165,13 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     const int c4 = (lane % LANES_PER_TILE) * 4;
     constexpr uint32_t SHARE_BYTES = 4u * PASSES * 64u * 16u; // a unit's share in the workspace: [wave][pass][lane] 16-byte pieces
 
-    const int g = (int)blockIdx.x;
+    // Workgroups are dealt to the eight XCDs in turn; stretch number g puts the workgroups of one XCD on neighbouring
+    // stretches, and the units are ordered by column block first, so that an XCD's workgroups read the same slab of the
+    // filter (which then stays in that XCD's L2) while each streams its own tiles.  With the tiles' order first, the
+    // workgroups of an XCD were on all column blocks at once and the filter, 4-17 MB in the transform domain, was
+    // fetched from memory once per unit.
+    const int G = (int)gridDim.x;
+    const int g = G % 8 == 0 ? ((int)blockIdx.x % 8) * (G / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
     const int spu = p.cin / 8; // steps per unit
     // stretches: the first p.longer of them hold p.per_wg + 1 steps, the others p.per_wg (32-bit arithmetic throughout:
     // a 64-bit division costs more than a hundred instructions, and this runs once per unit)
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     };
     const int end = stretch_begin(g + 1);
     auto view_of = [&](bool live, int unit, UnitView& v) {
-        const int mb = unit / p.n_blocks, nb = unit - mb * p.n_blocks;
+        const int nb = unit / p.m_blocks, mb = unit - nb * p.m_blocks;
         // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
         const int tile = mb * WINO_TM + fr;
         const bool tile_ok = live && tile < p.tiles;
@@ -227,7 +233,7 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     while (pos < end) {
         const int unit_begin = unit * spu;
         const int s0 = pos - unit_begin, s1 = end - unit_begin < spu ? end - unit_begin : spu;
-        const int n0 = (unit % p.n_blocks) * NC;
+        const int n0 = (unit / p.m_blocks) * NC;
         if (xi == 0 && fh == 0) {
             tile_desc[fr * 2] = cur.desc0;
             tile_desc[fr * 2 + 1] = cur.desc1;
@@ -434,6 +440,7 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     // (128-channel units -- NT = 4 -- were measured: the second register set of operands no longer fits beside 256
     // accumulators, and with one set the loads are not hidden: slower than 64-channel units on every ResNet50 shape)
     constexpr int nt = 2;
+    p.m_blocks = m_blocks;
     p.n_blocks = cout / (nt * 32);
     if ((int64_t)m_blocks * p.n_blocks > kWinoTickets) {
         set_error("conv2d_winograd: more than %d units of work in one launch", kWinoTickets);
