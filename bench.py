@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file and scaled by a plain copy of known size (a process cannot read these counters for itself; the
 # summaries under profiles/ give the commands and the raw readings).  Valid for the default configurations only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm, ResNet50 b64": 165.7e6, "skinny_gemm, GPT-2 decode b16": 11.0e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm + wino, ResNet50 b64": 161.2e6, "skinny_gemm, GPT-2 decode b16": 11.0e6}
 
 
 def load_package():
@@ -176,7 +176,8 @@ def bench_resnet(fdx, modelgen, args):
         "model_roofline_frac": round(img_s * flops_per_image / (PEAK_FP32_MFMA_TFLOPS * 1e12), 4),
         "roofline": {
             "bound": "mfma",
-            "kernel": "igemm_fast_kernel (implicit-GEMM Conv2D / GEMM, fp32 MFMA, all tile instantiations)",
+            "kernel": "igemm_fast_kernel (implicit-GEMM Conv2D / GEMM, fp32 MFMA, all tile instantiations) + wino_kernel (3x3 stride-1 "
+                      "convolutions, Winograd F(2x2,3x3) on fp32 MFMA); flops are the algorithmic direct-sum count of every launch",
             "achieved": round(achieved, 3),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
@@ -184,7 +185,7 @@ def bench_resnet(fdx, modelgen, args):
             "flops_per_launch": round(mf_flops / max(mf_launches, 1), 1),
             "avg_launch_ms": round(mf_ms / max(mf_launches, 1), 5),
             "share_of_step_time": round(mf_ms / total_ms, 4) if total_ms else None,
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["igemm, ResNet50 b64"] if batch == 64 else None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["igemm + wino, ResNet50 b64"] if batch == 64 else None,
         },
         "kernel_ms_per_step": {k: round(v["ms"] / prof_steps, 4) for k, v in sorted(fams.items())},
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
