@@ -482,8 +482,11 @@ void tune_store(const TuneKey& key, int choice)
 }
 bool tune_frozen()
 {
+    // FDX_AUTOTUNE=0 times nothing anywhere: the plan-level choices (block forms, direct against Winograd) that ask
+    // here take their fixed rule for shapes the table does not hold, like the tile tuner below
+    static const bool never_time = [] { const char* e = std::getenv("FDX_AUTOTUNE"); return e && e[0] == '0'; }();
     std::lock_guard<std::mutex> lock(g_tune_mutex);
-    return g_tune_frozen;
+    return g_tune_frozen || never_time;
 }
 static int g_autotune = -1;
 static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range per tile
