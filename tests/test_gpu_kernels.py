@@ -136,7 +136,10 @@ def test_gemm_vs_oracle_dense(fdx, oracle, m, n, k, tile):
     (3, 28, 28, 96, 3, 3, (2, 2), (1, 1), "valid"), (2, 14, 14, 144, 3, 3, (1, 1), (1, 1), "same"),
     # the column-tiled 3x3 kernel: widths that are not a multiple of its four-column tile, one-column images, same / valid
     (2, 7, 7, 32, 3, 3, (1, 1), (1, 1), "same"), (1, 5, 1, 8, 3, 3, (1, 1), (1, 1), "same"), (2, 9, 13, 16, 3, 3, (2, 2), (1, 1), "same"),
-    (1, 8, 10, 12, 3, 3, (1, 1), (1, 1), "valid"), (1, 3, 3, 4, 3, 3, (2, 2), (1, 1), "valid"), (2, 6, 5, 8, 5, 5, (1, 1), (1, 1), "same")])
+    (1, 8, 10, 12, 3, 3, (1, 1), (1, 1), "valid"), (1, 3, 3, 4, 3, 3, (2, 2), (1, 1), "valid"), (2, 6, 5, 8, 5, 5, (1, 1), (1, 1), "same"),
+    # enough items for the sliding-window 3x3 kernel with row tiles of 4: column tiles of 7 and of 8, extents that end inside a tile
+    (16, 14, 14, 256, 3, 3, (1, 1), (1, 1), "same"), (32, 7, 7, 480, 3, 3, (1, 1), (1, 1), "same"), (8, 9, 11, 512, 3, 3, (1, 1), (1, 1), "same"),
+    (8, 21, 16, 256, 3, 3, (1, 1), (1, 1), "valid")])
 def test_dwconv_vs_oracle(fdx, oracle, case):
     n, h, w, c, kh, kw, strides, dilation, padding = case
     say("dwconv", case)
@@ -150,6 +153,21 @@ def test_dwconv_vs_oracle(fdx, oracle, case):
     want6 = np.stack([oracle.relu(oracle.depthwise_conv2d(x[i], wj, None, kh, kw, strides, dilation, padding), 6.0, 0.0, 0.0)
                       for i in range(n)])
     assert rel(got6, want6) <= TOL
+
+
+@pytest.mark.parametrize("case", [(64, 14, 14, 1024, "same"), (64, 16, 16, 1024, "same"), (64, 16, 14, 1024, "same"), (64, 14, 16, 1024, "same"),
+                                  (64, 15, 13, 1024, "same"), (64, 18, 18, 1024, "valid")])
+def test_dwconv_sliding_window_tall_tiles(fdx, oracle, case):
+    """The sliding-window 3x3 kernel with row tiles of 7 and 8 (taken where they leave at least 65536 items): all four
+    (column tile, row tile) forms, extents that end inside a tile, both paddings; every image against the oracle."""
+    n, h, w, c, padding = case
+    say("dwconv sliding window", case)
+    r = rng_for("dwslide", case)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    wj = r.standard_normal((c, 3, 3)).astype(np.float32)
+    b = r.standard_normal(c).astype(np.float32)
+    want = np.stack([oracle.relu(oracle.depthwise_conv2d(x[i], wj, b, 3, 3, (1, 1), (1, 1), padding), 6.0, 0.0, 0.0) for i in range(n)])
+    assert rel(fdx.dwconv2d(x, wj, b, (1, 1), (1, 1), padding, act=fdx.relu_act(6.0)), want) <= TOL
 
 
 @pytest.mark.parametrize("case", [
