@@ -16,6 +16,15 @@
 #include "common.hpp"
 #include "igemm_params.hpp"
 
+// a size the kernel's 32-bit offsets do not cover: not an error of the caller, who has the layer-by-layer launches
+#define FDX_FUSED_LIMIT(cond, ...)                                                                        \
+    do {                                                                                                  \
+        if (!(cond)) {                                                                                    \
+            fdx::set_error(__VA_ARGS__);                                                                  \
+            return FDX_ERR_UNSUPPORTED;                                                                   \
+        }                                                                                                 \
+    } while (0)
+
 namespace fdx {
 
 struct DwPwParams {
@@ -291,12 +300,12 @@ extern "C" fdx_status fdx_dwconv_pointwise_nhwc_f32(const float* in, int n, int 
     p.in = in; p.dw_w = dw_weights_hwc; p.dw_b = dw_bias; p.pw_w = pw_weights_nc; p.pw_b = pw_bias; p.residual = residual; p.out = out;
     p.n = n; p.h = h; p.w = w; p.c = c; p.pad_top = pad_top; p.pad_left = pad_left; p.oh = out_h; p.ow = out_w; p.N = n_out;
     p.xt = (out_w + DWPW_TX - 1) / DWPW_TX;
-    FDX_REQUIRE((int64_t)n * out_h * p.xt < (1LL << 31) - 64, "dwconv_pointwise: too many output pixels for one launch");
+    FDX_FUSED_LIMIT((int64_t)n * out_h * p.xt < (1LL << 31) - 64, "dwconv_pointwise: too many output pixels for one launch");
     p.runs = n * out_h * p.xt;
     p.c_pad = (c + DWPW_KC - 1) / DWPW_KC * DWPW_KC;
-    FDX_REQUIRE((int64_t)n * h * w * c * 4 < (1LL << 31), "dwconv_pointwise: input tensor beyond 2 GiB");
+    FDX_FUSED_LIMIT((int64_t)n * h * w * c * 4 < (1LL << 31), "dwconv_pointwise: input tensor beyond 2 GiB");
     p.in_bytes = (uint32_t)((int64_t)n * h * w * c * 4);
-    FDX_REQUIRE((int64_t)n * out_h * out_w * n_out * 4 < (1LL << 31), "dwconv_pointwise: output tensor beyond 2 GiB");
+    FDX_FUSED_LIMIT((int64_t)n * out_h * out_w * n_out * 4 < (1LL << 31), "dwconv_pointwise: output tensor beyond 2 GiB");
     p.out_bytes = (uint32_t)((int64_t)n * out_h * out_w * n_out * 4);
     p.act1 = make_act(dw_act);
     p.act2 = make_act(act);

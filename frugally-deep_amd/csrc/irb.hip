@@ -25,6 +25,15 @@
 #include "common.hpp"
 #include "igemm_params.hpp"
 
+// a size the kernel's 32-bit offsets do not cover: not an error of the caller, who has the layer-by-layer launches
+#define FDX_FUSED_LIMIT(cond, ...)                                                                        \
+    do {                                                                                                  \
+        if (!(cond)) {                                                                                    \
+            fdx::set_error(__VA_ARGS__);                                                                  \
+            return FDX_ERR_UNSUPPORTED;                                                                   \
+        }                                                                                                 \
+    } while (0)
+
 namespace fdx {
 
 struct IrbParams {
@@ -422,12 +431,12 @@ static fdx_status irb_launch(IrbParams& p, int cin, int n_out, int stride, bool 
 {
     p.tiles_x = (p.ow + IRB_TW - 1) / IRB_TW;
     p.tiles_y = (p.oh + IRB_TH - 1) / IRB_TH;
-    FDX_REQUIRE((int64_t)p.n * p.tiles_x * p.tiles_y < (1LL << 30), "inverted_residual: too many output pixels for one launch");
+    FDX_FUSED_LIMIT((int64_t)p.n * p.tiles_x * p.tiles_y < (1LL << 30), "inverted_residual: too many output pixels for one launch");
     p.tiles = p.n * p.tiles_x * p.tiles_y;
     p.ce_pad = (p.ce + IRB_KC - 1) / IRB_KC * IRB_KC;
-    FDX_REQUIRE(in_floats * 4 < (1LL << 31), "inverted_residual: input tensor beyond 2 GiB");
+    FDX_FUSED_LIMIT(in_floats * 4 < (1LL << 31), "inverted_residual: input tensor beyond 2 GiB");
     p.in_bytes = (uint32_t)(in_floats * 4);
-    FDX_REQUIRE((int64_t)p.n * p.oh * p.ow * n_out * 4 < (1LL << 31), "inverted_residual: output tensor beyond 2 GiB");
+    FDX_FUSED_LIMIT((int64_t)p.n * p.oh * p.ow * n_out * 4 < (1LL << 31), "inverted_residual: output tensor beyond 2 GiB");
     p.out_bytes = (uint32_t)((int64_t)p.n * p.oh * p.ow * n_out * 4);
     const int ct = (n_out + 31) / 32, kin = cin / 8;
     const int nw = irb_waves(cin, p.ce, n_out, stride);
@@ -554,7 +563,7 @@ extern "C" fdx_status fdx_stem_block_nhwc_f32(const float* in, int n, int ih, in
         "stem_block: the convolution's output size does not fit the image");
     FDX_REQUIRE(pad_top >= 0 && pad_left >= 0 && (int64_t)(out_h - 1) * stride - pad_top < h && (int64_t)(out_w - 1) * stride - pad_left < w,
         "stem_block: output size does not fit the convolution's output");
-    FDX_REQUIRE((int64_t)iw * ic * ek * 4 < (1LL << 24), "stem_block: image rows too long");
+    FDX_FUSED_LIMIT((int64_t)iw * ic * ek * 4 < (1LL << 24), "stem_block: image rows too long");
     IrbParams p;
     std::memset(&p, 0, sizeof p);
     p.in = in; p.exp_w = conv_weights_nk; p.exp_b = conv_bias; p.dw_w = dw_weights_hwc; p.dw_b = dw_bias; p.pw_w = pw_weights_nc;

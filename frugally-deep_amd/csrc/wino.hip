@@ -406,6 +406,15 @@ extern "C" fdx_status fdx_conv2d_winograd_prepare(const float* weights_nkkc, int
     return FDX_OK;
 }
 
+// a size the kernel's 32-bit offsets and tickets do not cover: not an error of the caller, who has the direct kernel
+#define FDX_WINO_LIMIT(cond, ...)                                                                         \
+    do {                                                                                                  \
+        if (!(cond)) {                                                                                    \
+            fdx::set_error(__VA_ARGS__);                                                                  \
+            return FDX_ERR_UNSUPPORTED;                                                                   \
+        }                                                                                                 \
+    } while (0)
+
 extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h, int w, int cin, const float* u_weights, const float* bias,
     int cout, int pad_top, int pad_left, int out_h, int out_w, const float* residual, const fdx_act* act, float* out)
 {
@@ -426,13 +435,13 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     p.n = n; p.h = h; p.w = w; p.cin = cin; p.cout = cout; p.pad_top = pad_top; p.pad_left = pad_left; p.oh = out_h; p.ow = out_w;
     p.tiles_x = (out_w + 1) / 2;
     p.tiles_y = (out_h + 1) / 2;
-    FDX_REQUIRE((int64_t)n * p.tiles_x * p.tiles_y < (1LL << 30), "conv2d_winograd: too many output pixels for one launch");
+    FDX_WINO_LIMIT((int64_t)n * p.tiles_x * p.tiles_y < (1LL << 30), "conv2d_winograd: too many output pixels for one launch");
     p.tiles = n * p.tiles_x * p.tiles_y;
-    FDX_REQUIRE((int64_t)n * h * w * cin * 4 < (1LL << 31), "conv2d_winograd: input tensor beyond 2 GiB");
+    FDX_WINO_LIMIT((int64_t)n * h * w * cin * 4 < (1LL << 31), "conv2d_winograd: input tensor beyond 2 GiB");
     p.in_bytes = (uint32_t)((int64_t)n * h * w * cin * 4);
-    FDX_REQUIRE((int64_t)n * out_h * out_w * cout * 4 < (1LL << 31), "conv2d_winograd: output tensor beyond 2 GiB");
+    FDX_WINO_LIMIT((int64_t)n * out_h * out_w * cout * 4 < (1LL << 31), "conv2d_winograd: output tensor beyond 2 GiB");
     p.out_bytes = (uint32_t)((int64_t)n * out_h * out_w * cout * 4);
-    FDX_REQUIRE((int64_t)16 * cout * cin * 4 < (1LL << 31), "conv2d_winograd: filter beyond 2 GiB");
+    FDX_WINO_LIMIT((int64_t)16 * cout * cin * 4 < (1LL << 31), "conv2d_winograd: filter beyond 2 GiB");
     p.u_bytes = (uint32_t)((int64_t)16 * cout * cin * 4);
     p.act = make_act(act);
     FDX_REQUIRE(wino_prepare(), "conv2d_winograd: no device memory for the workspace");
@@ -452,7 +461,7 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     p.tickets = g_wino_tickets;
     // every workgroup gets at least four steps; none gets an empty stretch
     const int64_t total_steps = (int64_t)p.units * (cin / 8);
-    FDX_REQUIRE(total_steps < (1LL << 30), "conv2d_winograd: too many steps for one launch");
+    FDX_WINO_LIMIT(total_steps < (1LL << 30), "conv2d_winograd: too many steps for one launch");
     const int64_t by_steps = total_steps / 4 > 0 ? total_steps / 4 : 1;
     const dim3 grid((unsigned)(by_steps < g_wino_grid ? by_steps : g_wino_grid));
     p.per_wg = (int)(total_steps / grid.x);
@@ -461,7 +470,7 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     profile_begin();
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(wino_kernel<2>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)wino_lds_bytes(2));
-    FDX_REQUIRE(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
+    FDX_WINO_LIMIT(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
     hipLaunchKernelGGL(wino_kernel<2>, grid, dim3(256), lds, stream(), p);
     const double pix = (double)n * out_h * out_w;
     profile_end("conv2d_winograd_f32", 2.0 * pix * 9.0 * cin * cout, 4.0 * ((double)n * h * w * cin + pix * cout * (residual ? 2.0 : 1.0) + 9.0 * cin * cout));
