@@ -112,6 +112,30 @@ def cpu_baseline_decode(js, cores, prompt=4, warmup=3, timed=5):
     return cores * timed / dt
 
 
+def shader_clock_during(fdx, run_step, steps, ms_per_step):
+    """Shader clock (GHz) while `steps` forward passes run: the library's probe samples the cycle counter against the
+    constant-rate wall counter every 100 us on a stream of its own.  Outside the timed region."""
+    period_us = 100
+    window_ms = steps * ms_per_step
+    samples = int(min(65536, max(8, window_ms * 1e3 / period_us * 1.05 + 4)))
+    fdx.sync()
+    fdx.check(fdx.lib.fdx_clock_probe_start(samples, period_us))
+    for _ in range(steps):
+        run_step()
+    fdx.sync()
+    mean, lo, hi = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    fdx.check(fdx.lib.fdx_clock_probe_stop(ctypes.c_double(window_ms), ctypes.byref(mean), ctypes.byref(lo), ctypes.byref(hi)))
+    # the same probe with nothing else running
+    fdx.check(fdx.lib.fdx_clock_probe_start(64, period_us))
+    imean, ilo, ihi = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    fdx.check(fdx.lib.fdx_clock_probe_stop(ctypes.c_double(6.0), ctypes.byref(imean), ctypes.byref(ilo), ctypes.byref(ihi)))
+    return {"mean_ghz": round(mean.value, 3), "min_ghz": round(lo.value, 3), "max_ghz": round(hi.value, 3),
+            "idle_ghz": round(imean.value, 3),
+            "what": "shader cycle counter against the 100 MHz wall counter, one sample per 100 us over %d forward passes "
+                    "run after the timed region (min / max: single periods); idle = the same probe with nothing else running. "
+                    "The published peak the roofline uses assumes 2.4 GHz" % steps}
+
+
 def bench_resnet(fdx, modelgen, args):
     batch = args.batch
     spec = modelgen.resnet50()
@@ -191,6 +215,9 @@ def bench_resnet(fdx, modelgen, args):
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
         "load_seconds": round(load_s, 2),
     }
+    if not args.no_clock_probe:
+        result["shader_clock"] = shader_clock_during(fdx, lambda: model.predict_dev(batch, [d_in], shapes, [d_out]), args.steps,
+                                                     seconds * 1e3 / args.steps)
     # what a model.predict caller with host tensors sees: the same batch through fdx_model_predict, host-to-device copy
     # of the 38.5 MB input and device-to-host copy of the outputs included (pageable host memory)
     model.predict([x])
@@ -212,7 +239,7 @@ def bench_resnet(fdx, modelgen, args):
     return result
 
 
-def bench_secondary(fdx, modelgen, name, spec, batch, inputs, steps, warmup):
+def bench_secondary(fdx, modelgen, name, spec, batch, inputs, steps, warmup, clock_probe=True):
     """Secondary configurations (MobileNetV2 b128, transformer encoder b32): samples / second of one batched predict
     with inputs resident, and per kernel family the HIP-event time with its own roofline (TFLOP/s against the fp32
     MFMA peak for the GEMM families, algorithmic GB/s against HBM for the memory-bound ones)."""
@@ -255,6 +282,9 @@ def bench_secondary(fdx, modelgen, name, spec, batch, inputs, steps, warmup):
     res = {"workload": name, "batch": batch, "value": round(batch / sec, 1), "unit": "samples/s", "ms_per_step": round(sec * 1e3, 4),
            "gflop_per_sample": round(flops / batch / 1e9, 4),
            "model_mfma_frac": round(flops / sec / (PEAK_FP32_MFMA_TFLOPS * 1e12), 4), "kernels": per_family}
+    if clock_probe:
+        res["shader_clock"] = shader_clock_during(fdx, lambda: model.predict_dev(batch, d_in, shapes, d_out), steps, sec * 1e3)
+        res["shader_clock"].pop("what")
     model.close()
     for b in d_in + d_out:
         b.free()
@@ -387,6 +417,7 @@ def main():
     ap.add_argument("--decode-reps", type=int, default=2)
     ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels", "mobilenet_v2", "encoder"], default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-clock-probe", action="store_true", help="skip the shader-clock pass after the timed region")
     ap.add_argument("--ring-mb", type=float, default=600.0,
                     help="gpt2_kernels: total size of the ring of weight copies a kernel cycles through (larger than the "
                          "caches by default, so every launch streams from HBM)")
@@ -421,12 +452,13 @@ def main():
     if args.workload in ("all", "mobilenet_v2"):
         x = rng.uniform(0, 1, (128, 224, 224, 3)).astype(np.float32)
         secondary["mobilenet_v2"] = bench_secondary(fdx, modelgen, "MobileNetV2 alpha 1.0 architecture, 224x224x3, batch 128",
-                                                    modelgen.mobilenet_v2(), 128, [x], max(3, args.steps // 2), 3)
+                                                    modelgen.mobilenet_v2(), 128, [x], max(3, args.steps // 2), 3,
+                                                    not args.no_clock_probe)
     if args.workload in ("all", "encoder"):
         x = rng.standard_normal((32, 256, 512)).astype(np.float32)
         secondary["encoder"] = bench_secondary(fdx, modelgen, "6-layer pre-LN transformer encoder, seq 256, d 512, 8 heads, "
                                                "ffn 2048 (erf-GELU), batch 32", modelgen.encoder(), 32, [x],
-                                               max(3, args.steps // 2), 3)
+                                               max(3, args.steps // 2), 3, not args.no_clock_probe)
     if secondary:
         if result:
             result["secondary"] = secondary

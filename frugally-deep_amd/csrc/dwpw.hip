@@ -239,15 +239,17 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
     }
 }
 
-// workgroups of `kernel` with `lds` bytes of dynamic LDS that are resident at once (remembered per LDS size: one static
-// table per kernel instantiation; launches are serialised by the caller's stream order, the table by this mutex)
+// workgroups of `kernel` with `lds` bytes of dynamic LDS that are resident at once, remembered per (kernel, LDS size):
+// the instantiations share one function type, so the table is keyed by the kernel's address (launches are serialised by
+// the caller's stream order, the table by this mutex)
 template <typename K>
 static int64_t dwpw_resident(K kernel, size_t lds)
 {
     static std::mutex mu;
-    static std::map<size_t, int64_t> known;
+    static std::map<std::pair<const void*, size_t>, int64_t> known;
+    const std::pair<const void*, size_t> key(reinterpret_cast<const void*>(kernel), lds);
     std::lock_guard<std::mutex> lock(mu);
-    auto it = known.find(lds);
+    auto it = known.find(key);
     if (it != known.end())
         return it->second;
     int per_cu = 1, dev = 0;
@@ -255,7 +257,7 @@ static int64_t dwpw_resident(K kernel, size_t lds)
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds) != hipSuccess || per_cu < 1)
         per_cu = 1;
     const int cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
-    return known[lds] = (int64_t)per_cu * cus;
+    return known[key] = (int64_t)per_cu * cus;
 }
 
 // LDS of a workgroup: the waves' A slabs, plus the whole 1x1 filter where that still leaves room for a second workgroup

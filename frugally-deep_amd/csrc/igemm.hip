@@ -301,7 +301,10 @@ static int g_persist_scale = 0; // 0 = resident workgroups; tests and tuning may
 template <typename K>
 static int resident_workgroups(K kernel, int threads)
 {
-    static int resident = 0; // one instance per kernel instantiation
+    // keyed by the kernel's address: every instantiation has the same function type, so a static inside this template
+    // would be one value for all of them (callers hold g_igemm_mutex)
+    static std::map<const void*, int> cache;
+    int& resident = cache[reinterpret_cast<const void*>(kernel)];
     if (resident == 0) {
         int per_cu = 1, dev = 0;
         hipDeviceProp_t prop;

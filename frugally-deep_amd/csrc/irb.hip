@@ -409,20 +409,23 @@ static int irb_waves(int cin, int ce, int n_out, int stride)
 template <typename K>
 static int64_t irb_resident(K kernel, int threads, size_t lds)
 {
+    // keyed by the kernel's address as well: the instantiations share one function type, and the dynamic LDS limit is
+    // an attribute of each of them
     static std::mutex mu;
-    static std::map<size_t, int64_t> known;
+    static std::map<std::pair<const void*, size_t>, int64_t> known;
+    const std::pair<const void*, size_t> key(reinterpret_cast<const void*>(kernel), lds);
     std::lock_guard<std::mutex> lock(mu);
-    auto it = known.find(lds);
+    auto it = known.find(key);
     if (it != known.end())
         return it->second;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return known[lds] = 0;
+        return known[key] = 0;
     int per_cu = 0, dev = 0;
     hipDeviceProp_t prop;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds) != hipSuccess || per_cu < 1)
-        return known[lds] = 0;
+        return known[key] = 0;
     const int cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
-    return known[lds] = (int64_t)per_cu * cus;
+    return known[key] = (int64_t)per_cu * cus;
 }
 
 // Fills the tile counts and extents of `p` (pointers, image / grid sizes, channel counts and activations are set) and

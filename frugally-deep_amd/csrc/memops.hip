@@ -2,9 +2,11 @@
 // LayerNorm, softmax, embedding gather, argmax, transpose.  All are channel-innermost
 // (NHWC) so consecutive lanes touch consecutive addresses; rows are reduced with wave64
 // shuffles and, across waves, a small LDS exchange.
+#include <algorithm>
 #include <cfloat>
-
 #include <cstdlib>
+#include <mutex>
+#include <vector>
 #include "common.hpp"
 
 namespace fdx {
@@ -911,4 +913,87 @@ fdx_status argmax_launch(const float* x, int64_t rows, int depth, int32_t* out_i
 extern "C" fdx_status fdx_argmax_f32(const float* x, int64_t rows, int depth, int32_t* out_idx, float* out_val)
 {
     return fdx::argmax_launch(x, rows, depth, out_idx, out_val, nullptr);
+}
+
+// ---- shader-clock probe (a measurement aid; nothing in the reference corresponds to it)
+//
+// One lane on a stream of its own records the shader cycle counter and the constant-rate wall counter once per
+// period while the library stream runs its work; the ratio of their steps is the clock the compute units ran at
+// during that period.  The wait between samples sleeps and is bounded, and the kernel ends after `samples` periods
+// whatever else happens.
+namespace fdx {
+__global__ void clock_probe_kernel(long long* out, int samples, long long period_ticks)
+{
+    long long next = wall_clock64();
+    for (int i = 0; i < samples; ++i) {
+        out[2 * i] = clock64();
+        out[2 * i + 1] = wall_clock64();
+        next += period_ticks;
+        for (int spin = 0; spin < (1 << 18) && wall_clock64() < next; ++spin)
+            __builtin_amdgcn_s_sleep(16);
+    }
+}
+
+static std::mutex g_probe_mutex;
+static hipStream_t g_probe_stream = nullptr;
+static long long* g_probe_buf = nullptr;
+static int g_probe_samples = 0;
+constexpr int kProbeMaxSamples = 1 << 16;
+}
+
+extern "C" fdx_status fdx_clock_probe_start(int samples, int period_us)
+{
+    FDX_REQUIRE(samples >= 2 && samples <= kProbeMaxSamples && period_us >= 10 && period_us <= 100000,
+        "clock_probe_start: 2..65536 samples, period 10..100000 us");
+    (void)stream(); // the library is initialised on its device
+    std::lock_guard<std::mutex> lock(g_probe_mutex);
+    FDX_REQUIRE(g_probe_samples == 0, "clock_probe_start: a probe is already running; call fdx_clock_probe_stop first");
+    if (!g_probe_stream)
+        FDX_HIP(hipStreamCreateWithFlags(&g_probe_stream, hipStreamNonBlocking));
+    if (!g_probe_buf)
+        FDX_HIP(hipMalloc(&g_probe_buf, (size_t)kProbeMaxSamples * 2 * sizeof(long long)));
+    int dev = 0, khz = 0;
+    FDX_HIP(hipGetDevice(&dev));
+    FDX_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    FDX_REQUIRE(khz > 0, "clock_probe_start: the device reports no wall clock rate");
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(1), 0, g_probe_stream, g_probe_buf, samples,
+        (long long)khz * period_us / 1000);
+    FDX_LAUNCH_CHECK();
+    g_probe_samples = samples;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_clock_probe_stop(double window_ms, double* mean_ghz, double* min_ghz, double* max_ghz)
+{
+    FDX_REQUIRE(mean_ghz && min_ghz && max_ghz && window_ms > 0, "clock_probe_stop: bad arguments");
+    std::lock_guard<std::mutex> lock(g_probe_mutex);
+    FDX_REQUIRE(g_probe_samples > 0, "clock_probe_stop: no probe was started");
+    const int n = g_probe_samples;
+    g_probe_samples = 0;
+    FDX_HIP(hipStreamSynchronize(g_probe_stream));
+    std::vector<long long> h((size_t)n * 2);
+    FDX_HIP(hipMemcpy(h.data(), g_probe_buf, h.size() * sizeof(long long), hipMemcpyDeviceToHost));
+    int dev = 0, khz = 0;
+    FDX_HIP(hipGetDevice(&dev));
+    FDX_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    const double window_ticks = window_ms * khz;
+    double lo = 1e30, hi = 0.0;
+    long long c_first = h[0], w_first = h[1], c_last = h[0], w_last = h[1];
+    for (int i = 1; i < n; ++i) {
+        const long long dw = h[2 * i + 1] - h[2 * i - 1], dc = h[2 * i] - h[2 * i - 2];
+        if ((double)(h[2 * i + 1] - w_first) > window_ticks)
+            break;
+        if (dw <= 0)
+            continue;
+        const double ghz = (double)dc / (double)dw * khz * 1e-6;
+        lo = std::min(lo, ghz);
+        hi = std::max(hi, ghz);
+        c_last = h[2 * i];
+        w_last = h[2 * i + 1];
+    }
+    FDX_REQUIRE(w_last > w_first, "clock_probe_stop: no complete period inside the window");
+    *mean_ghz = (double)(c_last - c_first) / (double)(w_last - w_first) * khz * 1e-6;
+    *min_ghz = lo;
+    *max_ghz = hi;
+    return FDX_OK;
 }

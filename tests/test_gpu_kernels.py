@@ -528,6 +528,29 @@ def test_launcher_argument_errors(fdx):
         fdx.window_geometry(0, 4, 3, 3, 1, 1, "same")
 
 
+def test_shader_clock_probe(fdx):
+    """The measurement aid bench.py uses: a sampler on its own stream, bounded, one at a time."""
+    say("clock probe")
+    c = fdx.ctypes
+    mean, lo, hi = c.c_double(), c.c_double(), c.c_double()
+    with pytest.raises(fdx.FdxError):  # nothing started
+        fdx.check(fdx.lib.fdx_clock_probe_stop(c.c_double(1.0), c.byref(mean), c.byref(lo), c.byref(hi)))
+    with pytest.raises(fdx.FdxError):
+        fdx.check(fdx.lib.fdx_clock_probe_start(1, 100))
+    fdx.check(fdx.lib.fdx_clock_probe_start(40, 100))
+    with pytest.raises(fdx.FdxError):  # one at a time
+        fdx.check(fdx.lib.fdx_clock_probe_start(40, 100))
+    x = fdx.DevBuf.from_host(np.ones((1 << 20,), np.float32))
+    y = fdx.DevBuf(4 << 20)
+    act = fdx.relu_act()
+    for _ in range(20):  # some work beside it on the library stream
+        fdx.check(fdx.lib.fdx_activation_f32(fdx._dp(x), c.c_size_t(1 << 20), c.byref(act), fdx._dp(y)))
+    fdx.sync()
+    fdx.check(fdx.lib.fdx_clock_probe_stop(c.c_double(3.5), c.byref(mean), c.byref(lo), c.byref(hi)))
+    assert 0.3 < lo.value <= mean.value <= hi.value < 4.0, (lo.value, mean.value, hi.value)
+    assert y.to_host((1 << 20,))[123] == 1.0
+
+
 DENSE_ROWS = [(16, 768, 2304), (16, 768, 768), (16, 3072, 768), (3, 64, 100), (16, 768, 50257), (5, 20, 33), (7, 1024, 40),
               (16, 100, 64), (1, 2048, 48)]
 
