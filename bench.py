@@ -418,6 +418,9 @@ def main():
     ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels", "mobilenet_v2", "encoder"], default="all")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-clock-probe", action="store_true", help="skip the shader-clock pass after the timed region")
+    ap.add_argument("--tuner-import", default=None, help="per-shape tuner table to load and freeze before anything runs "
+                                                         "(fdx_tuner_import + fdx_tuner_freeze: nothing is timed, every run picks the same kernels)")
+    ap.add_argument("--tuner-export", default=None, help="write the per-shape tuner table of this run to this file at the end")
     ap.add_argument("--ring-mb", type=float, default=600.0,
                     help="gpt2_kernels: total size of the ring of weight copies a kernel cycles through (larger than the "
                          "caches by default, so every launch streams from HBM)")
@@ -429,6 +432,9 @@ def main():
         sys.exit("bench.py: this build runs on one GPU only (samples are independent; more GPUs would each take a "
                  "slice of the batch with their own copy of the weights) -- use --gpus 1")
     fdx, modelgen = load_package()
+    if args.tuner_import:
+        fdx.tuner_import(open(args.tuner_import).read())
+        fdx.tuner_freeze(True)
     if args.calibrate_copy_mib > 0:
         n = args.calibrate_copy_mib * (1 << 20) // 4
         src, dst = fdx.DevBuf(4 * n), fdx.DevBuf(4 * n)
@@ -464,6 +470,9 @@ def main():
             result["secondary"] = secondary
         else:
             result = {"metric": "secondary configurations", "n_gpus": 1, "secondary": secondary}
+    if args.tuner_export:
+        with open(args.tuner_export, "w") as f:
+            f.write(fdx.tuner_export())
     print(json.dumps(result), flush=True)
 
 

@@ -597,7 +597,9 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     if (log_picks)
         std::fprintf(stderr, "[fdx tune] conv=%d M=%d N=%d K=%d Cin=%d k=%dx%d s=%d res=%d: plain %d %.1f us, split %d %.1f us\n", (int)conv,
             q.M, q.N, q.K, q.Cin, q.kh, q.kw, q.sy, (int)(q.residual != nullptr), best, best_ms * 1e3f / 3, best_split, best_split_ms * 1e3f / 3);
-    if (best_split >= 0 && (best < 0 || best_split_ms < best_ms))
+    // a split variant writes partial tiles and reads them back; it has to win by more than the timing noise to be
+    // worth that traffic
+    if (best_split >= 0 && (best < 0 || best_split_ms < 0.98f * best_ms))
         best = best_split;
     if (log_picks)
         std::fprintf(stderr, "[fdx tune]   -> %d\n", best);
@@ -649,25 +651,27 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         splits = mode == 2 ? 0 : std::max(1, (cfg % 10000) / 100);
         cfg %= 100;
     };
-    if (cfg >= 100)
-        unpack();
     const bool stream_ok = pw_stream_ok(p, conv, batch, a_bytes, b_bytes) && b_vec;
-    if (cfg == kStreamCfg && !stream_ok)
-        cfg = -1;
-    if (cfg >= 10 && cfg != kStreamCfg && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
-        cfg = -1;
-    if (cfg < 10 || mode > 2) {
-        splits = 1;
-        mode = 0;
-    }
-    if (cfg == kStreamCfg) {
-        splits = 1;
-        mode = 0;
-    }
-    if (cfg >= 10 && splits != 1 && (cfg > 15 || !split_prepare())) {
-        splits = 1;
-        mode = 0;
-    }
+    // A choice comes from a test hook, from this process's timing runs, or from an imported table: whatever its source, it
+    // is only taken where this problem meets the kernel's conditions, and a split choice only with the workspace in
+    // place (a process that imports its table has not timed anything, so nothing else would have allocated it).
+    auto settle = [&]() {
+        if (cfg >= 100)
+            unpack();
+        if (cfg == kStreamCfg && !stream_ok)
+            cfg = -1;
+        if (cfg >= 10 && cfg != kStreamCfg && (!fast_ok || (cfg >= 13 && unit % 32 != 0)))
+            cfg = -1;
+        if (cfg < 10 || mode > 2 || mode < 0 || splits < 0 || splits > 64 || cfg == kStreamCfg) {
+            splits = 1;
+            mode = 0;
+        }
+        if (cfg >= 10 && splits != 1 && (cfg > 15 || !split_prepare())) {
+            splits = 1;
+            mode = 0;
+        }
+    };
+    settle();
     auto launch_general = [&](int c) {
         switch (c) {
         case 0: launch_cfg<128, 128, 2, 2>(p, a_mode, b_vec, batch, s); break;
@@ -689,8 +693,7 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
             const int general_cfg = !general_ok ? -1 : p.N <= 32 ? 2 : (blocks(128, 64) >= 512 ? 1 : 3);
             cfg = autotune(q, conv, batch, unit, s, general_cfg, [&] { launch_general(general_cfg); }, stream_ok,
                 [&] { pw_stream_launch(p, a_bytes, b_bytes, s); });
-            if (cfg >= 100)
-                unpack();
+            settle();
         }
         if (cfg >= 0) {
         } else if (fast_ok && p.N >= 64) {

@@ -203,3 +203,36 @@ def test_predict_from_several_host_threads(fdx, modelgen):
         th.join(timeout=100)
     assert not errors, errors[:5]
     assert len(results) == 4
+
+
+FRESH_PROCESS_IMPORT = r"""
+import importlib, sys, numpy as np
+sys.path.insert(0, sys.argv[1])
+fdx = importlib.import_module("frugally-deep_amd")
+# conv M N K Cin kh kw sy sx batch res choice: every tile of a 2048 x 256 x 512 GEMM cut into two K ranges (64 x 64 x 32
+# tile), the same as only the last round (hybrid), and as stream-K
+m, n, k = 2048, 256, 512
+r = np.random.default_rng(5)
+a = r.standard_normal((m, k)).astype(np.float32)
+w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+b = r.standard_normal(n).astype(np.float32)
+want = a.astype(np.float64) @ w.astype(np.float64).T + b
+for choice in (215, 10215, 20015):
+    fdx.tuner_import("0 %d %d %d 0 0 0 0 0 1 0 %d\n" % (m, n, k, choice))
+    fdx.tuner_freeze(True)
+    got = fdx.gemm(a, w, b)
+    err = float(np.abs(got - want).max() / np.abs(want).max())
+    print("choice", choice, "err", err, flush=True)
+    assert err < 1e-5, err
+print("ok", flush=True)
+"""
+
+
+def test_imported_split_choice_in_a_fresh_process(fdx):
+    """A deployment imports its tuner table before anything has run: the split variants' workspace, which the timing
+    runs of a tuning process allocate on the way, has to be there for the first launch all the same."""
+    import os, subprocess, sys
+    say("imported table, fresh process")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", FRESH_PROCESS_IMPORT, root], capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), (out.returncode, out.stdout[-400:], out.stderr[-800:])
