@@ -412,7 +412,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=10,
+                    help="untimed passes before the timed ones (the shader clock needs about 30 ms of load to settle after an idle period)")
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--decode-reps", type=int, default=2)
     ap.add_argument("--workload", choices=["all", "resnet50", "gpt2", "gpt2_kernels", "mobilenet_v2", "encoder"], default="all")
@@ -458,13 +459,13 @@ def main():
     if args.workload in ("all", "mobilenet_v2"):
         x = rng.uniform(0, 1, (128, 224, 224, 3)).astype(np.float32)
         secondary["mobilenet_v2"] = bench_secondary(fdx, modelgen, "MobileNetV2 alpha 1.0 architecture, 224x224x3, batch 128",
-                                                    modelgen.mobilenet_v2(), 128, [x], max(3, args.steps // 2), 3,
+                                                    modelgen.mobilenet_v2(), 128, [x], max(3, args.steps), max(3, 3 * args.warmup),
                                                     not args.no_clock_probe)
     if args.workload in ("all", "encoder"):
         x = rng.standard_normal((32, 256, 512)).astype(np.float32)
         secondary["encoder"] = bench_secondary(fdx, modelgen, "6-layer pre-LN transformer encoder, seq 256, d 512, 8 heads, "
                                                "ffn 2048 (erf-GELU), batch 32", modelgen.encoder(), 32, [x],
-                                               max(3, args.steps // 2), 3, not args.no_clock_probe)
+                                               max(3, args.steps), max(3, 3 * args.warmup // 2), not args.no_clock_probe)
     if secondary:
         if result:
             result["secondary"] = secondary

@@ -13,6 +13,7 @@
 // LDS read into four MFMAs (the k order inside a slab is permuted identically for A and
 // B, which a sum does not notice).  Epilogue: alpha, bias (per column or per row),
 // residual add, activation, fused on the accumulators before the only store.
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -483,6 +484,32 @@ void tune_store(const TuneKey& key, int choice)
     std::lock_guard<std::mutex> lock(g_tune_mutex);
     g_tuned[key] = choice;
 }
+static std::chrono::steady_clock::time_point g_tune_end; // end of the last timing run (epoch = none yet)
+static std::mutex g_tune_end_mutex;
+void tune_mark()
+{
+    std::lock_guard<std::mutex> lock(g_tune_end_mutex);
+    g_tune_end = std::chrono::steady_clock::now();
+}
+void tune_settle_clock(const std::function<bool()>& launch)
+{
+    using namespace std::chrono;
+    {
+        std::lock_guard<std::mutex> lock(g_tune_end_mutex);
+        if (steady_clock::now() - g_tune_end < milliseconds(5))
+            return;
+    }
+    const auto t0 = steady_clock::now();
+    bool ok = true;
+    while (ok && steady_clock::now() - t0 < milliseconds(30)) {
+        for (int r = 0; r < 3 && ok; ++r)
+            ok = launch();
+        if (hipStreamSynchronize(stream()) != hipSuccess)
+            break;
+    }
+    tune_mark();
+}
+
 bool tune_frozen()
 {
     // FDX_AUTOTUNE=0 times nothing anywhere: the plan-level choices (block forms, direct against Winograd) that ask
@@ -540,6 +567,7 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
         }
         return best_round;
     };
+    bool clock_settled = false;
     for (int cfg = 10; cfg <= 18; ++cfg) {
         if (cfg >= 13 && unit % 32 != 0)
             continue;
@@ -563,6 +591,10 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
                 continue;
             if (!launch_fast(cfg, splits, mode, q, conv, batch, s)) // warm-up; false = the cut does not fit
                 continue;
+            if (!clock_settled) {
+                tune_settle_clock([&] { return launch_fast(cfg, splits, mode, q, conv, batch, s); });
+                clock_settled = true;
+            }
             const float ms = timed([&] { launch_fast(cfg, splits, mode, q, conv, batch, s); });
             if (splits == 1) {
                 if (ms < best_ms) {
@@ -601,6 +633,7 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
     }
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
+    tune_mark();
     static const bool log_picks = [] { const char* e = std::getenv("FDX_TUNE_LOG"); return e && e[0] == '1'; }();
     if (log_picks)
         std::fprintf(stderr, "[fdx tune] conv=%d M=%d N=%d K=%d Cin=%d k=%dx%d s=%d res=%d: plain %d %.1f us, split %d %.1f us with its handicap\n", (int)conv,

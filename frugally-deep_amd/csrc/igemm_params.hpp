@@ -1,6 +1,7 @@
 // Launch parameters shared by the implicit-GEMM kernels.
 #pragma once
 #include <cstring>
+#include <functional>
 #include "common.hpp"
 
 namespace fdx {
@@ -52,5 +53,12 @@ struct TuneKey {
 bool tune_lookup(const TuneKey& key, int* choice);
 void tune_store(const TuneKey& key, int choice);
 bool tune_frozen(); // fdx_tuner_freeze(1): shapes not in the table take the closed rules, nothing is timed
+// The shader clock climbs for about 30 ms after an idle period (2.0 -> 2.4 GHz measured), and candidates timed along the
+// climb are not comparable: the later ones look faster.  A timing run that starts after a pause first repeats `launch`
+// (rounds of three, a stream synchronisation after each; false from it ends the repetition) for that long; runs that
+// follow one another within a few milliseconds, as the shapes of a model's first pass do, find the clock where the one
+// before left it.  tune_mark() is called at the end of every timing run.
+void tune_settle_clock(const std::function<bool()>& launch);
+void tune_mark();
 
 } // namespace fdx

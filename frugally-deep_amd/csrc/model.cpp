@@ -1761,6 +1761,8 @@ namespace {
                 st = FDX_OK;
                 continue;
             }
+            if (st == FDX_OK && form == 0)
+                tune_settle_clock([&] { return run(0) == FDX_OK; });
             for (int round = 0; round < 3 && st == FDX_OK; ++round) {
                 (void)hipEventRecord(e0, stream());
                 for (int r = 0; r < 3 && st == FDX_OK; ++r)
@@ -1773,6 +1775,7 @@ namespace {
         }
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
+        tune_mark();
         if (st != FDX_OK)
             return st;
         const int best = ms[1] < ms[0] ? 1 : 0;
@@ -2301,6 +2304,8 @@ namespace {
             st = run_block_form(m, p, idx, forms[f]); // warm-up; tells whether the launcher takes the shape
             if (st != FDX_OK || p.dw_fused[idx] != forms[f])
                 continue;
+            if (f == 0)
+                tune_settle_clock([&] { return run_block_form(m, p, idx, forms[0]) == FDX_OK; });
             for (int round = 0; round < 4 && st == FDX_OK; ++round) { // the shortest of four rounds: a single one is too noisy to rank forms a few percent apart
                 (void)hipEventRecord(e0, stream());
                 for (int r = 0; r < 3 && st == FDX_OK; ++r)
@@ -2313,6 +2318,7 @@ namespace {
         }
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
+        tune_mark();
         if (st != FDX_OK)
             return st;
         int best = 0;
