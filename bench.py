@@ -350,6 +350,16 @@ def bench_gpt2(fdx, modelgen, args):
                      "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
         "load_seconds": round(load_s, 2),
     }
+    if not args.no_clock_probe:  # one more generation with the probe beside it
+        sess.reset()
+        fdx.check(fdx.lib.fdx_session_prefill(sess._h, fdx._dp(d_ids), prompt, None, fdx._dp(d_first)))
+        fdx.sync()
+        fdx.check(fdx.lib.fdx_clock_probe_start(int(min(65536, decode_ms * 10 * 1.05 + 4)), 100))
+        fdx.check(fdx.lib.fdx_session_decode_greedy(sess._h, fdx._dp(d_first), new, fdx._dp(d_tok), fdx._dp(d_log)))
+        fdx.sync()
+        mean, lo, hi = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        fdx.check(fdx.lib.fdx_clock_probe_stop(ctypes.c_double(decode_ms), ctypes.byref(mean), ctypes.byref(lo), ctypes.byref(hi)))
+        out["shader_clock"] = {"mean_ghz": round(mean.value, 3), "min_ghz": round(lo.value, 3), "max_ghz": round(hi.value, 3)}
     if cpu:
         out["cpu_baseline"] = cpu
     sess.close()
