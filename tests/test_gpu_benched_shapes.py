@@ -128,7 +128,7 @@ def _features(modelgen, oracle, spec, tap, sample):
 
 
 @pytest.mark.parametrize("name,batch,small", [("resnet50", 64, 2), ("mobilenet_v2", 128, 8)])
-def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batch, small):
+def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batch, small, tmp_path):
     """At the benchmark batch the tuner picks other kernel variants (split-K, stream-K, fused depthwise pairs) than at
     the small batches the oracle comparisons use.  Samples are independent (include/fdeep/model.hpp:28-42): rows of the
     large batch must equal the same images run at the small batch, one image must meet the oracle, and with the table
@@ -159,6 +159,17 @@ def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batc
             assert np.array_equal(u, v)
         for u, g in zip(a, big):
             assert np.array_equal(u, g)  # the same table picks the same kernels as the run that made it
+        # the deployment itself: a process that has tuned nothing imports the table, freezes it and predicts
+        (tmp_path / "table.txt").write_text(table)
+        (tmp_path / "model.json").write_bytes(js if isinstance(js, bytes) else js.encode())
+        np.save(tmp_path / "x.npy", x)
+        import os, subprocess, sys
+        root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+        say("  fresh process with the imported table")
+        run = subprocess.run([sys.executable, "-c", FRESH_PROCESS_MODEL, root, str(tmp_path)], capture_output=True, text=True, timeout=110)
+        assert run.returncode == 0 and run.stdout.strip().endswith("ok"), (run.returncode, run.stdout[-400:], run.stderr[-800:])
+        for i, u in enumerate(a):
+            assert np.array_equal(u, np.load(tmp_path / ("out%d.npy" % i)))
         # a shape the table has not seen takes the closed rule, and still meets the oracle
         c = fdx.Model(js, verify=False).predict([x[:3]])
         for u, g in zip(c, big):
@@ -203,6 +214,20 @@ def test_predict_from_several_host_threads(fdx, modelgen):
         th.join(timeout=100)
     assert not errors, errors[:5]
     assert len(results) == 4
+
+
+FRESH_PROCESS_MODEL = r"""
+import importlib, os, sys, numpy as np
+sys.path.insert(0, sys.argv[1])
+d = sys.argv[2]
+fdx = importlib.import_module("frugally-deep_amd")
+fdx.tuner_import(open(os.path.join(d, "table.txt")).read())
+fdx.tuner_freeze(True)
+model = fdx.Model(os.path.join(d, "model.json"), verify=False)
+for i, o in enumerate(model.predict([np.load(os.path.join(d, "x.npy"))])):
+    np.save(os.path.join(d, "out%d.npy" % i), o)
+print("ok", flush=True)
+"""
 
 
 FRESH_PROCESS_IMPORT = r"""
