@@ -736,13 +736,13 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         }
         if (cfg >= 0) {
         } else if (fast_ok && p.N >= 64) {
-            // the largest tile that still gives every CU a few workgroups
-            if (blocks(128, 128) >= 1024 && p.N % 128 == 0)
-                cfg = 10;
-            else if (blocks(128, 64) >= 1024)
-                cfg = 11;
+            // what the timing runs pick most often: the 64 x 64 tile at four or five workgroups per CU, with the
+            // 32-float slab where K is long enough for it; the 128 x 128 tile only for problems that are large in
+            // every dimension
+            if (p.K >= 1024 && p.N % 128 == 0 && blocks(128, 128) >= 2048)
+                cfg = unit % 32 == 0 ? 13 : 10;
             else
-                cfg = unit % 32 == 0 ? 15 : 12;
+                cfg = (unit % 32 == 0 && p.K >= 128) ? 15 : 12;
         } else if (p.N <= 32)
             cfg = 2;
         else if (p.N <= 64)

@@ -1742,10 +1742,15 @@ namespace {
         key.res = res != nullptr;
         int known = 0;
         hipEvent_t e0 = nullptr, e1 = nullptr;
-        if (tune_lookup(key, &known) || tune_frozen() || hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        const bool listed = tune_lookup(key, &known);
+        if (listed || tune_frozen() || hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
             if (e0)
                 (void)hipEventDestroy(e0);
-            p.conv_form[idx] = known == 1 ? 1 : 0; // frozen and unseen: the direct kernel
+            // Nothing is timed and the shape is not in the table: the Winograd kernel from a gigaflop of direct-sum work
+            // up (every 3x3 layer of ResNet50 from batch 5; timed, it wins all four of its shapes at batch 64 by 1.4-1.8
+            // times), the direct kernel below that, where a launch is too short for the kernel's fixed costs to pay.
+            const bool by_rule = 2.0 * key.M * (double)key.N * key.K >= 1e9;
+            p.conv_form[idx] = (listed ? known == 1 : by_rule) ? 1 : 0;
             fdx_status st = run(p.conv_form[idx]);
             if (st == FDX_ERR_UNSUPPORTED && p.conv_form[idx] == 1) {
                 p.conv_form[idx] = 0;
@@ -2286,8 +2291,16 @@ namespace {
             key.kh = c.fuse_exp >= 0 ? (int)p.shapes[m.ops[c.fuse_exp].in[0]].back() : 0; // input channels of a whole block
         }
         int known = 0;
-        if (tune_lookup(key, &known) || tune_frozen()) // frozen and unseen: a launch per layer
-            return run_block_form(m, p, idx, known == 1 || known == 3 ? known : 2);
+        const bool listed = tune_lookup(key, &known);
+        if (listed || tune_frozen()) {
+            // Nothing is timed and the block is not in the table: the forms that win when they are timed (MobileNetV2 at
+            // batch 128: the whole block as one launch on the 112- and 56-row feature maps, depthwise + projection on
+            // the 28-row ones, a launch per layer below that); a form the launchers do not cover falls back inside
+            // run_block_form.
+            const int by_rule = key.M >= 56 ? 3 : key.M >= 28 ? 1 : 2;
+            const int form = listed ? (known == 1 || known == 3 ? known : 2) : by_rule;
+            return run_block_form(m, p, idx, form);
+        }
         hipEvent_t e0, e1;
         if (hipEventCreate(&e0) != hipSuccess)
             return run_block_form(m, p, idx, 2);
