@@ -318,13 +318,48 @@ static int resident_workgroups(K kernel, int threads)
     return resident;
 }
 
+// Strip width (in column tiles) for a whole-tile launch of `grid` workgroups, from a model of what the eight L2s fetch:
+// with `ns` strips every strip reads all of A once (A x ns in total) and each XCD reads its strip's share of B, once if
+// that share stays in its L2 between rounds of workgroups and once per round otherwise.
+static int g_strips = -1; // FDX_STRIPS=0 keeps the row-by-row order
+static int g_forced_strips = 0; // fdx_debug_force_strips
+static int pick_strip_width(const GemmParams& q, int bm, int bn, int grid)
+{
+    if (g_strips < 0) {
+        const char* e = std::getenv("FDX_STRIPS");
+        g_strips = (e && e[0] == '0') ? 0 : 1;
+    }
+    if (q.batch != 1)
+        return 0;
+    const int tiles_m = (q.M + bm - 1) / bm, tiles_n = (q.N + bn - 1) / bn;
+    if (g_forced_strips > 0) // test hook: this many strips wherever there are as many column tiles
+        return g_forced_strips <= tiles_n ? (tiles_n + g_forced_strips - 1) / g_forced_strips : 0;
+    if (!g_strips)
+        return 0;
+    const double a_bytes = 4.0 * q.M * q.K, b_bytes = 4.0 * q.N * q.K;
+    const int rounds = (tiles_m * tiles_n + grid - 1) / grid;
+    int best_ns = 1;
+    double best_cost = 0.0;
+    for (int ns = 1; ns <= 8 && ns <= tiles_n; ns *= 2) {
+        const double share = b_bytes / ns;
+        const double cost = a_bytes * ns + 8.0 * share * (share <= 2.0e6 ? 1 : rounds);
+        if (ns == 1 || cost < 0.9 * best_cost) { // a change of order has to promise a tenth less traffic
+            best_cost = cost;
+            best_ns = ns;
+        }
+    }
+    return best_ns == 1 ? 0 : (tiles_n + best_ns - 1) / best_ns;
+}
+
 template <typename K>
-static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStream_t s, int threads = 256)
+static void launch_persistent(K kernel, int tiles, const GemmParams& q, hipStream_t s, int threads = 256, int bm = 0, int bn = 0)
 {
     const int resident = resident_workgroups(kernel, threads);
     const int cap = g_persist_scale > 0 ? g_persist_scale : resident;
     const int grid = tiles < cap ? tiles : cap;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), 0, s, q);
+    GemmParams r = q;
+    r.strip_w = bm > 0 ? pick_strip_width(q, bm, bn, grid) : 0;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), 0, s, r);
 }
 
 #include "pw_stream.hpp"
@@ -413,6 +448,8 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
     q.split_dp_tiles = 0;
     q.split_ws = g_split_ws;
     q.split_tickets = g_split_tickets;
+    q.strip_w = 0; // set per whole-tile launch
+
     bool ok = true;
 #define FDX_FAST(BM_, BN_, BK_)                                                                                  \
     {                                                                                                            \
@@ -428,9 +465,9 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
             else                                                                                                 \
                 ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles, splits, mode, cfg, q, s); \
         } else if (conv)                                                                                         \
-            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s);                        \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s, 256, BM_, BN_);         \
         else                                                                                                     \
-            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s);                       \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s, 256, BM_, BN_);        \
     }
         // eight-wave variants: more waves per SIMD to cover LDS and global latency, or a 256-row tile that halves the
         // operand traffic per FLOP
@@ -438,9 +475,9 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
     {                                                                                                            \
         const int tiles = ((q.M + BM_ - 1) / BM_) * ((q.N + BN_ - 1) / BN_) * batch;                             \
         if (conv)                                                                                                \
-            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, true>, tiles, q, s, 512);                \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, true>, tiles, q, s, 512, BM_, BN_);      \
         else                                                                                                     \
-            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, false>, tiles, q, s, 512);               \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, false>, tiles, q, s, 512, BM_, BN_);     \
     }
         switch (cfg) {
         case 10: FDX_FAST(128, 128, 16) break;
@@ -606,8 +643,9 @@ static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStre
                 // round of the hybrid form), and in the stream-K form every tile's operands fetched at a K phase of
                 // its own, so that tiles of one row block no longer share them in L2 (measured on ResNet50's
                 // 14 x 14 and 7 x 7 1x1 layers: 3.7 times the algorithmic bytes).  A cut has to win by more than that
-                // handicap to be taken.
-                const float score = ms * (mode == 2 ? 1.10f : 1.02f);
+                // handicap to be taken: 4 % of its time for K ranges, 15 % for stream-K (which wins by 9 % on those 1x1
+                // layers, by 15-20 % on deep 3x3 convolutions and by more on a Dense with few rows).
+                const float score = ms * (mode == 2 ? 1.15f : 1.04f);
                 if (score < best_split_ms) {
                     best_split_ms = score;
                     best_split = cfg + 100 * splits + 10000 * mode;
@@ -890,6 +928,13 @@ extern "C" fdx_status fdx_debug_force_tile(int cfg)
 }
 
 // tests: caps the persistent grid (0 = as many workgroups as are resident on the chip)
+extern "C" fdx_status fdx_debug_force_strips(int strips)
+{
+    FDX_REQUIRE(strips >= 0 && strips <= 64, "debug_force_strips: 0 (the traffic model decides) .. 64");
+    fdx::g_forced_strips = strips;
+    return FDX_OK;
+}
+
 extern "C" fdx_status fdx_debug_persist_cap(int workgroups)
 {
     // the tile walk hands every eighth workgroup one eighth of the tiles, so a capped grid keeps at least eight

@@ -120,8 +120,19 @@ void igemm_fast_kernel(GemmParams p)
         }
         cur_tile = tile;
         const int z = tile / per_problem, id = tile - z * per_problem;
-        m0 = (id / tiles_n) * BM;
-        n0 = (id % tiles_n) * BN;
+        if (p.strip_w > 0) {
+            const int per_strip = tiles_m * p.strip_w, last = (tiles_n - 1) / p.strip_w;
+            int strip = id / per_strip;
+            strip = strip < last ? strip : last; // the last strip may be narrower
+            const int rem = id - strip * per_strip, left = tiles_n - strip * p.strip_w;
+            const int w_eff = p.strip_w < left ? p.strip_w : left;
+            const int mt = rem / w_eff;
+            m0 = mt * BM;
+            n0 = (strip * p.strip_w + (rem - mt * w_eff)) * BN;
+        } else {
+            m0 = (id / tiles_n) * BM;
+            n0 = (id % tiles_n) * BN;
+        }
         const float* A = p.A + (z / p.inner) * p.a_outer + (z % p.inner) * p.a_inner;
         const float* B = p.B + (z / p.inner) * p.b_outer + (z % p.inner) * p.b_inner;
         c_off = (z / p.inner) * p.c_outer + (z % p.inner) * p.c_inner;

@@ -38,6 +38,10 @@ struct GemmParams {
     int split_dp_tiles; // leading tiles that are computed whole (one unit each); the rest are cut into `splits` K ranges
     float* split_ws;
     int* split_tickets;
+    // fast path, whole-tile launches: output tiles are numbered strip by strip (strip_w column tiles wide, row tiles
+    // inside a strip, columns fastest) instead of row by row, so that the contiguous tile range of an XCD needs only
+    // its strip's columns of B; 0 = one strip (row by row)
+    int strip_w;
 };
 
 // Key of the per-process tuning table (igemm.hip).  conv = 0 / 1: a GEMM / convolution shape and its tile choice

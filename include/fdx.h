@@ -459,6 +459,8 @@ fdx_status fdx_tuner_freeze(int on);
  *     kernel for K <= 128 (where it does not apply the tuner decides); + 100 * splits
  *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
  *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
+ *   fdx_debug_force_strips: whole-tile launches of the fast path number their output tiles in this many column strips
+ *     (wherever the output has as many column tiles) instead of letting the traffic model decide; 0 = the model decides.
  *   fdx_debug_force_dw_fusion: how plans built from now on run a depthwise 3x3 convolution and the 1x1 convolutions
  *     around it: -1 = the forms are timed once per block shape (the default), 0 = one launch per layer, 1 = depthwise +
  *     projection as one launch wherever the pair qualifies, 2 = expansion + depthwise + projection as one launch
@@ -469,6 +471,7 @@ fdx_status fdx_tuner_freeze(int on);
  */
 fdx_status fdx_debug_force_tile(int cfg);
 fdx_status fdx_debug_persist_cap(int workgroups);
+fdx_status fdx_debug_force_strips(int strips);
 fdx_status fdx_debug_force_dw_fusion(int mode);
 fdx_status fdx_debug_force_winograd(int mode);
 

@@ -652,6 +652,41 @@ def test_gemm_split_k_many_tiles(fdx, oracle, tile):
     assert rel(got, want) <= TOL
 
 
+@pytest.mark.parametrize("strips", [2, 3, 5, 8])
+@pytest.mark.parametrize("tile,cap", [(15, 0), (12, 24), (14, 10), (13, 0), (16, 0), (18, 0)])
+def test_gemm_and_conv_tiles_numbered_in_column_strips(fdx, oracle, strips, tile, cap):
+    """Whole-tile launches may number their output tiles strip by strip (so that an XCD's contiguous tile range needs
+    only its strip's columns of the weights); the order must not change a single value.  Column-tile counts that the
+    strip count does not divide, row counts that are no multiple of the tile, and a capped persistent grid (several
+    tiles per workgroup) are covered; the unstriped run is the reference."""
+    say("column strips", strips, "tile", tile, "cap", cap)
+    r = rng_for("strips", strips, tile)
+    m, n, k = 1000, 704, 256  # 11 column tiles of 64, 6 (5.5) of 128
+    a = r.standard_normal((m, k)).astype(np.float32)
+    w = (r.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    b = r.standard_normal(n).astype(np.float32)
+    res = r.standard_normal((m, n)).astype(np.float32)
+    x = r.standard_normal((2, 18, 17, 64)).astype(np.float32)
+    wj = (r.standard_normal((320, 3, 3, 64)) / 24.0).astype(np.float32)
+    bj = r.standard_normal(320).astype(np.float32)
+    fdx.lib.fdx_debug_force_tile(tile)
+    fdx.lib.fdx_debug_persist_cap(cap)
+    try:
+        plain = fdx.gemm(a, w, b, residual=res, act=fdx.relu_act())
+        plain_c = fdx.conv2d(x, wj, bj, (1, 1), (1, 1), "same", act=fdx.relu_act())
+        fdx.check(fdx.lib.fdx_debug_force_strips(strips))
+        got = fdx.gemm(a, w, b, residual=res, act=fdx.relu_act())
+        got_c = fdx.conv2d(x, wj, bj, (1, 1), (1, 1), "same", act=fdx.relu_act())
+    finally:
+        fdx.lib.fdx_debug_force_strips(0)
+        fdx.lib.fdx_debug_persist_cap(0)
+        fdx.lib.fdx_debug_force_tile(-1)
+    want = np.maximum(a.astype(np.float64) @ w.astype(np.float64).T + b + res, 0)
+    assert rel(plain, want) <= TOL
+    assert np.array_equal(got, plain)
+    assert np.array_equal(got_c, plain_c)
+
+
 @pytest.mark.parametrize("tile,cap", [(10215, 24), (10315, 24), (10413, 8), (10214, 16), (10612, 40), (10815, 9)])
 def test_conv2d_hybrid_whole_tiles_plus_split_remainder(fdx, oracle, tile, cap):
     """Persistent grid capped to `cap` workgroups: the tiles that fill whole rounds run as whole tiles, the last partial
