@@ -47,6 +47,7 @@ struct WinoParams {
     int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
     uint32_t in_bytes, out_bytes, u_bytes, ws_bytes;
     int m_blocks, n_blocks, units; // blocks of 32 tiles, column blocks of NT * 32 channels; units of work = their product
+    int tile_major;      // units ordered by tile block first (all column blocks of a tile block are neighbours)
     int per_wg, longer;  // steps per workgroup (total / workgroups) and how many workgroups take one more
     float* ws;           // shares of units that several workgroups work on: two places per workgroup
     int* tickets;        // one per unit, zero between launches
@@ -194,7 +195,8 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     };
     const int end = stretch_begin(g + 1);
     auto view_of = [&](bool live, int unit, UnitView& v) {
-        const int nb = unit / p.m_blocks, mb = unit - nb * p.m_blocks;
+        const int nb = p.tile_major ? unit % p.n_blocks : unit / p.m_blocks;
+        const int mb = p.tile_major ? unit / p.n_blocks : unit - nb * p.m_blocks;
         // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
         const int tile = mb * WINO_TM + fr;
         const bool tile_ok = live && tile < p.tiles;
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     while (pos < end) {
         const int unit_begin = unit * spu;
         const int s0 = pos - unit_begin, s1 = end - unit_begin < spu ? end - unit_begin : spu;
-        const int n0 = (unit / p.m_blocks) * NC;
+        const int n0 = (p.tile_major ? unit % p.n_blocks : unit / p.m_blocks) * NC;
         if (xi == 0 && fh == 0) {
             tile_desc[fr * 2] = cur.desc0;
             tile_desc[fr * 2 + 1] = cur.desc1;
@@ -323,11 +325,18 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
             }
             __syncthreads();
             if (last_flag != 0) {
+                // shares are added in stretch order whoever came last; this workgroup's own one is formed again from the
+                // exchange area (the same operations on the same values, so the same bits) instead of read back
+                const int my_part = g - g_a;
                 for (int pass = 0; pass < PASSES; ++pass) {
                     f32x4 y = { 0.f, 0.f, 0.f, 0.f };
-                    for (int sp = 0; sp < parts; ++sp)
-                        y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_ws,
-                            (int)(share_off(g_a + sp, unit) + lane_off + (uint32_t)pass * 1024u), 0, kAgentScope));
+                    for (int sp = 0; sp < parts; ++sp) {
+                        if (sp == my_part)
+                            y += combine(pass);
+                        else
+                            y += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_ws,
+                                (int)(share_off(g_a + sp, unit) + lane_off + (uint32_t)pass * 1024u), 0, kAgentScope));
+                    }
                     finish(pass, y);
                 }
             }
@@ -456,6 +465,11 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
         return FDX_ERR_UNSUPPORTED;
     }
     p.units = m_blocks * p.n_blocks;
+    // Column block first keeps one slab of the filter in an XCD's L2, at the price of the input crossing the fabric once
+    // per column block.  A filter that fits an L2 whole with room to spare (2 MB in the transform domain: 128 -> 128
+    // channels) takes the other order: a tile block's column blocks follow each other, and the input is fetched once.
+    static const bool lean = [] { const char* e = std::getenv("FDX_WINO_ORDER"); return !(e && e[0] == '0'); }();
+    p.tile_major = lean && p.n_blocks > 1 && fdx_conv2d_winograd_weight_floats(cin, cout) * sizeof(float) <= (2u << 20) ? 1 : 0;
     p.ws = g_wino_ws;
     p.ws_bytes = (uint32_t)(2 * kWinoShareBytes * (size_t)g_wino_grid);
     p.tickets = g_wino_tickets;
