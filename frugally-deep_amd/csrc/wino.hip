@@ -47,7 +47,7 @@ struct WinoParams {
     int tiles_x, tiles_y, tiles; // 2x2 output tiles per row, per image column, and all of them
     uint32_t in_bytes, out_bytes, u_bytes, ws_bytes;
     int m_blocks, n_blocks, units; // blocks of 32 tiles, column blocks of NT * 32 channels; units of work = their product
-    int tile_major;      // units ordered by tile block first (all column blocks of a tile block are neighbours)
+    int nb_group;        // column blocks per group: units are ordered group, tile block, column block inside the group
     int per_wg, longer;  // steps per workgroup (total / workgroups) and how many workgroups take one more
     float* ws;           // shares of units that several workgroups work on: two places per workgroup
     int* tickets;        // one per unit, zero between launches
@@ -195,8 +195,8 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     };
     const int end = stretch_begin(g + 1);
     auto view_of = [&](bool live, int unit, UnitView& v) {
-        const int nb = p.tile_major ? unit % p.n_blocks : unit / p.m_blocks;
-        const int mb = p.tile_major ? unit / p.n_blocks : unit - nb * p.m_blocks;
+        const int nb = (unit / (p.m_blocks * p.nb_group)) * p.nb_group + unit % p.nb_group;
+        const int mb = (unit / p.nb_group) % p.m_blocks;
         // this lane's tile and the eight patch pixels row xi of Bt reads: rows (0, 2), (1, 2), (1, 2), (1, 3) of the patch
         const int tile = mb * WINO_TM + fr;
         const bool tile_ok = live && tile < p.tiles;
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
     while (pos < end) {
         const int unit_begin = unit * spu;
         const int s0 = pos - unit_begin, s1 = end - unit_begin < spu ? end - unit_begin : spu;
-        const int n0 = (p.tile_major ? unit % p.n_blocks : unit / p.m_blocks) * NC;
+        const int n0 = ((unit / (p.m_blocks * p.nb_group)) * p.nb_group + unit % p.nb_group) * NC;
         if (xi == 0 && fh == 0) {
             tile_desc[fr * 2] = cur.desc0;
             tile_desc[fr * 2 + 1] = cur.desc1;
@@ -466,10 +466,17 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     }
     p.units = m_blocks * p.n_blocks;
     // Column block first keeps one slab of the filter in an XCD's L2, at the price of the input crossing the fabric once
-    // per column block.  A filter that fits an L2 whole with room to spare (2 MB in the transform domain: 128 -> 128
-    // channels) takes the other order: a tile block's column blocks follow each other, and the input is fetched once.
+    // per column block.  Column blocks whose slabs together stay within 2 MB (half an L2) form a group that shares the
+    // walk over the tile blocks: inside a group a tile block's column blocks follow each other, and the input is
+    // fetched once per group (128 -> 128 channels: one group, the tiles' order first; 256 -> 256: two groups of two;
+    // 512 -> 512: every column block on its own).
     static const bool lean = [] { const char* e = std::getenv("FDX_WINO_ORDER"); return !(e && e[0] == '0'); }();
-    p.tile_major = lean && p.n_blocks > 1 && fdx_conv2d_winograd_weight_floats(cin, cout) * sizeof(float) <= (2u << 20) ? 1 : 0;
+    const size_t slab_bytes = fdx_conv2d_winograd_weight_floats(cin, cout) * sizeof(float) / (size_t)p.n_blocks;
+    p.nb_group = 1;
+    if (lean)
+        for (int gsz = 2; gsz <= p.n_blocks; ++gsz)
+            if (p.n_blocks % gsz == 0 && (size_t)gsz * slab_bytes <= ((size_t)2 << 20))
+                p.nb_group = gsz;
     p.ws = g_wino_ws;
     p.ws_bytes = (uint32_t)(2 * kWinoShareBytes * (size_t)g_wino_grid);
     p.tickets = g_wino_tickets;
