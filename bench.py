@@ -47,7 +47,10 @@ def profile_families(fdx):
         if fdx.lib.fdx_profile_get(i, name, 128, ctypes.byref(launches), ctypes.byref(ms), ctypes.byref(flops),
                                    ctypes.byref(nbytes)) != 0:
             break
-        fams[name.value.decode()] = dict(launches=launches.value, ms=ms.value, flops=flops.value, bytes=nbytes.value)
+        executed = ctypes.c_double()
+        fdx.check(fdx.lib.fdx_profile_get_executed(i, ctypes.byref(executed)))
+        fams[name.value.decode()] = dict(launches=launches.value, ms=ms.value, flops=flops.value, bytes=nbytes.value,
+                                         executed=executed.value)
         i += 1
     return fams
 
@@ -72,10 +75,16 @@ def cpu_model_name():
     return "unknown"
 
 
+CPU_BUILD = None
+CPU_KIND_NOTE = "restated reference CPU path (no Eigen): the oracle's plain-C port of the reference algorithm, kind 'port'"
+
+
 def cpu_baseline_resnet(js, x, cores, warmup=3, passes=5):
     """The oracle (a port of the reference CPU path) timed with one prediction per core in parallel threads, 3 warm-up
     and 5 timed passes as the reference's own harness does (test/applications_performance.cpp:59-77)."""
     import fdeep_oracle
+    global CPU_BUILD
+    CPU_BUILD = fdeep_oracle.use_native_build()
     ref = fdeep_oracle.OracleModel(js)
     samples = [x[i % x.shape[0]] for i in range(cores)]
     with concurrent.futures.ThreadPoolExecutor(cores) as pool:
@@ -93,6 +102,8 @@ def cpu_baseline_decode(js, cores, prompt=4, warmup=3, timed=5):
     warm-up steps per sequence, then 5 timed steps each (a step streams every weight of the model once per sequence,
     whatever the context length, so the short context hardly changes its cost)."""
     import fdeep_oracle
+    global CPU_BUILD
+    CPU_BUILD = fdeep_oracle.use_native_build()
     ref = fdeep_oracle.OracleModel(js)
     rng = np.random.default_rng(7)
     decoders = [fdeep_oracle.CachedDecoder(ref) for _ in range(cores)]
@@ -150,6 +161,11 @@ def bench_resnet(fdx, modelgen, args):
     d_out = fdx.DevBuf(4 * batch * 1000)
     shapes = [(224, 224, 3)]
 
+    fdx.sync()
+    t0 = time.perf_counter()
+    model.predict_dev(batch, [d_in], shapes, [d_out])
+    fdx.sync()
+    first_call_ms = (time.perf_counter() - t0) * 1e3
     for _ in range(args.warmup):
         model.predict_dev(batch, [d_in], shapes, [d_out])
     fdx.sync()
@@ -180,6 +196,9 @@ def bench_resnet(fdx, modelgen, args):
     mf_ms = sum(v["ms"] for v in mfma.values())
     mf_launches = sum(v["launches"] for v in mfma.values())
     achieved = mf_flops / (mf_ms / 1e3) / 1e12 if mf_ms > 0 else 0.0
+    # what the matrix cores really issued: the Winograd launches carry 16 products per 2x2 output tile where the direct
+    # sum has 36, so their algorithmic figure can exceed the peak; this one cannot
+    executed = sum(v["executed"] for v in mfma.values()) / (mf_ms / 1e3) / 1e12 if mf_ms > 0 else 0.0
     total_ms = sum(v["ms"] for v in fams.values())
 
     result = {
@@ -206,6 +225,12 @@ def bench_resnet(fdx, modelgen, args):
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+            "executed_achieved": round(executed, 3),
+            "executed_frac": round(executed / PEAK_FP32_MFMA_TFLOPS, 4),
+            "executed_note": "multiply-adds the kernels issue (Winograd launches: 16 per 2x2 output tile and channel pair instead of "
+                             "36) / time / peak: the hardware utilisation, where frac is the algorithmic direct-sum rate",
+            "family_tflops": {k: {"algorithmic": round(v["flops"] / (v["ms"] / 1e3) / 1e12, 2),
+                                  "executed": round(v["executed"] / (v["ms"] / 1e3) / 1e12, 2)} for k, v in sorted(mfma.items()) if v["ms"] > 0},
             "flops_per_launch": round(mf_flops / max(mf_launches, 1), 1),
             "avg_launch_ms": round(mf_ms / max(mf_launches, 1), 5),
             "share_of_step_time": round(mf_ms / total_ms, 4) if total_ms else None,
@@ -214,6 +239,8 @@ def bench_resnet(fdx, modelgen, args):
         "kernel_ms_per_step": {k: round(v["ms"] / prof_steps, 4) for k, v in sorted(fams.items())},
         "wall_ms_per_step": round(wall_s * 1e3 / args.steps, 4),
         "load_seconds": round(load_s, 2),
+        "first_call_ms": round(first_call_ms, 1),
+        "kernel_choice": "timed per shape on first sight (--tune)" if args.tune else "closed rules, nothing timed (the library's default)",
     }
     if not args.no_clock_probe:
         result["shader_clock"] = shader_clock_during(fdx, lambda: model.predict_dev(batch, [d_in], shapes, [d_out]), args.steps,
@@ -232,7 +259,7 @@ def bench_resnet(fdx, modelgen, args):
         cores = host_cores()
         cpu = cpu_baseline_resnet(js, x, cores)
         result["cpu_baseline"] = {"value": round(cpu, 3), "unit": "img/s", "cores": cores, "kind": "port",
-                                  "cpu": cpu_model_name(),
+                                  "what": CPU_KIND_NOTE, "build": CPU_BUILD, "cpu": cpu_model_name(),
                                   "sample": "%d ResNet50 predictions per pass (one per core, in parallel threads), "
                                             "3 warm-up + 5 timed passes of the CPU oracle" % cores}
     model.close()
@@ -312,7 +339,7 @@ def bench_gpt2(fdx, modelgen, args):
     if not args.no_cpu_baseline:
         cores = host_cores()
         cpu = {"value": round(cpu_baseline_decode(js, cores), 2), "unit": "tok/s", "cores": cores, "kind": "port",
-               "cpu": cpu_model_name(),
+               "what": CPU_KIND_NOTE, "build": CPU_BUILD, "cpu": cpu_model_name(),
                "sample": "%d sequences (one per core, in parallel threads) on the CPU oracle's KV-cached decoder: 4 prompt + 3 "
                          "warm-up steps, then 5 timed greedy steps each" % cores}
     del js
@@ -347,7 +374,9 @@ def bench_gpt2(fdx, modelgen, args):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4), "bytes_per_step_mean": round(total_bytes / new),
                      "kernel": "skinny_gemm_kernel (Dense for 16 rows, weights streamed once; 48 of the step's 63 launches plus the LM head's striding variant)",
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"]},
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH["skinny_gemm, GPT-2 decode b16"],
+                     "traffic_note": "isolated-kernel run (--workload gpt2_kernels, the step's five Dense shapes against rings of "
+                                     "weight copies), not a counter run of the decode loop itself"},
         "load_seconds": round(load_s, 2),
     }
     if not args.no_clock_probe:  # one more generation with the probe beside it
@@ -431,6 +460,9 @@ def main():
     ap.add_argument("--no-clock-probe", action="store_true", help="skip the shader-clock pass after the timed region")
     ap.add_argument("--tuner-import", default=None, help="per-shape tuner table to load and freeze before anything runs "
                                                          "(fdx_tuner_import + fdx_tuner_freeze: nothing is timed, every run picks the same kernels)")
+    ap.add_argument("--tune", action="store_true", help="let the first sight of every shape time its candidate kernels "
+                                                        "(fdx_tuner_timing(1)); the default runs on the closed rules, as a "
+                                                        "caller who sets nothing does")
     ap.add_argument("--tuner-export", default=None, help="write the per-shape tuner table of this run to this file at the end")
     ap.add_argument("--ring-mb", type=float, default=600.0,
                     help="gpt2_kernels: total size of the ring of weight copies a kernel cycles through (larger than the "
@@ -446,6 +478,8 @@ def main():
     if args.tuner_import:
         fdx.tuner_import(open(args.tuner_import).read())
         fdx.tuner_freeze(True)
+    if args.tune:
+        fdx.tuner_timing(True)
     if args.calibrate_copy_mib > 0:
         n = args.calibrate_copy_mib * (1 << 20) // 4
         src, dst = fdx.DevBuf(4 * n), fdx.DevBuf(4 * n)

@@ -103,6 +103,11 @@ def tuner_import(text):
     check(lib.fdx_tuner_import(text.encode()))
 
 
+def tuner_timing(on=True):
+    """Timing runs on the first sight of a shape (off unless asked for; FDX_AUTOTUNE=1 asks for them too)."""
+    check(lib.fdx_tuner_timing(1 if on else 0))
+
+
 def tuner_freeze(on=True):
     check(lib.fdx_tuner_freeze(1 if on else 0))
 

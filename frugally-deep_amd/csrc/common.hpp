@@ -8,6 +8,7 @@
 #include <string>
 
 #include "../../include/fdx.h"
+#include "../../include/fdx_debug.h"
 
 namespace fdx {
 
@@ -18,9 +19,10 @@ bool profiling();
 // Clears library-owned scratch at set-up time, on the library stream (which does not synchronise with the null
 // stream) and waits for it, so that the first kernel that reads the cells sees zeros.  Not for use inside a stream capture.
 hipError_t zero_device(void* p, size_t bytes);
-// records one launch for the per-kernel profile (flops / bytes are algorithmic figures)
+// records one launch for the per-kernel profile (flops / bytes are algorithmic figures; executed_flops = the
+// multiply-adds the kernel really issues where that differs, as in the Winograd form; negative = the same)
 void profile_begin();
-void profile_end(const char* family, double flops, double bytes);
+void profile_end(const char* family, double flops, double bytes, double executed_flops = -1.0);
 
 struct Act {
     int kind;

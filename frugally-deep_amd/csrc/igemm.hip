@@ -547,15 +547,24 @@ void tune_settle_clock(const std::function<bool()>& launch)
     tune_mark();
 }
 
+// Whether first sights of a shape may be timed.  Off unless the caller asks (fdx_tuner_timing(1) or FDX_AUTOTUNE=1 in
+// the environment): a timing run launches a few thousand candidates, about a second for a ResNet50 at batch 64, which a
+// drop-in predict must not spend on its first call.  With timing off every choice (tile, K cut, direct against Winograd,
+// block forms) follows the closed rules, the same in every process.
+static int g_tune_timing = -1; // -1 = not read yet; guarded by g_tune_mutex
+static bool tune_timing_locked()
+{
+    if (g_tune_timing < 0) {
+        const char* e = std::getenv("FDX_AUTOTUNE");
+        g_tune_timing = (e && e[0] == '1') ? 1 : 0;
+    }
+    return g_tune_timing == 1;
+}
 bool tune_frozen()
 {
-    // FDX_AUTOTUNE=0 times nothing anywhere: the plan-level choices (block forms, direct against Winograd) that ask
-    // here take their fixed rule for shapes the table does not hold, like the tile tuner below
-    static const bool never_time = [] { const char* e = std::getenv("FDX_AUTOTUNE"); return e && e[0] == '0'; }();
     std::lock_guard<std::mutex> lock(g_tune_mutex);
-    return g_tune_frozen || never_time;
+    return g_tune_frozen || !tune_timing_locked();
 }
-static int g_autotune = -1;
 static int g_split_enabled = 1; // FDX_SPLITK=0 keeps the tuner to one K range per tile
 
 // general_cfg >= 0: the general kernel's configuration for this shape competes too (narrow outputs, where half of a
@@ -566,14 +575,8 @@ template <typename F, typename G>
 static int autotune(const GemmParams& q, bool conv, int batch, int unit, hipStream_t s, int general_cfg, F general_launch,
     bool stream_ok, G stream_launch)
 {
-    if (g_autotune < 0) {
-        const char* e = std::getenv("FDX_AUTOTUNE");
-        g_autotune = (e && e[0] == '0') ? 0 : 1;
-        const char* sp = std::getenv("FDX_SPLITK");
-        g_split_enabled = (sp && sp[0] == '0') ? 0 : 1;
-    }
-    if (!g_autotune)
-        return -1;
+    static const bool split_env = [] { const char* sp = std::getenv("FDX_SPLITK"); return !(sp && sp[0] == '0'); }();
+    g_split_enabled = split_env ? 1 : 0;
     TuneKey key;
     std::memset(&key, 0, sizeof key);
     key.conv = conv; key.M = q.M; key.N = q.N; key.K = q.K; key.Cin = conv ? q.Cin : 0; key.kh = conv ? q.kh : 0;
@@ -1069,6 +1072,13 @@ extern "C" fdx_status fdx_tuner_import(const char* text)
     std::lock_guard<std::mutex> lock(fdx::g_tune_mutex);
     for (const auto& r : rows)
         fdx::g_tuned[r.first] = r.second;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_tuner_timing(int on)
+{
+    std::lock_guard<std::mutex> lock(fdx::g_tune_mutex);
+    fdx::g_tune_timing = on != 0 ? 1 : 0;
     return FDX_OK;
 }
 

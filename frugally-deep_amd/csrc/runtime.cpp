@@ -20,11 +20,11 @@ static bool g_profile = false;
 struct Pending {
     hipEvent_t a, b;
     const char* family;
-    double flops, bytes;
+    double flops, bytes, executed;
 };
 struct Family {
     uint64_t launches = 0;
-    double ms = 0, flops = 0, bytes = 0;
+    double ms = 0, flops = 0, bytes = 0, executed = 0;
 };
 static std::vector<Pending> g_pending;
 static std::vector<hipEvent_t> g_event_pool;
@@ -82,7 +82,7 @@ void profile_begin()
         (void)hipEventRecord(g_cur, g_stream);
 }
 
-void profile_end(const char* family, double flops, double bytes)
+void profile_end(const char* family, double flops, double bytes, double executed_flops)
 {
     if (!g_profile || !g_cur)
         return;
@@ -90,7 +90,7 @@ void profile_end(const char* family, double flops, double bytes)
     if (!b)
         return;
     (void)hipEventRecord(b, g_stream);
-    g_pending.push_back({ g_cur, b, family, flops, bytes });
+    g_pending.push_back({ g_cur, b, family, flops, bytes, executed_flops < 0 ? flops : executed_flops });
     g_cur = nullptr;
 }
 
@@ -107,6 +107,7 @@ static void drain_profile()
             f.ms += ms;
             f.flops += p.flops;
             f.bytes += p.bytes;
+            f.executed += p.executed;
         }
         g_event_pool.push_back(p.a);
         g_event_pool.push_back(p.b);
@@ -244,6 +245,20 @@ extern "C" fdx_status fdx_profile_get(int index, char* name, size_t name_len, ui
     if (total_ms) *total_ms = it->second.ms;
     if (flops) *flops = it->second.flops;
     if (bytes) *bytes = it->second.bytes;
+    return FDX_OK;
+}
+
+extern "C" fdx_status fdx_profile_get_executed(int index, double* executed_flops)
+{
+    drain_profile();
+    FDX_REQUIRE(index >= 0 && executed_flops, "profile_get_executed: bad arguments");
+    if (index >= (int)g_families.size()) {
+        set_error("profile_get_executed: index out of range");
+        return FDX_ERR_INVALID;
+    }
+    auto it = g_families.begin();
+    std::advance(it, index);
+    *executed_flops = it->second.executed;
     return FDX_OK;
 }
 

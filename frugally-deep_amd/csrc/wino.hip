@@ -494,7 +494,9 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     FDX_WINO_LIMIT(attr == hipSuccess, "conv2d_winograd: the kernel's LDS request was refused");
     hipLaunchKernelGGL(wino_kernel<2>, grid, dim3(256), lds, stream(), p);
     const double pix = (double)n * out_h * out_w;
-    profile_end("conv2d_winograd_f32", 2.0 * pix * 9.0 * cin * cout, 4.0 * ((double)n * h * w * cin + pix * cout * (residual ? 2.0 : 1.0) + 9.0 * cin * cout));
+    const double tiles = (double)n * ((out_h + 1) / 2) * ((out_w + 1) / 2);
+    profile_end("conv2d_winograd_f32", 2.0 * pix * 9.0 * cin * cout, 4.0 * ((double)n * h * w * cin + pix * cout * (residual ? 2.0 : 1.0) + 9.0 * cin * cout),
+        2.0 * 16.0 * tiles * cin * cout);
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }

@@ -15,7 +15,8 @@
  *   - host threads: every call enqueues on the one library stream, so work from several
  *     threads runs in the order the calls were made; a model (and a session) serialises
  *     its own calls, the convolution / GEMM launcher serialises its tuner and scratch.
- *     The profile and stopwatch calls (fdx_profile_*, fdx_timer_*) are meant for one thread.
+ *   - measurement aids and test hooks (stopwatch, per-kernel profile, shader-clock probe, forced kernel choices) are
+ *     declared apart, in fdx_debug.h: nothing a caller of the reference's API needs.
  */
 #ifndef FDX_H
 #define FDX_H
@@ -71,22 +72,6 @@ fdx_status fdx_dev_free(void* p);
 fdx_status fdx_h2d(void* dst_dev, const void* src_host, size_t bytes);
 fdx_status fdx_d2h(void* dst_host, const void* src_dev, size_t bytes);
 fdx_status fdx_sync(void);
-/* HIP-event stopwatch on the library stream: start, run work, stop returns milliseconds */
-fdx_status fdx_timer_start(void);
-fdx_status fdx_timer_stop(float* ms);
-/* Shader-clock probe, a measurement aid with no counterpart in the reference (the clock of the compute units falls
- * under load, and with it what the matrix cores can deliver): one lane on a stream of its own samples the shader
- * cycle counter against the constant-rate wall counter every period_us (10..100000) while other work runs, and ends
- * by itself after `samples` (2..65536) periods.  stop waits for it and returns the clock in GHz over the first
- * window_ms milliseconds after the start: the mean, and the lowest and highest single period.  One probe at a time. */
-fdx_status fdx_clock_probe_start(int samples, int period_us);
-fdx_status fdx_clock_probe_stop(double window_ms, double* mean_ghz, double* min_ghz, double* max_ghz);
-/* name and average duration (ms) of the dominant kernel family since the last reset,
- * measured with HIP events around every launch while profiling is enabled */
-fdx_status fdx_profile_enable(int on);
-fdx_status fdx_profile_reset(void);
-fdx_status fdx_profile_get(int index, char* name, size_t name_len, uint64_t* launches, double* total_ms,
-    double* flops, double* bytes);
 
 /*
  * Conv2D, cross-correlation, implicit GEMM on fp32 MFMA:
@@ -439,41 +424,22 @@ fdx_status fdx_session_decode_greedy(fdx_session* s, const float* first_ids_dev,
 fdx_status fdx_session_length(const fdx_session* s, int* len);
 
 /*
- * The per-shape tuning table.  The first launch of a convolution / GEMM shape (and of a depthwise 3x3 + 1x1 pair) times
- * the candidate kernels once per process and keeps the winner; candidates sum in different orders, so two processes may
+ * The per-shape tuning table (no counterpart in the reference).  By default nothing is timed: every kernel choice
+ * (tile, K cut, direct against Winograd convolution, the form of a depthwise block) follows closed rules, the same in
+ * every process, and the first predict of a shape costs what any later one costs plus plan building.
+ * fdx_tuner_timing(1) (or FDX_AUTOTUNE=1 in the environment) lets the first launch of a convolution / GEMM shape (and of
+ * a depthwise 3x3 + 1x1 pair) time the candidate kernels once per process and keep the winner: about a second for a
+ * ResNet50 at batch 64, for 0-2 % more throughput.  Candidates sum in different orders, so two processes that time may
  * return results that differ in the last bits (all within the reference tolerance; the reference itself leaves the
- * summation order to Eigen, convolution.hpp:134-148).  For bit-identical results run to run, export the table of a
- * warmed-up process, import it at start-up and freeze it: under a frozen table a shape that is not listed takes a fixed
- * rule and nothing is timed.  Text format: one line per shape, "conv M N K Cin kh kw sy sx batch res choice".
+ * summation order to Eigen, convolution.hpp:134-148).  A deployment that wants the timed choices without timing exports
+ * the table of a warmed-up process, imports it at start-up and freezes it: a listed shape takes its row, an unlisted one
+ * the closed rule.  Text format: one line per shape, "conv M N K Cin kh kw sy sx batch res choice".
  * fdx_tuner_export: `needed` receives the size including the terminator; text may be NULL to query it.
  */
+fdx_status fdx_tuner_timing(int on);
 fdx_status fdx_tuner_export(char* text, size_t capacity, size_t* needed);
 fdx_status fdx_tuner_import(const char* text);
 fdx_status fdx_tuner_freeze(int on);
-
-/*
- * Test hooks (no counterpart in the reference; process-wide, meant for one thread): the parity tests use them to drive
- * every tile configuration and scheduling form of the convolution / GEMM kernels on small problems, where the tuner
- * would never pick them.
- *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; 30 = the row-streaming
- *     kernel for K <= 128 (where it does not apply the tuner decides); + 100 * splits
- *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
- *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
- *   fdx_debug_force_strips: whole-tile launches of the fast path number their output tiles in this many column strips
- *     (wherever the output has as many column tiles) instead of letting the traffic model decide; 0 = the model decides.
- *   fdx_debug_force_dw_fusion: how plans built from now on run a depthwise 3x3 convolution and the 1x1 convolutions
- *     around it: -1 = the forms are timed once per block shape (the default), 0 = one launch per layer, 1 = depthwise +
- *     projection as one launch wherever the pair qualifies, 2 = expansion + depthwise + projection as one launch
- *     wherever the block qualifies (other blocks as under 1).
- *   fdx_debug_force_winograd: which kernel plans built from now on run a 3x3 stride-1 convolution with: -1 = the direct and
- *     the Winograd kernel are timed once per shape (the default), 0 = always the direct kernel, 1 = the Winograd kernel
- *     wherever it covers the shape.
- */
-fdx_status fdx_debug_force_tile(int cfg);
-fdx_status fdx_debug_persist_cap(int workgroups);
-fdx_status fdx_debug_force_strips(int strips);
-fdx_status fdx_debug_force_dw_fusion(int mode);
-fdx_status fdx_debug_force_winograd(int mode);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,64 @@
+/*
+ * fdx_debug -- measurement aids and test hooks of libfdx.so.  None of these has a counterpart in the reference and no
+ * caller of fdeep::load_model / model::predict needs them: bench.py measures with them, the parity tests use them to
+ * force kernel forms that the closed rules and the tuner would not pick on small problems.  Process-wide, meant for
+ * one thread.
+ */
+#ifndef FDX_DEBUG_H
+#define FDX_DEBUG_H
+
+#include "fdx.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* HIP-event stopwatch on the library stream: start, run work, stop returns milliseconds */
+fdx_status fdx_timer_start(void);
+fdx_status fdx_timer_stop(float* ms);
+/* Shader-clock probe, a measurement aid with no counterpart in the reference (the clock of the compute units falls
+ * under load, and with it what the matrix cores can deliver): one lane on a stream of its own samples the shader
+ * cycle counter against the constant-rate wall counter every period_us (10..100000) while other work runs, and ends
+ * by itself after `samples` (2..65536) periods.  stop waits for it and returns the clock in GHz over the first
+ * window_ms milliseconds after the start: the mean, and the lowest and highest single period.  One probe at a time. */
+fdx_status fdx_clock_probe_start(int samples, int period_us);
+fdx_status fdx_clock_probe_stop(double window_ms, double* mean_ghz, double* min_ghz, double* max_ghz);
+/* name and average duration (ms) of the dominant kernel family since the last reset,
+ * measured with HIP events around every launch while profiling is enabled */
+fdx_status fdx_profile_enable(int on);
+fdx_status fdx_profile_reset(void);
+fdx_status fdx_profile_get(int index, char* name, size_t name_len, uint64_t* launches, double* total_ms,
+    double* flops, double* bytes);
+/* the multiply-add work the family's kernels really issued (2 per multiply-add), where that differs from the algorithmic
+ * direct-sum count fdx_profile_get reports: the Winograd convolution issues 16 products per 2x2 output tile and
+ * channel pair where the direct sum has 36 */
+fdx_status fdx_profile_get_executed(int index, double* executed_flops);
+
+/*
+ * Test hooks (no counterpart in the reference; process-wide, meant for one thread): the parity tests use them to drive
+ * every tile configuration and scheduling form of the convolution / GEMM kernels on small problems, where the tuner
+ * would never pick them.
+ *   fdx_debug_force_tile: -1 = tuner decides; 0..3 general kernel tiles; 10..18 fast-path tiles; 30 = the row-streaming
+ *     kernel for K <= 128 (where it does not apply the tuner decides); + 100 * splits
+ *     (every tile cut into `splits` K ranges), + 10000 (only the last partial round is cut), 20000 + tile = stream-K.
+ *   fdx_debug_persist_cap: caps the persistent grid at `workgroups` (at least 8; 0 = the resident count).
+ *   fdx_debug_force_strips: whole-tile launches of the fast path number their output tiles in this many column strips
+ *     (wherever the output has as many column tiles) instead of letting the traffic model decide; 0 = the model decides.
+ *   fdx_debug_force_dw_fusion: how plans built from now on run a depthwise 3x3 convolution and the 1x1 convolutions
+ *     around it: -1 = the forms are timed once per block shape (the default), 0 = one launch per layer, 1 = depthwise +
+ *     projection as one launch wherever the pair qualifies, 2 = expansion + depthwise + projection as one launch
+ *     wherever the block qualifies (other blocks as under 1).
+ *   fdx_debug_force_winograd: which kernel plans built from now on run a 3x3 stride-1 convolution with: -1 = the direct and
+ *     the Winograd kernel are timed once per shape (the default), 0 = always the direct kernel, 1 = the Winograd kernel
+ *     wherever it covers the shape.
+ */
+fdx_status fdx_debug_force_tile(int cfg);
+fdx_status fdx_debug_persist_cap(int workgroups);
+fdx_status fdx_debug_force_strips(int strips);
+fdx_status fdx_debug_force_dw_fusion(int mode);
+fdx_status fdx_debug_force_winograd(int mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -57,6 +57,24 @@ def build(force=False):
     return so
 
 
+def use_native_build():
+    """Builds the oracle for the CPU of this host (-march=native) and makes every later call use it: for the timed
+    CPU-baseline leg, which should not run an AVX2 build on an AVX-512 host.  Returns the compiler flags in use;
+    keeps the portable build when no compiler is at hand."""
+    global _LIB
+    so = os.path.join(_HERE, "liboracle_native.so")
+    try:
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle_native.so"], stdout=subprocess.DEVNULL,
+                              stderr=subprocess.DEVNULL)
+        native = ctypes.CDLL(so)
+        native.fdo_argmax.restype = ctypes.c_size_t
+        _LIB = native
+        return "-O3 -march=native, built on the measuring host"
+    except (OSError, subprocess.CalledProcessError):
+        lib()
+        return "-O3 -march=x86-64-v3 (AVX2 + FMA), prebuilt"
+
+
 def lib():
     global _LIB
     if _LIB is None:

@@ -1,4 +1,4 @@
-"""The C-ABI library loads without a GPU and exports every entry point include/fdx.h declares."""
+"""The C-ABI library loads without a GPU and exports every entry point include/fdx.h and include/fdx_debug.h declare."""
 import ctypes
 import os
 import re
@@ -9,8 +9,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "fdx.h")).read()
+def declared_symbols(headers=("fdx.h", "fdx_debug.h")):
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in headers)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     # function declarations only: "fdx_status (*callback)(...)" members and typedefs are not exported symbols
     return sorted(set(re.findall(r"\b(fdx_[a-z0-9_]+)\s*\((?!\*)", text)))
@@ -23,6 +23,9 @@ def test_header_declares_the_expected_surface():
                  "fdx_embedding_f32", "fdx_argmax_f32", "fdx_model_create", "fdx_model_predict", "fdx_session_create",
                  "fdx_session_decode_step", "fdx_last_error"):
         assert must in names
+    # the boundary header holds no measurement aids or test hooks: those live in fdx_debug.h
+    boundary = declared_symbols(("fdx.h",))
+    assert not [n for n in boundary if n.startswith(("fdx_debug_", "fdx_profile_", "fdx_timer_", "fdx_clock_probe_"))]
 
 
 def test_library_exports_every_declared_symbol(fdx):

@@ -279,11 +279,13 @@ def test_cnn_closed_rules_and_first_call_latency(fdx, oracle, modelgen, name, ba
     js = _features(modelgen, oracle, spec, tap, x[0])
     model = fdx.Model(js, verify=False)
     d_x = fdx.DevBuf.from_host(x)
+    shapes = [(224, 224, 3)]
+    d_outs = [fdx.DevBuf(4 * batch * int(np.prod(sh))) for sh in model.infer_shapes(shapes)]
     times = []
     for i in range(10):
         fdx.sync()
         t0 = time.perf_counter()
-        outs = model.predict_device([d_x], batch)
+        model.predict_dev(batch, [d_x], shapes, d_outs)
         fdx.sync()
         times.append((time.perf_counter() - t0) * 1e3)
     say("  first call %.1f ms, tenth %.1f ms" % (times[0], times[9]))
@@ -295,7 +297,6 @@ def test_cnn_closed_rules_and_first_call_latency(fdx, oracle, modelgen, name, ba
     again = fdx.Model(js, verify=False).predict([x])
     for g, a in zip(got, again):
         assert np.array_equal(g, a)
-    assert fdx.tuner_export().strip() == "" or True  # the table may hold rows other tests imported
 
 
 def test_predict_from_several_host_threads(fdx, modelgen):
