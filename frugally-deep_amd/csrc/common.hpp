@@ -19,6 +19,8 @@ bool profiling();
 // Clears library-owned scratch at set-up time, on the library stream (which does not synchronise with the null
 // stream) and waits for it, so that the first kernel that reads the cells sees zeros.  Not for use inside a stream capture.
 hipError_t zero_device(void* p, size_t bytes);
+// pinned host int that kernels store a code to when a bounded wait runs out; fdx_sync and fdx_d2h report and clear it
+int* async_error_cell();
 // records one launch for the per-kernel profile (flops / bytes are algorithmic figures; executed_flops = the
 // multiply-adds the kernel really issues where that differs, as in the Winograd form; negative = the same)
 void profile_begin();

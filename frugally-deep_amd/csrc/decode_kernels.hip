@@ -188,7 +188,61 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
         for (int w = 0; w < SK_WAVES; ++w)
             v += red[w * 256 + t];
     }
-    if (ksplit > 1) {
+    if (ksplit > 1 && p.local_split) {
+        // All K ranges of this column group run on one XCD (see SkinnyParams::local_split): partial tiles, flags and the
+        // final sum go through that XCD's L2 with group-scope accesses (they miss the CU's own cache and are served by
+        // the L2 the writers wrote through to), which costs a third of the exchange through memory below.  The last K
+        // range is the one that waits: workgroups start in the order of their linear index, so everything it waits for
+        // is already running or done, whatever else occupies the chip.
+        constexpr int kGroup = 1, kDevice = 16; // cache-policy bits of a buffer access: sc0 = group scope, sc1 = device scope
+        const int n_flags = p.ticket_count / 2;
+        const __amdgpu_buffer_rsrc_t ws_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.workspace, 0, (int)((int64_t)gx * ksplit * 1024), 0x00020000);
+        const __amdgpu_buffer_rsrc_t fl_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.tickets + n_flags, 0, n_flags * 4, 0x00020000);
+        const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u; // XCC_ID: which XCD this workgroup runs on
+        if (by != ksplit - 1) {
+            if (t < 256)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), ws_rsrc, ((by * gx + bx) * 256 + t) * 4, 0, kGroup);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (t == 0)
+                __builtin_amdgcn_raw_buffer_store_b32(1u + xcc, fl_rsrc, (bx * 8 + by) * 4, 0, kGroup);
+            return;
+        }
+        if (t < ksplit - 1) {
+            unsigned f = 0;
+            for (int spin = 0; spin < (1 << 18); ++spin) {
+                // Device scope for the flag: a group-scope load may be answered by this CU's own cache, which keeps the
+                // zero it saw first (measured: such polls never saw the flag); the line lies in this XCD's L2 either way.
+                // The compiler barriers keep the load inside the loop (as a read-only intrinsic it would be hoisted).
+                asm volatile("" ::: "memory");
+                f = __builtin_amdgcn_raw_buffer_load_b32(fl_rsrc, (bx * 8 + t) * 4, 0, kDevice);
+                asm volatile("" ::: "memory");
+                if (f)
+                    break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (f != 1u + xcc && p.err)
+                __hip_atomic_store(p.err, (int)(kErrSplitExchange | (f << 8) | (xcc << 16) | ((unsigned)t << 24)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        __syncthreads();
+        if (t < 256) {
+            float pv[8];
+#pragma unroll
+            for (int ks = 0; ks < 7; ++ks)
+                pv[ks] = ks < ksplit - 1
+                    ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ws_rsrc, ((ks * gx + bx) * 256 + t) * 4, 0, kGroup))
+                    : 0.f;
+            const float own = v;
+            v = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 7; ++ks)
+                if (ks < ksplit - 1)
+                    v += pv[ks];
+            v += own;
+        }
+        if (t < ksplit - 1)
+            __builtin_amdgcn_raw_buffer_store_b32(0u, fl_rsrc, (bx * 8 + t) * 4, 0, kGroup); // for the next launch
+    } else if (ksplit > 1) {
         // Publish this split's partial tile with device-scope stores (they go past the XCD's L2), wait for
         // them, then take a ticket; only the last arrival continues and adds the partials in split order,
         // which makes the sum independent of arrival order.  No fence that writes back the whole L2.
@@ -822,6 +876,13 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
             q.workspace = g_splitk_ws;
             q.tickets = g_splitk_tickets;
         }
+        // column groups in a multiple of 8: the K ranges of a group share an XCD and meet in its L2 (FDX_SPLIT_LOCAL=0
+        // keeps the exchange through memory, for comparison)
+        static const bool local_on = [] { const char* e = std::getenv("FDX_SPLIT_LOCAL"); return !(e && e[0] == '0'); }();
+        q.ticket_count = ticket_count;
+        q.workspace_floats = ws_floats;
+        q.local_split = (int)(local_on && ksplit > 1 && ksplit <= 8 && tiles % 8 == 0 && tiles * 8 <= ticket_count / 2 && tiles <= ticket_count / 2);
+        q.err = async_error_cell();
     }
     const int per_wg = ((p.K + ksplit * 16 - 1) / (ksplit * 16)) * 16; // as the kernel derives it
     const dim3 grid((unsigned)tiles, (unsigned)ksplit);

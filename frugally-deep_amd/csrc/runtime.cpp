@@ -15,6 +15,10 @@ static hipStream_t g_stream = nullptr;
 static bool g_inited = false;
 static std::mutex g_mutex;
 static hipEvent_t g_t0 = nullptr, g_t1 = nullptr;
+// One int in pinned host memory that kernels can reach: a kernel whose bounded wait ran out stores its code there, and
+// the calls that wait for the stream (fdx_sync, fdx_d2h) look at it, so a failed exchange comes back as an error from
+// the very call that would hand the results out.
+static int* g_async_err = nullptr;
 
 static bool g_profile = false;
 struct Pending {
@@ -50,6 +54,25 @@ hipStream_t stream()
     return g_stream;
 }
 bool profiling() { return g_profile; }
+int* async_error_cell()
+{
+    if (!g_inited)
+        (void)ensure_init();
+    return g_async_err;
+}
+// after the stream has drained: reports and clears what a kernel left in the cell
+static fdx_status check_async_error()
+{
+    if (!g_async_err)
+        return FDX_OK;
+    const int code = *static_cast<volatile int*>(g_async_err);
+    if (code == 0)
+        return FDX_OK;
+    *g_async_err = 0;
+    set_error("a kernel gave up a bounded wait for another workgroup's partial results (code %d): the results of the calls since the last "
+              "synchronisation are not valid", code);
+    return FDX_ERR_HIP;
+}
 
 hipError_t zero_device(void* p, size_t bytes)
 {
@@ -130,6 +153,8 @@ fdx_status ensure_init()
     FDX_HIP(hipEventCreate(&g_t0));
     FDX_HIP(hipEventCreate(&g_t1));
     FDX_HIP(noalloc_setup());
+    FDX_HIP(hipHostMalloc(reinterpret_cast<void**>(&g_async_err), sizeof(int), hipHostMallocDefault));
+    *g_async_err = 0;
     g_inited = true;
     return FDX_OK;
 }
@@ -181,7 +206,7 @@ extern "C" fdx_status fdx_d2h(void* dst, const void* src, size_t bytes)
 {
     FDX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
     FDX_HIP(hipStreamSynchronize(g_stream));
-    return FDX_OK;
+    return check_async_error();
 }
 
 extern "C" fdx_status fdx_sync(void)
@@ -190,7 +215,7 @@ extern "C" fdx_status fdx_sync(void)
     if (st != FDX_OK)
         return st;
     FDX_HIP(hipStreamSynchronize(g_stream));
-    return FDX_OK;
+    return check_async_error();
 }
 
 extern "C" fdx_status fdx_timer_start(void)

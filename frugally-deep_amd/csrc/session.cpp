@@ -618,7 +618,7 @@ bool build_fast_plan(fdx_session* s)
                 stp.g.W = packed;
                 stp.g.packed = 1;
             }
-            stp.g.workspace = nullptr; // split-K stays off: its device-scope fences cost more than the idle CUs
+            stp.g.workspace = nullptr; // launches that split K take the library's workspace and tickets
             stp.g.workspace_floats = fdx_session::kWsFloats;
             stp.g.tickets = s->splitk_tickets;
             stp.g.ticket_count = fdx_session::kTickets;

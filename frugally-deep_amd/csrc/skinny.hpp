@@ -33,10 +33,20 @@ struct SkinnyParams {
     int64_t workspace_floats;
     int* tickets;
     int ticket_count;
+    // The K ranges of a column group exchange their partial tiles inside their XCD's L2 instead of through memory:
+    // with a number of column groups that is a multiple of 8 the workgroups (bx, 0..splits-1) all run on XCD bx % 8
+    // (workgroups go round the XCDs by their linear index).  The last K range of a group waits, bounded, for flags the
+    // others store next to the tickets (tickets[ticket_count / 2 + bx * 8 + split], zero between launches), adds the
+    // partials in split order and runs the epilogue.  err (may be null) receives kErrSplitExchange if a wait runs out or
+    // the flags name another XCD.
+    int local_split;
+    int* err;
     // optional, wide-output launches only (skinny_wide_grid(p) > 0): every workgroup leaves the packed (value, column)
     // maximum of each row over the columns it produced in amax_parts[workgroup][16]; argmax_parts_launch picks the winner
     unsigned long long* amax_parts;
 };
+
+constexpr int kErrSplitExchange = 2; // value of the err cell: the partial tiles of a split launch did not meet
 
 fdx_status skinny_gemm_launch(const SkinnyParams& p);
 

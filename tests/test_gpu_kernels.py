@@ -551,8 +551,10 @@ def test_shader_clock_probe(fdx):
     assert y.to_host((1 << 20,))[123] == 1.0
 
 
+# (16, 3072, 768), (16, 4096, 1024), (9, 8192, 128): column groups in a multiple of 8, so the K ranges of a group (4, 4 and 8
+# of them) meet inside their XCD's L2; (1, 2048, 48): three column groups, the K ranges meet through memory
 DENSE_ROWS = [(16, 768, 2304), (16, 768, 768), (16, 3072, 768), (3, 64, 100), (16, 768, 50257), (5, 20, 33), (7, 1024, 40),
-              (16, 100, 64), (1, 2048, 48)]
+              (16, 100, 64), (1, 2048, 48), (16, 4096, 1024), (9, 8192, 128)]
 
 
 @pytest.mark.parametrize("m,k,n", DENSE_ROWS)
@@ -568,10 +570,13 @@ def test_dense_rows_decode_shape(fdx, oracle, m, k, n):
     dx, dw, db, dr = (fdx.DevBuf.from_host(a) for a in (x, w, b, res))
     out = fdx.DevBuf(4 * m * n)
     act = fdx.gelu_act()
-    for _ in range(2):  # twice: the split-K tickets must be back at zero after a launch
+    got = []
+    for _ in range(3):  # repeated: the split-K tickets and flags must be back at zero after a launch
         fdx.check(fdx.lib.fdx_dense_rows_f32(fdx._dp(dx), m, k, fdx._dp(dw), fdx._dp(db), n, fdx._dp(dr), fdx.ctypes.byref(act),
                                              fdx._dp(out)))
-        assert rel(out.to_host((m, n)), want) <= TOL
+        got.append(out.to_host((m, n)))
+        assert rel(got[-1], want) <= TOL
+    assert np.array_equal(got[0], got[1]) and np.array_equal(got[0], got[2])  # partial tiles are added in a fixed order
 
 
 @pytest.mark.parametrize("m,k,n", [(16, 768, 2304), (3, 64, 100), (16, 768, 50257), (7, 1024, 40), (16, 100, 64)])
