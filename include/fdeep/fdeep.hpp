@@ -78,6 +78,8 @@ public:
         return 1;
     }
     void shrink_rank() { rank_ = minimal_rank(); }
+    // include/fdeep/tensor_shape.hpp:143-146
+    void shrink_rank_with_min(std::size_t min_rank_to_keep) { rank_ = std::max(minimal_rank(), min_rank_to_keep); }
     void maximize_rank() { rank_ = 5; }
     // the extents the rank covers, outermost first (include/fdeep/tensor_shape.hpp:153-164)
     std::vector<std::size_t> dimensions() const
@@ -136,6 +138,14 @@ public:
     tensor_shape_variable(std::size_t rank, const std::vector<std::int64_t>& dims5)
         : rank_(rank), dims_(dims5) {}
     std::size_t rank() const { return rank_; }
+    // product of the known extents, unknown ones counting as 1 (include/fdeep/tensor_shape_variable.hpp:87-90)
+    std::size_t minimal_volume() const
+    {
+        std::size_t v = 1;
+        for (std::int64_t d : dims_)
+            v *= d >= 0 ? static_cast<std::size_t>(d) : 1;
+        return v;
+    }
     bool fixed(std::size_t i) const { return dims_[i] >= 0; }     // i indexes the 5 right-aligned dims
     std::int64_t dim(std::size_t i) const { return dims_[i]; }
     std::size_t rank_;
@@ -196,6 +206,19 @@ public:
     std::size_t z_;
 };
 
+// include/fdeep/tensor_pos.hpp:116-147
+inline tensor_pos create_tensor_pos_from_dims(const std::vector<std::size_t>& dimensions)
+{
+    internal::assertion(dimensions.size() >= 1 && dimensions.size() <= 5, "Invalid tensor-pos dimensions");
+    switch (dimensions.size()) {
+    case 1: return tensor_pos(dimensions[0]);
+    case 2: return tensor_pos(dimensions[0], dimensions[1]);
+    case 3: return tensor_pos(dimensions[0], dimensions[1], dimensions[2]);
+    case 4: return tensor_pos(dimensions[0], dimensions[1], dimensions[2], dimensions[3]);
+    default: return tensor_pos(dimensions[0], dimensions[1], dimensions[2], dimensions[3], dimensions[4]);
+    }
+}
+
 // Rank <= 5, right-aligned, row-major, channels-last fp32 values on a shared buffer:
 // copying a tensor shares the buffer.
 class tensor {
@@ -219,6 +242,27 @@ public:
         return get_ignore_rank(pos);
     }
     float_type get_ignore_rank(const tensor_pos& pos) const { return (*values_)[idx_ignore_rank(pos)]; }
+    const float_type& get_ref_ignore_rank(const tensor_pos& pos) const { return (*values_)[idx_ignore_rank(pos)]; }
+    float_type& get_ref_ignore_rank(const tensor_pos& pos) { return (*values_)[idx_ignore_rank(pos)]; }
+    // the value at a signed position, pad_value outside the tensor (include/fdeep/tensor.hpp:66-79)
+    float_type get_padded(float_type pad_value, int d5, int d4, int y, int x, int z) const
+    {
+        if (d5 < 0 || d5 >= static_cast<int>(shape_.size_dim_5_) || d4 < 0 || d4 >= static_cast<int>(shape_.size_dim_4_) || y < 0
+            || y >= static_cast<int>(shape_.height_) || x < 0 || x >= static_cast<int>(shape_.width_) || z < 0
+            || z >= static_cast<int>(shape_.depth_))
+            return pad_value;
+        return get_ignore_rank(tensor_pos(static_cast<std::size_t>(d5), static_cast<std::size_t>(d4), static_cast<std::size_t>(y),
+            static_cast<std::size_t>(x), static_cast<std::size_t>(z)));
+    }
+    // the five-index forms the reference keeps as deprecated (include/fdeep/tensor.hpp:95-112): rank is ignored
+    float_type get(std::size_t pos_dim_5, std::size_t pos_dim_4, std::size_t y, std::size_t x, std::size_t z) const
+    {
+        return get_ignore_rank(tensor_pos(pos_dim_5, pos_dim_4, y, x, z));
+    }
+    void set(std::size_t pos_dim_5, std::size_t pos_dim_4, std::size_t y, std::size_t x, std::size_t z, float_type value)
+    {
+        set_ignore_rank(tensor_pos(pos_dim_5, pos_dim_4, y, x, z), value);
+    }
     void set(const tensor_pos& pos, float_type value)
     {
         internal::assertion(pos.rank() == shape_.rank(), "Invalid position rank for tensor");
@@ -226,11 +270,15 @@ public:
     }
     void set_ignore_rank(const tensor_pos& pos, float_type value) { (*values_)[idx_ignore_rank(pos)] = value; }
     const tensor_shape& shape() const { return shape_; }
+    void shrink_rank() { shape_.shrink_rank(); }
+    void shrink_rank_with_min(std::size_t min_rank_to_keep) { shape_.shrink_rank_with_min(min_rank_to_keep); }
+    void maximize_rank() { shape_.maximize_rank(); }
     std::size_t depth() const { return shape_.depth_; }
     std::size_t height() const { return shape_.height_; }
     std::size_t width() const { return shape_.width_; }
     std::size_t rank() const { return shape_.rank(); }
     const shared_float_vec& as_vector() const { return values_; }
+    shared_float_vec& as_vector() { return values_; }
     float_vec to_vector() const { return *values_; }
 
 private:
@@ -321,6 +369,31 @@ inline std::vector<std::uint8_t> tensor_to_bytes(const tensor& t, float_type low
     std::vector<std::uint8_t> bytes(t.shape().volume(), 0);
     tensor_into_bytes(t, bytes.data(), bytes.size(), low, high);
     return bytes;
+}
+
+// All values of all tensors, in order, cut anew into vectors_size vectors of vector_size tensors of shape
+// (height, width, depth) (include/fdeep/tensor.hpp:1282-1303)
+inline tensors_vec reshape_tensor_vectors(std::size_t vectors_size, std::size_t vector_size, std::size_t depth, std::size_t height,
+    std::size_t width, const tensors_vec& tss)
+{
+    float_vec values;
+    for (const auto& ts : tss)
+        for (const auto& t : ts)
+            values.insert(values.end(), t.as_vector()->begin(), t.as_vector()->end());
+    internal::assertion(values.size() == vectors_size * vector_size * height * width * depth,
+        "Invalid number of values for reshape target.");
+    const std::size_t per_tensor = depth * height * width;
+    tensors_vec result;
+    std::size_t at = 0;
+    while (at < values.size()) {
+        if (result.empty() || result.back().size() == vector_size)
+            result.emplace_back();
+        const std::size_t n = std::min(per_tensor, values.size() - at);
+        result.back().push_back(tensor(tensor_shape(height, width, depth),
+            float_vec(values.begin() + static_cast<std::ptrdiff_t>(at), values.begin() + static_cast<std::ptrdiff_t>(at + n))));
+        at += n;
+    }
+    return result;
 }
 
 namespace internal {

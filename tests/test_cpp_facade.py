@@ -20,6 +20,18 @@ def compile_facade():
                            "-L", PKG, "-lfdx", "-Wl,-rpath," + PKG, "-Wl,-rpath,/opt/rocm/lib", "-pthread", "-o", EXE])
 
 
+def test_value_types_follow_the_reference(fdx):
+    """tensor / tensor_shape / tensor_shape_variable / tensor_pos members and reshape_tensor_vectors of the facade
+    (host code only: the program touches no GPU)."""
+    src = os.path.join(ROOT, "tests", "cpp", "value_types_test.cpp")
+    exe = os.path.join(ROOT, "tests", "cpp", "value_types_test.bin")
+    subprocess.check_call(["g++", "-std=c++14", "-O1", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), src,
+                           "-L", PKG, "-lfdx", "-Wl,-rpath," + PKG, "-Wl,-rpath,/opt/rocm/lib", "-pthread", "-o", exe])
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    print(out.stdout, out.stderr, flush=True)
+    assert out.returncode == 0 and "value_types_test ok" in out.stdout
+
+
 def test_facade_compiles_and_links(fdx):
     compile_facade()
     assert os.path.exists(EXE)
