@@ -103,6 +103,13 @@ def tuner_import(text):
     check(lib.fdx_tuner_import(text.encode()))
 
 
+def model_check(json_text, unknown_extent=7):
+    """The host half of loading a model file (parse, graph, parameter arrays, shapes) without touching a GPU
+    (fdx_model_check); raises FdxError with the loader's message for a defective file."""
+    data = json_text if isinstance(json_text, bytes) else json_text.encode()
+    check(lib.fdx_model_check(data, ctypes.c_size_t(len(data)), ctypes.c_int64(unknown_extent)))
+
+
 def tuner_timing(on=True):
     """Timing runs on the first sight of a shape (off unless asked for; FDX_AUTOTUNE=1 asks for them too)."""
     check(lib.fdx_tuner_timing(1 if on else 0))

@@ -116,6 +116,7 @@ __device__ __forceinline__ float apply_act_full(float x, const Act& a)
 // primitives: swaps inside quads, then the mirror inside each half row and inside the row (after the quad steps all lanes
 // of a quad agree, so the mirrored partner holds the other quads' sum).  __shfl_xor compiles to ds_bpermute_b32, a trip
 // through the LDS crossbar with an address register and a wait of its own per step.
+#if defined(__HIPCC__) // device-only builtins; a plain host compiler (the sanitizer build of the loader) skips them
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v)
 {
@@ -129,6 +130,7 @@ __device__ __forceinline__ float row16_sum(float v)
     v += dpp_move<0x140>(v); // row_mirror
     return v;
 }
+#endif
 
 // activations an epilogue can carry
 inline bool epilogue_act_ok(const fdx_act* a) { return !a || a->kind == FDX_ACT_NONE || a->kind == FDX_ACT_RELU || a->kind == FDX_ACT_GELU; }

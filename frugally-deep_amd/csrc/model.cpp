@@ -91,7 +91,8 @@ namespace {
         if (bytes.size() % 4 != 0)
             throw FormatError("invalid float vector data");
         out.resize(bytes.size() / 4);
-        std::memcpy(out.data(), bytes.data(), bytes.size());
+        if (!bytes.empty()) // an empty array has no buffer to copy from
+            std::memcpy(out.data(), bytes.data(), bytes.size());
         return out;
     }
 
@@ -282,6 +283,7 @@ namespace {
         std::string prefix;
         std::map<std::string, int> input_ops;
         std::map<std::tuple<std::string, int, int>, int> memo;
+        std::set<std::tuple<std::string, int, int>> building; // connections whose producers are being resolved right now
     };
 
     struct Builder {
@@ -387,6 +389,14 @@ namespace {
             auto lit = sc.layers.find(c.layer);
             if (lit == sc.layers.end())
                 throw FormatError("dangling connection to layer " + c.layer);
+            // a layer that (directly or through others) names itself as its input would recurse without end
+            if (!sc.building.insert(key).second)
+                throw FormatError("cyclic connection at layer " + c.layer);
+            struct Leave {
+                std::set<std::tuple<std::string, int, int>>& s;
+                std::tuple<std::string, int, int> k;
+                ~Leave() { s.erase(k); }
+            } leave { sc.building, key };
             const Value& L = *lit->second;
             const std::string cls = L.at("class_name").str();
             const Value& cfg = L.at("config");
@@ -2530,7 +2540,8 @@ namespace {
 
 fdx_model::~fdx_model()
 {
-    (void)hipStreamSynchronize(fdx::stream());
+    if (!device_allocs.empty() || err_flag || !plans.empty()) // a model that was only checked never reached the device
+        (void)hipStreamSynchronize(fdx::stream());
     for (auto& hl : host_layers)
         if (hl.vt.destroy && hl.instance)
             hl.vt.destroy(hl.instance);
@@ -2546,18 +2557,16 @@ extern "C" fdx_status fdx_model_create(const char* json_text, size_t len, int ve
     return fdx_model_create_custom(json_text, len, verify, verify_epsilon, nullptr, 0, out);
 }
 
-extern "C" fdx_status fdx_model_create_custom(const char* json_text, size_t len, int verify, float verify_epsilon,
-    const fdx_custom_layer* custom_layers, int n_custom_layers, fdx_model** out)
-{
-    FDX_REQUIRE(json_text && out, "model_create: null argument");
-    FDX_REQUIRE(n_custom_layers >= 0 && (n_custom_layers == 0 || custom_layers), "model_create: bad custom layer list");
-    *out = nullptr;
-    if (fdx_sync() != FDX_OK)
-        return FDX_ERR_HIP;
-    std::unique_ptr<fdx_model> m(new fdx_model);
-    try {
+namespace fdx {
+namespace {
+    // Host half of loading: text -> op list -> load-time fusion.  Touches no device; throws FormatError / Unsupported.
+    const Value& parse_and_build(const char* json_text, size_t len, const fdx_custom_layer* custom_layers, int n_custom_layers,
+        fdx_model& model, std::unique_ptr<Value>& root_holder)
+    {
+        fdx_model* m = &model;
         json::Parser parser(json_text, len);
-        const Value root = parser.parse();
+        root_holder.reset(new Value(parser.parse()));
+        const Value& root = *root_holder;
         const Value* fmt = root.find("image_data_format");
         if (!fmt || !fmt->is_string() || fmt->str() != "channels_last")
             throw FormatError("only channels_last data format supported");
@@ -2605,6 +2614,23 @@ extern "C" fdx_status fdx_model_create_custom(const char* json_text, size_t len,
         for (const auto& o : outs)
             m->outputs.push_back(b.build(top, o));
         fuse(*m);
+        return root;
+    }
+} // namespace
+} // namespace fdx
+
+extern "C" fdx_status fdx_model_create_custom(const char* json_text, size_t len, int verify, float verify_epsilon,
+    const fdx_custom_layer* custom_layers, int n_custom_layers, fdx_model** out)
+{
+    FDX_REQUIRE(json_text && out, "model_create: null argument");
+    FDX_REQUIRE(n_custom_layers >= 0 && (n_custom_layers == 0 || custom_layers), "model_create: bad custom layer list");
+    *out = nullptr;
+    if (fdx_sync() != FDX_OK)
+        return FDX_ERR_HIP;
+    std::unique_ptr<fdx_model> m(new fdx_model);
+    try {
+        std::unique_ptr<Value> holder;
+        const Value& root = parse_and_build(json_text, len, custom_layers, n_custom_layers, *m, holder);
         fdx_status st = upload(*m);
         if (st != FDX_OK)
             return st;
@@ -2622,6 +2648,54 @@ extern "C" fdx_status fdx_model_create_custom(const char* json_text, size_t len,
         return FDX_ERR_FORMAT;
     }
     *out = m.release();
+    return FDX_OK;
+}
+
+// The host half of fdx_model_create alone: parses the text, builds and fuses the op list, decodes every parameter array
+// and the embedded test tensors, and infers all shapes with unknown extents set to `unknown_extent`.  No device is
+// touched, so a file can be checked where there is no GPU; the status and message are the ones fdx_model_create would
+// give for the same defect.
+extern "C" fdx_status fdx_model_check(const char* json_text, size_t len, int64_t unknown_extent)
+{
+    FDX_REQUIRE(json_text, "model_check: null argument");
+    FDX_REQUIRE(unknown_extent > 0, "model_check: the stand-in for unknown extents must be positive");
+    fdx_model m;
+    try {
+        std::unique_ptr<Value> holder;
+        const Value& root = parse_and_build(json_text, len, nullptr, 0, m, holder);
+        std::vector<Shape> shapes;
+        for (const Shape& d : m.in_decl) {
+            Shape s = d;
+            for (auto& e : s)
+                if (e < 0)
+                    e = unknown_extent;
+            shapes.push_back(s);
+        }
+        std::vector<Shape> all;
+        const fdx_status st = infer_shapes(m, shapes, all, topo_order(m));
+        if (st != FDX_OK)
+            return st;
+        if (const Value* tests = root.find("tests"))
+            if (tests->is_array())
+                for (const auto& t : tests->arr) {
+                    const Value& ins = t.at("inputs");
+                    const Value& outs = t.at("outputs");
+                    FDX_REQUIRE(ins.is_array() && outs.is_array(), "test needs inputs and outputs");
+                    FDX_REQUIRE(ins.size() == m.inputs.size() && outs.size() == m.outputs.size(), "test case arity does not match the model");
+                    for (const Value* side : { &ins, &outs })
+                        for (const auto& tv : side->arr) {
+                            const Shape s = decl_shape(tv.at("shape"));
+                            const std::vector<float> vals = decode_floats(tv.at("values"));
+                            FDX_REQUIRE((int64_t)vals.size() == volume(s), "test tensor: values do not fill the shape");
+                        }
+                }
+    } catch (const Unsupported& e) {
+        set_error("%s", e.what());
+        return FDX_ERR_UNSUPPORTED;
+    } catch (const std::exception& e) {
+        set_error("%s", e.what());
+        return FDX_ERR_FORMAT;
+    }
     return FDX_OK;
 }
 

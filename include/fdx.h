@@ -356,6 +356,14 @@ typedef struct fdx_session fdx_session;
  * test cases with absolute tolerance verify_epsilon (model.hpp:254-267, import_model.hpp:1990-2021).
  */
 fdx_status fdx_model_create(const char* json, size_t len, int verify, float verify_epsilon, fdx_model** out);
+/*
+ * The host half of fdx_model_create alone, for machines without a GPU: what read_model does to a file before the first
+ * prediction (include/fdeep/model.hpp:198-253, import_model.hpp:274-297 for the parameter arrays): parses the text, builds the
+ * layer graph, decodes every parameter array and embedded test tensor and infers all shapes, with unknown extents set to
+ * unknown_extent (> 0).  Returns the status and message fdx_model_create would give for the same defect; touches no device.
+ * Files that need a custom layer creator answer FDX_ERR_UNSUPPORTED here.
+ */
+fdx_status fdx_model_check(const char* json, size_t len, int64_t unknown_extent);
 /* ---- host fallback for layer classes the device path does not implement ----
  * The counterpart of the reference's extension point: internal::layer_creators, a map from class name
  * to a factory of layer objects whose apply_impl runs on host tensors

@@ -70,3 +70,14 @@ def test_modelgen_flops_and_format(modelgen, oracle):
     for n in (0, 1, 191, 192, 193, 384):
         a = np.arange(n, dtype=np.float32)
         assert json.loads(modelgen._encode_floats_json(a)) == modelgen.encode_floats(a)
+
+
+def test_model_check_runs_without_a_gpu(fdx, modelgen):
+    """fdx_model_check is the loader's host half: a good file passes and a defective one comes back with the loader's own
+    message, on a machine with no GPU."""
+    fdx.model_check(modelgen.dumps(modelgen.small_cnn()))
+    fdx.model_check(modelgen.dumps(modelgen.gpt2(layers=1, d_model=16, heads=2, vocab=50, max_pos=16)))
+    with pytest.raises(fdx.FdxError, match="channels_last"):
+        fdx.model_check(b'{"image_data_format": "channels_first"}')
+    with pytest.raises(fdx.FdxError):
+        fdx.model_check(b'{"image_data_format": "channels_last", "architecture": {')
