@@ -32,6 +32,26 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm + wino, ResNet50 b64": 144.3e6, "skinny_gemm, GPT-2 decode b16": 11.0e6}
 
 
+def under_profiler():
+    """True when a ROCm profiler drives this process (rocprofv3 preloads its tool library and sets ROCPROF* variables)."""
+    pre = os.environ.get("LD_PRELOAD", "")
+    return "rocprofiler" in pre or "rocprof" in pre or any(k.startswith(("ROCPROF", "ROCPROFILER")) for k in os.environ)
+
+
+def log_address_map(stage):
+    """Under a profiler: keeps a copy of /proc/self/maps per stage, so that a fault address from a runtime or profiler
+    thread (none of the library's own: it starts no threads) can be attributed to a mapping afterwards."""
+    if not under_profiler():
+        return
+    try:
+        out_dir = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out_dir, exist_ok=True)
+        with open("/proc/self/maps") as src, open(os.path.join(out_dir, "bench_maps_%d_%s.txt" % (os.getpid(), stage)), "w") as dst:
+            dst.write(src.read())
+    except OSError:
+        pass
+
+
 def load_package():
     import __graft_entry__ as entry
     entry._ensure_built()
@@ -332,6 +352,7 @@ def bench_gpt2(fdx, modelgen, args):
     spec = modelgen.gpt2()
     js = modelgen.dumps(spec)
     del spec
+    log_address_map("gpt2_generated")
     t0 = time.perf_counter()
     model = fdx.Model(js, verify=False)
     load_s = time.perf_counter() - t0
@@ -474,7 +495,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (samples are independent; more GPUs would each take a "
                  "slice of the batch with their own copy of the weights) -- use --gpus 1")
+    log_address_map("start")
     fdx, modelgen = load_package()
+    log_address_map("library_loaded")
     if args.tuner_import:
         fdx.tuner_import(open(args.tuner_import).read())
         fdx.tuner_freeze(True)

@@ -719,6 +719,21 @@ class Model:
         check(lib.fdx_model_predict(self._h, batch, ip, dims, ranks, op, None, None))
         return outs
 
+    def predict_samples(self, samples):
+        """samples[b][i] = the array of input i of sample b (the form fdeep::model::predict_multi takes): every sample
+        stays where it is, the library gathers them on their way to the GPU (fdx_model_predict_samples)."""
+        batch = len(samples)
+        held = [[np.ascontiguousarray(samples[b][i], np.float32) for b in range(batch)] for i in range(self.n_inputs)]
+        sample_shapes = [held[i][0].shape for i in range(self.n_inputs)]
+        dims, ranks = self._dims(sample_shapes)
+        out_shapes = self.infer_shapes(sample_shapes)
+        outs = [np.empty((batch,) + s, np.float32) for s in out_shapes]
+        ip = (c_float_p * (self.n_inputs * batch))(*[held[i][b].ctypes.data_as(c_float_p) for i in range(self.n_inputs)
+                                                      for b in range(batch)])
+        op = (c_float_p * self.n_outputs)(*[o.ctypes.data_as(c_float_p) for o in outs])
+        check(lib.fdx_model_predict_samples(self._h, batch, ip, dims, ranks, op, None, None))
+        return outs
+
     def predict_dev(self, batch, in_bufs, sample_shapes, out_bufs):
         """Device-resident variant: in_bufs / out_bufs are DevBuf objects; asynchronous (call sync())."""
         dims, ranks = self._dims(sample_shapes)

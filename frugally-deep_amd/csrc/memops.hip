@@ -945,6 +945,9 @@ extern "C" fdx_status fdx_clock_probe_start(int samples, int period_us)
 {
     FDX_REQUIRE(samples >= 2 && samples <= kProbeMaxSamples && period_us >= 10 && period_us <= 100000,
         "clock_probe_start: 2..65536 samples, period 10..100000 us");
+    // the probe kernel ends only by itself, and fdx_clock_probe_stop waits for it: keep its whole run within ten seconds
+    FDX_REQUIRE((long long)samples * period_us <= 10LL * 1000 * 1000,
+        "clock_probe_start: samples x period is %lld us; a probe may run for at most 10 s", (long long)samples * period_us);
     (void)stream(); // the library is initialised on its device
     std::lock_guard<std::mutex> lock(g_probe_mutex);
     FDX_REQUIRE(g_probe_samples == 0, "clock_probe_start: a probe is already running; call fdx_clock_probe_stop first");

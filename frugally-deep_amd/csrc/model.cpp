@@ -13,7 +13,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <condition_variable>
 #include <set>
+#include <thread>
 #include <tuple>
 
 #include "einsum.hpp"
@@ -2358,11 +2360,12 @@ namespace {
         return st;
     }
 
-    fdx_status execute(fdx_model& m, Plan& p)
+    // skip: an op that has already run for this call (the first convolution, behind the input copy), or -1
+    fdx_status execute(fdx_model& m, Plan& p, int skip = -1)
     {
         for (int idx : p.order) {
             const Op& o = m.ops[idx];
-            if (o.dead)
+            if (o.dead || idx == skip)
                 continue;
             fdx_status st = FDX_OK;
             if (o.fused_into >= 0 && p.dw_fused[o.fused_into] != 2)
@@ -2412,8 +2415,242 @@ namespace {
         return FDX_OK;
     }
 
+    // ---- host inputs on their way to the GPU ------------------------------------------------------------------------
+    // A large host input (a batch of images: tens of MB) is not handed to one pageable hipMemcpy, which stages it through
+    // the runtime's own bounce buffers on the calling thread at about half the link's rate and lets the GPU wait for all of
+    // it.  It goes through two pinned buffers of the library in pieces of whole samples: a few helper threads fill one
+    // buffer from the caller's memory while the DMA engine drains the other, and the first convolution of the network
+    // runs on each piece as soon as its copy has landed, so that only the rest of the network waits for the last piece.
+    // One stager per process; host threads that predict at the same time take turns.
+    struct Segment {
+        const char* src;
+        char* dst;
+        size_t bytes;
+    };
+    class Stager {
+    public:
+        static constexpr int kLanes = 4;          // the calling thread plus three helpers
+        static constexpr size_t kMinBytes = 4u << 20; // below this one plain copy is as fast
+        std::mutex use; // held for a whole staged input
+        char* pinned[2] = { nullptr, nullptr };
+        size_t pinned_bytes = 0;
+        hipStream_t copy_stream = nullptr;
+        hipEvent_t drained[2] = { nullptr, nullptr }; // the copy out of pinned[i] has finished
+        hipEvent_t landed = nullptr;                  // recorded per piece; the compute stream waits on it
+
+        fdx_status prepare(size_t piece_bytes)
+        {
+            if (!copy_stream) {
+                FDX_HIP(hipStreamCreateWithFlags(&copy_stream, hipStreamNonBlocking));
+                for (auto& e : drained)
+                    FDX_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+                FDX_HIP(hipEventCreateWithFlags(&landed, hipEventDisableTiming));
+            }
+            if (piece_bytes > pinned_bytes) {
+                for (auto& b : pinned) {
+                    if (b)
+                        FDX_HIP(hipHostFree(b));
+                    b = nullptr;
+                    FDX_HIP(hipHostMalloc(reinterpret_cast<void**>(&b), piece_bytes, hipHostMallocDefault));
+                }
+                pinned_bytes = piece_bytes;
+            }
+            if (workers.empty())
+                for (int i = 1; i < kLanes; ++i)
+                    workers.emplace_back([this, i] { work(i); });
+            return FDX_OK;
+        }
+        // copies the segments with all lanes; returns when every byte is in place
+        void gather(const std::vector<Segment>& segs)
+        {
+            size_t total = 0;
+            for (const auto& g : segs)
+                total += g.bytes;
+            const size_t share = (total + kLanes - 1) / kLanes;
+            std::vector<std::vector<Segment>> lanes(kLanes);
+            size_t lane = 0, room = share;
+            for (Segment g : segs)
+                while (g.bytes > 0) {
+                    const size_t take = std::min(g.bytes, room);
+                    lanes[lane].push_back({ g.src, g.dst, take });
+                    g.src += take; g.dst += take; g.bytes -= take; room -= take;
+                    if (room == 0 && lane + 1 < (size_t)kLanes) {
+                        ++lane;
+                        room = share;
+                    }
+                }
+            {
+                std::lock_guard<std::mutex> lock(mu);
+                for (int i = 1; i < kLanes; ++i)
+                    jobs[i] = &lanes[(size_t)i];
+                pending = kLanes - 1;
+                ++round;
+            }
+            wake.notify_all();
+            for (const auto& g : lanes[0])
+                std::memcpy(g.dst, g.src, g.bytes);
+            std::unique_lock<std::mutex> lock(mu);
+            done.wait(lock, [this] { return pending == 0; });
+        }
+        ~Stager()
+        {
+            {
+                std::lock_guard<std::mutex> lock(mu);
+                quit = true;
+            }
+            wake.notify_all();
+            for (auto& t : workers)
+                t.join();
+            // pinned buffers, stream and events live until the process ends (the runtime may be gone by now)
+        }
+
+    private:
+        void work(int lane)
+        {
+            unsigned seen = 0;
+            for (;;) {
+                const std::vector<Segment>* job = nullptr;
+                {
+                    std::unique_lock<std::mutex> lock(mu);
+                    wake.wait(lock, [&] { return quit || round != seen; });
+                    if (quit)
+                        return;
+                    seen = round;
+                    job = jobs[lane];
+                }
+                for (const auto& g : *job)
+                    std::memcpy(g.dst, g.src, g.bytes);
+                {
+                    std::lock_guard<std::mutex> lock(mu);
+                    if (--pending == 0)
+                        done.notify_all();
+                }
+            }
+        }
+        std::vector<std::thread> workers;
+        std::mutex mu;
+        std::condition_variable wake, done;
+        const std::vector<Segment>* jobs[kLanes] = {};
+        int pending = 0;
+        unsigned round = 0;
+        bool quit = false;
+    };
+    Stager& stager()
+    {
+        static Stager* s = new Stager; // never destroyed: its threads sleep until the process ends
+        return *s;
+    }
+
+    // The convolution that alone consumes the model's only input and can run on a range of samples by itself, or -1.
+    int first_conv_of(const fdx_model& m, const Plan& p)
+    {
+        if (m.inputs.size() != 1)
+            return -1;
+        const int in = m.inputs[0];
+        int found = -1;
+        for (int idx : p.order) {
+            const Op& o = m.ops[idx];
+            if (o.dead)
+                continue;
+            bool uses = o.residual == in;
+            for (int i : o.in)
+                uses = uses || i == in;
+            if (!uses)
+                continue;
+            if (found >= 0 || o.kind != OpKind::Conv2D || o.in.size() != 1 || o.residual >= 0 || o.fused_into >= 0 || o.exp_into >= 0
+                || o.fuse_dw >= 0 || o.softmax)
+                return -1;
+            if (o.dw.size() > 4 && o.dw[4] && p.conv_form[idx] < 0)
+                return -1; // its form is still to be timed on the whole batch
+            found = idx;
+        }
+        for (int out : m.outputs)
+            if (out == in || out == found)
+                return -1;
+        // a block that absorbs this convolution (first block of MobileNet-like networks) runs it inside its own launch
+        if (found >= 0)
+            for (int idx : p.order)
+                if (!m.ops[idx].dead && m.ops[idx].fuse_exp == found)
+                    return -1;
+        return found;
+    }
+
+    // One host input per model input, each either one contiguous block of `batch` samples or `batch` pointers to single
+    // samples; copies them to the plan's input buffers and, where the network starts with a convolution of its own
+    // launch, runs that convolution piece by piece behind the copy.  *conv_done receives the op already executed, or -1.
+    fdx_status stage_host_inputs(fdx_model* m, Plan* p, int batch, const float* const* in, bool per_sample, const std::vector<Shape>& shapes,
+        int* conv_done)
+    {
+        *conv_done = -1;
+        size_t total = 0;
+        for (size_t i = 0; i < m->inputs.size(); ++i)
+            total += sizeof(float) * (size_t)batch * (size_t)volume(shapes[i]);
+        if (total < Stager::kMinBytes) {
+            for (size_t i = 0; i < m->inputs.size(); ++i) {
+                const size_t sample = sizeof(float) * (size_t)volume(shapes[i]);
+                char* dst = reinterpret_cast<char*>(p->out[m->inputs[i]]);
+                if (!per_sample)
+                    FDX_HIP(hipMemcpyAsync(dst, in[i], sample * (size_t)batch, hipMemcpyHostToDevice, stream()));
+                else
+                    for (int b = 0; b < batch; ++b)
+                        FDX_HIP(hipMemcpyAsync(dst + sample * (size_t)b, in[i * (size_t)batch + (size_t)b], sample, hipMemcpyHostToDevice, stream()));
+            }
+            return FDX_OK;
+        }
+        Stager& st = stager();
+        std::lock_guard<std::mutex> lock(st.use);
+        const int conv = batch >= 8 ? first_conv_of(*m, *p) : -1;
+        // pieces of whole samples: four per input, more where a piece would exceed 16 MB
+        int piece = 0; // counted over all inputs: the two pinned buffers alternate across them
+        for (size_t i = 0; i < m->inputs.size(); ++i) {
+            const size_t sample = sizeof(float) * (size_t)volume(shapes[i]);
+            int per_piece = std::max(1, (batch + 3) / 4);
+            while (per_piece > 1 && sample * (size_t)per_piece > ((size_t)16 << 20))
+                per_piece = (per_piece + 1) / 2;
+            fdx_status fs = st.prepare(sample * (size_t)per_piece);
+            if (fs != FDX_OK)
+                return fs;
+            char* dst = reinterpret_cast<char*>(p->out[m->inputs[i]]);
+            for (int s0 = 0; s0 < batch; s0 += per_piece, ++piece) {
+                const int count = std::min(per_piece, batch - s0);
+                const int slot = piece & 1;
+                if (piece >= 2)
+                    FDX_HIP(hipEventSynchronize(st.drained[slot])); // the copy that last read this buffer
+                std::vector<Segment> segs;
+                if (!per_sample)
+                    segs.push_back({ reinterpret_cast<const char*>(in[i]) + sample * (size_t)s0, st.pinned[slot], sample * (size_t)count });
+                else
+                    for (int b = 0; b < count; ++b)
+                        segs.push_back({ reinterpret_cast<const char*>(in[i * (size_t)batch + (size_t)(s0 + b)]), st.pinned[slot] + sample * (size_t)b, sample });
+                st.gather(segs);
+                FDX_HIP(hipMemcpyAsync(dst + sample * (size_t)s0, st.pinned[slot], sample * (size_t)count, hipMemcpyHostToDevice, st.copy_stream));
+                FDX_HIP(hipEventRecord(st.drained[slot], st.copy_stream));
+                FDX_HIP(hipEventRecord(st.landed, st.copy_stream));
+                FDX_HIP(hipStreamWaitEvent(stream(), st.landed, 0));
+                if (conv >= 0) {
+                    // the first convolution on samples s0 .. s0 + count of its input and output
+                    const int src = m->inputs[0];
+                    const int saved_batch = p->batch;
+                    float* const saved_in = p->out[src];
+                    float* const saved_out = p->out[conv];
+                    p->batch = count;
+                    p->out[src] = saved_in + (size_t)s0 * (size_t)volume(p->shapes[src]);
+                    p->out[conv] = saved_out + (size_t)s0 * (size_t)volume(p->shapes[conv]);
+                    const fdx_status rs = run_op(*m, *p, conv);
+                    p->batch = saved_batch;
+                    p->out[src] = saved_in;
+                    p->out[conv] = saved_out;
+                    if (rs != FDX_OK)
+                        return rs;
+                }
+            }
+        }
+        *conv_done = conv;
+        return FDX_OK;
+    }
+
     fdx_status predict_impl(fdx_model* m, int batch, const float* const* in, bool in_on_device, const int64_t* in_dims,
-        const int* in_ranks, float* const* out, bool out_on_device, int64_t* out_dims, int* out_ranks)
+        const int* in_ranks, float* const* out, bool out_on_device, int64_t* out_dims, int* out_ranks, bool per_sample = false)
     {
         FDX_REQUIRE(m && in && in_dims && in_ranks && out, "predict: null argument");
         FDX_REQUIRE(batch > 0, "predict: batch must be positive");
@@ -2437,22 +2674,28 @@ namespace {
                     plan->out[kv.first] = kv.second;
             }
         } restore{ p, {} };
-        for (size_t i = 0; i < m->inputs.size(); ++i) {
-            FDX_REQUIRE(in[i], "predict: null input %zu", i);
-            const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(shapes[i]);
-            if (in_on_device && (reinterpret_cast<uintptr_t>(in[i]) & 15) == 0) {
-                float* own = p->out[m->inputs[i]];
-                for (size_t k = 0; k < p->out.size(); ++k)
-                    if (p->out[k] == own && own) {
-                        restore.saved.emplace_back((int)k, own);
-                        p->out[k] = const_cast<float*>(in[i]);
-                    }
-                continue;
+        int conv_done = -1;
+        if (!in_on_device) {
+            for (size_t i = 0; i < m->inputs.size() * (per_sample ? (size_t)batch : 1); ++i)
+                FDX_REQUIRE(in[i], "predict: null input %zu", i);
+            if ((st = stage_host_inputs(m, p, batch, in, per_sample, shapes, &conv_done)) != FDX_OK)
+                return st;
+        } else
+            for (size_t i = 0; i < m->inputs.size(); ++i) {
+                FDX_REQUIRE(in[i], "predict: null input %zu", i);
+                const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(shapes[i]);
+                if ((reinterpret_cast<uintptr_t>(in[i]) & 15) == 0) {
+                    float* own = p->out[m->inputs[i]];
+                    for (size_t k = 0; k < p->out.size(); ++k)
+                        if (p->out[k] == own && own) {
+                            restore.saved.emplace_back((int)k, own);
+                            p->out[k] = const_cast<float*>(in[i]);
+                        }
+                    continue;
+                }
+                FDX_HIP(hipMemcpyAsync(p->out[m->inputs[i]], in[i], bytes, hipMemcpyDeviceToDevice, stream()));
             }
-            FDX_HIP(hipMemcpyAsync(p->out[m->inputs[i]], in[i], bytes, in_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
-                stream()));
-        }
-        if ((st = execute(*m, *p)) != FDX_OK)
+        if ((st = execute(*m, *p, conv_done)) != FDX_OK)
             return st;
         for (size_t i = 0; i < m->outputs.size(); ++i) {
             FDX_REQUIRE(out[i], "predict: null output %zu", i);
@@ -2739,6 +2982,12 @@ extern "C" fdx_status fdx_model_predict(fdx_model* m, int batch, const float* co
     const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks)
 {
     return predict_impl(m, batch, in, false, in_dims, in_ranks, out, false, out_dims, out_ranks);
+}
+
+extern "C" fdx_status fdx_model_predict_samples(fdx_model* m, int batch, const float* const* in_samples, const int64_t* in_dims,
+    const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks)
+{
+    return predict_impl(m, batch, in_samples, false, in_dims, in_ranks, out, false, out_dims, out_ranks, true);
 }
 
 extern "C" fdx_status fdx_model_predict_dev(fdx_model* m, int batch, const float* const* in_dev, const int64_t* in_dims,

@@ -218,6 +218,16 @@ extern "C" fdx_status fdx_sync(void)
     return check_async_error();
 }
 
+extern "C" fdx_status fdx_dev_mem_info(size_t* free_bytes, size_t* total_bytes)
+{
+    FDX_REQUIRE(free_bytes && total_bytes, "dev_mem_info: null argument");
+    fdx_status st = ensure_init();
+    if (st != FDX_OK)
+        return st;
+    FDX_HIP(hipMemGetInfo(free_bytes, total_bytes));
+    return FDX_OK;
+}
+
 extern "C" fdx_status fdx_timer_start(void)
 {
     fdx_status st = ensure_init();

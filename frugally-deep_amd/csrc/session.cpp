@@ -332,7 +332,10 @@ bool build_fast_plan(fdx_session* s)
     auto alloc = [&](size_t floats) -> float* {
         const size_t bytes = (floats * sizeof(float) + 255) & ~(size_t)255;
         if (bytes > chunk_left) {
-            const size_t want = std::max(bytes, (size_t)256 << 20);
+            // 32 MiB first, doubling up to 256 MiB: a small model's session stays small, a large one still ends up in a
+            // handful of allocations
+            const size_t step = std::min((size_t)256 << 20, (size_t)32 << 20 << std::min<size_t>(s->owned.size(), 3));
+            const size_t want = std::max(bytes, step);
             void* p = nullptr;
             if (hipMalloc(&p, want) != hipSuccess)
                 return nullptr;

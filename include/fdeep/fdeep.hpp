@@ -496,8 +496,8 @@ public:
             if (!ok)
                 return predict_one_by_one(inputs_vec); // ragged shapes: still correct, one launch sequence each
         }
-        std::vector<float_vec> staged(n_in);
-        std::vector<const float*> in_ptrs(n_in);
+        // one pointer per sample and input: the library gathers them on their way to the GPU, nothing is concatenated here
+        std::vector<const float*> in_ptrs(n_in * batch);
         std::vector<std::int64_t> in_dims(5 * n_in);
         std::vector<int> in_ranks(n_in);
         for (std::size_t i = 0; i < n_in; ++i) {
@@ -506,14 +506,8 @@ public:
             for (int k = 0; k < 5; ++k)
                 in_dims[i * 5 + k] = static_cast<std::int64_t>(d[k]);
             in_ranks[i] = static_cast<int>(s.rank());
-            if (batch == 1) {
-                in_ptrs[i] = inputs_vec.front()[i].as_vector()->data();
-            } else {
-                staged[i].reserve(batch * s.volume());
-                for (const auto& ins : inputs_vec)
-                    staged[i].insert(staged[i].end(), ins[i].as_vector()->begin(), ins[i].as_vector()->end());
-                in_ptrs[i] = staged[i].data();
-            }
+            for (std::size_t b = 0; b < batch; ++b)
+                in_ptrs[i * batch + b] = inputs_vec[b][i].as_vector()->data();
         }
         std::vector<std::int64_t> out_dims(5 * n_out);
         std::vector<int> out_ranks(n_out);
@@ -529,7 +523,7 @@ public:
             outs[i].resize(batch * out_shapes.back().volume());
             out_ptrs[i] = outs[i].data();
         }
-        internal::check(fdx_model_predict(handle_.get(), static_cast<int>(batch), in_ptrs.data(), in_dims.data(),
+        internal::check(fdx_model_predict_samples(handle_.get(), static_cast<int>(batch), in_ptrs.data(), in_dims.data(),
             in_ranks.data(), out_ptrs.data(), nullptr, nullptr));
         std::vector<tensors> result(batch);
         for (std::size_t b = 0; b < batch; ++b)

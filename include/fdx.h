@@ -207,8 +207,11 @@ fdx_status fdx_dense_rows_f32(const float* x, int m, int k, const float* w_nk, c
  * workspace allocated on first use.  The call makes no hipMalloc / hipFree and uses no allocating library routine.
  * Needs fdx_init (or any earlier library call) to have run; limits: m <= 16, n <= 65536, k <= 32768 and
  * ceil(n / 16) * splits * 256 <= 1048576 floats (splits <= 8, chosen from k and n), otherwise FDX_ERR_INVALID with the
- * reason in fdx_last_error.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (other than
- * in order on the library's stream) race.
+ * reason in fdx_last_error; an activation other than NONE / RELU / GELU answers FDX_ERR_UNSUPPORTED as in every launcher
+ * with an epilogue.  One exception to "allocates nothing": while the per-kernel profile is switched on
+ * (fdx_profile_enable, fdx_debug.h) every launch records two HIP events, which the runtime creates on first use; leave the
+ * profile off where allocation is forbidden.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (other than in order on the library's stream) race.
  */
 fdx_status fdx_dense_rows_noalloc_f32(const float* x, int m, int k, const float* w_nk, const float* bias, int n,
     const float* residual, const fdx_act* act, float* out);
@@ -403,6 +406,11 @@ fdx_status fdx_model_io_shape(const fdx_model* m, int is_output, int index, int*
  * (others are copied first): such an input must stay unchanged until that work has completed.
  */
 fdx_status fdx_model_predict(fdx_model* m, int batch, const float* const* in, const int64_t* in_dims,
+    const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks);
+/* fdx_model_predict with every input given as `batch` pointers to single samples, in_samples[i * batch + b] = sample b of
+ * input i: the form predict_multi receives its tensors in (include/fdeep/model.hpp:28-42), so that a caller who holds
+ * one buffer per sample does not have to concatenate them first.  Host pointers; returns after the outputs are written. */
+fdx_status fdx_model_predict_samples(fdx_model* m, int batch, const float* const* in_samples, const int64_t* in_dims,
     const int* in_ranks, float* const* out, int64_t* out_dims, int* out_ranks);
 fdx_status fdx_model_predict_dev(fdx_model* m, int batch, const float* const* in_dev, const int64_t* in_dims,
     const int* in_ranks, float* const* out_dev, int64_t* out_dims, int* out_ranks);

@@ -13,13 +13,15 @@
 extern "C" {
 #endif
 
+/* free and total device memory in bytes (hipMemGetInfo): the tests use it to show that an entry point allocates nothing */
+fdx_status fdx_dev_mem_info(size_t* free_bytes, size_t* total_bytes);
 /* HIP-event stopwatch on the library stream: start, run work, stop returns milliseconds */
 fdx_status fdx_timer_start(void);
 fdx_status fdx_timer_stop(float* ms);
 /* Shader-clock probe, a measurement aid with no counterpart in the reference (the clock of the compute units falls
  * under load, and with it what the matrix cores can deliver): one lane on a stream of its own samples the shader
  * cycle counter against the constant-rate wall counter every period_us (10..100000) while other work runs, and ends
- * by itself after `samples` (2..65536) periods.  stop waits for it and returns the clock in GHz over the first
+ * by itself after `samples` (2..65536) periods, at most 10 s in all (samples x period_us <= 10^7).  stop waits for it and returns the clock in GHz over the first
  * window_ms milliseconds after the start: the mean, and the lowest and highest single period.  One probe at a time. */
 fdx_status fdx_clock_probe_start(int samples, int period_us);
 fdx_status fdx_clock_probe_stop(double window_ms, double* mean_ghz, double* min_ghz, double* max_ghz);

@@ -217,6 +217,43 @@ def test_predict_from_device_pointers(fdx, modelgen):
     assert np.array_equal(run(b.ptr.value + 4), want[1])
 
 
+@pytest.mark.parametrize("batch", [16, 13, 8])
+def test_large_host_inputs_are_staged_in_pieces(fdx, modelgen, batch):
+    """Host inputs of several MB travel through the library's pinned buffers in pieces of whole samples, and a network
+    that starts with a convolution runs it piece by piece behind the copy (include/fdeep/model.hpp:28-42: samples are
+    independent).  The result must be what the device-pointer call returns on the same data, for one contiguous block,
+    for one pointer per sample, for a batch that does not divide into equal pieces, and on a second call."""
+    say("staged host inputs, batch", batch)
+    spec = modelgen.resnet50(input_size=160, width=16, blocks=(1, 1, 1, 1), classes=10, random_bn=True)
+    model = fdx.Model(modelgen.dumps(spec))
+    r = np.random.default_rng(90 + batch)
+    x = r.uniform(0, 1, (batch, 160, 160, 3)).astype(np.float32)  # 4.9 MB at batch 16, 2.4 MB at batch 8 (the plain copy)
+    d_x = fdx.DevBuf.from_host(x)
+    d_out = fdx.DevBuf(4 * batch * 10)
+    model.predict_dev(batch, [d_x], [(160, 160, 3)], [d_out])
+    fdx.sync()
+    want = d_out.to_host((batch, 10))
+    for _ in range(2):
+        got = model.predict([x])[0]
+        assert rel(got, want) <= 3e-6, np.abs(got - want).max()
+    scattered = [[np.array(x[b])] for b in range(batch)]  # one allocation per sample
+    got = model.predict_samples(scattered)[0]
+    assert rel(got, want) <= 3e-6
+    # a network whose first layer is not a convolution of its own launch: pieces are copied, nothing runs behind them
+    b2 = modelgen.Builder("two_in", 5)
+    u = b2.input((256, 256, 4), "u")
+    v = b2.input((256, 256, 4), "v")
+    y = b2.add([u, v], "sum")
+    y = b2.conv2d(y, 8, 3, "c", padding="same", activation="relu")
+    m2 = fdx.Model(modelgen.dumps(b2.finish([b2.gap(y, "gap")])))
+    a, c = (r.standard_normal((batch, 256, 256, 4)).astype(np.float32) for _ in range(2))
+    d_a, d_c, d_o = fdx.DevBuf.from_host(a), fdx.DevBuf.from_host(c), fdx.DevBuf(4 * batch * 8)
+    m2.predict_dev(batch, [d_a, d_c], [(256, 256, 4)] * 2, [d_o])
+    fdx.sync()
+    assert rel(m2.predict([a, c])[0], d_o.to_host((batch, 8))) <= 3e-6
+    assert rel(m2.predict_samples([[a[b], c[b]] for b in range(batch)])[0], d_o.to_host((batch, 8))) <= 3e-6
+
+
 def test_input_shape_errors(fdx, modelgen):
     say("shape errors")
     model = fdx.Model(modelgen.dumps(modelgen.small_cnn()))
