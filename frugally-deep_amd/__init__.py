@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libfdx.so")
+# FDX_LIBRARY names another build of the same library (for comparing two builds in one session on one machine)
+LIB_PATH = os.environ.get("FDX_LIBRARY") or os.path.join(_HERE, "libfdx.so")
 
 c_float_p = ctypes.POINTER(ctypes.c_float)
 c_void_pp = ctypes.POINTER(ctypes.c_void_p)

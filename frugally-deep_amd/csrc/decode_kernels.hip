@@ -46,7 +46,8 @@ struct SkinnyShared {
 };
 
 // The work of workgroup (bx, by) of a (gx, gy) grid.
-template <int CHUNK, bool SINGLE>
+// EMB: the instantiation that knows the embedding prologue (SkinnyParams::emb_x / emb_res); the others carry none of its code
+template <int CHUNK, bool SINGLE, bool EMB = false>
 __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, int by, int gx, int gy, SkinnyShared& sh)
 {
     float* red = sh.red;
@@ -73,7 +74,22 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
     const gptr<const float> Wg = as_global(p.W);
     const gptr<const float> wrow = Wg + (int64_t)(n_ok ? n : 0) * p.ldw;
     const int spw = per_wave / 16; // slabs per wave in the packed layout
-    const gptr<const float> xrow = as_global(p.X) + (int64_t)(m_ok ? i : 0) * p.ldx;
+    const bool emb = EMB && p.emb_x != 0;
+    const bool emb_res = EMB && p.emb_res != 0;
+    // embedding rows of this lane's activation row: token id (a float in the model's input) and position, both checked
+    const int emb_pos = (emb || emb_res) ? *as_global(p.len_dev) : 0;
+    auto emb_row = [&](int row, bool& ok) -> int64_t {
+        const float f = as_global(p.emb_ids)[row];
+        const int64_t id = (f >= 0.f && f < 9.0e18f) ? (int64_t)f : -1;
+        ok = id >= 0 && id < p.emb_a_rows && emb_pos < p.emb_b_rows;
+        return ok ? id : 0;
+    };
+    bool emb_ok = true;
+    const int64_t emb_id = emb && m_ok ? emb_row(i, emb_ok) : 0;
+    if (emb && m_ok && !emb_ok && p.emb_err && bx == 0 && by == 0 && wave == 0 && kq == 0)
+        atomicExch(p.emb_err, 1);
+    const gptr<const float> xrow = emb ? as_global(p.emb_a) + emb_id * K : as_global(p.X) + (int64_t)(m_ok ? i : 0) * p.ldx;
+    const gptr<const float> xrow_b = emb ? as_global(p.emb_b) + (int64_t)(emb_ok ? emb_pos : 0) * K : xrow;
     // two named register sets (indexing one array with a run-time buffer number would push it to scratch)
     f32x4 w0[CHUNK], a0[CHUNK];
     auto load_chunk = [&](f32x4 (&wreg)[CHUNK], f32x4 (&areg)[CHUNK], int s0) {
@@ -85,11 +101,16 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
             if (p.packed) {
                 // pre-packed operand: this wave's slab is one contiguous 1 KB run, zeros baked in
                 if (s0 + s < spw)
-                    wv = reinterpret_cast<gptr<const f32x4>>(Wg)[(((int64_t)bx * SK_WAVES + wave) * spw + (s0 + s)) * 64 + lane];
+                    wv = __builtin_nontemporal_load(reinterpret_cast<gptr<const f32x4>>(Wg) + (((int64_t)bx * SK_WAVES + wave) * spw + (s0 + s)) * 64 + lane);
             } else if (n_ok && k_ok)
-                wv = *reinterpret_cast<gptr<const f32x4>>(wrow + k);
-            if (m_ok && k_ok)
+                wv = __builtin_nontemporal_load(reinterpret_cast<gptr<const f32x4>>(wrow + k)); // every weight is used once per launch
+            if (m_ok && k_ok) {
                 av = *reinterpret_cast<gptr<const f32x4>>(xrow + k);
+                if (emb) {
+                    const f32x4 bv = *reinterpret_cast<gptr<const f32x4>>(xrow_b + k);
+                    av = emb_ok ? av + bv : f32x4 { 0.f, 0.f, 0.f, 0.f };
+                }
+            }
             wreg[s] = wv;
             areg[s] = av;
         }
@@ -106,7 +127,11 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
     if (e_ok) {
         if (p.bias)
             e_bias = as_global(p.bias)[ecol];
-        if (p.residual)
+        if (emb_res) {
+            bool ok = true;
+            const int64_t id = emb_row(em, ok);
+            e_res = ok ? as_global(p.emb_a)[id * p.N + ecol] + as_global(p.emb_b)[(int64_t)emb_pos * p.N + ecol] : 0.f;
+        } else if (p.residual)
             e_res = as_global(p.residual)[(int64_t)em * p.ldr + ecol];
         if (p.ln)
             e_wsum = as_global(p.w_rowsum)[ecol];
@@ -295,11 +320,11 @@ __device__ __forceinline__ void skinny_gemm_body(const SkinnyParams& p, int bx, 
     }
 }
 
-template <int CHUNK, bool SINGLE>
+template <int CHUNK, bool SINGLE, bool EMB = false>
 __global__ __launch_bounds__(512) void skinny_gemm_kernel(SkinnyParams p)
 {
     __shared__ SkinnyShared sh;
-    skinny_gemm_body<CHUNK, SINGLE>(p, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, sh);
+    skinny_gemm_body<CHUNK, SINGLE, EMB>(p, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, sh);
 }
 
 
@@ -314,7 +339,10 @@ __device__ __forceinline__ unsigned long long pack_max(float v, int col);
 template <int CHUNK>
 __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int tiles)
 {
-    __shared__ float red[SK_WAVES * 256];
+    // two reduction buffers taken in turn: a column group's partial tiles are summed out of one while the next group's go
+    // into the other, so one barrier per group is enough (the barrier of group g + 1 orders every read of group g's
+    // buffer before the writes of group g + 2)
+    __shared__ float red_both[2][SK_WAVES * 256];
     __shared__ float stat[SK_WAVES * 16];
     __shared__ float row_mean[16], row_rstd[16];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -346,9 +374,9 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
             f32x4 wv = { 0.f, 0.f, 0.f, 0.f };
             if (p.packed) {
                 if (s < spw)
-                    wv = reinterpret_cast<const f32x4*>(p.W)[(((int64_t)tile * SK_WAVES + wave) * spw + s) * 64 + lane];
+                    wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p.W) + (((int64_t)tile * SK_WAVES + wave) * spw + s) * 64 + lane);
             } else if (n_ok && s < slabs && k < k_end)
-                wv = *reinterpret_cast<const f32x4*>(wrow + k);
+                wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow + k));
             wreg[s] = wv;
         }
     };
@@ -372,9 +400,9 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
     };
 
     int tile = blockIdx.x;
-    // short rows leave room for three register sets: the weights of the next TWO column groups are in flight while one
-    // is multiplied; longer rows keep one group ahead
-    constexpr bool AHEAD2 = CHUNK <= 6;
+    // one column group ahead: with the weights on non-temporal loads a second group in flight no longer pays (measured on
+    // the 768 -> 50257 shape: 28.5 us one ahead, 29.9 us two ahead, 32.9 us before either change)
+    constexpr bool AHEAD2 = false;
     f32x4 w0[CHUNK], w1[CHUNK], w2[AHEAD2 ? CHUNK : 1];
     load_w(w0, tile);
     Epi e0 = load_epi(tile);
@@ -433,7 +461,10 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
 
     const int64_t len_shift = p.seg[0].len_stride ? (int64_t)(*p.len_dev) : 0; // only read when a segment asks for it
     unsigned long long best = 0ull; // packed maximum of this thread's output elements (one row, one column per group)
+    int turn = 0;
     for (; tile < tiles; tile += gridDim.x) {
+        float* red = red_both[turn];
+        turn ^= 1;
         const int next = tile + (AHEAD2 ? 2 : 1) * gridDim.x;
         Epi e2 { 0.f, 0.f, 0.f };
         if (next < tiles) {
@@ -475,7 +506,6 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
             const int64_t shift = sg.len_stride ? (sgi == 0 ? len_shift : (int64_t)(*p.len_dev)) * sg.len_stride : 0;
             sg.ptr[shift + (int64_t)em * sg.ld + (col - sg.col_begin)] = v;
         }
-        __syncthreads(); // the reduction buffer is rewritten by the next column group
 #pragma unroll
         for (int s = 0; s < CHUNK; ++s) {
             w0[s] = w1[s];
@@ -853,7 +883,9 @@ static int skinny_ksplit(int K, int tiles)
 
 fdx_status skinny_gemm_launch(const SkinnyParams& p)
 {
-    FDX_REQUIRE(p.X && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0, "dense_rows: bad arguments");
+    FDX_REQUIRE((p.X || p.emb_x) && p.W && p.M > 0 && p.M <= 16 && p.N > 0 && p.K > 0, "dense_rows: bad arguments");
+    FDX_REQUIRE(!(p.emb_x || p.emb_res) || (p.emb_ids && p.emb_a && p.emb_b && p.len_dev && p.emb_a_rows > 0 && p.emb_b_rows > 0),
+        "dense_rows: the embedding prologue needs ids, both tables and the position counter");
     FDX_REQUIRE(p.K % 4 == 0 && p.ldx % 4 == 0 && p.ldw % 4 == 0, "dense_rows: K and row strides must be multiples of 4");
     FDX_REQUIRE(p.n_seg >= 1 && p.n_seg <= 3, "dense_rows: 1 to 3 output segments");
     FDX_REQUIRE(!p.ln || (p.K <= SK_WAVES * SK_CHUNK * 16 && p.w_rowsum), "dense_rows: the LayerNorm prologue needs K <= %d",
@@ -890,6 +922,9 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
     // many column groups and a short K: resident workgroups stride through the groups instead of one group each
     const int wide_grid = skinny_wide_grid(p);
     FDX_REQUIRE(!p.amax_parts || (wide_grid > 0 && ksplit == 1), "dense_rows: partial arg-max cells need the wide-output kernel");
+    FDX_REQUIRE(!(p.emb_x || p.emb_res) || (wide_grid == 0 && ksplit == 1 && per_wg <= SK_WAVES * 6 * 16),
+        "dense_rows: the embedding prologue needs K <= %d and runs neither with the wide-output kernel nor with K split across workgroups",
+        SK_WAVES * 6 * 16);
     if (ksplit == 1 && wide_grid > 0) {
         if (per_wg <= SK_WAVES * 6 * 16)
             hipLaunchKernelGGL((skinny_wide_kernel<6>), dim3((unsigned)wide_grid), dim3(512), 0, stream(), q, tiles);
@@ -900,7 +935,9 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p)
         return FDX_OK;
     }
     // every load of a workgroup in flight at once when its K range fits 8 (or 24) slabs per wave
-    if (per_wg <= SK_WAVES * 6 * 16) // K = 768 and the halves / quarters of longer rows: no empty register slots
+    if (p.emb_x || p.emb_res)
+        hipLaunchKernelGGL((skinny_gemm_kernel<6, true, true>), grid, dim3(512), 0, stream(), q);
+    else if (per_wg <= SK_WAVES * 6 * 16) // K = 768 and the halves / quarters of longer rows: no empty register slots
         hipLaunchKernelGGL((skinny_gemm_kernel<6, true>), grid, dim3(512), 0, stream(), q);
     else if (per_wg <= SK_WAVES * SK_CHUNK * 16)
         hipLaunchKernelGGL((skinny_gemm_kernel<SK_CHUNK, true>), grid, dim3(512), 0, stream(), q);

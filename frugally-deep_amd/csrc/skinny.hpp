@@ -41,6 +41,17 @@ struct SkinnyParams {
     // the flags name another XCD.
     int local_split;
     int* err;
+    // Optional: with emb_x != 0 the activation rows are not read from X but formed on the way in as the sum of two
+    // embedding rows, row i = emb_a[(int)emb_ids[i]][:] + emb_b[*len_dev][:] (token + position embedding of the token a
+    // decode step starts from, layers/embedding_layer.hpp:38-58 twice and an Add); with emb_res != 0 the residual operand
+    // is that sum (residual is then ignored; the tables' depth must equal N).  An id outside [0, emb_a_rows) or a position outside [0, emb_b_rows) sets *emb_err to 1
+    // and contributes zeros.  Not with the wide-output kernel and not with K split across workgroups.
+    const float* emb_ids;
+    const float* emb_a;
+    const float* emb_b;
+    int emb_a_rows, emb_b_rows;
+    int emb_x, emb_res;
+    int* emb_err;
     // optional, wide-output launches only (skinny_wide_grid(p) > 0): every workgroup leaves the packed (value, column)
     // maximum of each row over the columns it produced in amax_parts[workgroup][16]; argmax_parts_launch picks the winner
     unsigned long long* amax_parts;

@@ -55,6 +55,10 @@ fdx_status fdx_profile_get_executed(int index, double* executed_flops);
  *     wherever it covers the shape.
  */
 fdx_status fdx_debug_force_tile(int cfg);
+/* decode sessions created from now on: 1 = the token + position embedding launch of a step is folded into the two GEMMs
+ * that read its result (measured slower than the launch it saves, hence not the default), 0 = never, -1 = as the
+ * environment says (FDX_DECODE_EMBED_FOLD=1) */
+fdx_status fdx_debug_decode_embed_fold(int mode);
 fdx_status fdx_debug_persist_cap(int workgroups);
 fdx_status fdx_debug_force_strips(int strips);
 fdx_status fdx_debug_force_dw_fusion(int mode);

@@ -208,3 +208,29 @@ def test_attention_with_output_projection_in_one_launch(fdx, oracle, modelgen, m
         seq = np.concatenate([prompts[0], first[:1], want_tokens[:5, 0]]).astype(np.float32)
         want = oracle_logits(ref, seq)[-1]
         assert rel(lb[0], want) <= TOL
+
+
+def test_embedding_folded_into_its_readers_gives_the_same_tokens(fdx, modelgen):
+    """The opt-in form of the decode step in which the first projection GEMM and the first residual operand form the
+    token + position rows themselves (one launch fewer): same sums in the same order, so logits and tokens are
+    bit-identical to the default step."""
+    print("decode step with the embedding folded into its readers", flush=True)
+    js = modelgen.dumps(modelgen.gpt2(seed=61, layers=2, d_model=768, heads=12, vocab=50257, max_pos=128, bias_std=0.1,
+                                      random_affine=True))
+    model = fdx.Model(js, verify=False)
+    B, P, N = 16, 24, 12
+    prompts = np.random.default_rng(62).integers(0, 50257, (B, P))
+    outs = []
+    for mode in (0, 1):
+        fdx.check(fdx.lib.fdx_debug_decode_embed_fold(mode))
+        try:
+            sess = fdx.Session(model, B, 64)
+        finally:
+            fdx.check(fdx.lib.fdx_debug_decode_embed_fold(-1))
+        _, first = sess.prefill(prompts)
+        tokens, logits = sess.decode_greedy(first, N)
+        step_logits, step_next = sess.decode_step(tokens[-1])
+        outs.append((tokens, logits, step_logits, step_next))
+        sess.close()
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a, b)
