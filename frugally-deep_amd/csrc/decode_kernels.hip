@@ -376,7 +376,7 @@ __global__ __launch_bounds__(512, 4) void skinny_wide_kernel(SkinnyParams p, int
                 if (s < spw)
                     wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p.W) + (((int64_t)tile * SK_WAVES + wave) * spw + s) * 64 + lane);
             } else if (n_ok && s < slabs && k < k_end)
-                wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow + k));
+                wv = *reinterpret_cast<const f32x4*>(wrow + k); // 64-byte pieces of a row: the other half of the line is the next slab's
             wreg[s] = wv;
         }
     };
