@@ -254,6 +254,38 @@ def test_large_host_inputs_are_staged_in_pieces(fdx, modelgen, batch):
     assert rel(m2.predict_samples([[a[b], c[b]] for b in range(batch)])[0], d_o.to_host((batch, 8))) <= 3e-6
 
 
+def test_large_host_inputs_from_several_threads(fdx, modelgen):
+    """predict is callable from many host threads (FAQ.md:103-114); with inputs large enough for the pinned pieces the
+    threads take turns at the library's staging buffers.  Three threads, two models, three calls each: every result
+    equals the serial one."""
+    import threading
+    say("staged host inputs from three threads")
+    spec = modelgen.resnet50(input_size=160, width=16, blocks=(1, 1, 1, 1), classes=10, random_bn=True)
+    models = [fdx.Model(modelgen.dumps(spec)), fdx.Model(modelgen.dumps(spec))]
+    r = np.random.default_rng(95)
+    xs = [r.uniform(0, 1, (16 + 4 * i, 160, 160, 3)).astype(np.float32) for i in range(3)]
+    want = [models[i % 2].predict([xs[i]])[0] for i in range(3)]
+    got = [[None] * 3 for _ in range(3)]
+    errors = []
+
+    def work(i):
+        try:
+            for k in range(3):
+                got[i][k] = models[i % 2].predict([xs[i]])[0]
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(3):
+        for k in range(3):
+            assert np.array_equal(got[i][k], want[i]), (i, k)
+
+
 def test_input_shape_errors(fdx, modelgen):
     say("shape errors")
     model = fdx.Model(modelgen.dumps(modelgen.small_cnn()))
