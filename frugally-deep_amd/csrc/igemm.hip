@@ -775,15 +775,45 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
                 [&] { pw_stream_launch(p, a_bytes, b_bytes, s); });
             settle();
         }
+        static const bool closed_cuts = [] { const char* e = std::getenv("FDX_CLOSED_SPLIT"); return !(e && e[0] == '0'); }();
         if (cfg >= 0) {
+        } else if (stream_ok && p.K <= 32 && p.N <= 160 && p.M >= 65536) {
+            // very short rows over a long map (MobileNetV2's first expansions): the row-streaming kernel
+            cfg = kStreamCfg;
         } else if (fast_ok && p.N >= 64) {
             // what the timing runs pick most often: the 64 x 64 tile at four or five workgroups per CU, with the
             // 32-float slab where K is long enough for it; the 128 x 128 tile only for problems that are large in
-            // every dimension
+            // every dimension; the 128 x 64 tile with the short slab for wide outputs from short rows, where the
+            // stores dominate
             if (p.K >= 1024 && p.N % 128 == 0 && blocks(128, 128) >= 2048)
                 cfg = unit % 32 == 0 ? 13 : 10;
+            else if (p.K <= 96 && p.N >= 128 && blocks(128, 64) >= 1024)
+                cfg = 11;
             else
                 cfg = (unit % 32 == 0 && p.K >= 128) ? 15 : 12;
+            // Fewer 64 x 64 tiles than one round of resident workgroups (four per CU) and a long K: the chip is filled
+            // by cutting K instead.  Below one tile per CU every tile is cut into equal K ranges, about two workgroups
+            // per CU in total (a Dense with few rows: 2.8 times faster at 64 x 1000 x 2048); from there up to one
+            // round the stream-K form spreads the slabs of all tiles evenly over the resident workgroups (10-12 %
+            // faster on ResNet50's 14 x 14 and 7 x 7 1x1 layers).  Both forms add their partial tiles in a fixed order.
+            if (closed_cuts && (cfg == 15 || cfg == 12)) {
+                const int64_t t64 = blocks(64, 64);
+                const int slabs = p.K / (cfg == 15 ? 32 : 16);
+                if (t64 < 256 && p.K >= 512) {
+                    int want = (int)std::min<int64_t>(8, (512 + t64 - 1) / t64);
+                    while (want >= 2 && slabs < 4 * want)
+                        --want;
+                    if (want >= 2) {
+                        splits = want;
+                        mode = 0;
+                    }
+                } else if (t64 < 1024 && p.K >= 1024 && cfg == 15) {
+                    splits = 0;
+                    mode = 2;
+                }
+                if (splits != 1)
+                    settle(); // the cut needs its workspace
+            }
         } else if (p.N <= 32)
             cfg = 2;
         else if (p.N <= 64)

@@ -143,9 +143,11 @@ def test_mobilenet_v2_full_size_fusion_invariance(fdx, oracle, modelgen):
             outs.append(fdx.Model(js, verify=False).predict([x]))
     finally:
         fdx.check(fdx.lib.fdx_debug_force_dw_fusion(-1))
+    # the forms add the same products in different orders (one launch keeps a block's sums in registers, separate 1x1
+    # launches cut a long K into ranges on the small maps): a fifth of the bar against the oracle
     for other in outs[1:]:
         for a, b in zip(outs[0], other):
-            assert rel(a, b) <= 1e-5
+            assert rel(a, b) <= TOL / 5
     want = oracle.OracleModel(js).predict([x[0]])
     for g, w in zip(outs[0], want):
         assert rel(g[0], w) <= TOL
