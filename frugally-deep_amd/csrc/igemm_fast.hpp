@@ -278,6 +278,34 @@ void igemm_fast_kernel(GemmParams p)
         float* __restrict__ C = p.C + c_off;
         const float* __restrict__ R = p.residual ? p.residual + c_off : nullptr;
         const int su_done = cur_su, tile_done = cur_tile;
+        // What the epilogue reads from memory -- the bias and the residual rows of the first 32-row band -- is requested
+        // before the next tile's operands: loads complete in the order of their issue, so behind those operands their
+        // first use would wait for the whole prefetch.
+        constexpr int LPR = WTN / 4;  // lanes per scratch row
+        constexpr int RPS = 64 / LPR; // rows per store pass
+        const int srow = lane / LPR, scol = (lane % LPR) * 4;
+        const int n = en0 + wn * WTN + scol;
+        const bool n_ok = n < p.N; // N is a multiple of 4 on this path
+        f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
+        f32x4 rr[32 / RPS];
+        auto request_residual = [&](int i) {
+#pragma unroll
+            for (int ps = 0; ps < 32 / RPS; ++ps) {
+                const int m = em0 + wm * WTM + i * 32 + ps * RPS + srow;
+                rr[ps] = f32x4 { 0.f, 0.f, 0.f, 0.f };
+                if (R && m < p.M && n_ok)
+                    rr[ps] = *reinterpret_cast<const f32x4*>(R + (int64_t)m * p.ldc + n);
+            }
+        };
+        auto request_epilogue = [&]() {
+            if (p.bias && n_ok)
+                bias4 = *reinterpret_cast<const f32x4*>(p.bias + n);
+            request_residual(0);
+        };
+        // (the split variants hold partial tiles in registers across the exchange below; there the requests wait
+        // until the exchange is over)
+        if (!SPLIT)
+            request_epilogue();
         tile += unit_step;
         const bool more = tile < unit_end;
         if (more) {
@@ -366,26 +394,14 @@ void igemm_fast_kernel(GemmParams p)
 
         // ---- epilogue: accumulators -> per-wave LDS scratch [32][WTN] -> 16-byte row accesses
         float* scratch = smem + wave * 32 * OSTRIDE;
-        constexpr int LPR = WTN / 4;  // lanes per scratch row
-        constexpr int RPS = 64 / LPR; // rows per store pass
-        const int srow = lane / LPR, scol = (lane % LPR) * 4;
-        const int n = en0 + wn * WTN + scol;
-        const bool n_ok = n < p.N; // N is a multiple of 4 on this path
-        f32x4 bias4 = { 0.f, 0.f, 0.f, 0.f };
-        if (p.bias && n_ok)
-            bias4 = *reinterpret_cast<const f32x4*>(p.bias + n);
+        if (SPLIT)
+            request_epilogue();
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            // the residual rows of this 32-row band are requested before the accumulators go through LDS, so their
+            // the residual rows of a later 32-row band are requested before the accumulators go through LDS, so their
             // latency is covered by the transposition instead of stalling every store
-            f32x4 rr[32 / RPS];
-#pragma unroll
-            for (int ps = 0; ps < 32 / RPS; ++ps) {
-                const int m = em0 + wm * WTM + i * 32 + ps * RPS + srow;
-                rr[ps] = f32x4 { 0.f, 0.f, 0.f, 0.f };
-                if (R && m < p.M && n_ok)
-                    rr[ps] = *reinterpret_cast<const f32x4*>(R + (int64_t)m * p.ldc + n);
-            }
+            if (i > 0)
+                request_residual(i);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
