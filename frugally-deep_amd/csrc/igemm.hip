@@ -274,6 +274,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void igemm_kernel(GemmParam
 // ------------------------------------------------------------------ dispatch
 
 static int g_forced_tile = -1; // tests force a tile configuration through fdx_debug_force_tile
+static bool g_dual_one_launch = true; // tests run a two-input convolution as two launches through fdx_debug_dual_conv
 
 template <int BM, int BN, int WM, int WN>
 static void launch_cfg(const GemmParams& p, int a_mode, int b_vec, int batch, hipStream_t s)
@@ -466,6 +467,8 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
                 ok = launch_split(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, true>, tiles, splits, mode, cfg, q, s); \
         } else if (conv)                                                                                         \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, true>, tiles, q, s, 256, BM_, BN_);         \
+        else if (q.A2)                                                                                           \
+            launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false, false, false, true>, tiles, q, s, 256, BM_, BN_); \
         else                                                                                                     \
             launch_persistent(igemm_fast_kernel<BM_, BN_, 2, 2, BK_, false>, tiles, q, s, 256, BM_, BN_);        \
     }
@@ -760,7 +763,30 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
         }
     };
-    if (cfg < 0) {
+    if (p.A2) {
+        // two-source rows: whole tiles of the four-wave fast kernel only, nothing timed
+        const int64_t a2_bytes = (int64_t)(p.OH > 0 && p.OW > 0 ? p.M / (p.OH * p.OW) : 0) * p.H2 * p.W2 * p.C2 * 4;
+        const bool dual_ok = !conv && batch == 1 && fast_ok && p.a_valid_k == 0 && aligned16(p.A2) && p.C2 % 4 == 0 && p.K1 > 0
+            && p.K1 % 16 == 0 && p.K > p.K1 && (p.K - p.K1) % 16 == 0 && p.K - p.K1 <= p.C2 && a2_bytes > 0 && a2_bytes < (1LL << 31)
+            && p.s2y > 0 && p.s2x > 0 && (int64_t)(p.OH - 1) * p.s2y < p.H2 && (int64_t)(p.OW - 1) * p.s2x < p.W2
+            && p.M == (p.M / (p.OH * p.OW)) * p.OH * p.OW;
+        if (!dual_ok) {
+            set_error("igemm: this two-source problem needs the fast path");
+            return FDX_ERR_UNSUPPORTED;
+        }
+        p.a2_records = (uint32_t)a2_bytes;
+        const bool slab32 = p.K % 32 == 0 && p.K1 % 32 == 0;
+        if (cfg < 10 || cfg > 15 || (cfg >= 13 && !slab32))
+            cfg = -1;
+        splits = 1;
+        mode = 0;
+        if (cfg < 0) {
+            if (p.K >= 1024 && p.N % 128 == 0 && blocks(128, 128) >= 2048)
+                cfg = slab32 ? 13 : 10;
+            else
+                cfg = (slab32 && p.K >= 128) ? 15 : 12;
+        }
+    } else if (cfg < 0) {
         if (fast_ok && p.N >= 16 && 2.0 * p.M * (double)p.N * p.K * batch >= 2e8) {
             GemmParams q = p;
             q.A = p.A - a_shift;
@@ -960,6 +986,12 @@ extern "C" fdx_status fdx_debug_force_tile(int cfg)
     return FDX_OK;
 }
 
+extern "C" fdx_status fdx_debug_dual_conv(int one_launch)
+{
+    fdx::g_dual_one_launch = one_launch != 0;
+    return FDX_OK;
+}
+
 // tests: caps the persistent grid (0 = as many workgroups as are resident on the chip)
 extern "C" fdx_status fdx_debug_force_strips(int strips)
 {
@@ -1029,6 +1061,59 @@ fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const f
     p.inner = 1;
     p.a_valid_k = cin;
     return run_igemm(p, false, 1, "conv1x1_gemm_f32", 2.0 * (double)rows * cout * cin);
+}
+} // namespace fdx
+
+namespace fdx {
+// The sum of two pointwise convolutions with one epilogue,
+//     out[img][y][x][:] = act(W[:, :c1] . in1[img][y][x][:] + W[:, c1:] . in2[img][y * s2y][x * s2x][:] + bias),
+// as one GEMM over the concatenated channels (a residual block whose shortcut branch is a 1x1 convolution, strided or
+// not: Add(Conv2D(a), Conv2D(b)) of layers/add_layer.hpp:20-29 over layers/conv_2d_layer.hpp:52-56).  w_cat is
+// [cout][c1 + c2].  Where the fast path does not apply the two convolutions run one after the other on the same filter
+// array, the second adding to the first's result.
+fdx_status conv1x1_dual_launch(const float* in1, int n, int oh, int ow, int c1, const float* in2, int h2, int w2, int c2, int s2y, int s2x,
+    const float* w_cat, const float* bias, int cout, const fdx_act* act, float* out)
+{
+    FDX_REQUIRE(in1 && in2 && w_cat && out && n > 0 && oh > 0 && ow > 0 && c1 > 0 && c2 > 0 && h2 > 0 && w2 > 0 && s2y > 0 && s2x > 0
+            && cout > 0 && (int64_t)(oh - 1) * s2y < h2 && (int64_t)(ow - 1) * s2x < w2,
+        "conv1x1_dual: bad arguments");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    FDX_REQUIRE((int64_t)n * oh * ow < (1LL << 31) && (int64_t)h2 * w2 * c2 < (1LL << 31), "conv1x1_dual: dimension overflow");
+    const bool fused = g_dual_one_launch;
+    GemmParams p {};
+    p.A = in1; p.B = w_cat; p.C = out; p.bias = bias; p.residual = nullptr;
+    p.M = n * oh * ow; p.N = cout; p.K = c1 + c2;
+    p.lda = c1; p.ldb = p.K; p.ldc = cout;
+    p.alpha = 1.f; p.bias_per_row = 0; p.act = make_act(act);
+    p.inner = 1;
+    p.OH = oh; p.OW = ow;
+    p.A2 = in2; p.K1 = c1; p.H2 = h2; p.W2 = w2; p.C2 = c2; p.s2y = s2y; p.s2x = s2x;
+    if (fused) {
+        const fdx_status st = run_igemm(p, false, 1, "conv1x1_gemm_f32");
+        if (st != FDX_ERR_UNSUPPORTED)
+            return st;
+    }
+    // one after the other: the strided one first, without bias and activation, then the other on top of it
+    GemmParams a {};
+    a.A = in2; a.B = w_cat + c1; a.C = out;
+    a.M = p.M; a.N = cout; a.K = c2; a.lda = 0; a.ldb = p.K; a.ldc = cout;
+    a.alpha = 1.f; a.act = make_act(nullptr);
+    a.inner = 1;
+    a.H = h2; a.W = w2; a.Cin = c2; a.kh = 1; a.kw = 1; a.sy = s2y; a.sx = s2x; a.dy = 1; a.dx = 1; a.OH = oh; a.OW = ow;
+    fdx_status st;
+    if (s2y == 1 && s2x == 1 && h2 == oh && w2 == ow) {
+        a.lda = c2;
+        st = run_igemm(a, false, 1, "conv1x1_gemm_f32");
+    } else {
+        st = run_igemm(a, true, 1, "conv_igemm_f32");
+    }
+    if (st != FDX_OK)
+        return st;
+    GemmParams b = p;
+    b.A2 = nullptr;
+    b.K = c1;
+    b.residual = out;
+    return run_igemm(b, false, 1, "conv1x1_gemm_f32");
 }
 } // namespace fdx
 

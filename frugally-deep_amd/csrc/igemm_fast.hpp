@@ -31,7 +31,11 @@
 //    and their workspace slots computed from the cut points.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false, bool STREAMK = false>
+//  * DUAL (GEMM form, whole tiles only): the rows of A come from two tensors -- the first K1 columns from A with row
+//    stride lda, the other K - K1 from A2, whose row for output pixel (image, y, x) is pixel (y * s2y, x * s2x) of an
+//    [H2][W2][C2] map.  That is the sum of two pointwise convolutions as one GEMM over the concatenated channels
+//    (a residual block whose shortcut is a 1x1 convolution: the shortcut's output is never written or read back).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false, bool STREAMK = false, bool DUAL = false>
 // (the second bound asks for two waves per SIMD where the split variant of the largest four-wave tile would otherwise
 // settle for one: its reduction holds the accumulators in ordinary registers next to the prefetched operands)
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (SPLIT && WAVES_M * WAVES_N == 4 && BM * BN >= 128 * 128) ? 2 : 1)
@@ -39,6 +43,7 @@ void igemm_fast_kernel(GemmParams p)
 {
     constexpr int NT = 64 * WAVES_M * WAVES_N;
     static_assert(NT == 256 || NT == 512, "four or eight waves");
+    static_assert(!DUAL || (!CONV && !SPLIT), "the two-source form is a whole-tile GEMM");
     constexpr int STRIDE = BKT + 4;
     constexpr int CPR = BKT / 4;  // 16-byte chunks per tile row
     constexpr int RPP = NT / CPR; // tile rows filled per loader pass
@@ -89,8 +94,11 @@ void igemm_fast_kernel(GemmParams p)
 
     // ---- per-tile loader state
     uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+    uint32_t a2_voff[DUAL ? A_LOADS : 1];
     uint64_t a_mask[A_LOADS];
     __amdgpu_buffer_rsrc_t srd_a, srd_b;
+    const __amdgpu_buffer_rsrc_t srd_a2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(DUAL ? p.A2 : p.A), 0,
+        DUAL ? (int)p.a2_records : 0, 0x00020000);
     int tap, fx, fy, c0, soff_a, soff_b;
     f32x4 ra[A_LOADS], rb[B_LOADS];
     int kt_n = KT; // slabs of the current unit
@@ -165,6 +173,14 @@ void igemm_fast_kernel(GemmParams p)
                     a_mask[i] = ~0ull;
                 }
             }
+            if (DUAL) {
+                a2_voff[i] = OOB;
+                if (m < p.M) {
+                    const int img = m / (p.OH * p.OW), rm = m - img * (p.OH * p.OW);
+                    const int oy = rm / p.OW, ox = rm - oy * p.OW;
+                    a2_voff[i] = (uint32_t)(((img * p.H2 + oy * p.s2y) * p.W2 + ox * p.s2x) * p.C2) * 4u + kq * 16;
+                }
+            }
         }
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
@@ -188,10 +204,16 @@ void igemm_fast_kernel(GemmParams p)
         }
     };
     auto load_tiles = [&]() {
+        if (DUAL && soff_b >= p.K1 * 4) { // the slab lies in the second tensor's columns (uniform over the workgroup)
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            const uint32_t vo = CONV ? (((a_mask[i] >> tap) & 1) ? a_voff[i] : OOB) : a_voff[i];
-            ra[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_a, (int)vo, soff_a, 0));
+            for (int i = 0; i < A_LOADS; ++i)
+                ra[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_a2, (int)a2_voff[DUAL ? i : 0], soff_b - p.K1 * 4, 0));
+        } else {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t vo = CONV ? (((a_mask[i] >> tap) & 1) ? a_voff[i] : OOB) : a_voff[i];
+                ra[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_a, (int)vo, soff_a, 0));
+            }
         }
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i)

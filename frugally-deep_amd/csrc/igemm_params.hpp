@@ -42,6 +42,12 @@ struct GemmParams {
     // inside a strip, columns fastest) instead of row by row, so that the contiguous tile range of an XCD needs only
     // its strip's columns of B; 0 = one strip (row by row)
     int strip_w;
+    // fast path, GEMM form, whole tiles: a second source of A rows (see DUAL in igemm_fast.hpp); A2 == nullptr = none.
+    // K1 = columns taken from A (a multiple of the K slab), the remaining K - K1 come from A2; OH / OW above give the
+    // output map the rows are pixels of.
+    const float* A2;
+    int K1, H2, W2, C2, s2y, s2x;
+    uint32_t a2_records;
 };
 
 // Key of the per-process tuning table (igemm.hip).  conv = 0 / 1: a GEMM / convolution shape and its tile choice

@@ -1230,6 +1230,40 @@ namespace {
                 }
             }
         }
+        // 5. a residual operand that is itself a 1x1 convolution (the shortcut branch of a block that changes the channel
+        // count or the resolution: Add(Conv2D(a), Conv2D(b))) joins the 1x1 stride-1 convolution that adds it.  The two
+        // become one GEMM over both inputs' channels, and the shortcut's output is neither written nor read back.
+        static const bool dual_on = [] { const char* e = std::getenv("FDX_DUAL_CONV"); return !(e && e[0] == '0'); }();
+        for (size_t i = 0; i < m.ops.size() && have_shapes && dual_on; ++i) {
+            Op& c = m.ops[i];
+            auto plain_1x1 = [](const Op& o) {
+                return !o.dead && o.kind == OpKind::Conv2D && o.kh == 1 && o.kw == 1 && o.dy == 1 && o.dx == 1 && o.zp[0] == 0 && o.zp[1] == 0
+                    && o.zp[2] == 0 && o.zp[3] == 0 && !o.softmax && o.fuse_dw < 0 && o.fused_into < 0 && o.fuse_exp < 0 && o.exp_into < 0
+                    && o.dual_cin == 0 && o.hw.size() == 2 && o.n_in > 0 && o.n_in % 16 == 0 && o.cout >= 64 && o.cout % 4 == 0
+                    && o.hw[0].size() == (size_t)o.cout * (size_t)o.n_in && o.hw[1].size() == (size_t)o.cout;
+            };
+            if (c.residual < 0 || c.residual == c.in[0] || !plain_1x1(c) || c.sy != 1 || c.sx != 1)
+                continue;
+            Op& r = m.ops[c.residual];
+            if (!plain_1x1(r) || r.cout != c.cout || r.act.kind != FDX_ACT_NONE || r.consumers != 1 || r.residual >= 0 || r.in.size() != 1)
+                continue;
+            const int k1 = c.n_in, k2 = r.n_in;
+            c.hw.resize(6);
+            c.hw[5].resize((size_t)c.cout * (size_t)(k1 + k2));
+            for (int n = 0; n < c.cout; ++n) {
+                std::copy_n(&c.hw[0][(size_t)n * k1], k1, &c.hw[5][(size_t)n * (k1 + k2)]);
+                std::copy_n(&r.hw[0][(size_t)n * k2], k2, &c.hw[5][(size_t)n * (k1 + k2) + k1]);
+                c.hw[1][n] += r.hw[1][n];
+            }
+            c.hw[0].clear(); // the joint filter serves both inputs
+            c.dual_cin = k2;
+            c.dual_sy = r.sy;
+            c.dual_sx = r.sx;
+            c.in.push_back(r.in[0]);
+            c.residual = -1;
+            r.dead = true;
+            count_consumers(m);
+        }
         // last: depthwise 3x3 convolutions whose only consumer is a 1x1 convolution (the second half of an
         // inverted-residual block, a SeparableConv2D) are marked; whether the pair runs as one launch is decided per plan
         // by timing both forms
@@ -1237,7 +1271,7 @@ namespace {
         for (size_t i = 0; dwpw_on && i < m.ops.size(); ++i) {
             Op& c = m.ops[i];
             if (c.dead || c.kind != OpKind::Conv2D || c.kh != 1 || c.kw != 1 || c.sy != 1 || c.sx != 1 || c.softmax
-                || c.zp[0] || c.zp[1] || c.zp[2] || c.zp[3] || c.in.empty())
+                || c.zp[0] || c.zp[1] || c.zp[2] || c.zp[3] || c.in.empty() || c.dual_cin > 0)
                 continue;
             Op& d = m.ops[c.in[0]];
             if (d.dead || d.kind != OpKind::DWConv2D || d.kh != 3 || d.kw != 3 || d.dy != 1 || d.dx != 1 || d.sy != d.sx
@@ -1253,7 +1287,7 @@ namespace {
             Op& e = m.ops[d.in[0]];
             const bool act_ok = e.act.kind == FDX_ACT_NONE || e.act.kind == FDX_ACT_RELU || e.act.kind == FDX_ACT_GELU;
             if (e.dead || e.kind != OpKind::Conv2D || e.softmax || e.residual >= 0 || e.consumers != 1 || e.fuse_dw >= 0 || e.exp_into >= 0
-                || !act_ok || e.hw.empty() || e.cout <= 0 || e.hw[0].size() % (size_t)e.cout != 0)
+                || e.dual_cin > 0 || !act_ok || e.hw.empty() || e.cout <= 0 || e.hw[0].size() % (size_t)e.cout != 0)
                 continue;
             const bool pointwise = e.kh == 1 && e.kw == 1 && e.sy == 1 && e.sx == 1 && !e.zp[0] && !e.zp[1] && !e.zp[2] && !e.zp[3];
             // ... or the small convolution on the image a MobileNet-like network starts with (3x3 / 2 on RGB)
@@ -1569,7 +1603,7 @@ namespace {
     double op_flops(const Op& o, const Shape& out, const std::vector<Shape>& shapes, int batch)
     {
         switch (o.kind) {
-        case OpKind::Conv2D: return 2.0 * batch * volume(out) * o.kh * o.kw * o.n_in;
+        case OpKind::Conv2D: return 2.0 * batch * volume(out) * (o.kh * o.kw * o.n_in + o.dual_cin);
         case OpKind::Dense: return 2.0 * batch * volume(out) * o.n_in;
         case OpKind::Einsum: return o.gemm ? 2.0 * batch * volume(out) * o.n_in : 0.0;
         case OpKind::MHA: {
@@ -1869,6 +1903,18 @@ namespace {
             const int h = one_d ? 1 : (int)(*is)[0], w = (int)(*is)[one_d ? 0 : 1], c = (int)is->back();
             if ((st = window(h, w, o, true, g)) != FDX_OK)
                 return st;
+            if (o.kind == OpKind::Conv2D && o.dual_cin > 0) {
+                const Shape& s2 = p.shapes[o.in[1]];
+                FDX_REQUIRE(o.dw.size() > 5 && o.dw[5] && s2.size() == 3 && s2[2] == o.dual_cin && !one_d, "%s: bad two-input convolution",
+                    o.name.c_str());
+                // (what the absorbed convolution would have produced must be what the other one produces: the Add of the
+                // two needs equal shapes, layers/add_layer.hpp:20-29)
+                FDX_REQUIRE((s2[0] + o.dual_sy - 1) / o.dual_sy == g[4] && (s2[1] + o.dual_sx - 1) / o.dual_sx == g[5],
+                    "%s: the two convolutions of the sum give different shapes", o.name.c_str());
+                st = conv1x1_dual_launch(in0, B, g[4], g[5], c, p.out[o.in[1]], (int)s2[0], (int)s2[1], o.dual_cin, o.dual_sy, o.dual_sx,
+                    o.dw[5], o.dw[1], o.cout, actp, out);
+                break;
+            }
             if (o.kind == OpKind::Conv2D && o.dw.size() > 3 && o.dw[3] && g[0] + o.zp[0] == 0 && g[2] + o.zp[2] == 0 && g[4] == h && g[5] == w) {
                 st = conv1x1_padded_launch(in0, (int64_t)B * h * w, c, o.dw[3], (c + 15) / 16 * 16, o.dw[1], o.cout, res, actp, out);
                 if (st != FDX_ERR_UNSUPPORTED)

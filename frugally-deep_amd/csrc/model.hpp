@@ -35,6 +35,10 @@ struct Op {
     int fused_into = -1; // that depthwise op: the convolution which may absorb it
     int fuse_exp = -1;   // 1x1 Conv2D with fuse_dw >= 0: the 1x1 expansion in front of the depthwise op, if one launch can run all three (fdx_inverted_residual_nhwc_f32)
     int exp_into = -1;   // that expansion: the projection which may absorb it
+    // 1x1 stride-1 Conv2D that has absorbed the 1x1 convolution of its residual operand (conv1x1_dual_launch): input
+    // channels and strides of that convolution, whose input is in[1]; the filter over both inputs' channels is weight
+    // array 5
+    int dual_cin = 0, dual_sy = 1, dual_sx = 1;
     bool dead = false;
     int consumers = 0;
 
@@ -128,6 +132,8 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
 float* plan_alloc(Plan& p, size_t bytes, int* block_index);
 std::vector<int> topo_order(const fdx_model& m); // producers before consumers, dead ops skipped by callers
 fdx_status positions_launch(float* out, int batch, int t, int start);
+fdx_status conv1x1_dual_launch(const float* in1, int n, int oh, int ow, int c1, const float* in2, int h2, int w2, int c2, int s2y, int s2x,
+    const float* w_cat, const float* bias, int cout, const fdx_act* act, float* out);
 fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const float* w_padded, int k_padded, const float* bias,
     int cout, const float* residual, const fdx_act* act, float* out);
 fdx_status mha_prefill_strided(const float* q, int64_t ldq, int64_t q_batch, const float* k, int64_t ldk, int64_t k_batch,

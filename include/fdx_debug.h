@@ -55,6 +55,10 @@ fdx_status fdx_profile_get_executed(int index, double* executed_flops);
  *     wherever it covers the shape.
  */
 fdx_status fdx_debug_force_tile(int cfg);
+/* a 1x1 convolution that has absorbed the 1x1 convolution of its residual operand (a residual block with a convolution on
+ * its shortcut branch): 1 = one GEMM over both inputs' channels (the default), 0 = the two convolutions one after the
+ * other, the second adding to the first's result -- the form taken by itself where the one-launch kernel does not apply */
+fdx_status fdx_debug_dual_conv(int one_launch);
 /* decode sessions created from now on: 1 = the token + position embedding launch of a step is folded into the two GEMMs
  * that read its result (measured slower than the launch it saves, hence not the default), 0 = never, -1 = as the
  * environment says (FDX_DECODE_EMBED_FOLD=1) */

@@ -353,3 +353,35 @@ def test_pointwise_convolution_on_channel_counts_between_slabs(fdx, oracle, mode
     spec = b.finish([out, y])
     xs = np.random.default_rng(51).standard_normal((5, 9, 7, cin)).astype(np.float32)
     run_both(fdx, oracle, modelgen, spec, [xs])
+
+
+@pytest.mark.parametrize("stride,size,c_in,c_mid,c_out", [(1, (9, 7), 64, 32, 128), (2, (15, 13), 64, 48, 256), (2, (8, 8), 128, 64, 64),
+                                                           ((2, 1), (11, 6), 32, 16, 96)])
+@pytest.mark.parametrize("one_launch", [1, 0])
+def test_block_with_a_convolution_on_its_shortcut(fdx, oracle, modelgen, stride, size, c_in, c_mid, c_out, one_launch):
+    """Add(BatchNormalization(Conv2D 1x1(a)), BatchNormalization(Conv2D 1x1 / stride(b))) + ReLU: the two convolutions run
+    as one GEMM over the channels of both inputs (the strided one reads every stride-th pixel of its map), or one after
+    the other on the joint filter when the one-launch kernel is switched off.  Odd map sizes, a non-square stride, and a
+    second block behind the first so that the sum is read again."""
+    say("shortcut convolution", stride, size, c_in, c_mid, c_out, "one launch" if one_launch else "two launches")
+    b = modelgen.Builder("sc_%s_%d_%d" % (str(stride).replace(" ", ""), c_in, c_out), 61 + c_in + c_out)
+    x = b.input(size + (c_in,), "img")
+    y = b.conv2d(x, c_mid, 1, "c1", strides=stride, use_bias=False)
+    y = b.batchnorm(y, "c1_bn", random_stats=True)
+    y = b.relu(y, "c1_relu")
+    z = b.conv2d(y, c_out, 1, "c3", bias_std=0.2)
+    z = b.batchnorm(z, "c3_bn", random_stats=True)
+    sc = b.conv2d(x, c_out, 1, "sc", strides=stride, bias_std=0.1)
+    sc = b.batchnorm(sc, "sc_bn", random_stats=True)
+    out = b.add([sc, z], "sum")
+    out = b.relu(out, "sum_relu")
+    y2 = b.conv2d(out, c_mid, 1, "d1", activation="relu", bias_std=0.1)
+    z2 = b.conv2d(y2, c_out, 1, "d3", bias_std=0.1)
+    out2 = b.add([out, z2], "sum2")
+    spec = b.finish([out2, out])
+    xs = np.random.default_rng(62).standard_normal((5,) + size + (c_in,)).astype(np.float32)
+    fdx.check(fdx.lib.fdx_debug_dual_conv(one_launch))
+    try:
+        run_both(fdx, oracle, modelgen, spec, [xs])
+    finally:
+        fdx.check(fdx.lib.fdx_debug_dual_conv(1))
