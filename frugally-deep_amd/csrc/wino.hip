@@ -57,7 +57,10 @@ struct WinoParams {
 constexpr int WINO_TM = 32;  // tiles per workgroup
 constexpr int WINO_PAD = 4;  // padding of an LDS row of the exchange
 
-constexpr int WINO_SETS = 3; // register sets of step operands: a set is loaded WINO_SETS - 1 steps before its use
+// register sets of step operands: a set is loaded WINO_SETS - 1 steps before its use.  One step ahead is enough (a step is
+// 32 MFMAs, 0.9 us at the least, and the operands come from L2 or the memory-side cache): a third set, two steps ahead,
+// measured 2-3 % slower on the ResNet50 layers, and the kernel without any operand loads only 25 % faster than with them
+constexpr int WINO_SETS = 2;
 
 // one step's operands: the eight patch pixels of this lane's tile and the 4 x NT filter pieces of its positions
 template <int NT>
