@@ -1264,6 +1264,44 @@ namespace {
             r.dead = true;
             count_consumers(m);
         }
+        // 6. a 1x1 stride-1 convolution whose result another 1x1 stride-1 convolution reads (a block's last convolution, with
+        // its Add and ReLU in the epilogue, and the next block's first): marked as a pair that one launch can run, the
+        // second convolution taking the first's result from LDS (conv1x1_chain_launch).  Whether a plan does so is decided
+        // when the plan is made.
+        static const bool chain_env = [] { const char* e = std::getenv("FDX_CHAIN"); return !(e && e[0] == '0'); }();
+        // (FDX_CHAIN=0: no pair is marked and no packed filter kept; unset: pairs are marked so that the test hook can
+        // switch them on; FDX_CHAIN=1: plans with many pixels run them as one launch)
+        for (size_t i = 0; i < m.ops.size() && have_shapes && chain_env; ++i) {
+            Op& d = m.ops[i];
+            auto gemm_1x1 = [](const Op& o) {
+                return !o.dead && o.kind == OpKind::Conv2D && o.kh == 1 && o.kw == 1 && o.sy == 1 && o.sx == 1 && o.dy == 1 && o.dx == 1
+                    && o.zp[0] == 0 && o.zp[1] == 0 && o.zp[2] == 0 && o.zp[3] == 0 && !o.softmax && o.fuse_dw < 0 && o.fused_into < 0
+                    && o.fuse_exp < 0 && o.exp_into < 0 && o.chain < 0 && o.chained_from < 0 && o.n_in > 0
+                    && (o.act.kind == FDX_ACT_NONE || o.act.kind == FDX_ACT_RELU || o.act.kind == FDX_ACT_GELU)
+                    && o.hw.size() >= 2 && o.hw[1].size() == (size_t)o.cout;
+            };
+            if (!gemm_1x1(d) || d.in.size() != 1 || d.residual >= 0 || d.dual_cin > 0 || d.hw.size() != 2
+                || d.hw[0].size() != (size_t)d.cout * (size_t)d.n_in)
+                continue;
+            Op& c = m.ops[d.in[0]];
+            if (!gemm_1x1(c) || c.cout != d.n_in || !chain_supported(c.n_in, c.dual_cin, c.cout, d.cout))
+                continue;
+            const bool dual = c.dual_cin > 0;
+            if (dual ? !(c.hw.size() == 6 && c.hw[5].size() == (size_t)c.cout * (size_t)(c.n_in + c.dual_cin))
+                     : !(c.hw.size() == 2 && c.hw[0].size() == (size_t)c.cout * (size_t)c.n_in))
+                continue;
+            if (shapes[d.in[0]].size() != 3)
+                continue;
+            const int k = c.n_in + c.dual_cin;
+            c.hw.resize(7);
+            c.hw[6].resize(chain_first_floats(c.cout, k));
+            chain_pack_first(dual ? c.hw[5].data() : c.hw[0].data(), c.cout, k, c.hw[6].data());
+            d.hw.resize(7);
+            d.hw[6].resize(chain_second_floats(c.cout, d.cout));
+            chain_pack_second(d.hw[0].data(), c.cout, d.cout, d.hw[6].data());
+            c.chain = (int)i;
+            d.chained_from = d.in[0];
+        }
         // last: depthwise 3x3 convolutions whose only consumer is a 1x1 convolution (the second half of an
         // inverted-residual block, a SeparableConv2D) are marked; whether the pair runs as one launch is decided per plan
         // by timing both forms
@@ -1271,7 +1309,7 @@ namespace {
         for (size_t i = 0; dwpw_on && i < m.ops.size(); ++i) {
             Op& c = m.ops[i];
             if (c.dead || c.kind != OpKind::Conv2D || c.kh != 1 || c.kw != 1 || c.sy != 1 || c.sx != 1 || c.softmax
-                || c.zp[0] || c.zp[1] || c.zp[2] || c.zp[3] || c.in.empty() || c.dual_cin > 0)
+                || c.zp[0] || c.zp[1] || c.zp[2] || c.zp[3] || c.in.empty() || c.dual_cin > 0 || c.chain >= 0 || c.chained_from >= 0)
                 continue;
             Op& d = m.ops[c.in[0]];
             if (d.dead || d.kind != OpKind::DWConv2D || d.kh != 3 || d.kw != 3 || d.dy != 1 || d.dx != 1 || d.sy != d.sx
@@ -1287,7 +1325,7 @@ namespace {
             Op& e = m.ops[d.in[0]];
             const bool act_ok = e.act.kind == FDX_ACT_NONE || e.act.kind == FDX_ACT_RELU || e.act.kind == FDX_ACT_GELU;
             if (e.dead || e.kind != OpKind::Conv2D || e.softmax || e.residual >= 0 || e.consumers != 1 || e.fuse_dw >= 0 || e.exp_into >= 0
-                || e.dual_cin > 0 || !act_ok || e.hw.empty() || e.cout <= 0 || e.hw[0].size() % (size_t)e.cout != 0)
+                || e.dual_cin > 0 || e.chain >= 0 || e.chained_from >= 0 || !act_ok || e.hw.empty() || e.cout <= 0 || e.hw[0].size() % (size_t)e.cout != 0)
                 continue;
             const bool pointwise = e.kh == 1 && e.kw == 1 && e.sy == 1 && e.sx == 1 && !e.zp[0] && !e.zp[1] && !e.zp[2] && !e.zp[3];
             // ... or the small convolution on the image a MobileNet-like network starts with (3x3 / 2 on RGB)
@@ -1627,6 +1665,17 @@ extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
     return FDX_OK;
 }
 
+// test hook: -1 = plans run a pair of 1x1 convolutions as one launch where the closed rule says so, 0 = never, 1 = wherever
+// the kernel covers the pair
+static int g_force_chain = -1;
+
+extern "C" fdx_status fdx_debug_force_chain(int mode)
+{
+    FDX_REQUIRE(mode >= -1 && mode <= 1, "fdx_debug_force_chain: mode must be -1, 0 or 1");
+    g_force_chain = mode;
+    return FDX_OK;
+}
+
 // test hook: -1 = a plan times the direct and the Winograd kernel of a 3x3 stride-1 convolution, 0 = always direct, 1 = Winograd
 // wherever it applies
 static int g_force_winograd = -1;
@@ -1666,6 +1715,21 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
     p->temps.assign(n, {});
     p->dw_fused.assign(n, g_force_dw_fusion < 0 ? 0 : (g_force_dw_fusion == 1 ? 1 : (g_force_dw_fusion == 2 ? 3 : 2)));
     p->conv_form.assign(n, (signed char)g_force_winograd);
+    // Pairs of 1x1 convolutions that one launch can run: off unless asked for (FDX_CHAIN=1 or the test hook).  Measured on
+    // ResNet50's 56 x 56 stage at batch 64, the one launch takes as long as the two it replaces where the first convolution
+    // adds a residual (178 us either way) and longer where it sums two inputs (218 against 175 us): what it saves in
+    // memory traffic it loses to its serial phases at two workgroups per CU.
+    p->chain_on.assign(n, 0);
+    p->chain_done.assign(n, 0);
+    for (int idx : p->order) {
+        const Op& o = m->ops[idx];
+        if (o.dead || o.chain < 0 || m->ops[o.chain].dead || p->shapes[idx].size() != 3)
+            continue;
+        const int64_t rows = (int64_t)batch * p->shapes[idx][0] * p->shapes[idx][1];
+        static const bool chain_default = [] { const char* e = std::getenv("FDX_CHAIN"); return e && e[0] == '1'; }();
+        const bool wanted = g_force_chain >= 0 ? g_force_chain != 0 : (chain_default && rows >= 65536);
+        p->chain_on[idx] = wanted ? 1 : 0;
+    }
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -1713,10 +1777,19 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
             p->out[idx] = p->out[o.in[0]];
         } else {
             const size_t bytes = sizeof(float) * (size_t)batch * (size_t)volume(p->shapes[idx]);
-            p->out[idx] = plan_alloc(*p, bytes, &p->block_of[idx]);
+            if (!p->out[idx]) // (the second convolution of a pair run as one launch got its block with the first)
+                p->out[idx] = plan_alloc(*p, bytes, &p->block_of[idx]);
             if (!p->out[idx]) {
                 set_error("out of device memory while planning %s", o.name.c_str());
                 return FDX_ERR_HIP;
+            }
+            if (o.chain >= 0 && p->chain_on[idx]) { // this op's launch also writes its consumer's result
+                const int d = o.chain;
+                p->out[d] = plan_alloc(*p, sizeof(float) * (size_t)batch * (size_t)volume(p->shapes[d]), &p->block_of[d]);
+                if (!p->out[d]) {
+                    set_error("out of device memory while planning %s", m->ops[d].name.c_str());
+                    return FDX_ERR_HIP;
+                }
             }
         }
         if (o.kind == OpKind::Conv2D && o.dw.size() > 2 && o.dw[2] && p->shapes[idx].size() == 3)
@@ -1903,6 +1976,27 @@ namespace {
             const int h = one_d ? 1 : (int)(*is)[0], w = (int)(*is)[one_d ? 0 : 1], c = (int)is->back();
             if ((st = window(h, w, o, true, g)) != FDX_OK)
                 return st;
+            if (o.kind == OpKind::Conv2D && o.chained_from >= 0 && p.chain_done[idx]) {
+                p.chain_done[idx] = 0; // produced by the launch of the convolution in front
+                break;
+            }
+            if (o.kind == OpKind::Conv2D && o.chain >= 0 && p.chain_on[idx] && o.dw.size() > 6 && o.dw[6]) {
+                const Op& d = m.ops[o.chain];
+                const fdx_act act2 = to_c(d.act);
+                const bool dual = o.dual_cin > 0;
+                const Shape* s2 = dual ? &p.shapes[o.in[1]] : nullptr;
+                if ((!dual || (s2->size() == 3 && (*s2)[2] == o.dual_cin && ((*s2)[0] + o.dual_sy - 1) / o.dual_sy == g[4]
+                                  && ((*s2)[1] + o.dual_sx - 1) / o.dual_sx == g[5]))
+                    && !one_d && d.dw.size() > 6 && d.dw[6] && p.out[o.chain]) {
+                    st = conv1x1_chain_launch(in0, B, g[4], g[5], c, dual ? p.out[o.in[1]] : nullptr, dual ? (int)(*s2)[0] : 0,
+                        dual ? (int)(*s2)[1] : 0, dual ? o.dual_cin : 0, o.dual_sy, o.dual_sx, o.dual_cin, o.dw[6], o.dw[1], res, actp, o.cout,
+                        out, d.dw[6], d.dw[1], d.act.kind == FDX_ACT_NONE ? nullptr : &act2, d.cout, p.out[o.chain]);
+                    if (st == FDX_OK)
+                        p.chain_done[o.chain] = 1;
+                    if (st != FDX_ERR_UNSUPPORTED)
+                        break;
+                }
+            }
             if (o.kind == OpKind::Conv2D && o.dual_cin > 0) {
                 const Shape& s2 = p.shapes[o.in[1]];
                 FDX_REQUIRE(o.dw.size() > 5 && o.dw[5] && s2.size() == 3 && s2[2] == o.dual_cin && !one_d, "%s: bad two-input convolution",
@@ -2711,6 +2805,17 @@ namespace {
                     if (ib != ia && !m.ops[(size_t)ib].dead && p.block_of[(size_t)ib] == p.block_of[(size_t)ia])
                         clash = true;
                 }
+            }
+            // a pair of convolutions that one launch runs stays on one side of the cut
+            for (int a = 0; a < cut && !clash; ++a) {
+                const int ia = p.order[(size_t)a];
+                const Op& oa = m.ops[(size_t)ia];
+                if (oa.dead || oa.chain < 0 || !p.chain_on[(size_t)ia])
+                    continue;
+                bool inside = false;
+                for (int b = a + 1; b < cut; ++b)
+                    inside = inside || p.order[(size_t)b] == oa.chain;
+                clash = !inside;
             }
             if (ok && !clash)
                 break;

@@ -39,6 +39,11 @@ struct Op {
     // channels and strides of that convolution, whose input is in[1]; the filter over both inputs' channels is weight
     // array 5
     int dual_cin = 0, dual_sy = 1, dual_sx = 1;
+    // 1x1 stride-1 Conv2D whose result feeds another one (the tail of a residual block and the convolution that opens the
+    // next block): chain = that consumer, chained_from on the consumer = this op.  Where a plan runs the pair as one launch
+    // (conv1x1_chain_launch) the consumer's result is produced here and its own turn is skipped; the packed filters are
+    // weight array 6 of both ops.
+    int chain = -1, chained_from = -1;
     bool dead = false;
     int consumers = 0;
 
@@ -96,6 +101,8 @@ struct Plan {
     std::vector<std::vector<float*>> temps; // per op: scratch placed at plan time
     std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = depthwise + projection as one launch, 2 = one launch per layer, 3 = expansion + depthwise + projection as one launch
     std::vector<signed char> conv_form;     // per 3x3 stride-1 convolution with a Winograd filter: -1 = not timed yet, 0 = direct kernel, 1 = Winograd kernel
+    std::vector<signed char> chain_on;      // per 1x1 convolution with chain >= 0: 1 = this plan runs it and its consumer as one launch
+    std::vector<signed char> chain_done;    // per consumer of such a pair: its result was produced by the producer's launch in this run
     double flops = 0;
     ~Plan();
 };
@@ -132,6 +139,14 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
 float* plan_alloc(Plan& p, size_t bytes, int* block_index);
 std::vector<int> topo_order(const fdx_model& m); // producers before consumers, dead ops skipped by callers
 fdx_status positions_launch(float* out, int batch, int t, int start);
+bool chain_supported(int k1, int k2, int n1, int n2);
+size_t chain_first_floats(int n1, int k);
+size_t chain_second_floats(int n1, int n2);
+void chain_pack_first(const float* w, int n1, int k, float* out);
+void chain_pack_second(const float* w, int n1, int n2, float* out);
+fdx_status conv1x1_chain_launch(const float* a, int n, int oh, int ow, int k1, const float* b, int h2, int w2, int c2, int s2y, int s2x,
+    int k2, const float* w1, const float* bias1, const float* residual, const fdx_act* act1, int n1, float* y, const float* w2p,
+    const float* bias2, const fdx_act* act2, int n2, float* z);
 fdx_status conv1x1_dual_launch(const float* in1, int n, int oh, int ow, int c1, const float* in2, int h2, int w2, int c2, int s2y, int s2x,
     const float* w_cat, const float* bias, int cout, const fdx_act* act, float* out);
 fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const float* w_padded, int k_padded, const float* bias,

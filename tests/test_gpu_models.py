@@ -385,3 +385,39 @@ def test_block_with_a_convolution_on_its_shortcut(fdx, oracle, modelgen, stride,
         run_both(fdx, oracle, modelgen, spec, [xs])
     finally:
         fdx.check(fdx.lib.fdx_debug_dual_conv(1))
+
+
+@pytest.mark.parametrize("c_in,c_mid,c_out,stride", [(64, 64, 256, 1), (64, 64, 128, 2), (32, 128, 256, 1), (128, 128, 512, 2)])
+@pytest.mark.parametrize("mode", [1, 0])
+def test_block_tail_and_next_block_head_as_one_launch(fdx, oracle, modelgen, c_in, c_mid, c_out, stride, mode):
+    """Three bottleneck blocks of 1x1 convolutions: the last convolution of a block (with its shortcut convolution, or its
+    Add, and the ReLU in the epilogue) and the first convolution of the next block run as one launch, the second taking the
+    first's result from LDS -- forced on (at sizes the library's rule would leave alone) and off; every block's sum is a
+    model output, so both results of each launch are compared.  Pixel counts that are no multiple of the 64-row block."""
+    say("chained 1x1 convolutions", c_in, c_mid, c_out, stride, "one launch" if mode else "two launches")
+    b = modelgen.Builder("chain_%d_%d_%d_%d" % (c_in, c_mid, c_out, stride), 71 + c_in + c_out)
+    x = b.input((11, 9, c_in), "img")
+    sums = []
+    for blk in range(3):
+        first = blk == 0
+        y = b.conv2d(x, c_mid, 1, "b%d_c1" % blk, strides=stride if first else 1, use_bias=False)
+        y = b.batchnorm(y, "b%d_c1_bn" % blk, random_stats=True)
+        y = b.relu(y, "b%d_c1_relu" % blk)
+        z = b.conv2d(y, c_out, 1, "b%d_c3" % blk, bias_std=0.2)
+        z = b.batchnorm(z, "b%d_c3_bn" % blk, random_stats=True)
+        if first:
+            sc = b.conv2d(x, c_out, 1, "b0_sc", strides=stride, bias_std=0.1)
+            sc = b.batchnorm(sc, "b0_sc_bn", random_stats=True)
+        else:
+            sc = x
+        x = b.add([sc, z], "b%d_sum" % blk)
+        x = b.relu(x, "b%d_out" % blk)
+        sums.append(x)
+    tail = b.conv2d(x, 64, 1, "tail", activation="relu", bias_std=0.1)
+    spec = b.finish([tail] + sums)
+    xs = np.random.default_rng(72).standard_normal((5, 11, 9, c_in)).astype(np.float32)
+    fdx.check(fdx.lib.fdx_debug_force_chain(mode))
+    try:
+        run_both(fdx, oracle, modelgen, spec, [xs])
+    finally:
+        fdx.check(fdx.lib.fdx_debug_force_chain(-1))
