@@ -48,6 +48,17 @@ def good_models(modelgen):
     yield "mobilenet", modelgen.mobilenet_v2(input_size=32, alpha=0.25, classes=10, truncate=4)
     yield "encoder", modelgen.encoder(layers=1, seq=8, d_model=16, heads=2, ffn=32)
     yield "gpt2", modelgen.gpt2(layers=1, d_model=16, heads=2, vocab=50, max_pos=16)
+    # bottleneck blocks wide enough for the loader to join the shortcut convolution with the block's last convolution and to
+    # pack the filters of a block tail / next block head pair
+    b = modelgen.Builder("blocks", 8)
+    x = b.input((6, 6, 64), "img")
+    for blk in range(2):
+        y = b.conv2d(x, 64, 1, "b%d_c1" % blk, strides=2 if blk == 0 else 1, activation="relu")
+        z = b.conv2d(y, 128, 1, "b%d_c3" % blk, use_bias=False)
+        z = b.batchnorm(z, "b%d_bn" % blk, random_stats=True)
+        sc = b.conv2d(x, 128, 1, "b%d_sc" % blk, strides=2) if blk == 0 else x
+        x = b.relu(b.add([sc, z], "b%d_sum" % blk), "b%d_out" % blk)
+    yield "blocks", b.finish([b.conv2d(x, 64, 1, "tail")])
     b = modelgen.Builder("mixed", 7)
     x = b.input((8, 8, 4), "img")
     y = b.separable_conv2d(x, 6, 3, "sep", padding="same", activation="swish")
