@@ -482,6 +482,17 @@ static bool launch_fast(int cfg, int splits, int mode, const GemmParams& q0, boo
         else                                                                                                     \
             launch_persistent(igemm_fast_kernel<BM_, BN_, WM_, WN_, 32, false>, tiles, q, s, 512, BM_, BN_);     \
     }
+    if (q.ln_wsum) { // rows normalised on the way: whole tiles of the 32-float slab configurations
+        switch (cfg) {
+        case 13: launch_persistent(igemm_fast_kernel<128, 128, 2, 2, 32, false, false, false, false, true>,
+            ((q.M + 127) / 128) * ((q.N + 127) / 128) * batch, q, s, 256, 128, 128); break;
+        case 14: launch_persistent(igemm_fast_kernel<128, 64, 2, 2, 32, false, false, false, false, true>,
+            ((q.M + 127) / 128) * ((q.N + 63) / 64) * batch, q, s, 256, 128, 64); break;
+        default: launch_persistent(igemm_fast_kernel<64, 64, 2, 2, 32, false, false, false, false, true>,
+            ((q.M + 63) / 64) * ((q.N + 63) / 64) * batch, q, s, 256, 64, 64); break;
+        }
+        return true;
+    }
         switch (cfg) {
         case 10: FDX_FAST(128, 128, 16) break;
         case 11: FDX_FAST(128, 64, 16) break;
@@ -763,7 +774,20 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         default: launch_cfg<64, 64, 2, 2>(p, a_mode, b_vec, batch, s); break;
         }
     };
-    if (p.A2) {
+    if (p.ln_wsum) {
+        // rows normalised on the way: whole tiles, 32-float slab, nothing timed
+        const bool ln_ok = !conv && batch == 1 && fast_ok && p.a_valid_k == 0 && !p.A2 && p.K % 32 == 0 && p.alpha == 1.f && aligned16(p.ln_wsum);
+        if (!ln_ok) {
+            set_error("igemm: this normalising problem needs the fast path");
+            return FDX_ERR_UNSUPPORTED;
+        }
+        if (cfg < 13 || cfg > 15)
+            cfg = -1;
+        splits = 1;
+        mode = 0;
+        if (cfg < 0)
+            cfg = (p.K >= 1024 && p.N % 128 == 0 && blocks(128, 128) >= 2048) ? 13 : 15;
+    } else if (p.A2) {
         // two-source rows: whole tiles of the four-wave fast kernel only, nothing timed
         const int64_t a2_bytes = (int64_t)(p.OH > 0 && p.OW > 0 ? p.M / (p.OH * p.OW) : 0) * p.H2 * p.W2 * p.C2 * 4;
         const bool dual_ok = !conv && batch == 1 && fast_ok && p.a_valid_k == 0 && aligned16(p.A2) && p.C2 % 4 == 0 && p.K1 > 0
@@ -985,6 +1009,31 @@ extern "C" fdx_status fdx_debug_force_tile(int cfg)
     fdx::g_forced_tile = cfg;
     return FDX_OK;
 }
+
+namespace fdx {
+// out[M][n] = act(LN(x)[M][k] . w^T + bias + residual), the rows of x normalised over k inside the GEMM (LNF in
+// igemm_fast.hpp): w is the filter with LayerNormalization's gamma folded in ([n][k]), bias the bias with beta folded in,
+// wsum[n] the row sums of w.  FDX_ERR_UNSUPPORTED, with nothing launched, where the fast path does not apply.
+bool gemm_ln_supported(int64_t m, int n, int k)
+{
+    return m > 0 && m < (1LL << 31) && n >= 16 && n % 4 == 0 && k >= 32 && k % 32 == 0 && (m * k) * 4 < (1LL << 31);
+}
+
+fdx_status gemm_ln_launch(const float* x, int64_t m, int k, const float* w, const float* bias, const float* wsum, float eps, const float* residual,
+    const fdx_act* act, float* out, int n)
+{
+    FDX_REQUIRE(x && w && wsum && out && gemm_ln_supported(m, n, k), "gemm_ln: bad arguments");
+    FDX_REQUIRE_EPILOGUE_ACT(act);
+    GemmParams p {};
+    p.A = x; p.B = w; p.C = out; p.bias = bias; p.residual = residual;
+    p.M = (int)m; p.N = n; p.K = k; p.lda = k; p.ldb = k; p.ldc = n;
+    p.alpha = 1.f; p.bias_per_row = 0; p.act = make_act(act);
+    p.inner = 1;
+    p.ln_wsum = wsum;
+    p.ln_eps = eps;
+    return run_igemm(p, false, 1, "gemm_ln_f32");
+}
+} // namespace fdx
 
 extern "C" fdx_status fdx_debug_dual_conv(int one_launch)
 {

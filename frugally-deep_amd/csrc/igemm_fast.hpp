@@ -35,7 +35,16 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 //    stride lda, the other K - K1 from A2, whose row for output pixel (image, y, x) is pixel (y * s2y, x * s2x) of an
 //    [H2][W2][C2] map.  That is the sum of two pointwise convolutions as one GEMM over the concatenated channels
 //    (a residual block whose shortcut is a 1x1 convolution: the shortcut's output is never written or read back).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false, bool STREAMK = false, bool DUAL = false>
+//  * LNF (GEMM form, whole tiles only, K = the whole row): the rows of A are layer-normalised over K on the way,
+//        C = act(LN(A) . B^T + bias)  with  LN(a) = (a - mean) / sqrt(var + eps)   (gamma folded into B, beta into bias
+//    by the caller; include/fdeep/layers/layer_normalization_layer.hpp:37-63).  A tile's K loop reads its rows from end
+//    to end anyway, so the row statistics are gathered from the operand registers on their way to LDS (sums of the
+//    differences to the row's first value a thread sees, which keeps them small whatever the row's mean), merged over
+//    the lanes that share a row after the loop, and applied in the epilogue as
+//        rstd * (acc - mean * rowsum(B)) + bias:
+//    no pass over A of its own, and the normalised tensor never exists.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKT, bool CONV, bool SPLIT = false, bool STREAMK = false, bool DUAL = false,
+    bool LNF = false>
 // (the second bound asks for two waves per SIMD where the split variant of the largest four-wave tile would otherwise
 // settle for one: its reduction holds the accumulators in ordinary registers next to the prefetched operands)
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (SPLIT && WAVES_M * WAVES_N == 4 && BM * BN >= 128 * 128) ? 2 : 1)
@@ -44,6 +53,7 @@ void igemm_fast_kernel(GemmParams p)
     constexpr int NT = 64 * WAVES_M * WAVES_N;
     static_assert(NT == 256 || NT == 512, "four or eight waves");
     static_assert(!DUAL || (!CONV && !SPLIT), "the two-source form is a whole-tile GEMM");
+    static_assert(!LNF || (!CONV && !SPLIT && !DUAL), "the normalising form is a whole-tile GEMM");
     constexpr int STRIDE = BKT + 4;
     constexpr int CPR = BKT / 4;  // 16-byte chunks per tile row
     constexpr int RPP = NT / CPR; // tile rows filled per loader pass
@@ -57,6 +67,7 @@ void igemm_fast_kernel(GemmParams p)
 
     __shared__ __attribute__((aligned(16))) float smem[2 * (BM + BN) * STRIDE];
     __shared__ int last_flag;
+    __shared__ float ln_stats[LNF ? 2 * BM : 2]; // (mean, 1 / sqrt(var + eps)) per tile row
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -234,9 +245,26 @@ void igemm_fast_kernel(GemmParams p)
             soff_a += BKT * 4;
         }
     };
-    auto store_tiles = [&](int buf) {
+    float ln_shift[LNF ? A_LOADS : 1], ln_s[LNF ? A_LOADS : 1], ln_q[LNF ? A_LOADS : 1];
+    auto store_tiles = [&](int buf, bool first = false) {
         float* as = smem + buf * (BM + BN) * STRIDE;
         float* bs = as + BM * STRIDE;
+        if (LNF) {
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                if (first) {
+                    ln_shift[LNF ? i : 0] = ra[i][0];
+                    ln_s[LNF ? i : 0] = 0.f;
+                    ln_q[LNF ? i : 0] = 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float dlt = ra[i][e] - ln_shift[LNF ? i : 0];
+                    ln_s[LNF ? i : 0] += dlt;
+                    ln_q[LNF ? i : 0] += dlt * dlt;
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
             *reinterpret_cast<f32x4*>(&as[(r0 + i * RPP) * STRIDE + kq * 4]) = ra[i];
@@ -264,7 +292,7 @@ void igemm_fast_kernel(GemmParams p)
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0.f;
 
-        store_tiles(0);
+        store_tiles(0, true);
         __syncthreads();
         const int kt_end = kt_n;
         for (int kt = 0; kt < kt_end; ++kt) {
@@ -292,8 +320,37 @@ void igemm_fast_kernel(GemmParams p)
             }
             if (kt + 1 < kt_end)
                 store_tiles(buf ^ 1);
+            if (LNF && kt + 1 == kt_end) {
+                // Every slab has passed through store_tiles by now, so every thread has seen 4 * KT values of each of its
+                // rows.  The eight lanes that share a row (consecutive lanes, CPR = 8) merge their means and sums of
+                // squared deviations pairwise, equal counts on both sides at every step, on the VALU's lane swaps: inside
+                // quads twice, then with the mirrored lane of the row's eight, whose quad holds the other half's result.
+                // Done here, behind the last slab's MFMAs and in front of the loop's last barrier, it costs no barrier of
+                // its own.
+                static_assert(!LNF || CPR == 8, "the merge below is written for eight lanes per row");
+#pragma unroll
+                for (int i = 0; i < A_LOADS; ++i) {
+                    float cnt = 4.0f * (float)KT;
+                    float mean = ln_shift[LNF ? i : 0] + ln_s[LNF ? i : 0] / cnt;
+                    float m2 = ln_q[LNF ? i : 0] - ln_s[LNF ? i : 0] * ln_s[LNF ? i : 0] / cnt;
+                    auto merge = [&](float om, float o2) {
+                        const float dlt = om - mean;
+                        mean = 0.5f * (mean + om);
+                        m2 = m2 + o2 + dlt * dlt * (0.5f * cnt);
+                        cnt *= 2.0f;
+                    };
+                    merge(dpp_move<0xB1>(mean), dpp_move<0xB1>(m2));   // quad_perm [1, 0, 3, 2]
+                    merge(dpp_move<0x4E>(mean), dpp_move<0x4E>(m2));   // quad_perm [2, 3, 0, 1]
+                    merge(dpp_move<0x141>(mean), dpp_move<0x141>(m2)); // row_half_mirror
+                    if (kq == 0) {
+                        ln_stats[2 * (r0 + i * RPP)] = mean;
+                        ln_stats[2 * (r0 + i * RPP) + 1] = 1.0f / sqrtf(fmaxf(m2, 0.f) / cnt + p.ln_eps);
+                    }
+                }
+            }
             __syncthreads();
         }
+
 
         // this tile's coordinates for the epilogue; the loader state moves on to the next tile
         const int em0 = m0, en0 = n0;
@@ -319,9 +376,12 @@ void igemm_fast_kernel(GemmParams p)
                     rr[ps] = *reinterpret_cast<const f32x4*>(R + (int64_t)m * p.ldc + n);
             }
         };
+        f32x4 wsum4 = { 0.f, 0.f, 0.f, 0.f };
         auto request_epilogue = [&]() {
             if (p.bias && n_ok)
                 bias4 = *reinterpret_cast<const f32x4*>(p.bias + n);
+            if (LNF && n_ok)
+                wsum4 = *reinterpret_cast<const f32x4*>(p.ln_wsum + n);
             request_residual(0);
         };
         // (the split variants hold partial tiles in registers across the exchange below; there the requests wait
@@ -441,9 +501,17 @@ void igemm_fast_kernel(GemmParams p)
                 const int row = ps * RPS + srow;
                 const f32x4 v = *reinterpret_cast<const f32x4*>(&scratch[row * OSTRIDE + scol]);
                 float r[4];
+                if (LNF) {
+                    const int trow = wm * WTM + i * 32 + row;
+                    const float mu = ln_stats[2 * trow], rs = ln_stats[2 * trow + 1];
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    r[e] = v[e] * p.alpha + bias4[e] + rr[ps][e];
+                    for (int e = 0; e < 4; ++e)
+                        r[e] = rs * (v[e] - mu * wsum4[e]) + bias4[e] + rr[ps][e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        r[e] = v[e] * p.alpha + bias4[e] + rr[ps][e];
+                }
                 apply_act_block(r, p.act);
                 done[ps] = f32x4 { r[0], r[1], r[2], r[3] };
             }

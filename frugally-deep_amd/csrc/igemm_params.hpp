@@ -48,6 +48,10 @@ struct GemmParams {
     const float* A2;
     int K1, H2, W2, C2, s2y, s2x;
     uint32_t a2_records;
+    // fast path, GEMM form, whole tiles: rows of A layer-normalised over K on the way (see LNF in igemm_fast.hpp);
+    // ln_wsum = per output column the sum of its (gamma-folded) filter row, nullptr = no normalisation
+    const float* ln_wsum;
+    float ln_eps;
 };
 
 // Key of the per-process tuning table (igemm.hip).  conv = 0 / 1: a GEMM / convolution shape and its tile choice

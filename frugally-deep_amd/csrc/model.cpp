@@ -9,6 +9,7 @@
 #include "model.hpp"
 
 #include <algorithm>
+#include <map>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -1264,6 +1265,60 @@ namespace {
             r.dead = true;
             count_consumers(m);
         }
+        // 7. a LayerNormalization over the last axis whose only readers are Dense layers and self-attention layers (all of
+        // query, value and key): the readers are marked, and get their filters with gamma / beta folded in when the weights
+        // are uploaded; a plan may then normalise inside their GEMMs and skip the LayerNormalization launch.  The op itself
+        // and the readers' own filters stay (a decode session folds them its own way, and sizes the GEMM kernel does not
+        // cover run as before).
+        // (Readers are marked unless FDX_LN_FOLD=0; plans use the marks only on request, FDX_LN_FOLD=1 or the test hook: on the
+        // benched encoder -- 8192 rows of 512, 12 LayerNormalization launches of 11 us -- the statistics cost the two GEMMs
+        // that gather them 12 % of their time, 0.7 % more per step than the launches they save.)
+        static const bool ln_fold_env = [] { const char* e = std::getenv("FDX_LN_FOLD"); return !(e && e[0] == '0'); }();
+        for (size_t i = 0; i < m.ops.size() && have_shapes && ln_fold_env; ++i) {
+            Op& ln = m.ops[i];
+            if (ln.dead || ln.kind != OpKind::LayerNorm || ln.rms || ln.act.kind != FDX_ACT_NONE || ln.in.size() != 1 || ln.target_shape.size() != 1)
+                continue;
+            const Shape& xs = shapes[ln.in[0]];
+            if (xs.empty())
+                continue;
+            const int64_t a = ln.target_shape[0];
+            const int64_t C = xs.back();
+            if (!(a == -1 || a == (int64_t)xs.size()) || C < 32 || C % 32 != 0)
+                continue;
+            if ((ln.hw.size() > 0 && !ln.hw[0].empty() && (int64_t)ln.hw[0].size() != C) || (ln.hw.size() > 1 && !ln.hw[1].empty() && (int64_t)ln.hw[1].size() != C))
+                continue;
+            bool is_output = false;
+            for (int out : m.outputs)
+                is_output = is_output || out == (int)i;
+            std::vector<int> readers;
+            bool ok = !is_output;
+            for (size_t q = 0; q < m.ops.size() && ok; ++q) {
+                const Op& r = m.ops[q];
+                if (r.dead)
+                    continue;
+                const bool reads = std::find(r.in.begin(), r.in.end(), (int)i) != r.in.end();
+                if (r.residual == (int)i)
+                    ok = false;
+                if (!reads)
+                    continue;
+                if (r.kind == OpKind::Dense && r.in.size() == 1 && r.n_in == C && r.hw.size() == 2 && r.ln_src < 0
+                    && r.hw[0].size() == (size_t)r.units * (size_t)C && r.hw[1].size() == (size_t)r.units && r.units % 4 == 0 && r.units >= 16) {
+                    readers.push_back((int)q);
+                } else if (r.kind == OpKind::MHA && r.ln_src < 0 && !r.gate && r.d_in == C && r.hw.size() >= 6 && r.in.size() >= 2
+                    && r.in[0] == (int)i && r.in[1] == (int)i && (r.in.size() == 2 || r.in[2] == (int)i) && (r.heads * r.dk) % 4 == 0
+                    && (r.heads * r.dv) % 4 == 0) {
+                    readers.push_back((int)q);
+                } else {
+                    ok = false;
+                }
+            }
+            if (!ok || readers.empty())
+                continue;
+            for (int q : readers) {
+                m.ops[q].ln_src = (int)i;
+                m.ops[q].ln_eps = ln.eps;
+            }
+        }
         // 6. a 1x1 stride-1 convolution whose result another 1x1 stride-1 convolution reads (a block's last convolution, with
         // its Add and ReLU in the epilogue, and the next block's first): marked as a pair that one launch can run, the
         // second convolution taking the first's result from LDS (conv1x1_chain_launch).  Whether a plan does so is decided
@@ -1340,6 +1395,35 @@ namespace {
 
     fdx_status upload(fdx_model& m)
     {
+        // gamma / beta of the LayerNormalization ops some reader folds into its filter (the op's own arrays are released when
+        // it is uploaded, before its readers' turn)
+        std::map<int, std::pair<std::vector<float>, std::vector<float>>> ln_affine;
+        for (auto& o : m.ops)
+            if (!o.dead && o.ln_src >= 0 && !ln_affine.count(o.ln_src)) {
+                const Op& ln = m.ops[(size_t)o.ln_src];
+                ln_affine[o.ln_src] = { ln.hw.size() > 0 ? ln.hw[0] : std::vector<float>(), ln.hw.size() > 1 ? ln.hw[1] : std::vector<float>() };
+            }
+        // filter [n][k] with gamma folded in, bias with beta folded in, row sums of the folded filter
+        auto fold_ln = [&](int ln_idx, const std::vector<float>& w, const std::vector<float>& b, int n, int k, std::vector<float>& wf,
+                           std::vector<float>& bf, std::vector<float>& ws) {
+            const auto& gb = ln_affine[ln_idx];
+            wf.resize((size_t)n * k);
+            bf.assign((size_t)n, 0.f);
+            ws.assign((size_t)n, 0.f);
+            for (int r = 0; r < n; ++r) {
+                double sum = 0.0, shift = b.empty() ? 0.0 : (double)b[(size_t)r];
+                for (int c = 0; c < k; ++c) {
+                    const float wv = w[(size_t)r * k + c];
+                    const float f = gb.first.empty() ? wv : wv * gb.first[(size_t)c];
+                    wf[(size_t)r * k + c] = f;
+                    sum += (double)f;
+                    if (!gb.second.empty())
+                        shift += (double)wv * (double)gb.second[(size_t)c];
+                }
+                ws[(size_t)r] = (float)sum;
+                bf[(size_t)r] = (float)shift;
+            }
+        };
         for (auto& o : m.ops) {
             if (o.dead) {
                 o.hw.clear();
@@ -1382,6 +1466,16 @@ namespace {
                     o.hw[10].insert(o.hw[10].end(), o.hw[(size_t)2 * part].begin(), o.hw[(size_t)2 * part].end());
                     o.hw[11].insert(o.hw[11].end(), o.hw[(size_t)2 * part + 1].begin(), o.hw[(size_t)2 * part + 1].end());
                 }
+            }
+            if (o.ln_src >= 0 && o.kind == OpKind::Dense && o.hw.size() == 2) {
+                o.hw.resize(5);
+                fold_ln(o.ln_src, o.hw[0], o.hw[1], o.units, o.n_in, o.hw[2], o.hw[3], o.hw[4]);
+            } else if (o.ln_src >= 0 && o.kind == OpKind::MHA && o.hw.size() >= 12 && !o.hw[10].empty()) {
+                const int nt = 2 * o.heads * o.dk + o.heads * o.dv;
+                o.hw.resize(15);
+                fold_ln(o.ln_src, o.hw[10], o.hw[11], nt, o.d_in, o.hw[12], o.hw[13], o.hw[14]);
+            } else {
+                o.ln_src = -1; // (an attention op whose projections were not stacked, ...: it reads the LayerNormalization's result)
             }
             o.dw.assign(o.hw.size(), nullptr);
             for (size_t i = 0; i < o.hw.size(); ++i) {
@@ -1665,6 +1759,18 @@ extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
     return FDX_OK;
 }
 
+// test hook: 0 = plans built from now on run every LayerNormalization as a launch of its own, 1 = they normalise inside the
+// readers' GEMMs where those are Dense / self-attention layers of a size the kernel covers, -1 = as the environment says
+// (FDX_LN_FOLD=1: inside the GEMMs; otherwise launches of their own)
+static int g_force_ln_fold = -1;
+
+extern "C" fdx_status fdx_debug_force_ln_fold(int mode)
+{
+    FDX_REQUIRE(mode >= -1 && mode <= 1, "fdx_debug_force_ln_fold: mode must be -1, 0 or 1");
+    g_force_ln_fold = mode;
+    return FDX_OK;
+}
+
 // test hook: -1 = plans run a pair of 1x1 convolutions as one launch where the closed rule says so, 0 = never, 1 = wherever
 // the kernel covers the pair
 static int g_force_chain = -1;
@@ -1730,6 +1836,34 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
         const bool wanted = g_force_chain >= 0 ? g_force_chain != 0 : (chain_default && rows >= 65536);
         p->chain_on[idx] = wanted ? 1 : 0;
     }
+    // LayerNormalization ops whose readers all normalise inside their own GEMM in this plan: no launch of their own
+    p->ln_fold_on.assign(n, 0);
+    p->ln_skip.assign(n, 0);
+    for (int idx : p->order) {
+        const Op& ln = m->ops[idx];
+        static const bool ln_fold_default = [] { const char* e = std::getenv("FDX_LN_FOLD"); return e && e[0] == '1'; }();
+        if (ln.dead || ln.kind != OpKind::LayerNorm || !(g_force_ln_fold == 1 || (g_force_ln_fold < 0 && ln_fold_default)))
+            continue;
+        bool all = true, any = false;
+        for (int q : p->order) {
+            const Op& r = m->ops[q];
+            if (r.dead || std::find(r.in.begin(), r.in.end(), idx) == r.in.end())
+                continue;
+            any = true;
+            const Shape& xs = p->shapes[ln.in[0]];
+            const int64_t rows = xs.empty() ? 0 : (int64_t)batch * volume(xs) / xs.back();
+            const int n_out = r.kind == OpKind::Dense ? r.units : 2 * r.heads * r.dk + r.heads * r.dv;
+            const size_t folded = r.kind == OpKind::Dense ? 2 : 12;
+            all = all && r.ln_src == idx && r.dw.size() > folded + 2 && r.dw[folded] && !xs.empty() && rows > 16
+                && gemm_ln_supported(rows, n_out, (int)xs.back());
+        }
+        if (!any || !all)
+            continue;
+        p->ln_skip[idx] = 1;
+        for (int q : p->order)
+            if (!m->ops[q].dead && m->ops[q].ln_src == idx)
+                p->ln_fold_on[q] = 1;
+    }
     std::vector<int> s2d_ops;
     // lifetime: position of the last consumer; a View extends the life of the buffer it aliases
     std::vector<int> root(n);
@@ -1743,6 +1877,9 @@ fdx_status get_plan(fdx_model* m, int batch, const std::vector<Shape>& in_shapes
             p->last_use[root[i]] = (int)pos;
         if (o.residual >= 0)
             p->last_use[root[o.residual]] = (int)pos;
+        if (o.ln_src >= 0 && p->ln_fold_on[p->order[pos]]) // normalising inside its GEMM, the op reads the LayerNormalization's input
+            for (int i : m->ops[o.ln_src].in)
+                p->last_use[root[i]] = (int)pos;
         if (o.fuse_dw >= 0) // run as one launch, the pair reads the depthwise convolution's input here
             for (int i : m->ops[o.fuse_dw].in)
                 p->last_use[root[i]] = (int)pos;
@@ -2040,6 +2177,10 @@ namespace {
         case OpKind::Dense: {
             const int64_t rows = (int64_t)B * volume(*is) / o.n_in;
             FDX_REQUIRE(rows < (1LL << 31), "%s: too many rows", o.name.c_str());
+            if (o.ln_src >= 0 && p.ln_fold_on[idx]) { // the LayerNormalization in front happens inside the GEMM
+                st = gemm_ln_launch(p.out[m.ops[o.ln_src].in[0]], rows, o.n_in, o.dw[2], o.dw[3], o.dw[4], o.ln_eps, res, actp, out, o.units);
+                break;
+            }
             st = fdx_gemm_bias_act_f32(in0, o.n_in, o.dw[0], o.n_in, (int)rows, o.units, o.n_in, 1.0f, o.dw[1], 0, res, actp,
                 out, o.units, nullptr);
             break;
@@ -2059,6 +2200,8 @@ namespace {
             break;
         }
         case OpKind::LayerNorm: {
+            if (p.ln_skip[idx])
+                return FDX_OK; // every reader normalises inside its own GEMM
             // axes are 1-based positions in the sample's own rank (negative from the end)
             const int rank = (int)is->size();
             int64_t dims5[5] = { 1, 1, 1, 1, 1 };
@@ -2292,7 +2435,12 @@ namespace {
             float *q = tmp[0], *k = tmp[1], *v = tmp[2], *merged = tmp[3], *scratch = tmp[4];
             if (o.dw.size() > 11 && o.dw[10]) {
                 const int64_t nt = 2 * nk + nv;
-                if ((st = fdx_gemm_bias_act_f32(xq, D, o.dw[10], D, B * T, (int)nt, D, 1.f, o.dw[11], 0, nullptr, nullptr, q, nt, nullptr)) != FDX_OK)
+                if (o.ln_src >= 0 && p.ln_fold_on[idx])
+                    st = gemm_ln_launch(p.out[m.ops[o.ln_src].in[0]], (int64_t)B * T, D, o.dw[12], o.dw[13], o.dw[14], o.ln_eps, nullptr, nullptr, q,
+                        (int)nt);
+                else
+                    st = fdx_gemm_bias_act_f32(xq, D, o.dw[10], D, B * T, (int)nt, D, 1.f, o.dw[11], 0, nullptr, nullptr, q, nt, nullptr);
+                if (st != FDX_OK)
                     return st;
                 if ((st = mha_prefill_strided(q, nt, T * nt, q + nk, nt, T * nt, q + 2 * nk, nt, T * nt, B, T, S, H, o.dk, o.dv, 0, merged,
                          nv, T * nv, scratch)) != FDX_OK)

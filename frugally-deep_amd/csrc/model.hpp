@@ -44,6 +44,13 @@ struct Op {
     // (conv1x1_chain_launch) the consumer's result is produced here and its own turn is skipped; the packed filters are
     // weight array 6 of both ops.
     int chain = -1, chained_from = -1;
+    // Dense / self-attention op whose input is a LayerNormalization over the last axis that feeds nothing else but such
+    // ops: ln_src = that op, ln_eps its epsilon.  Where a plan normalises inside the GEMM (gemm_ln_launch) the op reads the
+    // LayerNormalization's own input and the weight arrays with gamma / beta folded in (Dense: arrays 2-4 = filter, bias,
+    // filter row sums; attention: arrays 12-14, the same for the stacked query / key / value projection), and the
+    // LayerNormalization launch is skipped.
+    int ln_src = -1;
+    float ln_eps = 0.f;
     bool dead = false;
     int consumers = 0;
 
@@ -102,6 +109,8 @@ struct Plan {
     std::vector<signed char> dw_fused;      // per 1x1 convolution with fuse_dw >= 0: 0 = not timed yet, 1 = depthwise + projection as one launch, 2 = one launch per layer, 3 = expansion + depthwise + projection as one launch
     std::vector<signed char> conv_form;     // per 3x3 stride-1 convolution with a Winograd filter: -1 = not timed yet, 0 = direct kernel, 1 = Winograd kernel
     std::vector<signed char> chain_on;      // per 1x1 convolution with chain >= 0: 1 = this plan runs it and its consumer as one launch
+    std::vector<signed char> ln_fold_on;    // per Dense / attention op with ln_src >= 0: 1 = this plan normalises inside its GEMM
+    std::vector<signed char> ln_skip;       // per LayerNormalization op: 1 = every reader normalises for itself, no launch
     std::vector<signed char> chain_done;    // per consumer of such a pair: its result was produced by the producer's launch in this run
     double flops = 0;
     ~Plan();
@@ -147,6 +156,9 @@ void chain_pack_second(const float* w, int n1, int n2, float* out);
 fdx_status conv1x1_chain_launch(const float* a, int n, int oh, int ow, int k1, const float* b, int h2, int w2, int c2, int s2y, int s2x,
     int k2, const float* w1, const float* bias1, const float* residual, const fdx_act* act1, int n1, float* y, const float* w2p,
     const float* bias2, const fdx_act* act2, int n2, float* z);
+bool gemm_ln_supported(int64_t m, int n, int k);
+fdx_status gemm_ln_launch(const float* x, int64_t m, int k, const float* w, const float* bias, const float* wsum, float eps, const float* residual,
+    const fdx_act* act, float* out, int n);
 fdx_status conv1x1_dual_launch(const float* in1, int n, int oh, int ow, int c1, const float* in2, int h2, int w2, int c2, int s2y, int s2x,
     const float* w_cat, const float* bias, int cout, const fdx_act* act, float* out);
 fdx_status conv1x1_padded_launch(const float* in, int64_t rows, int cin, const float* w_padded, int k_padded, const float* bias,

@@ -421,3 +421,54 @@ def test_block_tail_and_next_block_head_as_one_launch(fdx, oracle, modelgen, c_i
         run_both(fdx, oracle, modelgen, spec, [xs])
     finally:
         fdx.check(fdx.lib.fdx_debug_force_chain(-1))
+
+
+@pytest.mark.parametrize("center,scale,offset", [(True, True, 0.0), (False, True, 0.0), (True, False, 3.0), (True, True, 40.0)])
+def test_layernorm_inside_the_readers_gemms(fdx, oracle, modelgen, center, scale, offset):
+    """A LayerNormalization over the last axis whose readers are Dense layers and a self-attention layer is computed inside
+    those layers' GEMMs (row statistics gathered in the K loop, gamma / beta folded into the filters): against the oracle,
+    and against the same model with the LayerNormalization as a launch of its own.  With and without gamma / beta, with
+    rows whose mean is far from zero (40 standard deviations: the sums behind the statistics are taken relative to a
+    value of the row), two Dense readers of one LayerNormalization, a residual Add in the reader's epilogue, and a
+    LayerNormalization that also feeds a plain Add (not folded)."""
+    say("layernorm inside the gemm", center, scale, offset)
+    b = modelgen.Builder("lnf_%d%d_%d" % (center, scale, int(offset)), 81 + int(offset))
+    x = b.input((24, 64), "tokens")
+    n1 = b.layernorm_axes(x, "ln1", [-1], eps=1e-5, center=center, scale=scale)
+    att = b.mha(n1, n1, "att", heads=4, key_dim=16, bias_std=0.1)
+    x1 = b.add([x, att], "res1")
+    n2 = b.layernorm_axes(x1, "ln2", [-1], eps=1e-3, center=center, scale=scale)
+    f1 = b.dense(n2, 128, "fc1", activation="gelu", bias_std=0.1)
+    g1 = b.dense(n2, 64, "gate", bias_std=0.1)          # a second reader of ln2
+    f2 = b.dense(f1, 64, "fc2", bias_std=0.1)
+    x2 = b.add([x1, f2], "res2")
+    x3 = b.add([x2, g1], "res3")
+    n3 = b.layernorm_axes(x3, "ln3", [-1], eps=1e-5, center=center, scale=scale)
+    f3 = b.dense(n3, 96, "head", bias_std=0.1)
+    mixed = b.add([n3, x3], "not_folded")                # ln3 has a reader that is no GEMM: it keeps its own launch
+    spec = b.finish([f3, x3, mixed])
+    xs = (np.random.default_rng(82).standard_normal((5, 24, 64)) + offset).astype(np.float32)
+    fdx.check(fdx.lib.fdx_debug_force_ln_fold(1))
+    try:
+        got, want, model = run_both(fdx, oracle, modelgen, spec, [xs])
+        fdx.check(fdx.lib.fdx_profile_enable(1))
+        fdx.check(fdx.lib.fdx_profile_reset())
+        model.predict([xs])
+        fdx.sync()
+        families, i = set(), 0
+        while True:
+            name = fdx.ctypes.create_string_buffer(128)
+            n, ms, fl, by = fdx.ctypes.c_uint64(), fdx.ctypes.c_double(), fdx.ctypes.c_double(), fdx.ctypes.c_double()
+            if fdx.lib.fdx_profile_get(i, name, 128, fdx.ctypes.byref(n), fdx.ctypes.byref(ms), fdx.ctypes.byref(fl), fdx.ctypes.byref(by)) != 0:
+                break
+            families.add(name.value.decode())
+            i += 1
+        fdx.check(fdx.lib.fdx_profile_enable(0))
+        fdx.check(fdx.lib.fdx_debug_force_ln_fold(0))
+        plain = fdx.Model(modelgen.dumps(spec), verify=False).predict([xs])
+    finally:
+        fdx.check(fdx.lib.fdx_profile_enable(0))
+        fdx.check(fdx.lib.fdx_debug_force_ln_fold(-1))
+    assert "gemm_ln_f32" in families, families  # the folded form really ran
+    for a, c in zip(got, plain):
+        assert rel(a, c) <= TOL / 5
