@@ -1079,6 +1079,7 @@ namespace {
     }
 
     bool is_gemm_like(const Op& o) { return o.kind == OpKind::Conv2D || o.kind == OpKind::Dense; }
+    bool fold_ln_requested(); // fdx_debug_force_ln_fold(1) is in force
 
     fdx_status infer_shapes(const fdx_model& m, const std::vector<Shape>& in_shapes, std::vector<Shape>& shapes,
         const std::vector<int>& order);
@@ -1270,11 +1271,11 @@ namespace {
         // are uploaded; a plan may then normalise inside their GEMMs and skip the LayerNormalization launch.  The op itself
         // and the readers' own filters stay (a decode session folds them its own way, and sizes the GEMM kernel does not
         // cover run as before).
-        // (Readers are marked unless FDX_LN_FOLD=0; plans use the marks only on request, FDX_LN_FOLD=1 or the test hook: on the
-        // benched encoder -- 8192 rows of 512, 12 LayerNormalization launches of 11 us -- the statistics cost the two GEMMs
-        // that gather them 12 % of their time, 0.7 % more per step than the launches they save.)
-        static const bool ln_fold_env = [] { const char* e = std::getenv("FDX_LN_FOLD"); return !(e && e[0] == '0'); }();
-        for (size_t i = 0; i < m.ops.size() && have_shapes && ln_fold_env; ++i) {
+        // (Only on request, FDX_LN_FOLD=1 or the test hook set when the model is loaded: on the benched encoder -- 8192 rows of
+        // 512, 12 LayerNormalization launches of 11 us -- the statistics cost the two GEMMs that gather them 12 % of their
+        // time, 0.7 % more per step than the launches they save; and the folded copies take as much memory as the filters.)
+        static const bool ln_fold_env = [] { const char* e = std::getenv("FDX_LN_FOLD"); return e && e[0] == '1'; }();
+        for (size_t i = 0; i < m.ops.size() && have_shapes && (ln_fold_env || fold_ln_requested()); ++i) {
             Op& ln = m.ops[i];
             if (ln.dead || ln.kind != OpKind::LayerNorm || ln.rms || ln.act.kind != FDX_ACT_NONE || ln.in.size() != 1 || ln.target_shape.size() != 1)
                 continue;
@@ -1763,6 +1764,10 @@ extern "C" fdx_status fdx_debug_force_dw_fusion(int mode)
 // readers' GEMMs where those are Dense / self-attention layers of a size the kernel covers, -1 = as the environment says
 // (FDX_LN_FOLD=1: inside the GEMMs; otherwise launches of their own)
 static int g_force_ln_fold = -1;
+
+namespace {
+bool fold_ln_requested() { return g_force_ln_fold == 1; }
+}
 
 extern "C" fdx_status fdx_debug_force_ln_fold(int mode)
 {

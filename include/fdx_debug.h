@@ -64,7 +64,7 @@ fdx_status fdx_debug_dual_conv(int one_launch);
  * 65536 pixels; otherwise never: the launch measured no faster than the two it replaces), 0 = never, 1 = wherever the
  * kernel covers the pair */
 fdx_status fdx_debug_force_chain(int mode);
-/* plans built from now on: 1 = a LayerNormalization over the last axis whose only readers are Dense / self-attention layers
+/* models loaded and plans built from now on: 1 = a LayerNormalization over the last axis whose only readers are Dense / self-attention layers
  * is computed inside those layers' GEMMs (row statistics gathered in the K loop, gamma / beta folded into the filters at
  * load); 0 = every LayerNormalization runs as a launch of its own; -1 = as the environment says (FDX_LN_FOLD=1: inside the
  * GEMMs; the default is a launch of its own, which measured 0.7 % faster on the benched encoder) */
