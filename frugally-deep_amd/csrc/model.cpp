@@ -1080,6 +1080,7 @@ namespace {
 
     bool is_gemm_like(const Op& o) { return o.kind == OpKind::Conv2D || o.kind == OpKind::Dense; }
     bool fold_ln_requested(); // fdx_debug_force_ln_fold(1) is in force
+    bool chain_requested();   // fdx_debug_force_chain(1) is in force
 
     fdx_status infer_shapes(const fdx_model& m, const std::vector<Shape>& in_shapes, std::vector<Shape>& shapes,
         const std::vector<int>& order);
@@ -1324,10 +1325,10 @@ namespace {
         // its Add and ReLU in the epilogue, and the next block's first): marked as a pair that one launch can run, the
         // second convolution taking the first's result from LDS (conv1x1_chain_launch).  Whether a plan does so is decided
         // when the plan is made.
-        static const bool chain_env = [] { const char* e = std::getenv("FDX_CHAIN"); return !(e && e[0] == '0'); }();
-        // (FDX_CHAIN=0: no pair is marked and no packed filter kept; unset: pairs are marked so that the test hook can
-        // switch them on; FDX_CHAIN=1: plans with many pixels run them as one launch)
-        for (size_t i = 0; i < m.ops.size() && have_shapes && chain_env; ++i) {
+        static const bool chain_env = [] { const char* e = std::getenv("FDX_CHAIN"); return e && e[0] == '1'; }();
+        // (pairs are marked, and their packed filters kept, only on request: FDX_CHAIN=1, or the test hook set when the model
+        // is loaded)
+        for (size_t i = 0; i < m.ops.size() && have_shapes && (chain_env || chain_requested()); ++i) {
             Op& d = m.ops[i];
             auto gemm_1x1 = [](const Op& o) {
                 return !o.dead && o.kind == OpKind::Conv2D && o.kh == 1 && o.kw == 1 && o.sy == 1 && o.sx == 1 && o.dy == 1 && o.dx == 1
@@ -1779,6 +1780,10 @@ extern "C" fdx_status fdx_debug_force_ln_fold(int mode)
 // test hook: -1 = plans run a pair of 1x1 convolutions as one launch where the closed rule says so, 0 = never, 1 = wherever
 // the kernel covers the pair
 static int g_force_chain = -1;
+
+namespace {
+bool chain_requested() { return g_force_chain == 1; }
+}
 
 extern "C" fdx_status fdx_debug_force_chain(int mode)
 {

@@ -59,7 +59,7 @@ fdx_status fdx_debug_force_tile(int cfg);
  * its shortcut branch): 1 = one GEMM over both inputs' channels (the default), 0 = the two convolutions one after the
  * other, the second adding to the first's result -- the form taken by itself where the one-launch kernel does not apply */
 fdx_status fdx_debug_dual_conv(int one_launch);
-/* plans built from now on: a 1x1 convolution whose result feeds another 1x1 convolution (the tail of one residual block and
+/* models loaded and plans built from now on: a 1x1 convolution whose result feeds another 1x1 convolution (the tail of one residual block and
  * the head of the next) and that convolution as one launch: -1 = as the environment says (FDX_CHAIN=1: plans with at least
  * 65536 pixels; otherwise never: the launch measured no faster than the two it replaces), 0 = never, 1 = wherever the
  * kernel covers the pair */

@@ -31,7 +31,9 @@ def harness(fdx, tmp_path_factory):
 def run(exe, paths, tmp_path):
     lst = tmp_path / "list.txt"
     lst.write_text("\n".join(str(p) for p in paths) + "\n")
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1")
+    # (the two opt-in fusions are switched on so that their load-time passes -- filter packing, gamma / beta folding -- run too)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1",
+               FDX_CHAIN="1", FDX_LN_FOLD="1")
     out = subprocess.run([exe, str(lst)], capture_output=True, text=True, timeout=600, env=env)
     assert out.returncode == 0 and "loader_sanitize done: %d files" % len(paths) in out.stdout, (out.stdout[-2000:], out.stderr[-4000:])
     status = {}
