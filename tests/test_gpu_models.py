@@ -472,3 +472,30 @@ def test_layernorm_inside_the_readers_gemms(fdx, oracle, modelgen, center, scale
     assert "gemm_ln_f32" in families, families  # the folded form really ran
     for a, c in zip(got, plain):
         assert rel(a, c) <= TOL / 5
+
+
+def test_shortcut_convolution_on_variable_input_sizes(fdx, oracle, modelgen):
+    """The joined shortcut convolution (stride 2) under variable height and width: odd and even sizes, each with a plan of
+    its own; the strided rows of the second input follow the size of the call."""
+    say("shortcut convolution, variable sizes")
+    b = modelgen.Builder("sc_var", 91)
+    x = b.input((12, 12, 32), "img")
+    y = b.conv2d(x, 32, 1, "c1", strides=2, activation="relu", bias_std=0.1)
+    z = b.conv2d(y, 64, 1, "c3", bias_std=0.1)
+    sc = b.conv2d(x, 64, 1, "sc", strides=2, bias_std=0.1)
+    out = b.relu(b.add([sc, z], "sum"), "out")
+    spec = b.finish([out])
+    spec["input_shapes"] = [[None, None, 32]]
+    spec["output_shapes"] = [[None, None, 64]]
+    for layer in spec["architecture"]["config"]["layers"]:
+        if layer["class_name"] == "InputLayer":
+            layer["config"]["batch_shape"] = [None, None, None, 32]
+    js = modelgen.dumps(spec)
+    ref = oracle.OracleModel(js)
+    model = fdx.Model(js)
+    r = np.random.default_rng(92)
+    for i, size in enumerate([(12, 12), (7, 9), (15, 4), (1, 1), (8, 13)]):
+        xi = r.standard_normal((2 + i % 3,) + size + (32,)).astype(np.float32)
+        want = np.stack([ref.predict([xi[k]])[0] for k in range(xi.shape[0])])
+        got = model.predict([xi])[0]
+        assert got.shape == want.shape and rel(got, want) <= TOL, size
