@@ -783,6 +783,53 @@ __global__ __launch_bounds__(1024) void argmax_parts_kernel(const unsigned long 
         *len_dev += 1;
 }
 
+// The same, and the embedding of the tokens just picked at the position they will take, x0[r][:] = table_a[id_r][:] +
+// table_b[new length][:]: inside a greedy loop this is the first launch of the next step (embed_add_kernel) riding in the
+// last launch of this one.  Ids beyond table_a cannot occur (they are column numbers of the head); a position beyond
+// table_b leaves zeros and reports nothing: the loop's last step embeds for a step that may never come (the caller keeps
+// loops that would run past the table on the stand-alone launch).
+__global__ __launch_bounds__(1024) void argmax_parts_embed_kernel(const unsigned long long* __restrict__ parts, int n_parts, int rows,
+    float* __restrict__ out_idx_f, int* __restrict__ len_dev, float* __restrict__ history, const float* __restrict__ ta, int dim_a,
+    const float* __restrict__ tb, int dim_b, int depth, float* __restrict__ x0, int* __restrict__ err)
+{
+    __shared__ unsigned long long sm[64][16];
+    __shared__ int ids_s[16];
+    __shared__ int pos_s;
+    const int r = threadIdx.x & 15, lane_part = threadIdx.x >> 4; // 64 threads per row
+    unsigned long long best = 0ull;
+    for (int q = lane_part; q < n_parts; q += 64) {
+        const unsigned long long pk = parts[(int64_t)q * 16 + r];
+        best = pk > best ? pk : best;
+    }
+    sm[lane_part][r] = best;
+    __syncthreads();
+    if (threadIdx.x < 16 && r < rows) {
+        for (int q = 0; q < 64; ++q)
+            best = sm[q][r] > best ? sm[q][r] : best;
+        const unsigned int col = best == 0ull ? 0u : 0xFFFFFFFFu - (unsigned int)(best & 0xFFFFFFFFull);
+        const float id = (float)col;
+        out_idx_f[r] = id;
+        history[(int64_t)(*len_dev) * rows + r] = id;
+        ids_s[r] = (int)col;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int pos = *len_dev + 1;
+        *len_dev = pos;
+        pos_s = pos;
+    }
+    __syncthreads();
+    const int pos = pos_s, quads = depth / 4;
+    for (int idx = threadIdx.x; idx < rows * quads; idx += 1024) {
+        const int row = idx / quads, c4 = (idx - row * quads) * 4;
+        const int id = ids_s[row];
+        f32x4 v = { 0.f, 0.f, 0.f, 0.f };
+        if (id < dim_a && pos < dim_b)
+            v = *reinterpret_cast<const f32x4*>(ta + (int64_t)id * depth + c4) + *reinterpret_cast<const f32x4*>(tb + (int64_t)pos * depth + c4);
+        *reinterpret_cast<f32x4*>(x0 + (int64_t)row * depth + c4) = v;
+    }
+}
+
 // packed winners -> float ids; optionally advances the session length (every other kernel of the step
 // has finished by stream order)
 __global__ void argmax_finish_kernel(const unsigned long long* __restrict__ amax, int rows, float* __restrict__ out_idx_f,
@@ -863,6 +910,21 @@ fdx_status argmax_parts_launch(const unsigned long long* amax_parts, int parts, 
     profile_begin();
     hipLaunchKernelGGL(argmax_parts_kernel, dim3(1), dim3(1024), 0, stream(), amax_parts, parts, rows, out_idx_f, len_dev, history);
     profile_end("argmax_f32", 0.0, 8.0 * parts * 16);
+    FDX_LAUNCH_CHECK();
+    return FDX_OK;
+}
+
+fdx_status argmax_parts_embed_launch(const unsigned long long* amax_parts, int parts, int rows, float* out_idx_f, int* len_dev, float* history,
+    const float* ta, int dim_a, const float* tb, int dim_b, int depth, float* x0, int* err)
+{
+    FDX_REQUIRE(amax_parts && out_idx_f && len_dev && history && ta && tb && x0 && parts > 0 && rows > 0 && rows <= 16 && depth > 0
+            && depth % 4 == 0 && (reinterpret_cast<uintptr_t>(ta) & 15) == 0 && (reinterpret_cast<uintptr_t>(tb) & 15) == 0
+            && (reinterpret_cast<uintptr_t>(x0) & 15) == 0,
+        "argmax_embed: bad arguments");
+    profile_begin();
+    hipLaunchKernelGGL(argmax_parts_embed_kernel, dim3(1), dim3(1024), 0, stream(), amax_parts, parts, rows, out_idx_f, len_dev, history, ta,
+        dim_a, tb, dim_b, depth, x0, err);
+    profile_end("argmax_f32", 0.0, 8.0 * parts * 16 + 12.0 * rows * depth);
     FDX_LAUNCH_CHECK();
     return FDX_OK;
 }

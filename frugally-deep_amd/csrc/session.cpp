@@ -58,6 +58,7 @@ struct fdx_session {
     int amax_part_count = 0;
     float* history = nullptr;           // [max_len][batch] greedy ids by the position that produced them
     hipGraphExec_t step_graph = nullptr; // one decode step (ids_buf -> ids_buf) captured for replay
+    hipGraphExec_t step_graph_merged = nullptr; // the same without the embedding launch, its last launch embedding the picked ids
     float* splitk_ws = nullptr;         // per-head partial rows of the attention + projection launches
     int* splitk_tickets = nullptr;      // their tickets, one per sequence, zero between launches
     static constexpr int64_t kWsFloats = 1 << 20;
@@ -77,6 +78,8 @@ struct fdx_session {
             (void)hipFree(p);
         if (step_graph)
             (void)hipGraphExecDestroy(step_graph);
+        if (step_graph_merged)
+            (void)hipGraphExecDestroy(step_graph_merged);
     }
     void arena_reset()
     {
@@ -703,13 +706,24 @@ bool build_fast_plan(fdx_session* s)
     return set_int_launch(s->len_dev, 0) == FDX_OK;
 }
 
-// enqueues the fused launches of one decode step; ids_dev [batch] floats, greedy ids go to next_dev
-fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
+// whether a greedy loop can let the last launch of a step embed the picked tokens for the next one: the step opens with
+// the token + position embedding and ends in the per-workgroup maxima of the head
+bool glue_mergeable(const fdx_session* s)
+{
+    static const bool on = [] { const char* e = std::getenv("FDX_DECODE_MERGE_GLUE"); return !(e && e[0] == '0'); }();
+    return on && s->amax_part_count > 0 && !s->steps.empty() && s->steps[0].kind == fdx_session::Step::EmbedAdd && s->steps[0].depth % 4 == 0
+        && s->history;
+}
+
+// enqueues the fused launches of one decode step; ids_dev [batch] floats, greedy ids go to next_dev.  merged: the step's
+// embedding is already in place (the previous step's last launch, or the loop's prologue, put it there) and this step's
+// last launch embeds the ids it picks.
+fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev, bool merged = false)
 {
     fdx_model& m = *s->m;
     const int B = s->batch;
     fdx_status st = FDX_OK;
-    for (size_t si = 0; si < s->steps.size(); ++si) {
+    for (size_t si = merged ? 1 : 0; si < s->steps.size(); ++si) {
         const auto& step = s->steps[si];
         const Op& o = m.ops[step.op];
         const fdx_act act = to_c(o.act);
@@ -755,6 +769,11 @@ fdx_status launch_steps(fdx_session* s, const float* ids_dev, float* next_dev)
     }
     // greedy ids (first maximum wins); the same launch records them by position and advances the cached
     // length on the device
+    if (merged) {
+        const auto& e = s->steps[0];
+        return argmax_parts_embed_launch(s->amax_parts, s->amax_part_count, B, next_dev, s->len_dev, s->history, e.a, e.g.M, e.b, e.g.N, e.depth,
+            e.out, m.err_flag);
+    }
     if (s->amax_part_count > 0)
         return argmax_parts_launch(s->amax_parts, s->amax_part_count, B, next_dev, s->len_dev, s->history);
     return argmax_bump_launch(s->logits_buf, B, s->vocab, next_dev, s->len_dev, s->amax, s->history);
@@ -787,10 +806,22 @@ fdx_status run_fast_greedy(fdx_session* s, const float* first_ids_dev, int steps
     const int B = s->batch;
     hipStream_t st = stream();
     FDX_HIP(hipMemcpyAsync(s->ids_buf, first_ids_dev, sizeof(float) * B, hipMemcpyDeviceToDevice, st));
-    if (!s->step_graph) {
+    // Where the step opens with the embedding launch and ends in the head's maxima, the replayed graph leaves the embedding
+    // out: the loop's first one runs here, every later one rides in the last launch of the step before (63 -> 62 launches
+    // per step on the GPT-2 shape).
+    // (not where the loop would run past the position table: those steps keep the stand-alone embedding launch)
+    const bool merged = glue_mergeable(s) && s->len + steps <= s->steps[0].g.N;
+    if (merged) {
+        const auto& e = s->steps[0];
+        const fdx_status es = embed_add_launch(s->ids_buf, B, e.a, e.g.M, e.b, e.g.N, s->len_dev, e.depth, e.out, m.err_flag, s->amax);
+        if (es != FDX_OK)
+            return es;
+    }
+    hipGraphExec_t& step_graph = merged ? s->step_graph_merged : s->step_graph;
+    if (!step_graph) {
         hipGraph_t graph = nullptr;
         FDX_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-        const fdx_status ls = launch_steps(s, s->ids_buf, s->ids_buf);
+        const fdx_status ls = launch_steps(s, s->ids_buf, s->ids_buf, merged);
         const hipError_t ce = hipStreamEndCapture(st, &graph);
         if (ls != FDX_OK) {
             if (graph)
@@ -798,13 +829,13 @@ fdx_status run_fast_greedy(fdx_session* s, const float* first_ids_dev, int steps
             return ls;
         }
         FDX_HIP(ce);
-        const hipError_t ie = hipGraphInstantiate(&s->step_graph, graph, nullptr, nullptr, 0);
+        const hipError_t ie = hipGraphInstantiate(&step_graph, graph, nullptr, nullptr, 0);
         (void)hipGraphDestroy(graph);
         FDX_HIP(ie);
     }
     const int start = s->len;
     for (int i = 0; i < steps; ++i)
-        FDX_HIP(hipGraphLaunch(s->step_graph, st));
+        FDX_HIP(hipGraphLaunch(step_graph, st));
     s->len += steps;
     FDX_HIP(hipMemcpyAsync(tokens_dev, s->history + (size_t)start * B, sizeof(float) * (size_t)steps * B, hipMemcpyDeviceToDevice, st));
     if (last_logits_dev)

@@ -65,6 +65,9 @@ fdx_status skinny_gemm_launch(const SkinnyParams& p);
 int skinny_wide_grid(const SkinnyParams& p);
 // greedy ids from per-workgroup partial maxima [parts][16] (first maximum wins), then as argmax_bump_launch
 fdx_status argmax_parts_launch(const unsigned long long* amax_parts, int parts, int rows, float* out_idx_f, int* len_dev, float* history);
+// ... and the token + position embedding of the picked ids at the position they take, into x0 (the next step's first launch)
+fdx_status argmax_parts_embed_launch(const unsigned long long* amax_parts, int parts, int rows, float* out_idx_f, int* len_dev, float* history,
+    const float* ta, int dim_a, const float* tb, int dim_b, int depth, float* x0, int* err);
 fdx_status skinny_prepare();
 int64_t packed_weight_floats(int n, int k);
 fdx_status pack_weights_launch(const float* w, int n, int k, int64_t ldw, float* out);

@@ -234,3 +234,38 @@ def test_embedding_folded_into_its_readers_gives_the_same_tokens(fdx, modelgen):
         sess.close()
     for a, b in zip(outs[0], outs[1]):
         assert np.array_equal(a, b)
+
+
+def test_greedy_loop_with_the_embedding_in_the_previous_steps_last_launch(fdx, modelgen):
+    """Inside a greedy loop over a vocabulary-sized head the token + position embedding of a step rides in the last launch
+    of the step before (the loop's first embedding runs ahead of the replays).  The loop, called twice with a single
+    step in between, must give the tokens of single steps; a loop that would run past the position table keeps the
+    stand-alone embedding launch."""
+    say("greedy loop, embedding merged into the arg-max launch")
+    cfg = dict(layers=2, d_model=64, heads=2, vocab=40009, max_pos=24)
+    js = modelgen.dumps(modelgen.gpt2(seed=63, bias_std=0.1, random_affine=True, std=0.2, **cfg))
+    model = fdx.Model(js)
+    B = 6
+    prompts = np.random.default_rng(64).integers(0, cfg["vocab"], (B, 5))
+    loop = fdx.Session(model, B, 32)
+    _, first = loop.prefill(prompts)
+    part1, _ = loop.decode_greedy(first, 6)            # positions 5 .. 10
+    _, mid = loop.decode_step(part1[-1])               # a single step between two loops (position 11)
+    part2, last_logits = loop.decode_greedy(mid, 7)    # positions 12 .. 18
+    single = fdx.Session(model, B, 32)
+    _, cur = single.prefill(prompts)
+    want = []
+    for i in range(6 + 1 + 7):
+        logits, cur_next = single.decode_step(cur)
+        want.append(cur_next)
+        cur = cur_next
+    got = list(part1) + [mid] + list(part2)
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert np.array_equal(g, w), i
+    assert rel(logits, last_logits) <= 1e-6
+    # positions 19 .. 23 exist, 24 does not: a loop of 6 from here runs past the table and takes the stand-alone embedding
+    # launches, like the single steps (a position without a row contributes zeros in both)
+    part3, _ = loop.decode_greedy(part2[-1], 6)
+    for i in range(6):
+        _, cur = single.decode_step(cur)
+        assert np.array_equal(part3[i], cur), i
