@@ -57,11 +57,6 @@ struct WinoParams {
 constexpr int WINO_TM = 32;  // tiles per workgroup
 constexpr int WINO_PAD = 4;  // padding of an LDS row of the exchange
 
-// register sets of step operands: a set is loaded WINO_SETS - 1 steps before its use.  One step ahead is enough (a step is
-// 32 MFMAs, 0.9 us at the least, and the operands come from L2 or the memory-side cache): a third set, two steps ahead,
-// measured 2-3 % slower on the ResNet50 layers, and the kernel without any operand loads only 25 % faster than with them
-constexpr int WINO_SETS = 2;
-
 // one step's operands: the eight patch pixels of this lane's tile and the 4 x NT filter pieces of its positions
 template <int NT>
 __device__ __forceinline__ void wino_load(f32x4 (&dd)[2][4], f32x4 (&bb)[4][NT], const uint32_t (&pix_off)[2][4],
@@ -79,64 +74,59 @@ __device__ __forceinline__ void wino_load(f32x4 (&dd)[2][4], f32x4 (&bb)[4][NT],
             bb[nu][nt] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], step * 16384, 0));
 }
 
-// The first WINO_SETS - 1 steps of a stretch of steps, requested ahead of wino_steps (for the first unit of a
-// workgroup at its start, for every later one before the previous unit's results are exchanged and stored, so that
-// they travel meanwhile).  Every load here and below is unconditional -- a step beyond the range is clamped to the last
-// one and its data never used: with loads behind branches the compiler has to assume the fewest outstanding ones at
-// every wait, which shortens the distance between a load and its use to nothing.
-template <int NT>
-__device__ __forceinline__ void wino_request(f32x4 (&d)[WINO_SETS][2][4], f32x4 (&b)[WINO_SETS][4][NT], const uint32_t (&pix_off)[2][4],
-    const uint32_t (&u_off)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u, int step_begin, int step_end)
+// One step: 8 input channels into the 4 x NT accumulators of this wave.  There is one register set of operands, and
+// with AHEAD each register is asked for its next step's value as soon as this step has read it -- the patch pixels right
+// after the input transform, the filter pieces of a position right after its MFMAs -- so that every load has a whole
+// step to arrive in while the registers of a second set stay free: at 128 accumulators + 64 operand registers two
+// workgroups fit on a CU, and the end of one's unit (exchange, barriers, stores) runs under the other's MFMAs.
+// NT = 32-column tiles of the output channels per workgroup, XI = this wave's row of the transform domain.
+template <int NT, int XI, bool AHEAD>
+__device__ __forceinline__ void wino_step(f32x4 (&d)[2][4], f32x4 (&b)[4][NT], const uint32_t (&pix_off)[2][4],
+    const uint32_t (&u_off)[4][NT], f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u,
+    int next)
 {
-    const int last = step_end - 1;
+    // row XI of Bt over the patch rows, then Bt again over the columns
+    f32x4 t[4], v[4];
 #pragma unroll
-    for (int s0 = 0; s0 < WINO_SETS - 1; ++s0)
-        wino_load<NT>(d[s0], b[s0], pix_off, u_off, srd_in, srd_u, step_begin + s0 < last ? step_begin + s0 : last);
+    for (int j = 0; j < 4; ++j)
+        t[j] = XI == 1 ? d[0][j] + d[1][j] : (XI == 2 ? d[1][j] - d[0][j] : d[0][j] - d[1][j]);
+    v[0] = t[0] - t[2];
+    v[1] = t[1] + t[2];
+    v[2] = t[2] - t[1];
+    v[3] = t[1] - t[3];
+    __builtin_amdgcn_sched_barrier(0);
+    if (AHEAD) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                d[r][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_in, (int)pix_off[r][j], next * 32, 0));
+    }
+#pragma unroll
+    for (int nu = 0; nu < 4; ++nu) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], b[nu][nt][e], acc[nu][nt], 0, 0, 0);
+        if (AHEAD) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                b[nu][nt] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(srd_u, (int)u_off[nu][nt], next * 16384, 0));
+        }
+        __builtin_amdgcn_sched_barrier(0); // (the scheduler would gather the loads at the end of the step, right before their use)
+    }
 }
 
-// NT = 32-column tiles of the output channels per workgroup, XI = this wave's row of the transform domain.  The loop
-// is unrolled over the register sets, so that nothing is ever copied from one set to another.
+// steps [step_begin, step_end) of a unit; the operands of step_begin have been requested (wino_load)
 template <int NT, int XI>
-__device__ __forceinline__ void wino_steps(f32x4 (&d)[WINO_SETS][2][4], f32x4 (&b)[WINO_SETS][4][NT], const uint32_t (&pix_off)[2][4],
+__device__ __forceinline__ void wino_steps(f32x4 (&d)[2][4], f32x4 (&b)[4][NT], const uint32_t (&pix_off)[2][4],
     const uint32_t (&u_off)[4][NT], f32x16 (&acc)[4][NT], const __amdgpu_buffer_rsrc_t& srd_in, const __amdgpu_buffer_rsrc_t& srd_u,
     int step_begin, int step_end)
 {
-    constexpr int SETS = WINO_SETS;
-    const int steps = step_end - step_begin, last = step_end - 1;
-    auto multiply = [&](const f32x4 (&dd)[2][4], const f32x4 (&bb)[4][NT]) {
-        // row XI of Bt over the patch rows, then Bt again over the columns
-        f32x4 t[4], v[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            t[j] = XI == 1 ? dd[0][j] + dd[1][j] : (XI == 2 ? dd[1][j] - dd[0][j] : dd[0][j] - dd[1][j]);
-        v[0] = t[0] - t[2];
-        v[1] = t[1] + t[2];
-        v[2] = t[2] - t[1];
-        v[3] = t[1] - t[3];
-#pragma unroll
-        for (int nu = 0; nu < 4; ++nu)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    acc[nu][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[nu][e], bb[nu][nt][e], acc[nu][nt], 0, 0, 0);
-    };
-    const int rounds = steps / SETS;
-    for (int r = 0; r < rounds; ++r) {
-#pragma unroll
-        for (int u = 0; u < SETS; ++u) {
-            const int ahead = step_begin + r * SETS + u + SETS - 1;
-            wino_load<NT>(d[(u + SETS - 1) % SETS], b[(u + SETS - 1) % SETS], pix_off, u_off, srd_in, srd_u, ahead < last ? ahead : last);
-            __builtin_amdgcn_sched_barrier(0); // the loads stay in front of the step they overlap with (the scheduler
-            multiply(d[u], b[u]);              // would gather them at the end of the loop body, right before their use)
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    const int rest = steps - rounds * SETS; // at most SETS - 1 steps, already loaded
-#pragma unroll
-    for (int u = 0; u < SETS - 1; ++u)
-        if (u < rest)
-            multiply(d[u], b[u]);
+    for (int s = step_begin; s < step_end - 1; ++s)
+        wino_step<NT, XI, true>(d, b, pix_off, u_off, acc, srd_in, srd_u, s + 1);
+    wino_step<NT, XI, false>(d, b, pix_off, u_off, acc, srd_in, srd_u, 0);
 }
 
 // Persistent workgroups, balanced over the chip: the units of work (32 tiles x NT * 32 channels, cin / 8 steps each)
@@ -148,7 +138,7 @@ __device__ __forceinline__ void wino_steps(f32x4 (&d)[WINO_SETS][2][4], f32x4 (&
 // then bias, residual and activation.  Nobody waits for anybody.  Without this a launch lasts a whole number of
 // units per CU: 392 units on 256 CUs take the time of 512.
 template <int NT>
-__global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
+__global__ __launch_bounds__(256, 2) void wino_kernel(WinoParams p)
 {
     constexpr int NC = NT * 32, LS = NC + WINO_PAD;
     constexpr int LANES_PER_TILE = NC / 4, TILES_PER_PASS = 64 / LANES_PER_TILE, PASSES = WINO_TM / TILES_PER_PASS;
@@ -226,14 +216,14 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
         v.desc0 = tile_ok ? (int)((uint32_t)(((img * p.oh + 2 * ty) * p.ow + 2 * tx) * p.cout) * 4u) : (int)OOB;
         v.desc1 = (2 * ty + 1 < p.oh ? 1 : 0) | (2 * tx + 1 < p.ow ? 2 : 0);
     };
-    f32x4 d[WINO_SETS][2][4], b[WINO_SETS][4][NT];
+    f32x4 d[2][4], b[4][NT];
     UnitView cur;
     int pos = stretch_begin(g);
     int unit = pos / spu; // (the only division by the step count: from here on units are counted up)
     if (pos < end) {
         const int unit_begin = unit * spu;
         view_of(true, unit, cur);
-        wino_request<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, pos - unit_begin, end - unit_begin < spu ? end - unit_begin : spu);
+        wino_load<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, pos - unit_begin);
     }
     while (pos < end) {
         const int unit_begin = unit * spu;
@@ -263,7 +253,7 @@ __global__ __launch_bounds__(256) void wino_kernel(WinoParams p)
         {
             const bool live = next_pos < end;
             view_of(live, unit + 1, cur);
-            wino_request<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, 0, !live || end - next_pos >= spu ? spu : end - next_pos);
+            wino_load<NT>(d, b, cur.pix_off, cur.u_off, srd_in, srd_u, 0);
         }
 
         // At along the row: z0 = m0 + m1 + m2, z1 = m1 - m2 - m3.  Element e of a lane is tile 8 * (e / 4) + 4 * fh +
@@ -370,7 +360,7 @@ static bool wino_prepare()
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount < 1)
         return false;
-    g_wino_grid = prop.multiProcessorCount;
+    g_wino_grid = 2 * prop.multiProcessorCount; // at most two workgroups per CU
     if (!g_wino_ws && hipMalloc(&g_wino_ws, 2 * kWinoShareBytes * (size_t)g_wino_grid) != hipSuccess)
         return false;
     if (!g_wino_tickets
@@ -458,8 +448,9 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     p.act = make_act(act);
     FDX_REQUIRE(wino_prepare(), "conv2d_winograd: no device memory for the workspace");
     const int m_blocks = (p.tiles + WINO_TM - 1) / WINO_TM;
-    // (128-channel units -- NT = 4 -- were measured: the second register set of operands no longer fits beside 256
-    // accumulators, and with one set the loads are not hidden: slower than 64-channel units on every ResNet50 shape)
+    // (128-channel units -- NT = 4, 256 accumulators, one workgroup per CU -- were measured: half the patch loads per
+    // MFMA, but 14x14 256 -> 256 takes 110 us instead of 87: half as many units, so every one is cut by a stretch
+    // boundary, and the exchange at a unit's end is twice as long with nothing beside it on the SIMD)
     constexpr int nt = 2;
     p.m_blocks = m_blocks;
     p.n_blocks = cout / (nt * 32);
@@ -487,7 +478,13 @@ extern "C" fdx_status fdx_conv2d_winograd_nhwc_f32(const float* in, int n, int h
     const int64_t total_steps = (int64_t)p.units * (cin / 8);
     FDX_WINO_LIMIT(total_steps < (1LL << 30), "conv2d_winograd: too many steps for one launch");
     const int64_t by_steps = total_steps / 4 > 0 ? total_steps / 4 : 1;
-    const dim3 grid((unsigned)(by_steps < g_wino_grid ? by_steps : g_wino_grid));
+    // Two workgroups fit on a CU.  The second one pays where units are short (64 input channels: 8 steps per unit, -9 %;
+    // 128: -3 %): the end of one's unit runs under the other's steps.  Units of 32 and 64 steps gain nothing there and
+    // lose 2-8 % to the shares of the units that twice as many stretches cut: one workgroup per CU for them.  (The
+    // steps themselves do not get faster with a second wave on the SIMD: their loads -- 16 per 32 MFMAs, the patch
+    // pieces 32 lines per instruction -- keep the CU's vector memory path as busy as the MFMAs keep the matrix pipe.)
+    const int resident = cin <= 128 ? g_wino_grid : g_wino_grid / 2;
+    const dim3 grid((unsigned)(by_steps < resident ? by_steps : resident));
     p.per_wg = (int)(total_steps / grid.x);
     p.longer = (int)(total_steps % grid.x);
     const size_t lds = wino_lds_bytes(nt);
