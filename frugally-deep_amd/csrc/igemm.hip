@@ -736,7 +736,7 @@ static fdx_status run_igemm(GemmParams& p, bool conv, int batch, const char* fam
         a_bytes = ((int64_t)(p.M - 1) * p.lda + (p.a_valid_k > 0 ? p.a_valid_k : p.K)) * 4;
         a_ok = a_mode == A_ROWS_VEC && p.K % 16 == 0;
     }
-    const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31);
+    const bool fast_ok = out_ok && a_ok && b_vec && a_bytes < (1LL << 31) && b_bytes < (1LL << 31) && p.ldc < (1LL << 24);
     const int unit = conv ? p.Cin : p.K;
 
     int cfg = g_forced_tile, splits = 1, mode = 0;

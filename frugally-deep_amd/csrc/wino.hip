@@ -292,7 +292,8 @@ __global__ __launch_bounds__(256, 2) void wino_kernel(WinoParams p)
             float v[4] = { y[0], y[1], y[2], y[3] };
             apply_act_block(v, p.act);
             const f32x4 r = { v[0], v[1], v[2], v[3] };
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), srd_out, (int)off, 0, 0);
+            // (agent scope: written through to memory instead of left dirty in this XCD's L2 until the kernel ends)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), srd_out, (int)off, 0, kAgentScope);
         };
         if (s0 == 0 && s1 == spu) {
 #pragma unroll 4
