@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file and scaled by a plain copy of known size (a process cannot read these counters for itself; the
 # summaries under profiles/ give the commands and the raw readings).  Valid for the default configurations only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm + wino, ResNet50 b64": 163.4e6, "skinny_gemm, GPT-2 decode b16": 11.3e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"igemm + wino, ResNet50 b64": 163.5e6, "skinny_gemm, GPT-2 decode b16": 11.3e6}
 
 
 def under_profiler():
