@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256) void dwpw_kernel(DwPwParams p)
             apply_act_block(v, p.act2);
 #pragma unroll
             for (int z = 0; z < 16; ++z)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[z]), srd_out, (int)off[z], 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[z]), srd_out, (int)off[z], 0, 16); // agent scope: written through to memory, nothing left dirty in L2 at the kernel's end
         }
     }
 }

@@ -381,7 +381,7 @@ __global__ __launch_bounds__(NW * 64) void irb_kernel(IrbParams p)
             irb_act(v, p.act_out, clamp_out);
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[e]), srd_out, (int)off[e], 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[e]), srd_out, (int)off[e], 0, 16); // agent scope: written through to memory, nothing left dirty in L2 at the kernel's end
         }
     }
 }

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void pw_stream_kernel(PwStreamParams q)
             apply_act_block(v, p.act);
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[e]), srd_c, (int)off[e], 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[e]), srd_c, (int)off[e], 0, 16); // agent scope: written through to memory, nothing left dirty in L2 at the kernel's end
         }
     }
 }
