@@ -2904,7 +2904,7 @@ namespace {
     // device op, so what has to hold is about buffers: pieces run piece-major, so an op of piece c + 1 must not write where
     // a result of piece c still waits for a reader behind the prefix.  Buffers are recycled by liveness, hence every prefix
     // op whose result is read behind the prefix has to own its block alone among the prefix ops.  The prefix is grown
-    // until it holds about as much arithmetic as the copy takes time (a sixth of the model's), and cut back until that holds.
+    // until it holds about as much arithmetic as the copy takes time, and cut back until that holds.
     int chunkable_prefix(const fdx_model& m, const Plan& p, int batch)
     {
         if (m.inputs.size() != 1)
@@ -2916,6 +2916,12 @@ namespace {
         // longest run of ops that can take a range of samples: device ops outside any fused block, every choice already made
         int longest = 0;
         double flops = 0, total = p.flops > 0 ? p.flops : 1;
+        // what the pieces behind the first need to travel (55 GB/s over the link) at the rate piece-sized launches compute
+        // at (75 TFLOP/s), and no more than a quarter of the model: ResNet50 b64 from host memory, prefix of 12 / 11 / 8 /
+        // 7 / 6 / 5 / 2 ops: 12.9 / 13.1-13.3 / 13.6 / 13.65 / 13.55 / 13.3 / 12.85 k img/s -- a longer prefix runs more
+        // of the model at a quarter of the batch than the copy can hide, a shorter one leaves the copy uncovered
+        const double in_bytes = 4.0 * (double)batch * (double)volume(p.shapes[(size_t)m.inputs[0]]);
+        const double enough = std::min(total / 4, in_bytes / 55e9 * 75e12);
         int wanted = -1;
         for (int pos = 0; pos < n_pos; ++pos) {
             const int idx = p.order[(size_t)pos];
@@ -2935,7 +2941,7 @@ namespace {
                 break;
             longest = pos + 1;
             flops += op_flops(o, p.shapes[(size_t)idx], p.shapes, batch);
-            if (wanted < 0 && flops >= total / 6)
+            if (wanted < 0 && flops >= enough)
                 wanted = pos + 1;
         }
         // a later op that absorbs a prefix op (blocks fused into one launch) keeps that op out of the prefix
