@@ -302,23 +302,42 @@ __global__ __launch_bounds__(256, 2) void wino_kernel(WinoParams p)
         } else {
             const uint32_t lane_off = (uint32_t)((xi * PASSES) * 64 + lane) * 16u;
             const uint32_t mine = share_off(g, unit) + lane_off;
-#pragma unroll 4
-            for (int pass = 0; pass < PASSES; ++pass)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, combine(pass)), srd_ws, (int)(mine + (uint32_t)pass * 1024u), 0,
-                    kAgentScope);
-            // every lane's share has left the CU before the ticket is taken
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
             const int g_a = owner_of(unit_begin), parts = owner_of(unit_begin + spu - 1) - g_a + 1;
-            if (t == 0) {
-                const int ticket = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const int last = ticket == parts - 1;
-                if (last)
-                    __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // for the next launch
-                last_flag = last;
+            // A stretch that ends inside this unit comes to it at the very end of its life; the stretches that hold the
+            // unit's later steps began with them and handed their shares in long ago.  One look at the ticket then shows
+            // everybody else in -- each took its ticket after its share had left its CU -- and this workgroup, certainly
+            // the last, neither stores a share of its own nor draws a ticket: two trips to memory fewer at the one place
+            // where nothing else is left to run beside them.
+            bool finish_here = false;
+            if (s1 < spu) {
+                if (t == 0)
+                    last_flag = __hip_atomic_load(p.tickets + unit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == parts - 1;
+                __syncthreads();
+                finish_here = last_flag != 0;
+                __syncthreads(); // last_flag is written again below
             }
-            __syncthreads();
-            if (last_flag != 0) {
+            if (finish_here) {
+                if (t == 0)
+                    __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // for the next launch
+            } else {
+#pragma unroll 4
+                for (int pass = 0; pass < PASSES; ++pass)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, combine(pass)), srd_ws, (int)(mine + (uint32_t)pass * 1024u),
+                        0, kAgentScope);
+                // every lane's share has left the CU before the ticket is taken
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (t == 0) {
+                    const int ticket = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const int last = ticket == parts - 1;
+                    if (last)
+                        __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // for the next launch
+                    last_flag = last;
+                }
+                __syncthreads();
+                finish_here = last_flag != 0;
+            }
+            if (finish_here) {
                 // shares are added in stretch order whoever came last; this workgroup's own one is formed again from the
                 // exchange area (the same operations on the same values, so the same bits) instead of read back
                 const int my_part = g - g_a;
